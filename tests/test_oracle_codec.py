@@ -1,0 +1,159 @@
+"""Pins the oracle's codec functions (e2m1 / e8m0 / e4m3) against the
+reference's golden vectors and against closed forms."""
+import json
+import os
+
+import numpy as np
+
+import oracle
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0], np.float64)
+
+
+def np_dequant(packed, scales, rows, cols):
+    """Independent closed form: LUT[nibble] * 2^(byte-127), low nibble = even column (ref/mxfp4_numpy.py:16-27)."""
+    packed = np.asarray(packed, np.uint8).reshape(rows, cols // 2)
+    idx = np.empty((rows, cols), np.uint8)
+    idx[:, 0::2] = packed & 0x0F
+    idx[:, 1::2] = packed >> 4
+    sc = np.exp2(np.asarray(scales, np.float64).reshape(rows, cols // 32) - 127.0)
+    return (E2M1[idx] * np.repeat(sc, 32, axis=1)).astype(np.float32)
+
+
+def test_fp4_golden_vector_bit_exact():
+    # src/selftest.rs:226-234 consumes the same vector (torch-generated)
+    g = json.load(open(os.path.join(G, "ds_golden_fp4.json")))
+    w = oracle.mxfp4_dequant(g["packed"], g["scales"], g["rows"], g["cols"])
+    want = np.asarray(g["dequant"], np.float64).astype(np.float32).reshape(g["rows"], g["cols"])
+    assert np.array_equal(np.abs(w).view(np.uint32), np.abs(want).view(np.uint32))  # the JSON renders -0.0 as "-0.0" or "0.0"
+    assert np.array_equal(w, want)
+
+
+def test_dequant_exhaustive_nibble_x_scale():
+    # all 16 nibbles x all 256 scale bytes; byte 0 is the subnormal 2^-127
+    for sb in range(256):
+        packed = np.array([n | (n << 4) for n in range(16)], np.uint8)
+        row = np.zeros(16, np.uint8)
+        row[:16] = packed
+        w = oracle.mxfp4_dequant(row, [sb], 1, 32)[0]
+        want = np_dequant(row, [min(sb, 254)], 1, 32)[0]
+        if sb == 255:  # 2^128 overflows f32: exp2_i builds the bit pattern of +inf
+            assert np.isinf(oracle.exp2_i(128))
+            continue
+        assert np.array_equal(w.view(np.uint32), want.view(np.uint32)), sb
+    assert np.float32(oracle.exp2_i(-127)).view(np.uint32) == 0x00400000
+    assert np.float32(oracle.scale_from_byte(0)).view(np.uint32) == 0x00400000
+    for sb in range(1, 255):
+        assert oracle.scale_from_byte(sb) == oracle.exp2_i(sb - 127) == 2.0 ** (sb - 127)
+    # nibble 8 is negative zero: the sign bit survives the scale
+    w = oracle.mxfp4_dequant(np.full(16, 0x88, np.uint8), [127], 1, 32)
+    assert np.all(w.view(np.uint32) == 0x80000000)
+
+
+def test_e4m3_decode_closed_form_and_roundtrip():
+    for b in range(256):
+        v = oracle.e4m3_to_f32(b)
+        s, e, m = b >> 7, (b >> 3) & 15, b & 7
+        if e == 15 and m == 7:
+            assert np.isnan(v)
+            continue
+        want = (-1.0) ** s * ((m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7))
+        assert v == want, b
+        # encode(decode(b)) == b for every finite code (negative zero keeps its sign)
+        assert oracle.f32_to_e4m3(v) == b, b
+    assert oracle.f32_to_e4m3(1e9) == 0x7E and oracle.f32_to_e4m3(-1e9) == 0xFE
+    assert oracle.f32_to_e4m3(float("nan")) == 0x7F
+    # ties to even mantissa: 1 + 1/16 is halfway between m=0 and m=1 -> m=0; 1 + 3/16 -> m=2
+    assert oracle.f32_to_e4m3(1.0625) == 0x38 and oracle.f32_to_e4m3(1.1875) == 0x3A
+    # subnormal carry into the smallest normal
+    assert oracle.f32_to_e4m3(2.0 ** -6 * (7.6 / 8)) == 0x08
+
+
+def test_fp8_golden_vector_byte_exact():
+    # src/selftest.rs:204-225: dequant matches torch, quantize reproduces torch's bytes with zero diffs
+    g = np.load(os.path.join(G, "ds_golden_fp8.npz"))
+    rows, cols = int(g["rows"]), int(g["cols"])
+    w = oracle.dequant_fp8(g["w_packed"], g["scales"], rows, cols)
+    assert np.array_equal(w.reshape(-1), g["dequant"])
+    qw, qs = oracle.quantize_fp8(g["w_orig"], rows, cols)
+    assert np.array_equal(qw.reshape(-1), g["w_packed"])
+    assert np.array_equal(qs.reshape(-1), g["scales"])
+
+
+def test_fp8_roundtrip_block32():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(256) * 3).astype(np.float32)
+    y, codes, exps = oracle.fp8_roundtrip(x, 32)
+    for b in range(8):
+        blk = x[b * 32:(b + 1) * 32]
+        e = int(np.ceil(np.log2(max(np.abs(blk).max(), 1e-4) / 448.0)))
+        assert exps[b] == e + 127
+        dec = np.array([oracle.e4m3_to_f32(int(c)) for c in codes[b * 32:(b + 1) * 32]], np.float32) * np.float32(2.0 ** e)
+        assert np.array_equal(dec, y[b * 32:(b + 1) * 32])
+        assert np.abs(y[b * 32:(b + 1) * 32] - blk).max() <= np.abs(blk).max() * 2.0 ** -4 + 1e-6
+
+
+def _block_errors(w, rows, cols, p, s):
+    wq = oracle.mxfp4_dequant(p, s, rows, cols).astype(np.float64).reshape(-1, 32)
+    return ((w.astype(np.float64).reshape(-1, 32) - wq) ** 2).sum(axis=1)
+
+
+def _never_worse(w, rows, cols):
+    p0, s0 = oracle.mxfp4_quantize(w, rows, cols, search=False)
+    p1, s1 = oracle.mxfp4_quantize(w, rows, cols, search=True)
+    e0, e1 = _block_errors(w, rows, cols, p0, s0), _block_errors(w, rows, cols, p1, s1)
+    assert np.all(e1 <= e0 * (1 + 1e-9) + 1e-20)
+
+
+def test_quantize_search_never_worse():
+    # src/mxfp4.rs:575-598 restated
+    for rows, cols in [(64, 128), (128, 64), (3, 64), (1, 32), (256, 1024)]:
+        _never_worse(oracle.pattern(0, rows * cols), rows, cols)
+    rows, cols = 16, 64
+    w = np.full(rows * cols, 0.01, np.float32)
+    for g in range(rows * cols // 32):
+        w[g * 32] = 3.7 if g % 2 == 0 else -5.9
+    _never_worse(w, rows, cols)
+    _never_worse(np.zeros(64, np.float32), 2, 32)
+    _never_worse((E2M1[np.arange(64) % 16] * 0.125).astype(np.float32), 2, 32)
+
+
+def test_quantize_roundtrip_exact_levels_and_zero_group():
+    # src/mxfp4.rs:600-611
+    rows, cols = 4, 64
+    w = (E2M1[np.arange(rows * cols) % 16] * 0.25).astype(np.float32)
+    p, s = oracle.mxfp4_quantize(w, rows, cols)
+    assert np.array_equal(oracle.mxfp4_dequant(p, s, rows, cols).reshape(-1), w)
+    # an all-zero group gets scale byte 0 (src/metal.rs:1332) and zero nibbles
+    p, s = oracle.mxfp4_quantize(np.zeros(64, np.float32), 2, 32)
+    assert np.all(s == 0) and np.all(p == 0)
+    # quantize(dequant(.)) is the identity on grids that use the top level (naive scale is then exact)
+    rng = np.random.default_rng(1)
+    packed = rng.integers(0, 256, (8, 32), dtype=np.uint8)
+    packed[:, 0] = 0x77
+    scales = rng.integers(110, 140, (8, 2), dtype=np.uint8)
+    w = oracle.mxfp4_dequant(packed, scales, 8, 64)
+    p2, s2 = oracle.mxfp4_quantize(w, 8, 64, search=False)
+    assert np.array_equal(s2, scales)
+    assert np.array_equal(oracle.mxfp4_dequant(p2, s2, 8, 64), w)
+
+
+def test_naive_scale_rule_matches_numpy_restatement():
+    # nano/export.py:23-41 states the same rule in numpy: e = ceil(log2(maxabs/6)), nearest level
+    rng = np.random.default_rng(7)
+    w = (rng.standard_normal((16, 64)) * 2).astype(np.float32)
+    p, s = oracle.mxfp4_quantize(w, 16, 64, search=False)
+    grp = w.reshape(16, 2, 32)
+    e = np.ceil(np.log2(np.abs(grp).max(axis=2) / np.float32(6.0))).astype(np.int32)
+    assert np.array_equal(s.astype(np.int32) - 127, e)
+    q = np.clip(grp / np.exp2(e)[..., None].astype(np.float32), -6, 6)
+    lv = np.abs(E2M1[:8])
+    idx = np.abs(np.abs(q)[..., None] - lv).argmin(-1)
+    # midpoints go up in the reference (mag >= bound): argmin picks the lower one, so compare off midpoints only
+    off_mid = ~np.isin(np.abs(q), [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
+    idx = np.where(np.signbit(q), idx + 8, idx).reshape(16, 64)
+    got = np.empty((16, 64), np.uint8)
+    got[:, 0::2] = p & 0x0F
+    got[:, 1::2] = p >> 4
+    assert np.array_equal(got[off_mid.reshape(16, 64)], idx[off_mid.reshape(16, 64)])

@@ -1,0 +1,95 @@
+"""Pins quantize_q8, block_dot and block_dot_i8 (src/q8.rs)."""
+import numpy as np
+
+import oracle
+
+LUT2 = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)
+
+
+def brute_block_dot(packed16, x32):
+    lo, hi = packed16 & 0x0F, packed16 >> 4
+    w = np.empty(32, np.int64)
+    w[0::2], w[1::2] = LUT2[lo], LUT2[hi]
+    return int((w * x32.astype(np.int64)).sum())
+
+
+def test_quantize_conventions():
+    # src/q8.rs:321-334
+    x = np.zeros(64, np.float32)
+    x[3], x[40] = 12.7, -3.3
+    q, s = oracle.quantize_q8(x)
+    assert s[0] == np.float32(12.7) / np.float32(127.0)
+    assert s[1] == np.float32(3.3) / np.float32(127.0)
+    assert q[3] == 127 and q[40] == -127
+    assert q.min() >= -127
+    q, s = oracle.quantize_q8(np.zeros(32, np.float32))
+    assert s[0] == 0.0 and not q.any()
+
+
+def test_quantize_bound_and_ties():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(4096).astype(np.float32)
+    q, s = oracle.quantize_q8(x)
+    assert np.abs(q.astype(np.int32)).max() <= 127
+    dx = np.repeat(s, 32)
+    assert np.all(np.abs(x - q * dx) <= dx * 0.5 * (1 + 1e-6))
+    # each block's largest magnitude maps to +-127
+    assert np.all(np.abs(q.reshape(-1, 32)).max(axis=1) == 127)
+    # round half away from zero: with max 127 the step is exactly 1
+    x = np.zeros(32, np.float32)
+    x[0], x[1], x[2], x[3], x[4] = 127.0, 0.5, -0.5, 1.5, 2.5
+    q, s = oracle.quantize_q8(x)
+    assert s[0] == 1.0 and list(q[:5]) == [127, 1, -1, 2, 3]
+
+
+def test_block_dot_matches_brute_force_on_reference_stream():
+    # src/q8.rs:283-296: seed 0xDEADBEEF, 2000 cases, x = (u8 % 255) as i8
+    for scalar in (0, 1):
+        oracle.force_scalar(scalar)
+        rng = oracle.Rng(0xDEADBEEF)
+        for _ in range(2000):
+            packed = rng.u8(16)
+            x = (rng.u8(32) % 255).astype(np.uint8).view(np.int8)
+            assert oracle.block_dot(packed, x) == brute_block_dot(packed, x)
+        x = np.full(32, 127, np.int8)
+        assert oracle.block_dot(np.full(16, 0x77, np.uint8), x) == 32 * 12 * 127
+        assert oracle.block_dot(np.full(16, 0xFF, np.uint8), x) == -32 * 12 * 127
+        assert oracle.block_dot(np.full(16, 0x88, np.uint8), x) == 0  # negative zero nibble counts 0
+    oracle.force_scalar(0)
+
+
+def test_block_dot_i8_matches_brute_force_on_reference_stream():
+    # src/q8.rs:301-316: seed 0x12345678
+    for scalar in (0, 1):
+        oracle.force_scalar(scalar)
+        rng = oracle.Rng(0x12345678)
+        for _ in range(2000):
+            w = (rng.u8(32) % 255).astype(np.uint8).view(np.int8)
+            x = (rng.u8(32) % 255).astype(np.uint8).view(np.int8)
+            if not scalar:
+                # the stream holds -128 (128 as i8); the AVX2 kernel is only exact for |q| <= 127
+                # (src/q8.rs:147-150), which quantize_q8 guarantees: keep the SIMD cases in that domain
+                w, x = np.maximum(w, -127), np.maximum(x, -127)
+            assert oracle.block_dot_i8(w, x) == int((w.astype(np.int64) * x.astype(np.int64)).sum())
+        p, n = np.full(32, 127, np.int8), np.full(32, -127, np.int8)
+        assert oracle.block_dot_i8(p, p) == 32 * 127 * 127
+        assert oracle.block_dot_i8(n, p) == -32 * 127 * 127
+        assert oracle.block_dot_i8(n, n) == 32 * 127 * 127
+    oracle.force_scalar(0)
+
+
+def test_dot_order():
+    # src/model.rs:63-82: 8 accumulators, ((p01+p23)+p45)+p67, sequential tail
+    rng = oracle.Rng(0xABCDEF)
+    for n in [0, 1, 7, 8, 9, 15, 16, 17, 64, 100, 1024, 1027]:
+        a, b = rng.f32(n), rng.f32(n)
+        acc = np.zeros(8, np.float32)
+        i = 0
+        while i + 8 <= n:
+            acc = (acc + a[i:i + 8] * b[i:i + 8]).astype(np.float32)
+            i += 8
+        s = np.float32(np.float32(np.float32(acc[0] + acc[1]) + np.float32(acc[2] + acc[3])) + np.float32(acc[4] + acc[5]))
+        s = np.float32(s + np.float32(acc[6] + acc[7]))
+        for j in range(i, n):
+            s = np.float32(s + np.float32(a[j] * b[j]))
+        assert np.float32(oracle.dot(a, b)).view(np.uint32) == s.view(np.uint32), n
