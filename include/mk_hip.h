@@ -1,0 +1,248 @@
+/*
+ * mk_hip.h -- C ABI of libmk_hip.so: microkimi's quantized-weight hot path on
+ * one AMD MI355X (gfx950).  Plain pointers and sizes only; no C++ or torch types.
+ *
+ * Two levels:
+ *
+ *   mk_dev_*   device level.  Every pointer is DEVICE memory, `stream` is a
+ *              hipStream_t passed as void* (NULL = the default stream).  The call
+ *              enqueues kernels and returns; nothing is allocated or synchronised.
+ *              This is the level a resident engine (weights and activations kept
+ *              in HBM) binds, and the level the benchmark measures.
+ *
+ *   mk_*       host level: the drop-in for the reference's operator entry points.
+ *              Pointers are HOST memory, as the Rust slices are; weights are
+ *              uploaded once into a device cache keyed by (pointer, rows, cols)
+ *              exactly like the reference's Metal weight cache
+ *              (src/metal.rs:874-936), inputs and outputs are staged per call and
+ *              the call returns after the result is in `out`.
+ *
+ * There is NO CPU fallback in this library: when no device is present or a HIP
+ * call fails the function returns a negative status, leaves `out` untouched and
+ * mk_last_error() says why.  (The reference's Metal path falls back to its CPU
+ * kernels, src/metal.rs:949-960; a caller that wants that keeps its own CPU path
+ * and takes it on a negative status.)
+ *
+ * Status: 0 = done on the GPU, < 0 = error, nothing written.
+ * All entry points are thread-safe; host-level calls serialise on one lock, as
+ * the reference's Metal path does (src/metal.rs:432-439).
+ */
+#ifndef MK_HIP_H
+#define MK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MK_OK 0
+#define MK_ERR_INVALID (-1)     /* bad argument (shape, alignment, null pointer) */
+#define MK_ERR_NO_DEVICE (-2)   /* no gfx950 device / mk_init not possible */
+#define MK_ERR_HIP (-3)         /* a HIP runtime call failed */
+#define MK_ERR_UNSUPPORTED (-4) /* valid request the kernels do not cover */
+#define MK_ERR_NOMEM (-5)       /* device cache budget or allocation exhausted */
+
+/* Arithmetic of the MXFP4 matvec, the reference's q8 toggle (src/q8.rs:71-89):
+ * MK_MODE_Q8  activation quantized to q8 per 32, exact integer block dots (reference default)
+ * MK_MODE_F32 exact f32 path (MICROKIMI_NO_Q8=1 / force_q8(0)) */
+#define MK_MODE_F32 0
+#define MK_MODE_Q8 1
+
+/* Activation rule of a packed expert (see mk_dev_moe_decode). */
+#define MK_ACT_SWIGLU 0 /* silu(g) * u, silu(x) = x / (1 + exp(-x))            (src/deepseek.rs:1086) */
+#define MK_ACT_SITU 1   /* 4 tanh(g/4) sigmoid(g) * 25 tanh(u/25)                (src/model.rs:619-621)  */
+#define MK_ACT_DS 2     /* w * silu(min(g,L)) * clamp(u,-L,L), weight before W2  (src/deepseek.rs:1083-1087) */
+
+/* ------------------------------------------------------------- lifecycle */
+
+/* Replaces metal::gpu_available / init_ctx (src/metal.rs:445-593): binds the
+ * library to HIP device `device` (first call wins; later calls return the same
+ * status).  mk_available() = 1 once a gfx950 device is bound. */
+int mk_init(int device);
+int mk_available(void);
+void mk_shutdown(void);
+const char *mk_last_error(void);
+/* Device-cache budget in MiB for the host-level weight cache (MICROKIMI_GPU_CACHE_MB,
+ * src/metal.rs:554-558).  0 = unlimited (default). */
+void mk_set_cache_mb(size_t mb);
+/* q8::force_q8 / q8::q8_enabled (src/q8.rs:77-89): -1 follows the environment
+ * (MICROKIMI_NO_Q8=1 selects the f32 path), 0 forces f32, 1 forces q8. */
+void mk_force_q8(int v);
+int mk_q8_enabled(void);
+
+/* ---------------------------------------------------- device level: codec */
+
+/* mxfp4::dequant (src/mxfp4.rs:19-31) = dequant::dequant_fp4 (src/dequant.rs:43-45).
+ * packed [rows][cols/2] u8 (low nibble = even column), scales [rows][cols/32] e8m0,
+ * out [rows][cols] f32, bit-exact (nibble 8 gives -0.0, byte 0 gives 2^-127). */
+int mk_dev_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out, void *stream);
+
+/* dequant::dequant_fp8 (src/dequant.rs:27-39): e4m3fn bytes [rows][cols] with e8m0
+ * scales per 128x128 block -> f32, bit-exact. */
+int mk_dev_fp8_dequant(const uint8_t *w, const uint8_t *scales, size_t rows, size_t cols, float *out, void *stream);
+
+/* q8::quantize_q8_into (src/q8.rs:49-69) for `nvec` vectors of `n` floats each
+ * (n % 32 == 0): q [nvec][n] i8, scales [nvec][n/32] f32.  dx = max|x|/127,
+ * q = round-half-away(x/dx) clamped to +-127, zero block -> scale 0. */
+int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *scales, void *stream);
+
+/* deepseek::fp8_roundtrip with block 32 (src/deepseek.rs:312-322) kept in coded
+ * form: codes [nvec][n] e4m3 bytes, exps [nvec][n/32] e8m0 bytes (MXFP8).  This
+ * is the activation format of mk_dev_mxfp4_grouped_gemm. */
+int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream);
+
+/* ------------------------------------------- device level: MXFP4 matvecs */
+
+/* mxfp4::matvec_packed_q8 (src/mxfp4.rs:405-443): out[r] = sum_g idot_g * (2^(sb_g-128) * xs_g).
+ * cols % 32 == 0; packed, xq 16-byte aligned. */
+int mk_dev_mxfp4_matvec_q8(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const int8_t *xq, const float *xs,
+                           float *out, void *stream);
+
+/* mxfp4::matvec_packed, exact f32 path (src/mxfp4.rs:488-538): out[r] = sum_g (sum_j E2M1[nib]*x) * 2^(sb_g-127). */
+int mk_dev_mxfp4_matvec_f32(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out,
+                            void *stream);
+
+/* mxfp4::matvec_packed (src/mxfp4.rs:458-539), the operator entry point: mode
+ * MK_MODE_Q8 quantizes x (into `xq_ws`, `xs_ws`: device scratch of cols bytes and
+ * cols/32 floats supplied by the caller) and runs the integer path; MK_MODE_F32
+ * ignores the scratch. */
+int mk_dev_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out, int mode,
+                        int8_t *xq_ws, float *xs_ws, void *stream);
+
+/* The same q8 matvec over `nmat` matrices of one shape in ONE launch: the
+ * grouped-expert form.  packed_ptrs / scales_ptrs / out_ptrs: device arrays of
+ * nmat device pointers; xq [nx][cols], xs [nx][cols/32]; x_index[nmat] (device,
+ * may be NULL = all use vector 0) picks the activation of each matrix. */
+int mk_dev_mxfp4_matvec_q8_grouped(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t nmat, size_t rows,
+                                   size_t cols, const int8_t *xq, const float *xs, const int32_t *x_index, float *const *out_ptrs,
+                                   void *stream);
+
+/* model::matvec_packed_nt (src/model.rs:2412-2447): exact-f32 batched matvec.
+ * x [m][cols] position-major (the kernel needs no transposed copy and no
+ * padding to 8), out [m][rows]. */
+int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m, float *out,
+                           void *stream);
+
+/* ------------------------------------------------- device level: q8 head */
+
+/* Q8Head::matvec / row_dot (src/model.rs:290-347) on `batch` already-quantized
+ * activations: out[b][r] = sum_g (ws[r][g] * xs[b][g]) * idot.
+ * q [rows][cols] i8; scales [rows][cols/32], f16 when scales_f16 != 0 (the q8_0
+ * storage form) else f32 (the reference's in-memory form); xq [batch][cols],
+ * xs [batch][cols/32]; out [batch][rows].  batch <= 8. */
+int mk_dev_q8_matvec(const int8_t *q, const void *scales, int scales_f16, size_t rows, size_t cols, const int8_t *xq, const float *xs,
+                     size_t batch, float *out, void *stream);
+
+/* The greedy token of model::top_k_probs (src/model.rs:3271-3291): index of the
+ * largest logit per row, ties to the lowest index.  logits [batch][n];
+ * ws: device scratch of 2 * batch * 1024 * 4 bytes; out_idx [batch] int32. */
+int mk_dev_argmax(const float *logits, size_t batch, size_t n, void *ws, int32_t *out_idx, void *stream);
+
+/* Q8Head::from_f32 (src/model.rs:274-286) on device: row-wise q8_0 of w [rows][cols];
+ * scales written as f16 (scales_f16 != 0; the rounded value is what the matvec
+ * then uses) or f32. */
+int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, void *scales, int scales_f16, void *stream);
+
+/* ------------------------------------------------ device level: MoE layer */
+
+/* Expert table: device arrays of per-expert device pointers, indexed by expert
+ * id.  w1, w3: [inter][d] (gate, up); w2: [d][inter] (down); each MXFP4 as
+ * (packed, scales) in the reference layout. */
+typedef struct {
+    const uint8_t *const *w1p, *const *w1s;
+    const uint8_t *const *w3p, *const *w3s;
+    const uint8_t *const *w2p, *const *w2s;
+    size_t d, inter;
+} mk_expert_table;
+
+/* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
+size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
+
+/* The expert section of moe_forward / ds_moe for B decode tokens in one grouped
+ * pass (src/model.rs:2227-2264,2346-2351; src/deepseek.rs:1069-1106):
+ *   per token t and slot s: e = ids[t][s];
+ *     a = W1_e x_t ; u = W3_e x_t ; act = ACT(a, u) ; o = W2_e act     (matvec_packed, `mode`)
+ *   out_t = sum_s w[t][s] * o   in slot order   (MK_ACT_DS: plain sum, weight inside act)
+ *         + o(shared expert)    when shared >= 0, unweighted.
+ * ids [B][topk] int32, weights [B][topk] f32, x [B][d], out [B][d]; all device.
+ * mode MK_MODE_Q8 re-quantizes x and act per 32 exactly as matvec_packed does on
+ * each call. */
+int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
+                      const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
+
+/* Router of the benchmark MoE layer on device: softmax over logits [B][n], top-k
+ * with the reference's rule (strict '>' insertion: ties to the lowest index;
+ * src/model.rs:2157-2173), weights renormalised.  ids [B][k] int32, weights [B][k]. */
+int mk_dev_router_softmax_topk(const float *logits, size_t B, size_t n, size_t k, int32_t *ids, float *weights, void *stream);
+
+/* ------------------------------------------- device level: MLA attention */
+
+/* mla_attn_flash_q8_mqa (src/model.rs:1804-1908) in the weight-absorbed form:
+ * one shared q8_0 latent row per position is K (with the rope row) and V of
+ * every head.
+ *   lat_q [n][L] i8, lat_s [n][L/32] f16; rope_q [n][R] i8, rope_s [n][R/32] f16
+ *   q [nh][L+R] f32 (latent part first), out [nh][L] f32
+ * score = (dot(q_rope, dequant(rope)) + sum_g (qs_g*ks_g)*idot_g) * scale over the
+ * q8-quantized latent query; online softmax; out = sum p * dequant(latent) / l.
+ * Positions 0..=pos are attended (pos < n).  L % 32 == 0, R % 32 == 0.
+ * workspace: mk_mla_decode_workspace_bytes(nh, L, pos + 1). */
+size_t mk_mla_decode_workspace_bytes(size_t nh, size_t L, size_t n_pos);
+int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos, const float *q,
+                         size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream);
+
+/* MlaCache::push (src/model.rs:1583-1618) for the shared-latent cache: quantize
+ * one position (latent [L] f32, rope [R] f32) into row `pos` of the cache arrays. */
+int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, size_t R, size_t pos, int8_t *lat_q, void *lat_s,
+                            int8_t *rope_q, void *rope_s, void *stream);
+
+/* ---------------------------------- device level: prefill expert GEMM */
+
+/* The per-expert batched evaluation of moe_prefill (src/model.rs:2539-2602) as a
+ * grouped GEMM on the block-scaled FP8/FP4 matrix cores.
+ *   y[i][r] = sum_k dequant(W_e)[r][k] * dequant(xa)[i][k]  for the rows i of group e
+ * xa: MXFP8 activations from mk_dev_quantize_mxfp8: codes [m][cols], exps [m][cols/32];
+ * rows of one expert are contiguous: group e covers rows offsets[e] .. offsets[e+1].
+ * packed_ptrs/scales_ptrs [n_groups]: the weight of each group; out [m][rows] f32. */
+int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                              size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
+                              void *stream);
+
+/* ------------------------------------------------------------ host level */
+
+/* metal::gpu_matvec_fp4 (src/metal.rs:943-1017), i.e. the GPU branch of
+ * mxfp4::matvec_packed (src/mxfp4.rs:467-473).  Host slices; the weight is
+ * cached on device by (packed pointer, rows, cols) and re-validated against the
+ * first 16 host bytes on every hit.  Arithmetic follows mk_q8_enabled(). */
+int mk_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out);
+
+/* mxfp4::dequant on host slices (upload, kernel, download). */
+int mk_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out);
+
+/* q8::quantize_q8_into on host slices. */
+int mk_quantize_q8(const float *x, size_t n, int8_t *q, float *scales);
+
+/* Q8Head (src/model.rs:261-348): built once, kept on device. */
+typedef struct mk_q8head mk_q8head;
+int mk_q8head_from_f32(const float *w, size_t rows, size_t cols, int scales_f16, mk_q8head **out);
+int mk_q8head_from_q8(const int8_t *q, const float *scales, size_t rows, size_t cols, int scales_f16, mk_q8head **out);
+/* logits for `batch` host rows x [batch][cols] -> out [batch][rows]; argmax_out (may be NULL) [batch] */
+int mk_q8head_matvec(mk_q8head *h, const float *x, size_t batch, float *out, int32_t *argmax_out);
+void mk_q8head_free(mk_q8head *h);
+
+/* Shared-latent q8 MLA cache kept on device (MlaCache, src/model.rs:765-781,1556-1618). */
+typedef struct mk_mla_cache mk_mla_cache;
+int mk_mla_cache_new(size_t nh, size_t L, size_t R, size_t capacity, mk_mla_cache **out);
+int mk_mla_cache_push(mk_mla_cache *c, const float *latent, const float *rope);
+size_t mk_mla_cache_positions(const mk_mla_cache *c);
+/* MlaCache::to_f32 (src/model.rs:1623-1676): dequantized rows, latent [n][L], rope [n][R] */
+int mk_mla_cache_to_f32(const mk_mla_cache *c, float *latent, float *rope);
+/* attention of all heads over positions 0..=positions-1: q [nh][L+R] host, out [nh][L] host */
+int mk_mla_attn(mk_mla_cache *c, const float *q, float scale, float *out);
+void mk_mla_cache_free(mk_mla_cache *c);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MK_HIP_H */

@@ -1,0 +1,111 @@
+"""ctypes binding of libmk_hip.so (the C ABI declared in include/mk_hip.h).
+
+The library is the product: there is no Python or CPU stand-in for it.  If it
+has not been built (python -m microkimi_amd.build) loading fails with an error.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmk_hip.so")
+
+MK_OK = 0
+MODE_F32, MODE_Q8 = 0, 1
+ACT_SWIGLU, ACT_SITU, ACT_DS = 0, 1, 2
+
+
+class MkError(RuntimeError):
+    def __init__(self, status, msg):
+        super().__init__(f"libmk_hip status {status}: {msg}")
+        self.status = status
+
+
+class ExpertTable(C.Structure):
+    _fields_ = [("w1p", C.c_void_p), ("w1s", C.c_void_p), ("w3p", C.c_void_p), ("w3s", C.c_void_p), ("w2p", C.c_void_p),
+                ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t)]
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python -m microkimi_amd.build` (needs hipcc); "
+                          "there is no fallback implementation")
+    lib = C.CDLL(LIB_PATH)
+    vp, sz, i32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_float
+    sig = {
+        "mk_init": (i32, [i32]),
+        "mk_available": (i32, []),
+        "mk_shutdown": (None, []),
+        "mk_last_error": (C.c_char_p, []),
+        "mk_set_cache_mb": (None, [sz]),
+        "mk_force_q8": (None, [i32]),
+        "mk_q8_enabled": (i32, []),
+        "mk_dev_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
+        "mk_dev_fp8_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
+        "mk_dev_quantize_q8": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_quantize_mxfp8": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec_q8": (i32, [vp, vp, sz, sz, vp, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec_f32": (i32, [vp, vp, sz, sz, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp, i32, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec_q8_grouped": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec_nt": (i32, [vp, vp, sz, sz, vp, sz, vp, vp]),
+        "mk_dev_q8_matvec": (i32, [vp, vp, i32, sz, sz, vp, vp, sz, vp, vp]),
+        "mk_dev_argmax": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_q8head_from_f32": (i32, [vp, sz, sz, vp, vp, i32, vp]),
+        "mk_moe_decode_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
+        "mk_dev_moe_decode": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),
+        "mk_dev_router_softmax_topk": (i32, [vp, sz, sz, sz, vp, vp, vp]),
+        "mk_mla_decode_workspace_bytes": (sz, [sz, sz, sz]),
+        "mk_dev_mla_q8_decode": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp, vp]),
+        "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
+        "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
+        "mk_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp]),
+        "mk_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp]),
+        "mk_quantize_q8": (i32, [vp, sz, vp, vp]),
+        "mk_q8head_from_f32": (i32, [vp, sz, sz, i32, C.POINTER(vp)]),
+        "mk_q8head_from_q8": (i32, [vp, vp, sz, sz, i32, C.POINTER(vp)]),
+        "mk_q8head_matvec": (i32, [vp, vp, sz, vp, vp]),
+        "mk_q8head_free": (None, [vp]),
+        "mk_mla_cache_new": (i32, [sz, sz, sz, sz, C.POINTER(vp)]),
+        "mk_mla_cache_push": (i32, [vp, vp, vp]),
+        "mk_mla_cache_positions": (sz, [vp]),
+        "mk_mla_cache_to_f32": (i32, [vp, vp, vp]),
+        "mk_mla_attn": (i32, [vp, vp, f32, vp]),
+        "mk_mla_cache_free": (None, [vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)  # AttributeError here = the library does not export a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    return lib, sorted(sig)
+
+
+lib, SYMBOLS = _load()
+
+
+def check(status):
+    if status != MK_OK:
+        raise MkError(status, lib.mk_last_error().decode("utf-8", "replace"))
+
+
+def require_device():
+    """Binds device 0; raises if no gfx950 device is usable (no fallback)."""
+    check(lib.mk_init(0))
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (must be contiguous) or None."""
+    if t is None:
+        return None
+    assert t.is_contiguous(), "tensor must be contiguous"
+    return C.c_void_p(t.data_ptr())
+
+
+def hptr(a):
+    """Host pointer of a contiguous numpy array."""
+    assert a.flags["C_CONTIGUOUS"]
+    return C.c_void_p(a.ctypes.data)
+
+
+def cur_stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)

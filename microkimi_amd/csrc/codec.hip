@@ -1,0 +1,189 @@
+// Codec kernels: MXFP4 / FP8 dequantization (bit-exact), q8_0 and MXFP8
+// activation quantization.  All HBM-bound elementwise work: 128-bit accesses,
+// one pass over the data.
+#include "mk_common.h"
+
+// ---------------------------------------------------------------- mxfp4::dequant
+// One thread decodes 8 nibbles (one dword of packed bytes) into two float4
+// stores.  W[r,c] = E2M1[nibble] * 2^(sb-127), low nibble = even column
+// (src/mxfp4.rs:19-31).  The product is one IEEE multiply, as in the reference.
+__global__ __launch_bounds__(256) void mk_mxfp4_dequant_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales,
+                                                               size_t n_words, float *__restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_words) return;
+    uint32_t w = packed[i];
+    // word i holds elements 8i .. 8i+7; 4 words per 32-block
+    float s = mk_scale_from_byte(scales[i >> 2]);
+    mk_f4 lo, hi;
+    lo.x = mk_e2m1(w & 15u) * s;
+    lo.y = mk_e2m1((w >> 4) & 15u) * s;
+    lo.z = mk_e2m1((w >> 8) & 15u) * s;
+    lo.w = mk_e2m1((w >> 12) & 15u) * s;
+    hi.x = mk_e2m1((w >> 16) & 15u) * s;
+    hi.y = mk_e2m1((w >> 20) & 15u) * s;
+    hi.z = mk_e2m1((w >> 24) & 15u) * s;
+    hi.w = mk_e2m1((w >> 28) & 15u) * s;
+    mk_f4 *o = reinterpret_cast<mk_f4 *>(out + i * 8);
+    o[0] = lo;
+    o[1] = hi;
+}
+
+// ---------------------------------------------------------------- dequant::dequant_fp8
+// e4m3fn byte -> f32 by bit construction (src/dequant.rs:12-23): normal
+// (-1)^s 2^(e-7) (1+m/8), subnormal (-1)^s (m/8) 2^-6, 0x7F/0xFF NaN.
+__device__ __forceinline__ float mk_e4m3_to_f32(uint32_t b) {
+    uint32_t sign = (b & 0x80u) << 24;
+    uint32_t e = (b >> 3) & 15u, m = b & 7u;
+    if (e == 15u && m == 7u) return __uint_as_float(0x7FC00000u);
+    if (e == 0u) {
+        float v = (float)m * 0.001953125f;  // m * 2^-9, exact
+        return __uint_as_float(__float_as_uint(v) | sign);
+    }
+    return __uint_as_float(sign | ((e + 120u) << 23) | (m << 20));
+}
+
+__global__ __launch_bounds__(256) void mk_fp8_dequant_kernel(const uint8_t *__restrict__ w, const uint8_t *__restrict__ scales, size_t rows,
+                                                             size_t cols, float *__restrict__ out) {
+    // one thread = 4 consecutive columns of one row (cols % 4 == 0)
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t per_row = cols / 4;
+    if (i >= rows * per_row) return;
+    size_t r = i / per_row, c = (i % per_row) * 4;
+    size_t scols = (cols + 127) / 128;
+    float s = mk_scale_from_byte(scales[(r / 128) * scols + c / 128]);
+    // byte 0 must mean 2^-127 here as well (exp2_i(-127)); mk_scale_from_byte gives that
+    uint32_t v = *reinterpret_cast<const uint32_t *>(w + r * cols + c);
+    mk_f4 o;
+    o.x = mk_e4m3_to_f32(v & 255u) * s;
+    o.y = mk_e4m3_to_f32((v >> 8) & 255u) * s;
+    o.z = mk_e4m3_to_f32((v >> 16) & 255u) * s;
+    o.w = mk_e4m3_to_f32(v >> 24) * s;
+    *reinterpret_cast<mk_f4 *>(out + r * cols + c) = o;
+}
+
+// ---------------------------------------------------------------- q8::quantize_q8_into
+// One half-wave (32 lanes) per block of 32 values: lane j holds x[32 g + j],
+// the block maximum comes from 5 cross-lane steps, every lane rounds its own
+// value (src/q8.rs:57-68).  SCALE_F16: the scale is stored as f16 (q8_0 storage
+// form) after the quantization used the f32 value.
+template <bool SCALE_F16>
+__global__ __launch_bounds__(256) void mk_quantize_q8_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ q,
+                                                             void *__restrict__ scales) {
+    size_t g = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    int j = threadIdx.x & 31;
+    if (g >= n_blocks) return;  // whole half-waves leave together
+    float v = x[g * 32 + j];
+    float mx = mk_half_wave_max(fabsf(v));
+    float dx = mx / 127.0f;
+    int qi = 0;
+    if (dx != 0.0f) qi = mk_q8_round(v, dx);
+    q[g * 32 + j] = (int8_t)qi;
+    if (j == 0) {
+        if (SCALE_F16)
+            reinterpret_cast<uint16_t *>(scales)[g] = mk_f32_to_f16_bits(dx);
+        else
+            reinterpret_cast<float *>(scales)[g] = dx;
+    }
+}
+
+// ---------------------------------------------------------------- MXFP8 activations
+// f32 -> e4m3fn, round to nearest even, saturating at 448 (src/dequant.rs:92-120).
+__device__ __forceinline__ uint32_t mk_f32_to_e4m3(float v) {
+    if (v != v) return 0x7Fu;
+    uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    float a = fminf(fabsf(v), 448.0f);
+    if (a < 0.015625f) {  // below the smallest normal 2^-6: m = rne(a * 2^9), 8 carries into e=1
+        return sign | (uint32_t)rintf(a * 512.0f);
+    }
+    uint32_t bits = __float_as_uint(a);
+    uint32_t r = (bits + 0x7FFFFu + ((bits >> 20) & 1u)) >> 20;  // exponent and 3 mantissa bits, RNE with carry
+    return sign | (r - (120u << 3));
+}
+
+// One half-wave per block of 32: scale exponent e = ceil(log2(max(amax,1e-4)/448))
+// clamped to [-127, 8], code = e4m3(clamp(x / 2^e)) (src/deepseek.rs:312-322).
+// The reference takes a float log2; a correctly rounded float log2 is what
+// (float)log2((double)r) gives, so the exponent matches the host libm.
+__global__ __launch_bounds__(256) void mk_quantize_mxfp8_kernel(const float *__restrict__ x, size_t n_blocks, uint8_t *__restrict__ codes,
+                                                                uint8_t *__restrict__ exps) {
+    size_t g = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    int j = threadIdx.x & 31;
+    if (g >= n_blocks) return;
+    float v = x[g * 32 + j];
+    float amax = fmaxf(mk_half_wave_max(fabsf(v)), 1e-4f);
+    int e = (int)ceilf((float)log2((double)(amax / 448.0f)));
+    e = max(-127, min(8, e));
+    float s = mk_scale_from_byte((uint32_t)(e + 127));
+    float qv = fminf(fmaxf(v / s, -448.0f), 448.0f);
+    codes[g * 32 + j] = (uint8_t)mk_f32_to_e4m3(qv);
+    if (j == 0) exps[g] = (uint8_t)(e + 127);
+}
+
+// ------------------------------------------------------------------ C ABI
+extern "C" int mk_dev_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out, void *stream) {
+    MK_REQUIRE(packed && scales && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0, "cols must be a multiple of 32");
+    MK_REQUIRE(((uintptr_t)packed & 3) == 0 && ((uintptr_t)out & 15) == 0, "packed must be 4-byte and out 16-byte aligned");
+    size_t n_words = rows * cols / 8;
+    if (n_words == 0) return MK_OK;
+    unsigned grid = (unsigned)((n_words + 255) / 256);
+    hipLaunchKernelGGL(mk_mxfp4_dequant_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)packed, scales, n_words,
+                       out);
+    return mk_launch_status("mxfp4_dequant");
+}
+
+extern "C" int mk_dev_fp8_dequant(const uint8_t *w, const uint8_t *scales, size_t rows, size_t cols, float *out, void *stream) {
+    MK_REQUIRE(w && scales && out, "null pointer");
+    MK_REQUIRE(cols % 4 == 0, "cols must be a multiple of 4");
+    MK_REQUIRE(((uintptr_t)w & 3) == 0 && ((uintptr_t)out & 15) == 0, "w must be 4-byte and out 16-byte aligned");
+    size_t n = rows * cols / 4;
+    if (n == 0) return MK_OK;
+    unsigned grid = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(mk_fp8_dequant_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, scales, rows, cols, out);
+    return mk_launch_status("fp8_dequant");
+}
+
+extern "C" int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *scales, void *stream) {
+    MK_REQUIRE(x && q && scales, "null pointer");
+    MK_REQUIRE(n % 32 == 0, "q8 blocks are 32 wide");
+    size_t n_blocks = nvec * n / 32;
+    if (n_blocks == 0) return MK_OK;
+    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    hipLaunchKernelGGL(mk_quantize_q8_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, x, n_blocks, q, (void *)scales);
+    return mk_launch_status("quantize_q8");
+}
+
+extern "C" int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, void *scales, int scales_f16, void *stream) {
+    MK_REQUIRE(w && q && scales, "null pointer");
+    MK_REQUIRE(cols % 32 == 0, "q8 blocks are 32 wide");
+    size_t n_blocks = rows * cols / 32;
+    if (n_blocks == 0) return MK_OK;
+    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    if (scales_f16)
+        hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, n_blocks, q, scales);
+    else
+        hipLaunchKernelGGL(mk_quantize_q8_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, n_blocks, q, scales);
+    return mk_launch_status("q8head_from_f32");
+}
+
+extern "C" int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream) {
+    MK_REQUIRE(x && codes && exps, "null pointer");
+    MK_REQUIRE(n % 32 == 0, "MXFP8 blocks are 32 wide");
+    size_t n_blocks = nvec * n / 32;
+    if (n_blocks == 0) return MK_OK;
+    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    hipLaunchKernelGGL(mk_quantize_mxfp8_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, x, n_blocks, codes, exps);
+    return mk_launch_status("quantize_mxfp8");
+}
+
+extern "C" int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, size_t R, size_t pos, int8_t *lat_q, void *lat_s,
+                                       int8_t *rope_q, void *rope_s, void *stream) {
+    MK_REQUIRE(latent && rope && lat_q && lat_s && rope_q && rope_s, "null pointer");
+    MK_REQUIRE(L % 32 == 0 && R % 32 == 0, "q8 blocks are 32 wide");
+    unsigned g1 = (unsigned)((L / 32 + 7) / 8), g2 = (unsigned)((R / 32 + 7) / 8);
+    hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(g1), dim3(256), 0, (hipStream_t)stream, latent, L / 32, lat_q + pos * L,
+                       (void *)((uint16_t *)lat_s + pos * (L / 32)));
+    hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(g2), dim3(256), 0, (hipStream_t)stream, rope, R / 32, rope_q + pos * R,
+                       (void *)((uint16_t *)rope_s + pos * (R / 32)));
+    return mk_launch_status("mla_cache_append");
+}

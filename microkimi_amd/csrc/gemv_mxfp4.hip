@@ -1,0 +1,444 @@
+// MXFP4 decode GEMV (mxfp4::matvec_packed and friends) for gfx950.
+//
+// HBM-bound: every weight byte is read exactly once with 128-bit loads, in the
+// reference's own layout (packed [rows][cols/2], scales [rows][cols/32]; rows are
+// contiguous, so a tile of rows is one contiguous byte range).  No repacking.
+//
+// Fast path (template on NB = cols/32):
+//   * a tile is lcm(NB,64) blocks = RT rows; T = tile/64 wave iterations.
+//     Lane l of iteration t owns block t*64+l of the tile: one 16-byte load of
+//     32 nibbles plus one scale byte; the wave's T loads cover RT rows with
+//     perfectly coalesced 1 KiB requests.
+//   * the block index a lane owns repeats from tile to tile, so the lane keeps
+//     "its" 32 activations (as f16 pairs) and block scale in registers for the
+//     whole kernel: the activation is staged once per workgroup through LDS.
+//   * q8 mode: nibbles -> f16 by v_cvt_scalef32_pk_f16_fp4, activation bytes as
+//     f16 integers, v_dot2_f32_f16 accumulation.  Every term is a multiple of 0.5
+//     below 2^15, so the f32 accumulation is exact: h = idot/2 and the block
+//     contribution is (h+h) * (2^(sb-128) * dx), the reference's expression.
+//   * one butterfly reduction per row, fixed order (deterministic).
+// Generic path: one wave per row, any cols % 32 == 0.
+#include "mk_common.h"
+
+namespace {
+
+constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
+constexpr int lcm_c(int a, int b) { return a / gcd_c(a, b) * b; }
+
+struct GemvArgs {
+    // single-matrix form
+    const uint8_t *packed;
+    const uint8_t *scales;
+    float *out;
+    // grouped form (device arrays), used when packed == nullptr
+    const uint8_t *const *packed_ptrs;
+    const uint8_t *const *scales_ptrs;
+    float *const *out_ptrs;
+    const int32_t *x_index;
+    // activation(s)
+    const int8_t *xq;  // [nx][cols]
+    const float *xs;   // [nx][cols/32]
+    const float *xf;   // f32 mode: [nx][cols]
+    int rows;
+    int tiles_per_wave;
+};
+
+__device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
+    float h = 0.0f;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        uint32_t wd = (uint32_t)w[d];
+        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 0), xr[d * 4 + 0], h, false);
+        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 1), xr[d * 4 + 1], h, false);
+        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 2), xr[d * 4 + 2], h, false);
+        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 3), xr[d * 4 + 3], h, false);
+    }
+    return h;
+}
+
+// ------------------------------------------------------------ q8 fast path
+template <int NB>
+__global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
+    constexpr int TILE = lcm_c(NB, 64);
+    constexpr int T = TILE / 64;
+    constexpr int RT = TILE / NB;
+    static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
+    __shared__ __attribute__((aligned(16))) _Float16 xh[NB * 32];
+    __shared__ float xsc[NB];
+
+    const int mat = blockIdx.y;
+    const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
+    const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    float *out = a.packed ? a.out : a.out_ptrs[mat];
+    const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
+    const int8_t *xq = a.xq + (size_t)xi * NB * 32;
+    const float *xs = a.xs + (size_t)xi * NB;
+
+    // stage the activation: int8 -> f16 (exact), 4 values per thread per step
+    for (int i = threadIdx.x; i < NB * 8; i += 256) {
+        uint32_t v = reinterpret_cast<const uint32_t *>(xq)[i];
+        mk_h2 lo, hi;
+        lo.x = (_Float16)(float)(int8_t)(v & 255u);
+        lo.y = (_Float16)(float)(int8_t)((v >> 8) & 255u);
+        hi.x = (_Float16)(float)(int8_t)((v >> 16) & 255u);
+        hi.y = (_Float16)(float)(int8_t)(v >> 24);
+        reinterpret_cast<mk_h2 *>(xh)[i * 2] = lo;
+        reinterpret_cast<mk_h2 *>(xh)[i * 2 + 1] = hi;
+    }
+    for (int i = threadIdx.x; i < NB; i += 256) xsc[i] = xs[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    mk_h2 xr[T][16];
+    float cf[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        const int g = (t * 64 + lane) % NB;
+        const mk_i4 *src = reinterpret_cast<const mk_i4 *>(xh + g * 32);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            mk_i4 v = src[k];
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[t][k * 4 + e] = __builtin_bit_cast(mk_h2, v[e]);
+        }
+        cf[t] = xsc[g];
+    }
+
+    const int n_tiles = (a.rows + RT - 1) / RT;
+    const int tile0 = (blockIdx.x * 4 + wave) * a.tiles_per_wave;
+    const int tile1 = min(tile0 + a.tiles_per_wave, n_tiles);
+
+    mk_i4 w[T];
+    uint32_t sb[T];
+    auto load_tile = [&](int tile) {
+        const size_t blk0 = (size_t)tile * TILE;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const int bi = t * 64 + lane;
+            const bool ok = tile * RT + bi / NB < a.rows;
+            w[t] = ok ? *reinterpret_cast<const mk_i4 *>(packed + (blk0 + bi) * 16) : mk_i4{0, 0, 0, 0};
+            sb[t] = ok ? (uint32_t)scales[blk0 + bi] : 0u;
+        }
+    };
+    if (tile0 < tile1) load_tile(tile0);
+    for (int tile = tile0; tile < tile1; tile++) {
+        mk_i4 wc[T];
+        uint32_t sc[T];
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            wc[t] = w[t];
+            sc[t] = sb[t];
+        }
+        if (tile + 1 < tile1) load_tile(tile + 1);  // next tile in flight while this one is reduced
+        float acc[RT];
+#pragma unroll
+        for (int r = 0; r < RT; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            float h = dot32_fp4_f16(wc[t], xr[t]);
+            float term = (h + h) * (mk_half_scale_from_byte(sc[t]) * cf[t]);
+            const int rit = (t * 64 + lane) / NB;
+#pragma unroll
+            for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < RT; r++) acc[r] = mk_wave_sum(acc[r]);
+        if (lane < RT) {
+            const int row = tile * RT + lane;
+            if (row < a.rows) out[row] = (RT == 2 && lane == 1) ? acc[RT - 1] : acc[0];
+        }
+    }
+}
+
+// ----------------------------------------------------------- f32 fast path
+// Same tiling; the f32 activation stays in LDS (28 KiB at cols 7168) and each
+// lane walks its block in column order with separate multiply and add, so the
+// per-block sum gsum and the term gsum * 2^(sb-127) are the reference's values
+// bit for bit (src/mxfp4.rs:494-505); only the order of the sum over blocks differs.
+template <int NB>
+__global__ __launch_bounds__(256) void mxfp4_gemv_f32_kernel(GemvArgs a) {
+    constexpr int TILE = lcm_c(NB, 64);
+    constexpr int T = TILE / 64;
+    constexpr int RT = TILE / NB;
+    static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
+    __shared__ __attribute__((aligned(16))) float xl[NB * 32];
+    const int mat = blockIdx.y;
+    const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
+    const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    float *out = a.packed ? a.out : a.out_ptrs[mat];
+    const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
+    const float *xf = a.xf + (size_t)xi * NB * 32;
+    for (int i = threadIdx.x; i < NB * 8; i += 256) reinterpret_cast<mk_f4 *>(xl)[i] = reinterpret_cast<const mk_f4 *>(xf)[i];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_tiles = (a.rows + RT - 1) / RT;
+    const int tile0 = (blockIdx.x * 4 + wave) * a.tiles_per_wave;
+    const int tile1 = min(tile0 + a.tiles_per_wave, n_tiles);
+    for (int tile = tile0; tile < tile1; tile++) {
+        const size_t blk0 = (size_t)tile * TILE;
+        mk_i4 w[T];
+        uint32_t sb[T];
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const int bi = t * 64 + lane;
+            const bool ok = tile * RT + bi / NB < a.rows;
+            w[t] = ok ? *reinterpret_cast<const mk_i4 *>(packed + (blk0 + bi) * 16) : mk_i4{0, 0, 0, 0};
+            sb[t] = ok ? (uint32_t)scales[blk0 + bi] : 0u;
+        }
+        float acc[RT];
+#pragma unroll
+        for (int r = 0; r < RT; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const int bi = t * 64 + lane;
+            const int g = bi % NB;
+            const mk_f4 *xv = reinterpret_cast<const mk_f4 *>(xl + g * 32);
+            float gsum = 0.0f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                uint32_t wd = (uint32_t)w[t][d];
+                mk_f4 x0 = xv[d * 2], x1 = xv[d * 2 + 1];
+                mk_f2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 0);
+                mk_f2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 1);
+                mk_f2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 2);
+                mk_f2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 3);
+                gsum = __fadd_rn(gsum, __fmul_rn(p0.x, x0.x));
+                gsum = __fadd_rn(gsum, __fmul_rn(p0.y, x0.y));
+                gsum = __fadd_rn(gsum, __fmul_rn(p1.x, x0.z));
+                gsum = __fadd_rn(gsum, __fmul_rn(p1.y, x0.w));
+                gsum = __fadd_rn(gsum, __fmul_rn(p2.x, x1.x));
+                gsum = __fadd_rn(gsum, __fmul_rn(p2.y, x1.y));
+                gsum = __fadd_rn(gsum, __fmul_rn(p3.x, x1.z));
+                gsum = __fadd_rn(gsum, __fmul_rn(p3.y, x1.w));
+            }
+            float term = __fmul_rn(gsum, mk_scale_from_byte(sb[t]));
+            const int rit = bi / NB;
+#pragma unroll
+            for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < RT; r++) acc[r] = mk_wave_sum(acc[r]);
+        if (lane < RT) {
+            const int row = tile * RT + lane;
+            if (row < a.rows) out[row] = (RT == 2 && lane == 1) ? acc[RT - 1] : acc[0];
+        }
+    }
+}
+
+// ------------------------------------------------------------ generic path
+// One wave per row, lanes stride over the row's blocks; activations come from
+// global memory (L2-resident).  Any cols % 32 == 0.
+template <bool Q8>
+__global__ __launch_bounds__(256) void mxfp4_gemv_generic_kernel(GemvArgs a, int nb) {
+    const int mat = blockIdx.y;
+    const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
+    const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    float *out = a.packed ? a.out : a.out_ptrs[mat];
+    const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= a.rows) return;
+    float acc = 0.0f;
+    for (int g = lane; g < nb; g += 64) {
+        const size_t blk = (size_t)row * nb + g;
+        mk_i4 w = *reinterpret_cast<const mk_i4 *>(packed + blk * 16);
+        uint32_t sb = scales[blk];
+        if (Q8) {
+            const int8_t *xq = a.xq + ((size_t)xi * nb + g) * 32;
+            mk_h2 xr[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                xr[k].x = (_Float16)(float)xq[2 * k];
+                xr[k].y = (_Float16)(float)xq[2 * k + 1];
+            }
+            float h = dot32_fp4_f16(w, xr);
+            acc += (h + h) * (mk_half_scale_from_byte(sb) * a.xs[(size_t)xi * nb + g]);
+        } else {
+            const float *x = a.xf + ((size_t)xi * nb + g) * 32;
+            float gsum = 0.0f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                uint32_t wd = (uint32_t)w[d];
+#pragma unroll
+                for (int k = 0; k < 8; k++) gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> (4 * k)) & 15u), x[d * 8 + k]));
+            }
+            acc += __fmul_rn(gsum, mk_scale_from_byte(sb));
+        }
+    }
+    acc = mk_wave_sum(acc);
+    if (lane == 0) out[row] = acc;
+}
+
+// ---------------------------------------------------------- batched f32 (nt)
+// model::matvec_packed_nt (src/model.rs:2412-2447): exact-f32 arithmetic for m
+// positions against one packed matrix.  One wave per row; the row's nibbles are
+// decoded once per 8-position group from registers, the activations stream from
+// L2.  Per position and block the sum runs in column order with separate
+// multiply and add (the reference's gsum), then gsum * scale; blocks are summed
+// across lanes.  This is the exact-arithmetic twin of the MFMA GEMM, not the
+// fast prefill path.
+__global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scales, int rows,
+                                                            int nb, const float *__restrict__ x, int m, float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const size_t cols = (size_t)nb * 32;
+    for (int p0 = 0; p0 < m; p0 += 4) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int g = lane; g < nb; g += 64) {
+            const size_t blk = (size_t)row * nb + g;
+            mk_i4 w = *reinterpret_cast<const mk_i4 *>(packed + blk * 16);
+            float s = mk_scale_from_byte(scales[blk]);
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                if (p0 + p < m) {
+                    const mk_f4 *xv = reinterpret_cast<const mk_f4 *>(x + (size_t)(p0 + p) * cols + (size_t)g * 32);
+                    float gsum = 0.0f;
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        uint32_t wd = (uint32_t)w[d];
+                        mk_f4 x0 = xv[d * 2], x1 = xv[d * 2 + 1];
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1(wd & 15u), x0.x));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 4) & 15u), x0.y));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 8) & 15u), x0.z));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 12) & 15u), x0.w));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 16) & 15u), x1.x));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 20) & 15u), x1.y));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 24) & 15u), x1.z));
+                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 28) & 15u), x1.w));
+                    }
+                    acc[p] += __fmul_rn(gsum, s);
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            float v = mk_wave_sum(acc[p]);
+            if (lane == 0 && p0 + p < m) out[(size_t)(p0 + p) * rows + row] = v;
+        }
+    }
+}
+
+template <int NB>
+int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
+    constexpr int RT = lcm_c(NB, 64) / NB;
+    GemvArgs a = a0;
+    const int n_tiles = (a.rows + RT - 1) / RT;
+    // enough waves to fill 256 CUs several times over, but several tiles per
+    // wave so the activation staging is amortised
+    int tpw = 1;
+    while (tpw < 16 && (size_t)n_tiles * nmat / (tpw * 2) >= 256 * 4 * 4) tpw *= 2;
+    a.tiles_per_wave = tpw;
+    const unsigned gx = (unsigned)((n_tiles + 4 * tpw - 1) / (4 * tpw));
+    if (q8)
+        hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL(mxfp4_gemv_f32_kernel<NB>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a);
+    return mk_launch_status("mxfp4_gemv");
+}
+
+int launch_gemv(const GemvArgs &a, bool q8, size_t nmat, size_t cols, hipStream_t st) {
+    const int nb = (int)(cols / 32);
+    if (a.rows == 0 || nmat == 0) return MK_OK;
+    switch (nb) {
+        case 32: return launch_fast<32>(a, q8, nmat, st);
+        case 64: return launch_fast<64>(a, q8, nmat, st);
+        case 128: return launch_fast<128>(a, q8, nmat, st);
+        case 224: return launch_fast<224>(a, q8, nmat, st);
+        default: break;
+    }
+    const unsigned gx = (unsigned)((a.rows + 3) / 4);
+    if (q8)
+        hipLaunchKernelGGL(mxfp4_gemv_generic_kernel<true>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a, nb);
+    else
+        hipLaunchKernelGGL(mxfp4_gemv_generic_kernel<false>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a, nb);
+    return mk_launch_status("mxfp4_gemv_generic");
+}
+
+bool shape_ok(size_t rows, size_t cols) { return cols % 32 == 0 && cols > 0 && rows <= 0x7FFFFFFF / 64 && cols <= (1u << 24); }
+
+}  // namespace
+
+extern "C" int mk_dev_mxfp4_matvec_q8(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const int8_t *xq,
+                                      const float *xs, float *out, void *stream) {
+    MK_REQUIRE(packed && scales && xq && xs && out, "null pointer");
+    MK_REQUIRE(shape_ok(rows, cols), "cols must be a positive multiple of 32");
+    MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)xq & 3) == 0, "packed must be 16-byte and xq 4-byte aligned");
+    GemvArgs a = {};
+    a.packed = packed;
+    a.scales = scales;
+    a.out = out;
+    a.xq = xq;
+    a.xs = xs;
+    a.rows = (int)rows;
+    return launch_gemv(a, true, 1, cols, (hipStream_t)stream);
+}
+
+extern "C" int mk_dev_mxfp4_matvec_f32(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out,
+                                       void *stream) {
+    MK_REQUIRE(packed && scales && x && out, "null pointer");
+    MK_REQUIRE(shape_ok(rows, cols), "cols must be a positive multiple of 32");
+    MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)x & 15) == 0, "packed and x must be 16-byte aligned");
+    GemvArgs a = {};
+    a.packed = packed;
+    a.scales = scales;
+    a.out = out;
+    a.xf = x;
+    a.rows = (int)rows;
+    return launch_gemv(a, false, 1, cols, (hipStream_t)stream);
+}
+
+extern "C" int mk_dev_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out,
+                                   int mode, int8_t *xq_ws, float *xs_ws, void *stream) {
+    if (mode == MK_MODE_F32) return mk_dev_mxfp4_matvec_f32(packed, scales, rows, cols, x, out, stream);
+    MK_REQUIRE(mode == MK_MODE_Q8, "mode must be MK_MODE_F32 or MK_MODE_Q8");
+    MK_REQUIRE(xq_ws && xs_ws, "q8 mode needs the xq/xs scratch");
+    int s = mk_dev_quantize_q8(x, 1, cols, xq_ws, xs_ws, stream);
+    if (s != MK_OK) return s;
+    return mk_dev_mxfp4_matvec_q8(packed, scales, rows, cols, xq_ws, xs_ws, out, stream);
+}
+
+extern "C" int mk_dev_mxfp4_matvec_q8_grouped(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t nmat,
+                                              size_t rows, size_t cols, const int8_t *xq, const float *xs, const int32_t *x_index,
+                                              float *const *out_ptrs, void *stream) {
+    MK_REQUIRE(packed_ptrs && scales_ptrs && xq && xs && out_ptrs, "null pointer");
+    MK_REQUIRE(shape_ok(rows, cols), "cols must be a positive multiple of 32");
+    MK_REQUIRE(nmat <= 65535, "at most 65535 matrices per launch");
+    GemvArgs a = {};
+    a.packed_ptrs = packed_ptrs;
+    a.scales_ptrs = scales_ptrs;
+    a.out_ptrs = out_ptrs;
+    a.x_index = x_index;
+    a.xq = xq;
+    a.xs = xs;
+    a.rows = (int)rows;
+    return launch_gemv(a, true, nmat, cols, (hipStream_t)stream);
+}
+
+int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t nmat, size_t rows,
+                             size_t cols, const int8_t *xq, const float *xs, const float *xf, const int32_t *x_index, float *const *out_ptrs,
+                             hipStream_t st) {
+    GemvArgs a = {};
+    a.packed_ptrs = packed_ptrs;
+    a.scales_ptrs = scales_ptrs;
+    a.out_ptrs = out_ptrs;
+    a.x_index = x_index;
+    a.xq = xq;
+    a.xs = xs;
+    a.xf = xf;
+    a.rows = (int)rows;
+    return launch_gemv(a, q8, nmat, cols, st);
+}
+
+extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m,
+                                      float *out, void *stream) {
+    MK_REQUIRE(packed && scales && x && out, "null pointer");
+    MK_REQUIRE(shape_ok(rows, cols), "cols must be a positive multiple of 32");
+    MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)x & 15) == 0, "packed and x must be 16-byte aligned");
+    if (rows == 0 || m == 0) return MK_OK;
+    hipLaunchKernelGGL(mxfp4_gemv_nt_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, packed, scales, (int)rows,
+                       (int)(cols / 32), x, (int)m, out);
+    return mk_launch_status("mxfp4_gemv_nt");
+}

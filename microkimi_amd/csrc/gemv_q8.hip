@@ -1,0 +1,305 @@
+// q8_0 GEMV (Q8Head::matvec, src/model.rs:290-347) for gfx950: int8 weights
+// [rows][cols] + one scale per 32 (f16 storage form or f32), q8 activations.
+//
+// out[b][r] = sum_g (ws[r][g] * xs[b][g]) * idot(r, b, g), idot exact int32.
+//
+// batch 1   VALU path.  Lane l of wave iteration t owns the 16-byte half block
+//           t*64+l of the row (perfectly coalesced 1 KiB wave loads, no repack)
+//           and keeps the matching 16 activation bytes and block scale in
+//           registers for the whole kernel; 4 x v_dot4_i32_i8 per load.
+// batch 2-8 matrix-core path.  One v_mfma_i32_16x16x64_i8 per 16 rows x 64
+//           columns.  The MFMA sums over K = 64 = two q8 blocks, whose scales
+//           differ, so the activation operand is laid out as 16 "columns" =
+//           8 batch rows x 2 block parities, each holding the activation bytes of
+//           one block and zeros for the other: the 16x16 result then holds the
+//           per-block integer dots, and the per-block scale product is applied in
+//           f32 exactly as the reference does.  Weights are read once for the
+//           whole batch.
+// generic   one wave per row, any cols % 32 == 0, any batch <= 8.
+#include "mk_common.h"
+
+namespace {
+
+template <bool F16>
+__device__ __forceinline__ float load_scale(const void *scales, size_t idx) {
+    if (F16) return mk_f16_bits_to_f32(reinterpret_cast<const uint16_t *>(scales)[idx]);
+    return reinterpret_cast<const float *>(scales)[idx];
+}
+
+// ------------------------------------------------------------- batch 1
+template <int NB, bool F16>
+__global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows,
+                                                         const int8_t *__restrict__ xq, const float *__restrict__ xs,
+                                                         float *__restrict__ out, int rows_per_wave) {
+    constexpr int T = NB * 2 / 64;  // half blocks per row / 64 lanes
+    static_assert(NB % 32 == 0 && T >= 1 && T <= 8, "row shape not covered by the fast path");
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    mk_i4 xr[T];
+    float cf[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        const int hb = t * 64 + lane;
+        xr[t] = *reinterpret_cast<const mk_i4 *>(xq + hb * 16);
+        cf[t] = xs[hb >> 1];
+    }
+    const int r0 = wave * rows_per_wave;
+    const int r1 = min(r0 + rows_per_wave, rows);
+    mk_i4 w[T];
+    float ws[T];
+    auto load_row = [&](int r) {
+        const int8_t *row = q + (size_t)r * NB * 32;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const int hb = t * 64 + lane;
+            w[t] = *reinterpret_cast<const mk_i4 *>(row + hb * 16);
+            ws[t] = load_scale<F16>(scales, (size_t)r * NB + (hb >> 1));
+        }
+    };
+    if (r0 < r1) load_row(r0);
+    for (int r = r0; r < r1; r++) {
+        mk_i4 wc[T];
+        float wsc[T];
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            wc[t] = w[t];
+            wsc[t] = ws[t];
+        }
+        if (r + 1 < r1) load_row(r + 1);
+        float acc = 0.0f;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            int d = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) d = __builtin_amdgcn_sdot4(wc[t][k], xr[t][k], d, false);
+            acc += (wsc[t] * cf[t]) * (float)d;
+        }
+        acc = mk_wave_sum(acc);
+        if (lane == 0) out[r] = acc;
+    }
+}
+
+// ------------------------------------------------------- batch 2..8 (MFMA)
+// Workgroup: 512 threads = 8 waves; LDS holds the batch's activation bytes in
+// the operand order ([K/16 chunks][8 batch rows][16 bytes]) and the activation
+// block scales ([NB][8]).  Each wave walks 16-row groups.
+template <bool F16>
+__global__ __launch_bounds__(512) void q8_gemv_mfma_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows, int nb,
+                                                           const int8_t *__restrict__ xq, const float *__restrict__ xs, int batch,
+                                                           float *__restrict__ out, int groups_per_wave) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int cols = nb * 32;
+    mk_i4 *xl = reinterpret_cast<mk_i4 *>(lds);                      // [cols/16][8]
+    float *xsl = reinterpret_cast<float *>(lds + (size_t)cols * 8);  // [nb][8]
+    for (int i = threadIdx.x; i < (cols / 16) * 8; i += 512) {
+        const int c = i >> 3, b = i & 7;
+        mk_i4 v = {0, 0, 0, 0};
+        if (b < batch) v = *reinterpret_cast<const mk_i4 *>(xq + (size_t)b * cols + c * 16);
+        xl[i] = v;
+    }
+    for (int i = threadIdx.x; i < nb * 8; i += 512) {
+        const int g = i >> 3, b = i & 7;
+        xsl[i] = b < batch ? xs[(size_t)b * nb + g] : 0.0f;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 15;   // weight row inside the group (B operand column / result column)
+    const int kb = lane >> 4;  // 16-byte K chunk inside the 64-wide step; also the result row group
+    const int par = kb >> 1;   // which of the step's two q8 blocks this lane's result rows belong to
+    const int a_batch = n & 7, a_par = n >> 3;  // A operand row m = n: batch row and block parity
+    const bool a_live = (kb >> 1) == a_par;
+    const int steps = nb / 2;
+    const int wave = blockIdx.x * 8 + (threadIdx.x >> 6);
+    const int n_groups = (rows + 15) / 16;
+    const int g0 = wave * groups_per_wave, g1 = min(g0 + groups_per_wave, n_groups);
+    for (int grp = g0; grp < g1; grp++) {
+        const int row = grp * 16 + n;
+        const bool row_ok = row < rows;
+        const int8_t *wrow = q + (size_t)(row_ok ? row : 0) * cols + kb * 16;
+        const size_t srow = (size_t)(row_ok ? row : 0) * nb + par;
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 4
+        for (int s = 0; s < steps; s++) {
+            mk_i4 wv = *reinterpret_cast<const mk_i4 *>(wrow + s * 64);
+            float wsf = load_scale<F16>(scales, srow + 2 * s);
+            mk_i4 xa = xl[(s * 4 + kb) * 8 + a_batch];
+            if (!a_live) xa = mk_i4{0, 0, 0, 0};
+            mk_i4 c = {0, 0, 0, 0};
+            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wv, c, 0, 0, 0);
+            const mk_f4 x4 = *reinterpret_cast<const mk_f4 *>(xsl + (2 * s + par) * 8 + 4 * (kb & 1));
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] += (wsf * x4[i]) * (float)c[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32, MK_WAVE);  // the two block parities
+        if (lane < 32 && row_ok) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int b = 4 * (kb & 1) + i;
+                if (b < batch) out[(size_t)b * rows + row] = acc[i];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- generic
+template <bool F16>
+__global__ __launch_bounds__(256) void q8_gemv_generic_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows, int nb,
+                                                              const int8_t *__restrict__ xq, const float *__restrict__ xs, int batch,
+                                                              float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const size_t cols = (size_t)nb * 32;
+    float acc[8];
+#pragma unroll
+    for (int b = 0; b < 8; b++) acc[b] = 0.0f;
+    for (int hb = lane; hb < nb * 2; hb += 64) {
+        mk_i4 w = *reinterpret_cast<const mk_i4 *>(q + (size_t)row * cols + hb * 16);
+        float wsf = load_scale<F16>(scales, (size_t)row * nb + (hb >> 1));
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            if (b < batch) {
+                mk_i4 x = *reinterpret_cast<const mk_i4 *>(xq + (size_t)b * cols + hb * 16);
+                int d = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) d = __builtin_amdgcn_sdot4(w[k], x[k], d, false);
+                acc[b] += (wsf * xs[(size_t)b * nb + (hb >> 1)]) * (float)d;
+            }
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        if (b < batch) {
+            float v = mk_wave_sum(acc[b]);
+            if (lane == 0) out[(size_t)b * rows + row] = v;
+        }
+    }
+}
+
+// ----------------------------------------------------------------- argmax
+// Greedy token: largest value, ties to the lowest index (the strict '>' of
+// top_k_probs, src/model.rs:3283-3287).  Stage 1: up to 1024 blocks per row
+// write (value, index) partials; stage 2: one block per row folds them.
+__device__ __forceinline__ void argmax_fold(float &bv, int &bi, float v, int i) {
+    if (v > bv || (v == bv && i < bi)) {
+        bv = v;
+        bi = i;
+    }
+}
+
+__device__ void argmax_block_reduce(float &bv, int &bi) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        float ov = __shfl_xor(bv, off, MK_WAVE);
+        int oi = __shfl_xor(bi, off, MK_WAVE);
+        argmax_fold(bv, bi, ov, oi);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        sv[wave] = bv;
+        si[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) argmax_fold(bv, bi, sv[w], si[w]);
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_stage1_kernel(const float *__restrict__ logits, int n, int chunk, float *__restrict__ pv,
+                                                            int *__restrict__ pi) {
+    const int b = blockIdx.y;
+    const float *row = logits + (size_t)b * n;
+    const int i0 = blockIdx.x * chunk, i1 = min(i0 + chunk, n);
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = i0 + threadIdx.x; i < i1; i += 256) argmax_fold(bv, bi, row[i], i);
+    argmax_block_reduce(bv, bi);
+    if (threadIdx.x == 0) {
+        pv[b * gridDim.x + blockIdx.x] = bv;
+        pi[b * gridDim.x + blockIdx.x] = bi;
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_stage2_kernel(const float *__restrict__ pv, const int *__restrict__ pi, int parts,
+                                                            int32_t *__restrict__ out) {
+    const int b = blockIdx.x;
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < parts; i += 256) argmax_fold(bv, bi, pv[b * parts + i], pi[b * parts + i]);
+    argmax_block_reduce(bv, bi);
+    if (threadIdx.x == 0) out[b] = bi == 0x7FFFFFFF ? 0 : bi;
+}
+
+template <int NB, bool F16>
+void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
+    // about 8 waves per SIMD-slot on 256 CUs, at least 4 rows per wave to amortise the activation registers
+    int rpw = (rows + 256 * 16 - 1) / (256 * 16);
+    if (rpw < 4) rpw = 4;
+    const int waves = (rows + rpw - 1) / rpw;
+    hipLaunchKernelGGL((q8_gemv_b1_kernel<NB, F16>), dim3((waves + 3) / 4), dim3(256), 0, st, q, scales, rows, xq, xs, out, rpw);
+}
+
+template <bool F16>
+int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, const int8_t *xq, const float *xs, size_t batch, float *out,
+              hipStream_t st) {
+    const int nb = (int)(cols / 32);
+    if (batch == 1) {
+        switch (nb) {
+            case 32: launch_b1<32, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
+            case 64: launch_b1<64, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
+            case 128: launch_b1<128, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
+            case 224: launch_b1<224, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
+            default: break;
+        }
+    } else if (nb % 2 == 0 && cols * 8 + (size_t)nb * 32 <= 150 * 1024) {
+        const int n_groups = (int)((rows + 15) / 16);
+        int gpw = (n_groups + 256 * 16 - 1) / (256 * 16);
+        if (gpw < 1) gpw = 1;
+        const int waves = (n_groups + gpw - 1) / gpw;
+        const size_t lds = cols * 8 + (size_t)nb * 32;
+        hipLaunchKernelGGL(q8_gemv_mfma_kernel<F16>, dim3((waves + 7) / 8), dim3(512), lds, st, q, scales, (int)rows, nb, xq, xs, (int)batch,
+                           out, gpw);
+        return mk_launch_status("q8_gemv_mfma");
+    }
+    hipLaunchKernelGGL(q8_gemv_generic_kernel<F16>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, q, scales, (int)rows, nb, xq, xs,
+                       (int)batch, out);
+    return mk_launch_status("q8_gemv_generic");
+}
+
+}  // namespace
+
+extern "C" int mk_dev_q8_matvec(const int8_t *q, const void *scales, int scales_f16, size_t rows, size_t cols, const int8_t *xq,
+                                const float *xs, size_t batch, float *out, void *stream) {
+    MK_REQUIRE(q && scales && xq && xs && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0 && cols > 0, "cols must be a positive multiple of 32");
+    MK_REQUIRE(batch >= 1 && batch <= 8, "batch must be 1..8");
+    MK_REQUIRE(rows <= 0x7FFFFFF0u && cols <= (1u << 24), "shape too large");
+    MK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)xq & 15) == 0, "q and xq must be 16-byte aligned");
+    if (rows == 0) return MK_OK;
+    static bool lds_opt_in = false;
+    if (!lds_opt_in) {
+        // the batch kernel stages up to 150 KiB of activations in the 160 KiB LDS
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        lds_opt_in = true;
+    }
+    if (scales_f16) return launch_q8<true>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);
+    return launch_q8<false>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);
+}
+
+extern "C" int mk_dev_argmax(const float *logits, size_t batch, size_t n, void *ws, int32_t *out_idx, void *stream) {
+    MK_REQUIRE(logits && ws && out_idx, "null pointer");
+    MK_REQUIRE(batch >= 1 && batch <= 65535 && n >= 1 && n <= 0x7FFFFFF0u, "bad shape");
+    int parts = (int)((n + 4095) / 4096);
+    if (parts > 1024) parts = 1024;
+    const int chunk = (int)((n + parts - 1) / parts);
+    float *pv = reinterpret_cast<float *>(ws);
+    int *pi = reinterpret_cast<int *>(pv + batch * 1024);
+    hipLaunchKernelGGL(argmax_stage1_kernel, dim3(parts, (unsigned)batch), dim3(256), 0, (hipStream_t)stream, logits, (int)n, chunk, pv, pi);
+    hipLaunchKernelGGL(argmax_stage2_kernel, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, pv, pi, parts, out_idx);
+    return mk_launch_status("argmax");
+}

@@ -1,0 +1,498 @@
+// Host side of libmk_hip.so: device context, error reporting, the pointer-keyed
+// weight cache and the host-slice entry points that stand where the reference's
+// Metal calls stand (src/metal.rs:441-451,599-665,874-1017).
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <vector>
+
+#include "mk_common.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+std::mutex g_mu;  // serialises host-level calls (the reference's io mutex)
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    int ensure(size_t bytes) {
+        if (bytes <= cap) return MK_OK;
+        if (p) hipFree(p);
+        p = nullptr;
+        cap = 0;
+        size_t want = bytes < 4096 ? 4096 : bytes;
+        if (mk_check_hip(hipMalloc(&p, want), "hipMalloc(staging)") != MK_OK) return MK_ERR_NOMEM;
+        cap = want;
+        return MK_OK;
+    }
+};
+
+struct CachedWeight {
+    void *packed = nullptr;
+    void *scales = nullptr;
+    size_t bytes = 0;
+};
+
+struct Ctx {
+    bool ready = false;
+    int status = MK_ERR_NO_DEVICE;
+    int device = -1;
+    hipStream_t stream = nullptr;
+    size_t cache_cap = 0;  // bytes, 0 = unlimited
+    size_t cache_bytes = 0;
+    std::map<std::tuple<const void *, size_t, size_t>, CachedWeight> cache;
+    DevBuf x, y, xq, xs, tmp;
+    int force_q8 = -1;
+};
+Ctx g_ctx;
+
+int ensure_init() {
+    if (g_ctx.ready) return MK_OK;
+    return mk_init(0);
+}
+
+}  // namespace
+
+void mk_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int mk_check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return MK_OK;
+    mk_set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+    return MK_ERR_HIP;
+}
+
+int mk_launch_status(const char *kernel) {
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return MK_OK;
+    mk_set_error("launch of %s failed: %d (%s)", kernel, (int)e, hipGetErrorString(e));
+    return MK_ERR_HIP;
+}
+
+extern "C" const char *mk_last_error(void) { return g_err; }
+
+extern "C" int mk_init(int device) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_ctx.ready) return MK_OK;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        mk_set_error("no HIP device visible");
+        return g_ctx.status = MK_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= n) {
+        mk_set_error("device %d out of range (%d visible)", device, n);
+        return g_ctx.status = MK_ERR_NO_DEVICE;
+    }
+    hipDeviceProp_t prop;
+    if (mk_check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties") != MK_OK) return g_ctx.status = MK_ERR_NO_DEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        mk_set_error("device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+        return g_ctx.status = MK_ERR_NO_DEVICE;
+    }
+    if (mk_check_hip(hipSetDevice(device), "hipSetDevice") != MK_OK) return g_ctx.status = MK_ERR_HIP;
+    if (mk_check_hip(hipStreamCreate(&g_ctx.stream), "hipStreamCreate") != MK_OK) return g_ctx.status = MK_ERR_HIP;
+    const char *mb = getenv("MK_GPU_CACHE_MB");
+    if (mb && *mb) g_ctx.cache_cap = (size_t)strtoull(mb, nullptr, 10) << 20;
+    g_ctx.device = device;
+    g_ctx.ready = true;
+    return g_ctx.status = MK_OK;
+}
+
+extern "C" int mk_available(void) { return g_ctx.ready ? 1 : 0; }
+
+extern "C" void mk_shutdown(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_ctx.ready) return;
+    hipStreamSynchronize(g_ctx.stream);
+    for (auto &kv : g_ctx.cache) {
+        hipFree(kv.second.packed);
+        hipFree(kv.second.scales);
+    }
+    g_ctx.cache.clear();
+    g_ctx.cache_bytes = 0;
+    for (DevBuf *b : {&g_ctx.x, &g_ctx.y, &g_ctx.xq, &g_ctx.xs, &g_ctx.tmp}) {
+        if (b->p) hipFree(b->p);
+        b->p = nullptr;
+        b->cap = 0;
+    }
+    hipStreamDestroy(g_ctx.stream);
+    g_ctx.stream = nullptr;
+    g_ctx.ready = false;
+    g_ctx.status = MK_ERR_NO_DEVICE;
+}
+
+extern "C" void mk_set_cache_mb(size_t mb) { g_ctx.cache_cap = mb << 20; }
+
+extern "C" void mk_force_q8(int v) { g_ctx.force_q8 = v < 0 ? -1 : (v ? 1 : 0); }
+
+extern "C" int mk_q8_enabled(void) {
+    if (g_ctx.force_q8 >= 0) return g_ctx.force_q8;
+    const char *e = getenv("MICROKIMI_NO_Q8");
+    return (e && strcmp(e, "1") == 0) ? 0 : 1;
+}
+
+namespace {
+
+// (host pointer, rows, cols) -> device copy, uploaded on first use; a hit is
+// re-validated against the first 16 host bytes because a freed host buffer can
+// come back at the same address with other contents (src/metal.rs:417-430).
+int cached_weight(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, CachedWeight *out) {
+    const size_t pb = rows * cols / 2, sb = rows * cols / 32;
+    auto key = std::make_tuple((const void *)packed, rows, cols);
+    auto it = g_ctx.cache.find(key);
+    if (it != g_ctx.cache.end()) {
+        uint8_t head[16];
+        size_t nh = pb < 16 ? pb : 16;
+        MK_HIP_TRY(hipMemcpyAsync(head, it->second.packed, nh, hipMemcpyDeviceToHost, g_ctx.stream));
+        MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+        if (memcmp(head, packed, nh) == 0) {
+            *out = it->second;
+            return MK_OK;
+        }
+        hipFree(it->second.packed);
+        hipFree(it->second.scales);
+        g_ctx.cache_bytes -= it->second.bytes;
+        g_ctx.cache.erase(it);
+    }
+    if (g_ctx.cache_cap && g_ctx.cache_bytes + pb + sb > g_ctx.cache_cap) {
+        mk_set_error("device weight cache budget exhausted (%zu MiB)", g_ctx.cache_cap >> 20);
+        return MK_ERR_NOMEM;
+    }
+    CachedWeight w;
+    if (mk_check_hip(hipMalloc(&w.packed, pb ? pb : 16), "hipMalloc(weight)") != MK_OK) return MK_ERR_NOMEM;
+    if (mk_check_hip(hipMalloc(&w.scales, sb ? sb : 16), "hipMalloc(weight scales)") != MK_OK) {
+        hipFree(w.packed);
+        return MK_ERR_NOMEM;
+    }
+    w.bytes = pb + sb;
+    int s = mk_check_hip(hipMemcpyAsync(w.packed, packed, pb, hipMemcpyHostToDevice, g_ctx.stream), "upload packed");
+    if (s == MK_OK) s = mk_check_hip(hipMemcpyAsync(w.scales, scales, sb, hipMemcpyHostToDevice, g_ctx.stream), "upload scales");
+    if (s == MK_OK) s = mk_check_hip(hipStreamSynchronize(g_ctx.stream), "upload sync");
+    if (s != MK_OK) {
+        hipFree(w.packed);
+        hipFree(w.scales);
+        return s;
+    }
+    g_ctx.cache[key] = w;
+    g_ctx.cache_bytes += w.bytes;
+    *out = w;
+    return MK_OK;
+}
+
+}  // namespace
+
+extern "C" int mk_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out) {
+    MK_REQUIRE(packed && scales && x && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0 && cols > 0, "cols must be a positive multiple of 32");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    if (rows == 0) return MK_OK;
+    std::lock_guard<std::mutex> lk(g_mu);
+    CachedWeight w;
+    if ((s = cached_weight(packed, scales, rows, cols, &w)) != MK_OK) return s;
+    if ((s = g_ctx.x.ensure(cols * 4)) != MK_OK) return s;
+    if ((s = g_ctx.y.ensure(rows * 4)) != MK_OK) return s;
+    if ((s = g_ctx.xq.ensure(cols)) != MK_OK) return s;
+    if ((s = g_ctx.xs.ensure(cols / 32 * 4)) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(g_ctx.x.p, x, cols * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    s = mk_dev_mxfp4_matvec((const uint8_t *)w.packed, (const uint8_t *)w.scales, rows, cols, (const float *)g_ctx.x.p, (float *)g_ctx.y.p,
+                            mk_q8_enabled() ? MK_MODE_Q8 : MK_MODE_F32, (int8_t *)g_ctx.xq.p, (float *)g_ctx.xs.p, g_ctx.stream);
+    if (s != MK_OK) return s;
+    std::vector<float> host(rows);  // `out` stays untouched unless everything succeeded
+    MK_HIP_TRY(hipMemcpyAsync(host.data(), g_ctx.y.p, rows * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    memcpy(out, host.data(), rows * 4);
+    return MK_OK;
+}
+
+extern "C" int mk_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out) {
+    MK_REQUIRE(packed && scales && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0, "cols must be a multiple of 32");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    if (rows * cols == 0) return MK_OK;
+    std::lock_guard<std::mutex> lk(g_mu);
+    const size_t pb = rows * cols / 2, sb = rows * cols / 32;
+    if ((s = g_ctx.tmp.ensure(pb + sb + 16)) != MK_OK) return s;
+    if ((s = g_ctx.y.ensure(rows * cols * 4)) != MK_OK) return s;
+    uint8_t *dp = (uint8_t *)g_ctx.tmp.p, *ds = dp + ((pb + 15) & ~(size_t)15);
+    MK_HIP_TRY(hipMemcpyAsync(dp, packed, pb, hipMemcpyHostToDevice, g_ctx.stream));
+    MK_HIP_TRY(hipMemcpyAsync(ds, scales, sb, hipMemcpyHostToDevice, g_ctx.stream));
+    if ((s = mk_dev_mxfp4_dequant(dp, ds, rows, cols, (float *)g_ctx.y.p, g_ctx.stream)) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(out, g_ctx.y.p, rows * cols * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    return MK_OK;
+}
+
+extern "C" int mk_quantize_q8(const float *x, size_t n, int8_t *q, float *scales) {
+    MK_REQUIRE(x && q && scales, "null pointer");
+    MK_REQUIRE(n % 32 == 0, "q8 blocks are 32 wide");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    if (n == 0) return MK_OK;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if ((s = g_ctx.x.ensure(n * 4)) != MK_OK) return s;
+    if ((s = g_ctx.xq.ensure(n)) != MK_OK) return s;
+    if ((s = g_ctx.xs.ensure(n / 32 * 4)) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(g_ctx.x.p, x, n * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    if ((s = mk_dev_quantize_q8((const float *)g_ctx.x.p, 1, n, (int8_t *)g_ctx.xq.p, (float *)g_ctx.xs.p, g_ctx.stream)) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(q, g_ctx.xq.p, n, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipMemcpyAsync(scales, g_ctx.xs.p, n / 32 * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    return MK_OK;
+}
+
+// ------------------------------------------------------------------ Q8Head
+struct mk_q8head {
+    int8_t *q = nullptr;
+    void *scales = nullptr;
+    int f16 = 0;
+    size_t rows = 0, cols = 0;
+    DevBuf x, xq, xs, y, ws, idx;
+};
+
+extern "C" void mk_q8head_free(mk_q8head *h) {
+    if (!h) return;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (h->q) hipFree(h->q);
+    if (h->scales) hipFree(h->scales);
+    for (DevBuf *b : {&h->x, &h->xq, &h->xs, &h->y, &h->ws, &h->idx})
+        if (b->p) hipFree(b->p);
+    delete h;
+}
+
+namespace {
+int q8head_alloc(size_t rows, size_t cols, int f16, mk_q8head **out) {
+    mk_q8head *h = new mk_q8head();
+    h->rows = rows;
+    h->cols = cols;
+    h->f16 = f16 ? 1 : 0;
+    const size_t nsc = rows * cols / 32;
+    if (mk_check_hip(hipMalloc((void **)&h->q, rows * cols + 16), "hipMalloc(q8 head)") != MK_OK ||
+        mk_check_hip(hipMalloc(&h->scales, nsc * (f16 ? 2 : 4) + 16), "hipMalloc(q8 head scales)") != MK_OK) {
+        if (h->q) hipFree(h->q);
+        delete h;
+        return MK_ERR_NOMEM;
+    }
+    *out = h;
+    return MK_OK;
+}
+}  // namespace
+
+extern "C" int mk_q8head_from_f32(const float *w, size_t rows, size_t cols, int scales_f16, mk_q8head **out) {
+    MK_REQUIRE(w && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0, "cols must be a positive multiple of 32");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    std::lock_guard<std::mutex> lk(g_mu);
+    mk_q8head *h = nullptr;
+    if ((s = q8head_alloc(rows, cols, scales_f16, &h)) != MK_OK) return s;
+    // quantize on the device in row chunks of at most 256 MiB of f32
+    size_t chunk = (256u << 20) / (cols * 4);
+    if (chunk == 0) chunk = 1;
+    if (chunk > rows) chunk = rows;
+    s = g_ctx.tmp.ensure(chunk * cols * 4);
+    for (size_t r0 = 0; s == MK_OK && r0 < rows; r0 += chunk) {
+        size_t nr = rows - r0 < chunk ? rows - r0 : chunk;
+        s = mk_check_hip(hipMemcpyAsync(g_ctx.tmp.p, w + r0 * cols, nr * cols * 4, hipMemcpyHostToDevice, g_ctx.stream), "upload f32 rows");
+        if (s == MK_OK)
+            s = mk_dev_q8head_from_f32((const float *)g_ctx.tmp.p, nr, cols, h->q + r0 * cols,
+                                       (uint8_t *)h->scales + r0 * (cols / 32) * (scales_f16 ? 2 : 4), scales_f16, g_ctx.stream);
+        if (s == MK_OK) s = mk_check_hip(hipStreamSynchronize(g_ctx.stream), "quantize sync");
+    }
+    if (s != MK_OK) {
+        hipFree(h->q);
+        hipFree(h->scales);
+        delete h;
+        return s;
+    }
+    *out = h;
+    return MK_OK;
+}
+
+extern "C" int mk_q8head_from_q8(const int8_t *q, const float *scales, size_t rows, size_t cols, int scales_f16, mk_q8head **out) {
+    MK_REQUIRE(q && scales && out, "null pointer");
+    MK_REQUIRE(cols % 32 == 0 && cols > 0 && rows > 0, "cols must be a positive multiple of 32");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    std::lock_guard<std::mutex> lk(g_mu);
+    mk_q8head *h = nullptr;
+    if ((s = q8head_alloc(rows, cols, scales_f16, &h)) != MK_OK) return s;
+    const size_t nsc = rows * cols / 32;
+    s = mk_check_hip(hipMemcpyAsync(h->q, q, rows * cols, hipMemcpyHostToDevice, g_ctx.stream), "upload q8 rows");
+    std::vector<uint16_t> half;
+    if (s == MK_OK) {
+        if (scales_f16) {
+            half.resize(nsc);
+            for (size_t i = 0; i < nsc; i++) {
+                _Float16 hv = (_Float16)scales[i];
+                memcpy(&half[i], &hv, 2);
+            }
+            s = mk_check_hip(hipMemcpyAsync(h->scales, half.data(), nsc * 2, hipMemcpyHostToDevice, g_ctx.stream), "upload f16 scales");
+        } else {
+            s = mk_check_hip(hipMemcpyAsync(h->scales, scales, nsc * 4, hipMemcpyHostToDevice, g_ctx.stream), "upload f32 scales");
+        }
+    }
+    if (s == MK_OK) s = mk_check_hip(hipStreamSynchronize(g_ctx.stream), "upload sync");
+    if (s != MK_OK) {
+        hipFree(h->q);
+        hipFree(h->scales);
+        delete h;
+        return s;
+    }
+    *out = h;
+    return MK_OK;
+}
+
+extern "C" int mk_q8head_matvec(mk_q8head *h, const float *x, size_t batch, float *out, int32_t *argmax_out) {
+    MK_REQUIRE(h && x && out, "null pointer");
+    MK_REQUIRE(batch >= 1, "batch must be at least 1");
+    std::lock_guard<std::mutex> lk(g_mu);
+    int s;
+    if ((s = h->x.ensure(batch * h->cols * 4)) != MK_OK) return s;
+    if ((s = h->xq.ensure(batch * h->cols)) != MK_OK) return s;
+    if ((s = h->xs.ensure(batch * h->cols / 32 * 4)) != MK_OK) return s;
+    if ((s = h->y.ensure(batch * h->rows * 4)) != MK_OK) return s;
+    if ((s = h->ws.ensure(2 * batch * 1024 * 4)) != MK_OK) return s;
+    if ((s = h->idx.ensure(batch * 4)) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(h->x.p, x, batch * h->cols * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    if ((s = mk_dev_quantize_q8((const float *)h->x.p, batch, h->cols, (int8_t *)h->xq.p, (float *)h->xs.p, g_ctx.stream)) != MK_OK) return s;
+    for (size_t b0 = 0; b0 < batch; b0 += 8) {
+        size_t nb = batch - b0 < 8 ? batch - b0 : 8;
+        s = mk_dev_q8_matvec(h->q, h->scales, h->f16, h->rows, h->cols, (const int8_t *)h->xq.p + b0 * h->cols,
+                             (const float *)h->xs.p + b0 * (h->cols / 32), nb, (float *)h->y.p + b0 * h->rows, g_ctx.stream);
+        if (s != MK_OK) return s;
+    }
+    if (argmax_out) {
+        if ((s = mk_dev_argmax((const float *)h->y.p, batch, h->rows, h->ws.p, (int32_t *)h->idx.p, g_ctx.stream)) != MK_OK) return s;
+    }
+    std::vector<float> host(batch * h->rows);
+    std::vector<int32_t> hidx(batch);
+    MK_HIP_TRY(hipMemcpyAsync(host.data(), h->y.p, batch * h->rows * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    if (argmax_out) MK_HIP_TRY(hipMemcpyAsync(hidx.data(), h->idx.p, batch * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    memcpy(out, host.data(), batch * h->rows * 4);
+    if (argmax_out) memcpy(argmax_out, hidx.data(), batch * 4);
+    return MK_OK;
+}
+
+// --------------------------------------------------------------- MLA cache
+struct mk_mla_cache {
+    size_t nh = 0, L = 0, R = 0, cap = 0, n = 0;
+    int8_t *lat_q = nullptr, *rope_q = nullptr;
+    void *lat_s = nullptr, *rope_s = nullptr;
+    DevBuf in, q, out, ws;
+};
+
+extern "C" void mk_mla_cache_free(mk_mla_cache *c) {
+    if (!c) return;
+    std::lock_guard<std::mutex> lk(g_mu);
+    for (void *p : {(void *)c->lat_q, (void *)c->rope_q, c->lat_s, c->rope_s})
+        if (p) hipFree(p);
+    for (DevBuf *b : {&c->in, &c->q, &c->out, &c->ws})
+        if (b->p) hipFree(b->p);
+    delete c;
+}
+
+extern "C" int mk_mla_cache_new(size_t nh, size_t L, size_t R, size_t capacity, mk_mla_cache **out) {
+    MK_REQUIRE(out, "null pointer");
+    MK_REQUIRE(nh > 0 && L % 32 == 0 && R % 32 == 0 && L > 0 && capacity > 0, "bad cache shape");
+    int s = ensure_init();
+    if (s != MK_OK) return s;
+    std::lock_guard<std::mutex> lk(g_mu);
+    mk_mla_cache *c = new mk_mla_cache();
+    c->nh = nh;
+    c->L = L;
+    c->R = R;
+    c->cap = capacity;
+    bool ok = hipMalloc((void **)&c->lat_q, capacity * L + 64) == hipSuccess && hipMalloc(&c->lat_s, capacity * (L / 32) * 2 + 64) == hipSuccess &&
+              hipMalloc((void **)&c->rope_q, capacity * (R ? R : 1) + 64) == hipSuccess &&
+              hipMalloc(&c->rope_s, capacity * (R / 32 + 1) * 2 + 64) == hipSuccess;
+    if (!ok) {
+        mk_set_error("hipMalloc(mla cache) failed");
+        for (void *p : {(void *)c->lat_q, (void *)c->rope_q, c->lat_s, c->rope_s})
+            if (p) hipFree(p);
+        delete c;
+        return MK_ERR_NOMEM;
+    }
+    *out = c;
+    return MK_OK;
+}
+
+extern "C" size_t mk_mla_cache_positions(const mk_mla_cache *c) { return c ? c->n : 0; }
+
+extern "C" int mk_mla_cache_push(mk_mla_cache *c, const float *latent, const float *rope) {
+    MK_REQUIRE(c && latent && (rope || c->R == 0), "null pointer");
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (c->n >= c->cap) {
+        mk_set_error("mla cache full (%zu positions)", c->cap);
+        return MK_ERR_NOMEM;
+    }
+    int s;
+    if ((s = c->in.ensure((c->L + c->R) * 4)) != MK_OK) return s;
+    float *dl = (float *)c->in.p, *dr = dl + c->L;
+    MK_HIP_TRY(hipMemcpyAsync(dl, latent, c->L * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    if (c->R) MK_HIP_TRY(hipMemcpyAsync(dr, rope, c->R * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    if ((s = mk_dev_mla_cache_append(dl, dr, c->L, c->R, c->n, c->lat_q, c->lat_s, c->rope_q, c->rope_s, g_ctx.stream)) != MK_OK) return s;
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    c->n++;
+    return MK_OK;
+}
+
+extern "C" int mk_mla_cache_to_f32(const mk_mla_cache *c, float *latent, float *rope) {
+    MK_REQUIRE(c && latent && (rope || c->R == 0), "null pointer");
+    std::lock_guard<std::mutex> lk(g_mu);
+    const size_t n = c->n, L = c->L, R = c->R;
+    if (n == 0) return MK_OK;
+    std::vector<int8_t> lq(n * L), rq(n * R);
+    std::vector<uint16_t> ls(n * L / 32), rs(n * R / 32);
+    MK_HIP_TRY(hipMemcpyAsync(lq.data(), c->lat_q, n * L, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipMemcpyAsync(ls.data(), c->lat_s, n * L / 32 * 2, hipMemcpyDeviceToHost, g_ctx.stream));
+    if (R) {
+        MK_HIP_TRY(hipMemcpyAsync(rq.data(), c->rope_q, n * R, hipMemcpyDeviceToHost, g_ctx.stream));
+        MK_HIP_TRY(hipMemcpyAsync(rs.data(), c->rope_s, n * R / 32 * 2, hipMemcpyDeviceToHost, g_ctx.stream));
+    }
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    // the byte-level dequantization q * s of MlaCache::to_f32 (src/model.rs:1641-1646)
+    auto h2f = [](uint16_t b) {
+        _Float16 h;
+        memcpy(&h, &b, 2);
+        return (float)h;
+    };
+    for (size_t i = 0; i < n * L; i++) latent[i] = (float)lq[i] * h2f(ls[i / 32]);
+    for (size_t i = 0; i < n * R; i++) rope[i] = (float)rq[i] * h2f(rs[i / 32]);
+    return MK_OK;
+}
+
+extern "C" int mk_mla_attn(mk_mla_cache *c, const float *q, float scale, float *out) {
+    MK_REQUIRE(c && q && out, "null pointer");
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (c->n == 0) {
+        mk_set_error("mla cache is empty");
+        return MK_ERR_INVALID;
+    }
+    int s;
+    const size_t qn = c->nh * (c->L + c->R), on = c->nh * c->L;
+    if ((s = c->q.ensure(qn * 4)) != MK_OK) return s;
+    if ((s = c->out.ensure(on * 4)) != MK_OK) return s;
+    if ((s = c->ws.ensure(mk_mla_decode_workspace_bytes(c->nh, c->L, c->cap))) != MK_OK) return s;
+    MK_HIP_TRY(hipMemcpyAsync(c->q.p, q, qn * 4, hipMemcpyHostToDevice, g_ctx.stream));
+    if ((s = mk_dev_mla_q8_decode(c->lat_q, c->lat_s, c->rope_q, c->rope_s, c->n - 1, (const float *)c->q.p, c->nh, c->L, c->R, scale,
+                                  c->ws.p, (float *)c->out.p, g_ctx.stream)) != MK_OK)
+        return s;
+    std::vector<float> host(on);
+    MK_HIP_TRY(hipMemcpyAsync(host.data(), c->out.p, on * 4, hipMemcpyDeviceToHost, g_ctx.stream));
+    MK_HIP_TRY(hipStreamSynchronize(g_ctx.stream));
+    memcpy(out, host.data(), on * 4);
+    return MK_OK;
+}

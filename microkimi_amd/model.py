@@ -1,0 +1,188 @@
+"""Host mirror of the hot-path operators inside src/model.rs and src/deepseek.rs:
+Q8Head, MlaCache + mla_attn_flash_q8_mqa, matvec_packed_nt, the MoE expert section."""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib, q8 as _q8
+from ._lib import ACT_SWIGLU, MODE_F32, MODE_Q8, ExpertTable, check, cur_stream, hptr, lib, ptr
+
+
+class Q8Head:
+    """model::Q8Head (src/model.rs:261-348) resident on the device.
+
+    from_f32 / from_q8 take device tensors; matvec takes x [batch, cols] f32 on the device and returns logits
+    [batch, rows].  scales_f16 selects the q8_0 storage form (f16 scales) or the reference's f32 scales."""
+
+    def __init__(self, q, scales, rows, cols):
+        self.q, self.scales, self.rows, self.cols = q, scales, rows, cols
+        import torch
+        self.scales_f16 = scales.dtype == torch.float16
+
+    @staticmethod
+    def from_f32(w, rows, cols, scales_f16=True):
+        import torch
+        if cols % 32 != 0:
+            raise ValueError("q8 blocks are 32 wide")
+        _lib.require_device()
+        q = torch.empty((rows, cols), dtype=torch.int8, device=w.device)
+        s = torch.empty((rows, cols // 32), dtype=torch.float16 if scales_f16 else torch.float32, device=w.device)
+        check(lib.mk_dev_q8head_from_f32(ptr(w.contiguous()), rows, cols, ptr(q), ptr(s), int(scales_f16), cur_stream()))
+        return Q8Head(q, s, rows, cols)
+
+    @staticmethod
+    def from_q8(q, scales, rows, cols):
+        return Q8Head(q.contiguous(), scales.contiguous(), rows, cols)
+
+    def matvec_q8(self, xq, out=None):
+        """Rows against already-quantized activations (Q8Head::row_dot, src/model.rs:337-347)."""
+        import torch
+        batch = xq.q.numel() // self.cols
+        if out is None:
+            out = torch.empty((batch, self.rows), dtype=torch.float32, device=self.q.device)
+        for b0 in range(0, batch, 8):
+            nb = min(8, batch - b0)
+            check(lib.mk_dev_q8_matvec(ptr(self.q), ptr(self.scales), int(self.scales_f16), self.rows, self.cols,
+                                       C.c_void_p(xq.q.data_ptr() + b0 * self.cols), C.c_void_p(xq.scales.data_ptr() + b0 * (self.cols // 32) * 4),
+                                       nb, C.c_void_p(out.data_ptr() + b0 * self.rows * 4), cur_stream()))
+        return out
+
+    def matvec(self, x, out=None):
+        """Q8Head::matvec (src/model.rs:290-335): quantize x, integer block dots, f32 rescale."""
+        _lib.require_device()
+        x = x.contiguous().reshape(-1, self.cols)
+        return self.matvec_q8(_q8.quantize_q8(x), out)
+
+    def argmax(self, logits):
+        """Greedy token per row, ties to the lowest index (src/model.rs:3271-3291)."""
+        import torch
+        batch, n = logits.shape
+        ws = torch.empty(2 * batch * 1024, dtype=torch.float32, device=logits.device)
+        idx = torch.empty(batch, dtype=torch.int32, device=logits.device)
+        check(lib.mk_dev_argmax(ptr(logits.contiguous()), batch, n, ptr(ws), ptr(idx), cur_stream()))
+        return idx
+
+
+def matvec_packed_nt(packed, scales, rows, cols, x, m):
+    """model::matvec_packed_nt (src/model.rs:2412-2447), exact f32: x [m, cols] (position-major) -> [m, rows]."""
+    import torch
+    _lib.require_device()
+    out = torch.empty((m, rows), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_mxfp4_matvec_nt(ptr(packed), ptr(scales), rows, cols, ptr(x.contiguous()), m, ptr(out), cur_stream()))
+    return out
+
+
+class MlaCache:
+    """Shared-latent q8_0 MLA cache on the device (MlaCache, src/model.rs:765-781,1556-1618, in the absorbed form):
+    per position L int8 + L/32 f16 scales (latent) and R int8 + R/32 f16 scales (decoupled rope key)."""
+
+    def __init__(self, L, R, capacity, device="cuda"):
+        import torch
+        self.L, self.R, self.cap, self.n = L, R, capacity, 0
+        self.lat_q = torch.zeros((capacity, L), dtype=torch.int8, device=device)
+        self.lat_s = torch.zeros((capacity, L // 32), dtype=torch.float16, device=device)
+        self.rope_q = torch.zeros((capacity, max(R, 1)), dtype=torch.int8, device=device)
+        self.rope_s = torch.zeros((capacity, max(R // 32, 1)), dtype=torch.float16, device=device)
+        self._ws = None
+
+    def positions(self):
+        return self.n
+
+    def push(self, latent, rope):
+        """MlaCache::push (src/model.rs:1583-1618): quantize one position at append."""
+        if self.n >= self.cap:
+            raise RuntimeError("MlaCache is full")
+        _lib.require_device()
+        check(lib.mk_dev_mla_cache_append(ptr(latent.contiguous()), ptr(rope.contiguous()), self.L, self.R, self.n, ptr(self.lat_q),
+                                          ptr(self.lat_s), ptr(self.rope_q), ptr(self.rope_s), cur_stream()))
+        self.n += 1
+
+    def assign_q8(self, lat_q, lat_s, rope_q, rope_s):
+        n = lat_q.shape[0]
+        self.lat_q[:n], self.lat_s[:n], self.rope_q[:n, :self.R], self.rope_s[:n, :self.R // 32] = lat_q, lat_s, rope_q, rope_s
+        self.n = n
+
+    def to_f32(self):
+        """MlaCache::to_f32 (src/model.rs:1623-1676): q * s."""
+        n, L, R = self.n, self.L, self.R
+        lat = (self.lat_q[:n].float().view(n, L // 32, 32) * self.lat_s[:n].float().unsqueeze(-1)).view(n, L)
+        rope = (self.rope_q[:n, :R].float().view(n, R // 32, 32) * self.rope_s[:n, :R // 32].float().unsqueeze(-1)).view(n, R)
+        return lat, rope
+
+
+def mla_attn_flash_q8_mqa(cache, q, pos, scale, out=None):
+    """model::mla_attn_flash_q8_mqa (src/model.rs:1804-1908) over the shared-latent cache: q [nh, L+R] f32 on the
+    device, positions 0..=pos attended, returns [nh, L]."""
+    import torch
+    _lib.require_device()
+    nh = q.shape[0]
+    if q.shape[1] != cache.L + cache.R:
+        raise ValueError("query width must be L + R")
+    if pos >= cache.n:
+        raise ValueError("pos is beyond the cached positions")
+    need = lib.mk_mla_decode_workspace_bytes(nh, cache.L, pos + 1)
+    if cache._ws is None or cache._ws.numel() < need:
+        cache._ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    if out is None:
+        out = torch.empty((nh, cache.L), dtype=torch.float32, device=q.device)
+    check(lib.mk_dev_mla_q8_decode(ptr(cache.lat_q), ptr(cache.lat_s), ptr(cache.rope_q), ptr(cache.rope_s), pos, ptr(q.contiguous()), nh,
+                                   cache.L, cache.R, float(scale), ptr(cache._ws), ptr(out), cur_stream()))
+    return out
+
+
+class PackedExperts:
+    """Expert table of an MoE layer on the device: per expert w1, w3 [inter, d] and w2 [d, inter], each MXFP4
+    (packed, scales) in the reference layout.  Built from lists of device tensors."""
+
+    def __init__(self, w1, w3, w2, d, inter):
+        import torch
+        self.d, self.inter, self.n = d, inter, len(w1)
+        self._keep = (w1, w3, w2)
+        dev = w1[0][0].device
+        arr = lambda lst, k: torch.tensor([t[k].data_ptr() for t in lst], dtype=torch.int64, device=dev)
+        self._ptrs = [arr(w1, 0), arr(w1, 1), arr(w3, 0), arr(w3, 1), arr(w2, 0), arr(w2, 1)]
+        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter)
+        self._ws = None
+
+
+def moe_decode(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_SWIGLU, limit=0.0, out=None):
+    """The expert section of moe_forward / ds_moe for B decode tokens in one grouped pass
+    (src/model.rs:2227-2264,2346-2351; src/deepseek.rs:1069-1106).  ids [B, topk] int32, weights [B, topk] f32,
+    x [B, d] f32, all on the device; returns [B, d]."""
+    import torch
+    _lib.require_device()
+    B, topk = ids.shape
+    need = lib.mk_moe_decode_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    if experts._ws is None or experts._ws.numel() < need:
+        experts._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((B, experts.d), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_moe_decode(C.byref(experts.table), B, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), shared,
+                                ptr(x.contiguous()), mode, act_kind, float(limit), ptr(experts._ws), ptr(out), cur_stream()))
+    return out
+
+
+def router_softmax_topk(logits, k):
+    """Router of the benchmark MoE layer: softmax, top-k with the reference's tie rule, renormalised weights."""
+    import torch
+    _lib.require_device()
+    B, n = logits.shape
+    ids = torch.empty((B, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((B, k), dtype=torch.float32, device=logits.device)
+    check(lib.mk_dev_router_softmax_topk(ptr(logits.contiguous()), B, n, k, ptr(ids), ptr(w), cur_stream()))
+    return ids, w
+
+
+def grouped_gemm_mxfp8(packed_list, scales_list, rows, cols, codes, exps, offsets):
+    """Per-expert batched evaluation of moe_prefill (src/model.rs:2539-2602) on the block-scaled matrix cores:
+    rows offsets[e]..offsets[e+1] of the MXFP8 activations (codes, exps) against expert e -> [m, rows] f32."""
+    import torch
+    _lib.require_device()
+    dev = codes.device
+    pp = torch.tensor([t.data_ptr() for t in packed_list], dtype=torch.int64, device=dev)
+    sp = torch.tensor([t.data_ptr() for t in scales_list], dtype=torch.int64, device=dev)
+    m = codes.shape[0]
+    out = torch.empty((m, rows), dtype=torch.float32, device=dev)
+    check(lib.mk_dev_mxfp4_grouped_gemm(ptr(pp), ptr(sp), len(packed_list), rows, cols, ptr(codes), ptr(exps), ptr(offsets), m, ptr(out),
+                                        cur_stream()))
+    return out

@@ -1,0 +1,73 @@
+"""The C ABI without a GPU: the library loads, exports every symbol include/mk_hip.h declares, and fails loudly
+(negative status, message, nothing written) when no device is present."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mk_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from microkimi_amd import _lib
+    names = declared_symbols()
+    assert len(names) >= 35
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert not missing, missing
+    assert set(names) == set(_lib.SYMBOLS)  # the Python binding covers the whole header
+
+
+def test_no_oracle_in_product_path():
+    # the product package must not import, load or name the CPU oracle
+    pkg = os.path.join(ROOT, "microkimi_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "libmk_oracle" not in text and "from oracle" not in text, f
+
+
+def test_fails_loudly_without_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a device is present")
+    from microkimi_amd import _lib, mxfp4
+    assert _lib.lib.mk_available() == 0
+    packed = np.zeros((4, 16), np.uint8)
+    scales = np.full((4, 1), 127, np.uint8)
+    out = np.full(4, 7.0, np.float32)
+    with pytest.raises(_lib.MkError) as e:
+        mxfp4.matvec_packed(packed, scales, 4, 32, np.ones(32, np.float32), out)
+    assert e.value.status == -2 and "device" in str(e.value)
+    assert np.all(out == 7.0)  # untouched: there is no CPU fallback
+
+
+def test_argument_checks_need_no_device():
+    from microkimi_amd import _lib, mxfp4
+    with pytest.raises(ValueError):
+        mxfp4.matvec_packed(np.zeros(8, np.uint8), np.zeros(1, np.uint8), 1, 16, np.zeros(16, np.float32), np.zeros(1, np.float32))
+    # the C ABI itself rejects a cols that is not a multiple of 32 before touching the device
+    st = _lib.lib.mk_dev_mxfp4_dequant(ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 48, ctypes.c_void_p(16), None)
+    assert st == -1 and b"multiple of 32" in _lib.lib.mk_last_error()
+    st = _lib.lib.mk_dev_q8_matvec(ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 4, 64, ctypes.c_void_p(16), ctypes.c_void_p(16), 9,
+                                   ctypes.c_void_p(16), None)
+    assert st == -1 and b"batch" in _lib.lib.mk_last_error()
+
+
+def test_workloads_are_reproducible():
+    from microkimi_amd import workloads as w
+    p, s, x = w.config0(rows=8, cols=64)
+    p2, s2, x2 = w.config0(rows=8, cols=64)
+    assert np.array_equal(p, p2) and np.array_equal(s, s2) and np.array_equal(x, x2)
+    assert s.min() >= 118 and s.max() <= 130
+    q, sc, xx = w.config1(rows=64, cols=64, batch=2)
+    assert q.min() >= -127 and sc.dtype == np.float16 and xx.shape == (2, 64)

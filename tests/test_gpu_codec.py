@@ -1,0 +1,90 @@
+"""GPU parity, codec kernels: bit-exact against the oracle."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from gpu_util import dev, torch_cuda
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def test_mxfp4_dequant_golden_and_exhaustive():
+    from microkimi_amd import mxfp4
+    g = json.load(open(os.path.join(G, "ds_golden_fp4.json")))
+    p, s = np.asarray(g["packed"], np.uint8), np.asarray(g["scales"], np.uint8)
+    w = mxfp4.dequant(dev(p), dev(s), g["rows"], g["cols"]).cpu().numpy()
+    assert np.array_equal(bits(w), bits(oracle.mxfp4_dequant(p, s, g["rows"], g["cols"])))
+    # every nibble x every scale byte 0..254 (255 is NaN in e8m0 and unused), sign of -0.0 included
+    rows = 255
+    p = np.tile(np.array([n | (n << 4) for n in range(16)], np.uint8), (rows, 1))
+    s = np.arange(rows, dtype=np.uint8).reshape(rows, 1)
+    w = mxfp4.dequant(dev(p), dev(s), rows, 32).cpu().numpy()
+    assert np.array_equal(bits(w), bits(oracle.mxfp4_dequant(p, s, rows, 32)))
+    # host-level entry point (numpy in, numpy out)
+    w2 = mxfp4.dequant(p, s, rows, 32)
+    assert np.array_equal(bits(w2), bits(w))
+
+
+def test_mxfp4_dequant_config_shape():
+    from microkimi_amd import mxfp4, workloads
+    p, s, _ = workloads.config0()
+    w = mxfp4.dequant(dev(p), dev(s), 2048, 7168).cpu().numpy()
+    assert np.array_equal(bits(w), bits(oracle.mxfp4_dequant(p, s, 2048, 7168)))
+
+
+def test_fp8_dequant_golden():
+    from microkimi_amd import dequant
+    g = np.load(os.path.join(G, "ds_golden_fp8.npz"))
+    rows, cols = int(g["rows"]), int(g["cols"])
+    w = dequant.dequant_fp8(dev(g["w_packed"]), dev(g["scales"]), rows, cols).cpu().numpy()
+    assert np.array_equal(bits(w.reshape(-1)), bits(g["dequant"]))
+    # all 256 codes, NaN codes included (compare as bits of the oracle's value, NaN == NaN)
+    codes = np.tile(np.arange(256, dtype=np.uint8), (128, 1))
+    sc = np.array([[120, 131]], np.uint8)
+    w = dequant.dequant_fp8(dev(codes), dev(sc), 128, 256).cpu().numpy()
+    want = oracle.dequant_fp8(codes, sc, 128, 256)
+    assert np.array_equal(np.isnan(w), np.isnan(want))
+    assert np.array_equal(bits(w)[~np.isnan(want)], bits(want)[~np.isnan(want)])
+
+
+def test_quantize_q8_bit_exact():
+    from microkimi_amd import q8
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((16, 7168)).astype(np.float32)
+    x[1, :64] = 0.0                      # zero blocks
+    x[2, :32] = np.float32(1e-30)        # tiny block
+    x[3, 0:5] = [127.0, 0.5, -0.5, 1.5, 2.5]
+    x[3, 5:32] = 0.25                    # scale exactly 1: ties round away from zero
+    x[4] *= 1e4
+    v = q8.quantize_q8(dev(x))
+    q, s = v.q.cpu().numpy(), v.scales.cpu().numpy()
+    for r in range(16):
+        qo, so = oracle.quantize_q8(x[r])
+        assert np.array_equal(q[r], qo), r
+        assert np.array_equal(bits(s[r]), bits(so)), r
+    # host-level entry point
+    hv = q8.quantize_q8(x[0])
+    assert np.array_equal(hv.q, q[0]) and np.array_equal(hv.scales, s[0])
+
+
+def test_quantize_mxfp8_bit_exact():
+    from microkimi_amd import dequant
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((8, 2048)) * np.array([1e-3, 0.1, 1, 3, 30, 300, 1e4, 1])[:, None]).astype(np.float32)
+    x[7, :64] = 0.0
+    x[7, 64:96] = np.float32(448.0)  # amax / 448 is an exact power of two
+    x[7, 96:128] = np.float32(0.875)
+    codes, exps = dequant.quantize_mxfp8(dev(x))
+    codes, exps = codes.cpu().numpy(), exps.cpu().numpy()
+    for r in range(8):
+        _, c, e = oracle.fp8_roundtrip(x[r], 32)
+        assert np.array_equal(exps[r], e), r
+        assert np.array_equal(codes[r], c), r

@@ -1,0 +1,177 @@
+"""GPU parity, MXFP4 GEMV (mxfp4::matvec_packed, both modes) and the q8_0 head, against the oracle.
+Tolerance (north star): relative L2 <= 1e-5 with f32 accumulation; identical argmax on logits."""
+import numpy as np
+import pytest
+
+import oracle
+from gpu_util import dev, rel_l2, torch_cuda
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+SHAPES = [(128, 512), (512, 128), (64, 128), (3, 64), (1, 32), (256, 1024), (2048, 4096), (333, 1024), (4096, 2048), (77, 7168),
+          (5, 96), (130, 2048)]
+
+
+def quantized_case(rows, cols):
+    w = oracle.pattern(0, rows * cols)
+    p, s = oracle.mxfp4_quantize(w, rows, cols)
+    return p, s, oracle.pattern(4242, cols)
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+@pytest.mark.parametrize("mode", [1, 0])
+def test_matvec_packed_selftest_shapes(rows, cols, mode):
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8
+    p, s, x = quantized_case(rows, cols)
+    want = oracle.matvec_packed(p, s, rows, cols, x, mode=mode)
+    out = torch.full((rows,), 7.0, device="cuda")
+    q8.force_q8(mode)
+    try:
+        mxfp4.matvec_packed(dev(p), dev(s), rows, cols, dev(x), out)
+    finally:
+        q8.force_q8(-1)
+    assert rel_l2(out.cpu().numpy(), want) <= TOL
+
+
+def test_q8_block_terms_are_exact():
+    # one block per row: out = idot * (2^(sb-128) * dx) has no summation at all, so the result must be bit-identical
+    from microkimi_amd import mxfp4, q8
+    torch = torch_cuda()
+    rng = np.random.default_rng(4)
+    rows = 4096
+    p = rng.integers(0, 256, (rows, 16), dtype=np.uint8)
+    s = rng.integers(0, 255, (rows, 1), dtype=np.uint8)
+    x = rng.standard_normal(32).astype(np.float32)
+    xq, xs = oracle.quantize_q8(x)
+    want = oracle.matvec_packed_q8(p, s, rows, 32, xq, xs)
+    out = torch.empty(rows, device="cuda")
+    mxfp4.matvec_packed_q8(dev(p), dev(s), rows, 32, q8.Q8Vec(dev(xq), dev(xs)), out)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_zero_block_and_config0():
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8, workloads
+    rows, cols = 64, 128
+    w = oracle.pattern(0, rows * cols)
+    w[2 * cols:4 * cols] = 0
+    p, s = oracle.mxfp4_quantize(w, rows, cols)
+    x = oracle.pattern(4242, cols)
+    for mode in (1, 0):
+        out = torch.empty(rows, device="cuda")
+        q8.force_q8(mode)
+        mxfp4.matvec_packed(dev(p), dev(s), rows, cols, dev(x), out)
+        q8.force_q8(-1)
+        got = out.cpu().numpy()
+        assert np.all(got[2:4] == 0) and rel_l2(got, oracle.matvec_packed(p, s, rows, cols, x, mode=mode)) <= TOL
+    # benchmark configuration 0 at full size, both modes
+    p, s, x = workloads.config0()
+    for mode in (1, 0):
+        out = torch.empty(2048, device="cuda")
+        q8.force_q8(mode)
+        mxfp4.matvec_packed(dev(p), dev(s), 2048, 7168, dev(x), out)
+        q8.force_q8(-1)
+        assert rel_l2(out.cpu().numpy(), oracle.matvec_packed(p, s, 2048, 7168, x, mode=mode)) <= TOL
+
+
+def test_grouped_launch_matches_per_matrix():
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8, workloads
+    rows, cols, nmat = 256, 7168, 5
+    mats = [workloads.mxfp4_matrix(9, "g", rows, cols, i) for i in range(nmat)]
+    xs = workloads.normal(9, "x", (3, cols))
+    idx = np.array([0, 2, 1, 1, 0], np.int32)
+    pd, sd = [dev(m[0]) for m in mats], [dev(m[1]) for m in mats]
+    outs = [torch.empty(rows, device="cuda") for _ in range(nmat)]
+    xq = q8.quantize_q8(dev(xs))
+    keep = mxfp4.matvec_packed_grouped_q8(pd, sd, rows, cols, xq, dev(idx), outs)
+    torch.cuda.synchronize()
+    for i in range(nmat):
+        want = oracle.matvec_packed(mats[i][0], mats[i][1], rows, cols, xs[idx[i]], mode=1)
+        assert rel_l2(outs[i].cpu().numpy(), want) <= TOL
+    del keep
+
+
+@pytest.mark.parametrize("rows,cols,m", [(64, 128, 8), (33, 64, 5), (128, 512, 24), (40, 7168, 3)])
+def test_matvec_packed_nt(rows, cols, m):
+    from microkimi_amd import model
+    p, s, _ = quantized_case(rows, cols)
+    x = oracle.pattern(99, cols * m).reshape(m, cols)
+    got = model.matvec_packed_nt(dev(p), dev(s), rows, cols, dev(x), m).cpu().numpy()
+    m8 = (m + 7) // 8 * 8
+    xt = np.zeros((cols, m8), np.float32)
+    xt[:, :m] = x.T
+    want = oracle.matvec_packed_nt(p, s, rows, cols, xt, m8)[:m]
+    assert rel_l2(got, want) <= TOL
+
+
+@pytest.mark.parametrize("rows,cols,batch,f16", [(512, 1024, 1, True), (512, 1024, 8, True), (512, 1024, 3, False), (100, 7168, 1, True),
+                                                  (100, 7168, 8, True), (37, 96, 2, True), (37, 96, 1, False), (64, 2048, 5, True),
+                                                  (1000, 4096, 1, False)])
+def test_q8head_shapes(rows, cols, batch, f16):
+    torch = torch_cuda()
+    from microkimi_amd import model
+    rng = np.random.default_rng(rows + cols + batch)
+    q = rng.integers(-127, 128, (rows, cols), dtype=np.int8)
+    s = (np.abs(rng.standard_normal((rows, cols // 32))) * 0.02 / 127).astype(np.float32)
+    if f16:
+        s16 = s.astype(np.float16)
+        s = s16.astype(np.float32)
+        head = model.Q8Head.from_q8(dev(q), dev(s16), rows, cols)
+    else:
+        head = model.Q8Head.from_q8(dev(q), dev(s), rows, cols)
+    x = rng.standard_normal((batch, cols)).astype(np.float32)
+    got = head.matvec(dev(x)).cpu().numpy()
+    for b in range(batch):
+        want = oracle.q8head_matvec(q, s, rows, cols, x[b], workers=8)
+        assert rel_l2(got[b], want) <= TOL, b
+        assert int(np.argmax(got[b])) == oracle.argmax(want)
+
+
+def test_q8head_reference_unit_test():
+    # src/model.rs:3866-3881 through the device path: from_f32 on the device, err/span < 1e-2, same argmax as f32
+    from microkimi_amd import model
+    rows, cols = 512, 1024
+    rng = oracle.Rng(0xC0FFEE)
+    w = rng.f32(rows * cols) * np.float32(0.02)
+    x = rng.f32(cols)
+    head = model.Q8Head.from_f32(dev(w.reshape(rows, cols)), rows, cols, scales_f16=False)
+    qo, so = oracle.q8head_from_f32(w, rows, cols)
+    assert np.array_equal(head.q.cpu().numpy(), qo) and np.array_equal(head.scales.cpu().numpy(), so)  # bit-exact quantization
+    got = head.matvec(dev(x)).cpu().numpy()[0]
+    want = oracle.matvec_f32(w, rows, cols, x)
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-2
+    assert int(np.argmax(got)) == int(np.argmax(want))
+    assert rel_l2(got, oracle.q8head_matvec(qo, so, rows, cols, x)) <= TOL
+    assert int(head.argmax(head.matvec(dev(x)))[0]) == oracle.argmax(want)
+
+
+def test_argmax_ties_lowest_index():
+    torch = torch_cuda()
+    from microkimi_amd import model
+    logits = np.zeros((3, 163840), np.float32)
+    logits[0, [70000, 5, 163839]] = 3.0
+    logits[1, 163839] = 1.0
+    logits[2] = -1.0
+    head = model.Q8Head(torch.empty(0), torch.empty(0, dtype=torch.float16), 0, 0)
+    idx = head.argmax(dev(logits)).cpu().numpy()
+    assert idx.tolist() == [5, 163839, 0]
+
+
+def test_lm_head_full_size_argmax_and_parity():
+    # benchmark configuration 1: 163840 x 7168, batch 1 and 8; top-1 must match the CPU path
+    from microkimi_amd import model, workloads
+    q, s16, x = workloads.config1()
+    head = model.Q8Head.from_q8(dev(q), dev(s16), workloads.VOCAB, workloads.D_MODEL)
+    s = s16.astype(np.float32)
+    got8 = head.matvec(dev(x)).cpu().numpy()
+    got1 = head.matvec(dev(x[:1])).cpu().numpy()
+    am = head.argmax(dev(got8)).cpu().numpy()
+    for b in range(8):
+        want = oracle.q8head_matvec(q, s, workloads.VOCAB, workloads.D_MODEL, x[b], workers=16)
+        assert rel_l2(got8[b], want) <= TOL, b
+        assert int(am[b]) == oracle.argmax(want), b
+        if b == 0:
+            assert rel_l2(got1[0], want) <= TOL

@@ -1,0 +1,76 @@
+"""GPU parity, q8_0 MLA decode attention over the shared-latent cache against the oracle's
+mla_attn_flash_q8_mqa.  Tolerance: relative L2 <= 1e-5."""
+import numpy as np
+import pytest
+
+import oracle
+from gpu_util import dev, rel_l2, torch_cuda
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def make_cache(ctx, L, R, nh, seed):
+    from microkimi_amd import workloads
+    rng = np.random.default_rng(seed)
+    lat = rng.standard_normal((ctx, L)).astype(np.float32)
+    rope = rng.standard_normal((ctx, R)).astype(np.float32)
+    q = rng.standard_normal((nh, L + R)).astype(np.float32)
+    lq, ls = workloads.q8_0_rows(lat)
+    rq, rs = workloads.q8_0_rows(rope)
+    return lat, rope, q, lq, ls, rq, rs
+
+
+@pytest.mark.parametrize("ctx,L,R,nh", [(1, 128, 64, 6), (7, 128, 64, 6), (64, 128, 64, 6), (65, 128, 64, 6), (512, 128, 64, 6),
+                                        (300, 512, 64, 20), (1000, 256, 32, 16)])
+def test_small_shapes(ctx, L, R, nh):
+    from microkimi_amd import model
+    lat, rope, q, lq, ls, rq, rs = make_cache(ctx, L, R, nh, ctx)
+    cache = model.MlaCache(L, R, ctx)
+    cache.assign_q8(dev(lq), dev(ls), dev(rq), dev(rs))
+    scale = float(np.float32(L // 4 + R) ** np.float32(-0.5))
+    got = model.mla_attn_flash_q8_mqa(cache, dev(q), ctx - 1, scale).cpu().numpy()
+    want = oracle.mla_absorbed_decode(lq, ls.astype(np.float32), rq, rs.astype(np.float32), q, nh, scale)
+    assert rel_l2(got, want) <= TOL
+    if ctx > 10:  # a shorter window over the same cache
+        got = model.mla_attn_flash_q8_mqa(cache, dev(q), ctx // 2, scale).cpu().numpy()
+        want = oracle.mla_absorbed_decode(lq, ls.astype(np.float32), rq, rs.astype(np.float32), q, nh, scale, pos=ctx // 2)
+        assert rel_l2(got, want) <= TOL
+
+
+def test_append_quantizes_like_the_reference():
+    torch = torch_cuda()
+    from microkimi_amd import model
+    L, R, n = 512, 64, 40
+    lat, rope, q, lq, ls, rq, rs = make_cache(n, L, R, 4, 77)
+    lat[3, :32] = 0.0
+    lq, ls = __import__("microkimi_amd").workloads.q8_0_rows(lat)
+    cache = model.MlaCache(L, R, n)
+    for j in range(n):
+        cache.push(dev(lat[j]), dev(rope[j]))
+    assert cache.positions() == n
+    assert np.array_equal(cache.lat_q.cpu().numpy(), lq) and np.array_equal(cache.rope_q.cpu().numpy(), rq)
+    assert np.array_equal(cache.lat_s.cpu().numpy().view(np.uint16), ls.view(np.uint16))
+    assert np.array_equal(cache.rope_s.cpu().numpy().view(np.uint16), rs.view(np.uint16))
+    # round trip within the q8_0 bound dx/2 (+ the f16 rounding of the scale), src/selftest.rs:790-841
+    lat2, rope2 = cache.to_f32()
+    bound = np.abs(lat.reshape(n, L // 32, 32)).max(axis=2, keepdims=True) / 254.0
+    err = np.abs(lat2.cpu().numpy().reshape(n, L // 32, 32) - lat.reshape(n, L // 32, 32))
+    assert np.all(err <= bound * 1.02 + np.abs(lat.reshape(n, L // 32, 32)) * 2.0 ** -11)
+
+
+@pytest.mark.parametrize("ctx", [1024, 4096, 16384])
+def test_benchmark_shapes(ctx):
+    # configuration 3: 128 heads, latent 512 + rope 64, scale 1/sqrt(192)
+    from microkimi_amd import model, workloads
+    lat, rope, q = workloads.config3_raw(ctx)
+    lq, ls = workloads.q8_0_rows(lat)
+    rq, rs = workloads.q8_0_rows(rope)
+    cache = model.MlaCache(workloads.MLA_LATENT, workloads.MLA_ROPE, ctx)
+    cache.assign_q8(dev(lq), dev(ls), dev(rq), dev(rs))
+    got = model.mla_attn_flash_q8_mqa(cache, dev(q), ctx - 1, workloads.MLA_SCALE).cpu().numpy()
+    want = oracle.mla_absorbed_decode(lq, ls.astype(np.float32), rq, rs.astype(np.float32), q, workloads.MLA_HEADS, workloads.MLA_SCALE)
+    assert rel_l2(got, want) <= TOL
+    # softmax-weighted averages of the cache rows stay inside the rows' range (size-independent property)
+    v = lq.astype(np.float32) * np.repeat(ls.astype(np.float32), 32, axis=1)
+    assert np.all(got <= v.max(axis=0) + 1e-4) and np.all(got >= v.min(axis=0) - 1e-4)
