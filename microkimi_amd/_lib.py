@@ -26,6 +26,10 @@ class ExpertTable(C.Structure):
 
 
 def _load():
+    # torch ships its own HIP runtime (same soname as the system one).  Loading torch first makes the dynamic
+    # loader bind libmk_hip.so to that already-loaded copy; the other order leaves two runtimes in the process
+    # and the second one finds no device.
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise ImportError(f"{LIB_PATH} is missing: build it with `python -m microkimi_amd.build` (needs hipcc); "
                           "there is no fallback implementation")

@@ -19,7 +19,7 @@ def hipcc():
 
 def build(verbose=False):
     """Compile every HIP source for gfx950 and link the shared library."""
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wno-unused-value",
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wno-unused-value", "-fno-strict-aliasing",
            # wrong results have been seen from compiler-formed packed-f32 ops on this target: keep them off
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-DMK_BUILD=1"]

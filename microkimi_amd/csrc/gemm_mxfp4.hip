@@ -10,6 +10,14 @@
 // The A operand is the activation in MXFP8 (e4m3 codes + e8m0 per 32), 32 bytes
 // per lane.  Accumulation is f32 in the matrix core.
 //
+// Operand layout of the instruction (measured on the device with one-hot
+// operands, both formats):
+//   scales        lane i + 16 b supplies the e8m0 byte of row/column i, K block b (k in [32 b, 32 b + 32))
+//   4-bit operand lane i + 16 b holds k = 32 b + j in registers 0-3, nibble j (low nibble first): one MXFP4 block
+//   8-bit operand lane i + 16 g holds k = 16 g + j in registers 0-3 (bytes 0-15) and k = 64 + 16 g + j in
+//                 registers 4-7 (bytes 16-31): the K = 128 step is two K = 64 halves
+//   result        lane l holds column l % 16, rows 4 (l / 16) + r
+//
 // Tiling: workgroup = 4 waves = 64 weight rows of one expert; each wave owns 16
 // rows and up to 64 token rows (4 accumulator tiles), so an expert's weights are
 // streamed from HBM once for up to 64 tokens.  At the prefill shapes (about 16
@@ -49,7 +57,7 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 #pragma unroll
         for (int c = 0; c < MC; c++) {
             const int t = min(base + c * 16 + n, tok1 - 1);
-            arow[c] = codes + (size_t)t * cols + kb * 32;
+            arow[c] = codes + (size_t)t * cols + kb * 16;
             aexp[c] = exps + (size_t)t * nb + kb;
         }
         for (int s = 0; s < steps; s++) {
@@ -60,7 +68,7 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
             for (int c = 0; c < MC; c++) {
                 if (c < nchunk) {
                     const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow[c] + s * 128);
-                    const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow[c] + s * 128 + 16);
+                    const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow[c] + s * 128 + 64);
                     const int asb = aexp[c][s * 4];
                     mk_i8v a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                     acc[c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[c], 0 /*A: fp8 e4m3*/, 4 /*B: fp4 e2m1*/, 0, asb, 0, wsb);

@@ -85,8 +85,9 @@ extern "C" int mk_init(int device) {
     std::lock_guard<std::mutex> lk(g_mu);
     if (g_ctx.ready) return MK_OK;
     int n = 0;
-    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
-        mk_set_error("no HIP device visible");
+    hipError_t ce = hipGetDeviceCount(&n);
+    if (ce != hipSuccess || n <= 0) {
+        mk_set_error("no HIP device visible (hipGetDeviceCount: %d %s, count %d)", (int)ce, hipGetErrorString(ce), n);
         return g_ctx.status = MK_ERR_NO_DEVICE;
     }
     if (device < 0 || device >= n) {

@@ -128,7 +128,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_q8_kernel(PairTables pt, cons
     constexpr int T = TILE / 64;
     constexpr int RT = TILE / NB;
     static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
-    __shared__ __attribute__((aligned(16))) _Float16 xh[NB * 32];
+    // f16 pairs kept as 32-bit words: written and read through the same type
+    __shared__ __attribute__((aligned(16))) uint32_t xh[NB * 16];
     __shared__ float xsc[NB];
     const int p = blockIdx.y;
     const uint8_t *w1p = pt.w1p[p], *w1s = pt.w1s[p], *w3p = pt.w3p[p], *w3s = pt.w3s[p];
@@ -143,8 +144,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_q8_kernel(PairTables pt, cons
         lo.y = (_Float16)(float)(int8_t)((v >> 8) & 255u);
         hi.x = (_Float16)(float)(int8_t)((v >> 16) & 255u);
         hi.y = (_Float16)(float)(int8_t)(v >> 24);
-        reinterpret_cast<mk_h2 *>(xh)[i * 2] = lo;
-        reinterpret_cast<mk_h2 *>(xh)[i * 2 + 1] = hi;
+        xh[i * 2] = __builtin_bit_cast(uint32_t, lo);
+        xh[i * 2 + 1] = __builtin_bit_cast(uint32_t, hi);
     }
     for (int i = threadIdx.x; i < NB; i += 256) xsc[i] = xsv[i];
     __syncthreads();
@@ -156,13 +157,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_q8_kernel(PairTables pt, cons
 #pragma unroll
     for (int t = 0; t < T; t++) {
         const int g = (t * 64 + lane) % NB;
-        const mk_i4 *src = reinterpret_cast<const mk_i4 *>(xh + g * 32);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            mk_i4 v = src[k];
-#pragma unroll
-            for (int e = 0; e < 4; e++) xr[t][k * 4 + e] = __builtin_bit_cast(mk_h2, v[e]);
-        }
+        for (int k = 0; k < 16; k++) xr[t][k] = __builtin_bit_cast(mk_h2, xh[g * 16 + k]);
         cf[t] = xsc[g];
     }
     float myact = 0.0f;

@@ -47,7 +47,8 @@ def test_q8head_host_api():
     _lib.lib.mk_q8head_free(h)
     # from_q8 with f16 storage
     s16 = s.astype(np.float16)
-    _lib.check(_lib.lib.mk_q8head_from_q8(_lib.hptr(q), _lib.hptr(s16.astype(np.float32)), rows, cols, 1, ctypes.byref(h)))
+    s16_as_f32 = s16.astype(np.float32)  # must outlive the call: hptr() only takes the address
+    _lib.check(_lib.lib.mk_q8head_from_q8(_lib.hptr(q), _lib.hptr(s16_as_f32), rows, cols, 1, ctypes.byref(h)))
     _lib.check(_lib.lib.mk_q8head_matvec(h, _lib.hptr(x), 1, _lib.hptr(out), None))
     assert rel_l2(out[0], oracle.q8head_matvec(q, s16.astype(np.float32), rows, cols, x[0])) <= 1e-5
     _lib.lib.mk_q8head_free(h)
