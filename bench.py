@@ -1,0 +1,368 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
+
+Headline (the JSON line's `value`): the q8_0 lm_head GEMV of benchmark configuration 1 -- 163840 x 7168 int8 weights
+with one f16 scale per 32, batch 1 -- as algorithmic HBM GB/s.  A step is one Q8Head::matvec: quantize the hidden row
+to q8, then the GEMV over the whole head; inputs are resident in HBM before the timed region.
+
+`roofline` is the GEMV kernel alone (HIP events around each launch, on the stream it runs on) against the 8 TB/s HBM
+peak; `cpu_baseline` is the CPU oracle (a port of the reference's Rust kernels) on a bounded row sample of the same
+head, on this host's cores.  `extras` holds the other configurations (MXFP4 GEMV stream, MoE decode layer tok/s,
+q8 MLA decode, grouped expert GEMM), each with its own algorithmic-bytes roofline fraction.
+
+Prints exactly one JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+FP4_PEAK_TFLOPS = 10100.0   # dense FP4/FP6 MFMA
+FP8_PEAK_TFLOPS = 5000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_events(torch, fn, iters, warmup=3):
+    """Average milliseconds per call of fn(), each call bracketed by its own pair of events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        evs.append((a, b))
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return sum(ts) / len(ts), ts[len(ts) // 2]
+
+
+def time_region(torch, fn, iters, warmup=3):
+    """Milliseconds per call over one timed region of `iters` back-to-back calls."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / iters
+
+
+def bench_lm_head(torch, steps, warmup):
+    from microkimi_amd import model, q8, workloads as W
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    rows, cols = W.VOCAB, W.D_MODEL
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q = torch.randint(-127, 128, (rows, cols), dtype=torch.int8, device="cuda", generator=g)
+    s = (torch.randn((rows, cols // 32), device="cuda", generator=g).abs() * (0.02 / 127.0)).to(torch.float16)
+    x = torch.randn((8, cols), device="cuda", generator=g)
+    head = model.Q8Head.from_q8(q, s, rows, cols)
+    out1 = torch.empty((1, rows), device="cuda")
+    out8 = torch.empty((8, rows), device="cuda")
+    x1 = x[:1].contiguous()
+
+    def step():
+        head.matvec(x1, out1)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    alg1 = rows * cols + rows * (cols // 32) * 2 + cols * 4 + rows * 4           # 1 248 489 472 B
+    alg8 = rows * cols + rows * (cols // 32) * 2 + 8 * cols * 4 + 8 * rows * 4   # 1 253 277 696 B
+    xq1 = q8.quantize_q8(x1)
+    xq8 = q8.quantize_q8(x)
+
+    def k1():
+        check(lib.mk_dev_q8_matvec(ptr(head.q), ptr(head.scales), 1, rows, cols, ptr(xq1.q), ptr(xq1.scales), 1, ptr(out1), cur_stream()))
+
+    def k8():
+        check(lib.mk_dev_q8_matvec(ptr(head.q), ptr(head.scales), 1, rows, cols, ptr(xq8.q), ptr(xq8.scales), 8, ptr(out8), cur_stream()))
+
+    k1_ms, k1_med = time_events(torch, k1, max(20, min(steps, 200)))
+    k8_ms, k8_med = time_events(torch, k8, max(20, min(steps, 100)))
+    am = head.argmax(out8)
+    torch.cuda.synchronize()
+    res = {
+        "ms_per_step": ms_step,
+        "value_gbs": alg1 / (ms_step * 1e-3) / 1e9,
+        "kernel_ms": k1_ms,
+        "kernel_gbs": alg1 / (k1_ms * 1e-3) / 1e9,
+        "alg_bytes": alg1,
+        "batch8": {"kernel_ms": k8_ms, "gbs": alg8 / (k8_ms * 1e-3) / 1e9, "frac": alg8 / (k8_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                   "alg_bytes": alg8, "tok_s": 8 / (k8_ms * 1e-3)},
+    }
+    return res, (q, s, x, out8, am)
+
+
+def cpu_baseline_lm_head(torch, tensors, sample_rows=16384, budget_s=12.0):
+    """The CPU oracle's Q8Head::matvec on the first `sample_rows` rows of the same head (same pool split rule)."""
+    import numpy as np
+    import oracle
+    q, s, x, out8, am = tensors
+    cols = q.shape[1]
+    qh = q[:sample_rows].cpu().numpy()
+    sh = s[:sample_rows].float().cpu().numpy()
+    xh = x[0].cpu().numpy()
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    workers = max(1, min(cores, 16))
+    oracle.q8head_matvec(qh, sh, sample_rows, cols, xh, workers=workers)  # warm-up
+    ts = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end and len(ts) < 200:
+        t0 = time.perf_counter()
+        want = oracle.q8head_matvec(qh, sh, sample_rows, cols, xh, workers=workers)
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    med = ts[len(ts) // 2]
+    bytes_sample = sample_rows * cols + sample_rows * (cols // 32) * 4 + cols * 4 + sample_rows * 4  # f32 scales, as the reference keeps them
+    # parity of the GPU logits on the sample, and of the greedy token over the whole head for row 0
+    got = out8[0, :sample_rows].cpu().numpy()
+    rel = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
+    return {"value": bytes_sample / med / 1e9, "unit": "GB/s", "cores": workers, "kind": "port",
+            "sample": f"first {sample_rows} of 163840 rows x 7168, batch 1, median of {len(ts)} calls, {med * 1e3:.2f} ms/call "
+                      f"(full head would take about {med * 1e3 * 163840 / sample_rows:.1f} ms)",
+            "gpu_vs_cpu_rel_l2_on_sample": rel}
+
+
+def rand_mxfp4(torch, g, rows, cols):
+    p = torch.randint(0, 256, (rows, cols // 2), dtype=torch.uint8, device="cuda", generator=g)
+    s = torch.randint(118, 131, (rows, cols // 32), dtype=torch.uint8, device="cuda", generator=g)
+    return p, s
+
+
+def bench_mxfp4_gemv(torch):
+    """Configuration 0 as a stream over 64 distinct matrices (7.8 MB each, 500 MB in all: more than the 256 MB
+    Infinity Cache), as one grouped launch and as 64 back-to-back launches."""
+    from microkimi_amd import mxfp4, q8, workloads as W
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    rows, cols, nmat = 2048, W.D_MODEL, 64
+    g = torch.Generator(device="cuda").manual_seed(2)
+    mats = [rand_mxfp4(torch, g, rows, cols) for _ in range(nmat)]
+    x = torch.randn(cols, device="cuda", generator=g)
+    xq = q8.quantize_q8(x)
+    outs = [torch.empty(rows, device="cuda") for _ in range(nmat)]
+    mk = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device="cuda")
+    pp, sp, op = mk([m[0] for m in mats]), mk([m[1] for m in mats]), mk(outs)
+    per = rows * cols // 2 + rows * cols // 32 + cols * 4 + rows * 4  # 7 835 648 B
+
+    def grouped():
+        check(lib.mk_dev_mxfp4_matvec_q8_grouped(ptr(pp), ptr(sp), nmat, rows, cols, ptr(xq.q), ptr(xq.scales), None, ptr(op), cur_stream()))
+
+    def singles():
+        for i in range(nmat):
+            check(lib.mk_dev_mxfp4_matvec_q8(ptr(mats[i][0]), ptr(mats[i][1]), rows, cols, ptr(xq.q), ptr(xq.scales), ptr(outs[i]), cur_stream()))
+
+    g_ms, _ = time_events(torch, grouped, 30)
+    s_ms = time_region(torch, singles, 10)
+    xf = x.contiguous()
+
+    def singles_f32():
+        for i in range(nmat):
+            check(lib.mk_dev_mxfp4_matvec_f32(ptr(mats[i][0]), ptr(mats[i][1]), rows, cols, ptr(xf), ptr(outs[i]), cur_stream()))
+
+    f_ms = time_region(torch, singles_f32, 5)
+    gbs = lambda ms: per * nmat / (ms * 1e-3) / 1e9
+    return {"workload": "64 distinct 2048x7168 MXFP4 matrices, batch 1", "alg_bytes_per_matrix": per,
+            "q8_grouped_launch": {"ms": g_ms, "gbs": gbs(g_ms), "frac": gbs(g_ms) / HBM_PEAK_GBS},
+            "q8_back_to_back": {"ms": s_ms, "gbs": gbs(s_ms), "frac": gbs(s_ms) / HBM_PEAK_GBS, "us_per_gemv": s_ms * 1e3 / nmat},
+            "f32_back_to_back": {"ms": f_ms, "gbs": gbs(f_ms), "frac": gbs(f_ms) / HBM_PEAK_GBS}}
+
+
+def bench_moe(torch):
+    """Configuration 2: 256 routed + 1 shared MXFP4 experts (6.0 GB resident), softmax top-8 router, B in {1, 4, 16}."""
+    from microkimi_amd import model, workloads as W
+    d, inter, ne = W.D_MODEL, W.D_INTER, W.N_EXPERTS
+    g = torch.Generator(device="cuda").manual_seed(3)
+    w1 = [rand_mxfp4(torch, g, inter, d) for _ in range(ne + 1)]
+    w3 = [rand_mxfp4(torch, g, inter, d) for _ in range(ne + 1)]
+    w2 = [rand_mxfp4(torch, g, d, inter) for _ in range(ne + 1)]
+    experts = model.PackedExperts(w1, w3, w2, d, inter)
+    per_expert = 3 * (inter * d // 2 + inter * d // 32)  # 23 396 352 B
+    res = {"workload": "256 routed + 1 shared MXFP4 experts (2048x7168 gate/up, 7168x2048 down), top-8, q8 mode",
+           "bytes_per_expert": per_expert}
+    for B in (1, 4, 16):
+        logits_h, hidden_h = W.config2_tokens(B)
+        logits = torch.from_numpy(logits_h).cuda()
+        x = torch.from_numpy(hidden_h * 0.02).cuda()  # small hidden state keeps SwiGLU of random experts finite
+        ids, wts = model.router_softmax_topk(logits, W.TOP_K)
+        out = torch.empty((B, d), device="cuda")
+        n_distinct = len(set(ids.cpu().numpy().reshape(-1).tolist())) + 1
+        alg = n_distinct * per_expert + B * 2 * d * 4
+
+        def step():
+            model.moe_decode(experts, ids, wts, x, shared=ne, out=out)
+
+        ms = time_region(torch, step, 30, warmup=5)
+        res[f"B{B}"] = {"ms": ms, "tok_s": B / (ms * 1e-3), "distinct_experts": n_distinct, "pairs": B * (W.TOP_K + 1), "alg_bytes": alg,
+                        "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "finite": bool(torch.isfinite(out).all().item())}
+    return res
+
+
+def bench_mla(torch):
+    """Configuration 3: 128 heads over a shared q8_0 latent cache; 32 distinct caches are rotated at every context
+    length (a model has 24 MLA layers) so repeats are not served by the Infinity Cache."""
+    from microkimi_amd import model, workloads as W
+    L, R, nh = W.MLA_LATENT, W.MLA_ROPE, W.MLA_HEADS
+    g = torch.Generator(device="cuda").manual_seed(4)
+    res = {"workload": "128 heads, latent 512 + rope 64 q8_0 (612 B/position), 32 rotating caches"}
+    q = torch.randn((nh, L + R), device="cuda", generator=g)
+    out = torch.empty((nh, L), device="cuda")
+    from microkimi_amd._lib import lib
+    ws = torch.empty(lib.mk_mla_decode_workspace_bytes(nh, L, 16384), dtype=torch.uint8, device="cuda")  # one scratch for all caches
+    for ctx in (1024, 4096, 16384):
+        caches = []
+        for _ in range(32):
+            c = model.MlaCache(L, R, ctx)
+            c.lat_q.copy_(torch.randint(-127, 128, (ctx, L), dtype=torch.int8, device="cuda", generator=g))
+            c.lat_s.copy_((torch.rand((ctx, L // 32), device="cuda", generator=g) * 0.03 + 0.005).to(torch.float16))
+            c.rope_q.copy_(torch.randint(-127, 128, (ctx, R), dtype=torch.int8, device="cuda", generator=g))
+            c.rope_s.copy_((torch.rand((ctx, R // 32), device="cuda", generator=g) * 0.03 + 0.005).to(torch.float16))
+            c.n = ctx
+            c._ws = ws
+            caches.append(c)
+        it = [0]
+
+        def step():
+            c = caches[it[0] % 32]
+            it[0] += 1
+            model.mla_attn_flash_q8_mqa(c, q, ctx - 1, W.MLA_SCALE, out)
+
+        ms = time_region(torch, step, 64, warmup=4)
+        alg = ctx * 612 + nh * (L + R) * 4 + nh * L * 4
+        flops = 2.0 * nh * (L + R + L) * ctx
+        res[f"ctx{ctx}"] = {"us": ms * 1e3, "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                            "tflops": flops / (ms * 1e-3) / 1e12}
+        del caches
+    return res
+
+
+def bench_gemm(torch):
+    """Configuration 4: 512 tokens routed top-8 over 256 experts (about 16 rows per expert), gate GEMM 2048 x 7168 per
+    expert on the block-scaled MFMA; and a large-M variant (512 rows on each of 8 experts)."""
+    import numpy as np
+    from microkimi_amd import dequant, model, workloads as W
+    d, inter, ne = W.D_MODEL, W.D_INTER, W.N_EXPERTS
+    g = torch.Generator(device="cuda").manual_seed(5)
+    logits_h, x_h = W.config4_tokens()
+    ids, _ = model.router_softmax_topk(torch.from_numpy(logits_h).cuda(), W.TOP_K)
+    flat = ids.cpu().numpy().reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    counts = np.bincount(flat, minlength=ne)
+    offsets = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).cuda()
+    xg = torch.from_numpy(x_h[order // W.TOP_K]).cuda()
+    codes, exps = dequant.quantize_mxfp8(xg)
+    mats = [rand_mxfp4(torch, g, inter, d) for _ in range(ne)]
+    pl, sl = [m[0] for m in mats], [m[1] for m in mats]
+    m = int(xg.shape[0])
+
+    def step():
+        model.grouped_gemm_mxfp8(pl, sl, inter, d, codes, exps, offsets)
+
+    ms = time_region(torch, step, 10, warmup=2)
+    used = int((counts > 0).sum())
+    wbytes = used * (inter * d // 2 + inter * d // 32)
+    alg = wbytes + m * d + m * d // 32 + m * inter * 4
+    flops = 2.0 * m * inter * d
+    res = {"workload": "gate GEMM of 512 tokens x top-8 over 256 experts (4096 rows, 2048 x 7168 per expert), MXFP8 activations",
+           "prefill": {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "mfma_frac_fp8_peak": flops / (ms * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
+                       "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "rows_per_expert_max": int(counts.max()), "experts_used": used}}
+    # large-M variant: the kernel's own ceiling
+    M = 512
+    xl = torch.randn((8 * M, d), device="cuda", generator=g)
+    cl, el = dequant.quantize_mxfp8(xl)
+    off2 = torch.arange(0, 9, dtype=torch.int32, device="cuda") * M
+
+    def step2():
+        model.grouped_gemm_mxfp8(pl[:8], sl[:8], inter, d, cl, el, off2)
+
+    ms2 = time_region(torch, step2, 5, warmup=1)
+    fl2 = 2.0 * 8 * M * inter * d
+    res["large_m"] = {"rows_per_expert": M, "experts": 8, "ms": ms2, "tflops": fl2 / (ms2 * 1e-3) / 1e12,
+                      "mfma_frac_fp8_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (no CPU fallback exists for the measured path)", file=sys.stderr)
+        sys.exit(3)
+    from microkimi_amd import _lib
+    _lib.require_device()
+    torch.cuda.set_device(0)
+
+    log("lm_head ...")
+    head, tensors = bench_lm_head(torch, args.steps, args.warmup)
+    cpu = None
+    if not args.no_cpu:
+        log("cpu baseline ...")
+        cpu = cpu_baseline_lm_head(torch, tensors)
+    del tensors
+    torch.cuda.empty_cache()
+    extras = {"lm_head_batch8": head.pop("batch8")}
+    if not args.no_extras:
+        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("grouped_gemm", bench_gemm)):
+            log(name, "...")
+            try:
+                extras[name] = fn(torch)
+            except Exception as e:  # an extra must not hide the headline
+                extras[name] = {"error": repr(e)}
+            torch.cuda.empty_cache()
+
+    line = {
+        "metric": "q8_0 lm_head GEMV HBM GB/s",
+        "value": head["value_gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "config 1: q8_0 lm_head 163840x7168 (int8 + f16 scale per 32), batch 1; step = quantize_q8(x) + GEMV",
+                   "rows": 163840, "cols": 7168, "batch": 1, "algorithmic_bytes": head["alg_bytes"]},
+        "roofline": {"bound": "hbm", "achieved": head["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "q8_gemv_b1_kernel<224, f16 scales>", "kernel_ms": head["kernel_ms"]},
+        "cpu_baseline": cpu,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
