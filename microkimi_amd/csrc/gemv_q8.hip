@@ -16,6 +16,8 @@
 //           f32 exactly as the reference does.  Weights are read once for the
 //           whole batch.
 // generic   one wave per row, any cols % 32 == 0, any batch <= 8.
+#include <stdlib.h>
+
 #include "mk_common.h"
 
 namespace {
@@ -27,14 +29,18 @@ __device__ __forceinline__ float load_scale(const void *scales, size_t idx) {
 }
 
 // ------------------------------------------------------------- batch 1
+// Rows are dealt round-robin to a fixed number of resident waves: wave w takes
+// rows w, w + W, w + 2W, ...  Every wave has the same amount of work (no tail)
+// and at any moment the chip reads one compact window of W consecutive rows.
 template <int NB, bool F16>
 __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows,
                                                          const int8_t *__restrict__ xq, const float *__restrict__ xs,
-                                                         float *__restrict__ out, int rows_per_wave) {
+                                                         float *__restrict__ out) {
     constexpr int T = NB * 2 / 64;  // half blocks per row / 64 lanes
     static_assert(NB % 32 == 0 && T >= 1 && T <= 8, "row shape not covered by the fast path");
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int n_waves = gridDim.x * 4;
     mk_i4 xr[T];
     float cf[T];
 #pragma unroll
@@ -43,8 +49,6 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
         xr[t] = *reinterpret_cast<const mk_i4 *>(xq + hb * 16);
         cf[t] = xs[hb >> 1];
     }
-    const int r0 = wave * rows_per_wave;
-    const int r1 = min(r0 + rows_per_wave, rows);
     mk_i4 w[T];
     float ws[T];
     auto load_row = [&](int r) {
@@ -56,8 +60,8 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
             ws[t] = load_scale<F16>(scales, (size_t)r * NB + (hb >> 1));
         }
     };
-    if (r0 < r1) load_row(r0);
-    for (int r = r0; r < r1; r++) {
+    if (wave < rows) load_row(wave);
+    for (int r = wave; r < rows; r += n_waves) {
         mk_i4 wc[T];
         float wsc[T];
 #pragma unroll
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
             wc[t] = w[t];
             wsc[t] = ws[t];
         }
-        if (r + 1 < r1) load_row(r + 1);
+        if (r + n_waves < rows) load_row(r + n_waves);
         float acc = 0.0f;
 #pragma unroll
         for (int t = 0; t < T; t++) {
@@ -80,24 +84,32 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
 }
 
 // ------------------------------------------------------- batch 2..8 (MFMA)
-// Workgroup: 512 threads = 8 waves; LDS holds the batch's activation bytes in
-// the operand order ([K/16 chunks][8 batch rows][16 bytes]) and the activation
-// block scales ([NB][8]).  Each wave walks 16-row groups.
-template <bool F16>
-__global__ __launch_bounds__(512) void q8_gemv_mfma_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows, int nb,
-                                                           const int8_t *__restrict__ xq, const float *__restrict__ xs, int batch,
-                                                           float *__restrict__ out, int groups_per_wave) {
+// Workgroup of WAVES waves; LDS holds the batch's activation bytes in operand
+// order ([K/16 chunks][8 batch rows][16 bytes]), the activation block scales
+// ([NB][8]) and, per wave, the weight scales of the 16-row group the wave is
+// working on.  The scales of 16 consecutive rows are one contiguous range:
+// they are fetched with seven fully coalesced 1 KiB loads, one group ahead,
+// and read back from LDS per step -- scattered 2-byte global loads per step cost
+// a cache line each and halved the bandwidth.
+template <bool F16, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows,
+                                                                  int nb, const int8_t *__restrict__ xq, const float *__restrict__ xs,
+                                                                  int batch, float *__restrict__ out) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int SB = F16 ? 2 : 4;  // bytes per weight scale
+    constexpr int NIT = F16 ? 8 : 16;  // 1 KiB wave loads covering the scales of one group (nb <= 256)
     const int cols = nb * 32;
     mk_i4 *xl = reinterpret_cast<mk_i4 *>(lds);                      // [cols/16][8]
     float *xsl = reinterpret_cast<float *>(lds + (size_t)cols * 8);  // [nb][8]
-    for (int i = threadIdx.x; i < (cols / 16) * 8; i += 512) {
+    const int group_bytes = 16 * nb * SB;
+    uint8_t *sl = lds + (size_t)cols * 8 + (size_t)nb * 32 + (size_t)(threadIdx.x >> 6) * group_bytes;  // this wave's scale tile
+    for (int i = threadIdx.x; i < (cols / 16) * 8; i += WAVES * 64) {
         const int c = i >> 3, b = i & 7;
         mk_i4 v = {0, 0, 0, 0};
         if (b < batch) v = *reinterpret_cast<const mk_i4 *>(xq + (size_t)b * cols + c * 16);
         xl[i] = v;
     }
-    for (int i = threadIdx.x; i < nb * 8; i += 512) {
+    for (int i = threadIdx.x; i < nb * 8; i += WAVES * 64) {
         const int g = i >> 3, b = i & 7;
         xsl[i] = b < batch ? xs[(size_t)b * nb + g] : 0.0f;
     }
@@ -110,26 +122,68 @@ __global__ __launch_bounds__(512) void q8_gemv_mfma_kernel(const int8_t *__restr
     const int a_batch = n & 7, a_par = n >> 3;  // A operand row m = n: batch row and block parity
     const bool a_live = (kb >> 1) == a_par;
     const int steps = nb / 2;
-    const int wave = blockIdx.x * 8 + (threadIdx.x >> 6);
+    const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+    const int n_waves = gridDim.x * WAVES;
     const int n_groups = (rows + 15) / 16;
-    const int g0 = wave * groups_per_wave, g1 = min(g0 + groups_per_wave, n_groups);
-    for (int grp = g0; grp < g1; grp++) {
+    const size_t scale_bytes = (size_t)rows * nb * SB;
+    constexpr int S = 8;  // K steps per register block; two blocks (ping, pong) are in flight per lane
+
+    mk_i4 spre[NIT];  // scales of the next group, in flight while the current group is computed
+    auto prefetch_scales = [&](int grp) {
+        const size_t base = (size_t)grp * group_bytes;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const size_t off = (size_t)(it * 64 + lane) * 16;
+            spre[it] = (off < (size_t)group_bytes && base + off + 16 <= scale_bytes)
+                           ? *reinterpret_cast<const mk_i4 *>(reinterpret_cast<const uint8_t *>(scales) + base + off)
+                           : mk_i4{0, 0, 0, 0};
+        }
+    };
+    if (wave < n_groups) prefetch_scales(wave);
+    // 16-row groups are dealt round-robin to the resident waves
+    for (int grp = wave; grp < n_groups; grp += n_waves) {
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            const int off = (it * 64 + lane) * 16;
+            if (off < group_bytes) *reinterpret_cast<mk_i4 *>(sl + off) = spre[it];
+        }
+        if (grp + n_waves < n_groups) prefetch_scales(grp + n_waves);
         const int row = grp * 16 + n;
         const bool row_ok = row < rows;
         const int8_t *wrow = q + (size_t)(row_ok ? row : 0) * cols + kb * 16;
-        const size_t srow = (size_t)(row_ok ? row : 0) * nb + par;
+        const uint8_t *srow = sl + (size_t)(n * nb + par) * SB;
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll 4
-        for (int s = 0; s < steps; s++) {
-            mk_i4 wv = *reinterpret_cast<const mk_i4 *>(wrow + s * 64);
-            float wsf = load_scale<F16>(scales, srow + 2 * s);
-            mk_i4 xa = xl[(s * 4 + kb) * 8 + a_batch];
-            if (!a_live) xa = mk_i4{0, 0, 0, 0};
-            mk_i4 c = {0, 0, 0, 0};
-            c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wv, c, 0, 0, 0);
-            const mk_f4 x4 = *reinterpret_cast<const mk_f4 *>(xsl + (2 * s + par) * 8 + 4 * (kb & 1));
+        mk_i4 wa[S], wb[S];
+        auto load_block = [&](mk_i4 *wv, int s0) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] += (wsf * x4[i]) * (float)c[i];
+            for (int j = 0; j < S; j++) {
+                const int s = min(s0 + j, steps - 1);  // past the end: a repeated, unused load
+                wv[j] = *reinterpret_cast<const mk_i4 *>(wrow + s * 64);
+            }
+        };
+        auto compute_block = [&](const mk_i4 *wv, int s0) {
+#pragma unroll
+            for (int j = 0; j < S; j++) {
+                const int s = s0 + j;
+                if (s < steps) {
+                    mk_i4 xa = xl[(s * 4 + kb) * 8 + a_batch];
+                    if (!a_live) xa = mk_i4{0, 0, 0, 0};
+                    mk_i4 c = {0, 0, 0, 0};
+                    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa, wv[j], c, 0, 0, 0);
+                    const mk_f4 x4 = *reinterpret_cast<const mk_f4 *>(xsl + (2 * s + par) * 8 + 4 * (kb & 1));
+                    const float wsf = F16 ? mk_f16_bits_to_f32(*reinterpret_cast<const uint16_t *>(srow + 2 * s * SB))
+                                          : *reinterpret_cast<const float *>(srow + 2 * s * SB);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[i] += (wsf * x4[i]) * (float)c[i];
+                }
+            }
+        };
+        load_block(wa, 0);
+        for (int s0 = 0; s0 < steps; s0 += 2 * S) {
+            if (s0 + S < steps) load_block(wb, s0 + S);
+            compute_block(wa, s0);
+            if (s0 + 2 * S < steps) load_block(wa, s0 + 2 * S);
+            if (s0 + S < steps) compute_block(wb, s0 + S);
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32, MK_WAVE);  // the two block parities
@@ -234,13 +288,17 @@ __global__ __launch_bounds__(256) void argmax_stage2_kernel(const float *__restr
     if (threadIdx.x == 0) out[b] = bi == 0x7FFFFFFF ? 0 : bi;
 }
 
+int tune(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return (e && *e) ? atoi(e) : dflt;
+}
+
 template <int NB, bool F16>
 void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
-    // about 8 waves per SIMD-slot on 256 CUs, at least 4 rows per wave to amortise the activation registers
-    int rpw = (rows + 256 * 16 - 1) / (256 * 16);
-    if (rpw < 4) rpw = 4;
-    const int waves = (rows + rpw - 1) / rpw;
-    hipLaunchKernelGGL((q8_gemv_b1_kernel<NB, F16>), dim3((waves + 3) / 4), dim3(256), 0, st, q, scales, rows, xq, xs, out, rpw);
+    // a fixed, fully resident grid: blocks-per-CU x 256 CUs x 4 waves
+    int blocks = tune("MK_Q8_B1_BLOCKS", 512);
+    if (blocks * 4 > rows) blocks = (rows + 3) / 4;
+    hipLaunchKernelGGL((q8_gemv_b1_kernel<NB, F16>), dim3(blocks), dim3(256), 0, st, q, scales, rows, xq, xs, out);
 }
 
 template <bool F16>
@@ -255,14 +313,15 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
             case 224: launch_b1<224, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
             default: break;
         }
-    } else if (nb % 2 == 0 && cols * 8 + (size_t)nb * 32 <= 150 * 1024) {
+    } else if (nb % 2 == 0 && nb <= 256) {
+        // LDS: activations (cols * 8) + their scales (nb * 32) + one scale tile per wave (16 * nb * 2 or 4 bytes)
+        constexpr int WAVES = F16 ? 8 : 4;
         const int n_groups = (int)((rows + 15) / 16);
-        int gpw = (n_groups + 256 * 16 - 1) / (256 * 16);
-        if (gpw < 1) gpw = 1;
-        const int waves = (n_groups + gpw - 1) / gpw;
-        const size_t lds = cols * 8 + (size_t)nb * 32;
-        hipLaunchKernelGGL(q8_gemv_mfma_kernel<F16>, dim3((waves + 7) / 8), dim3(512), lds, st, q, scales, (int)rows, nb, xq, xs, (int)batch,
-                           out, gpw);
+        int blocks = tune("MK_Q8_MFMA_BLOCKS", 256);  // one per CU
+        if (blocks * WAVES > n_groups) blocks = (n_groups + WAVES - 1) / WAVES;
+        const size_t lds = cols * 8 + (size_t)nb * 32 + (size_t)WAVES * 16 * nb * (F16 ? 2 : 4);
+        hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq, xs,
+                           (int)batch, out);
         return mk_launch_status("q8_gemv_mfma");
     }
     hipLaunchKernelGGL(q8_gemv_generic_kernel<F16>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, q, scales, (int)rows, nb, xq, xs,
@@ -282,9 +341,9 @@ extern "C" int mk_dev_q8_matvec(const int8_t *q, const void *scales, int scales_
     if (rows == 0) return MK_OK;
     static bool lds_opt_in = false;
     if (!lds_opt_in) {
-        // the batch kernel stages up to 150 KiB of activations in the 160 KiB LDS
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        // the batch kernel uses up to 136 KiB of the 160 KiB LDS
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         lds_opt_in = true;
     }
     if (scales_f16) return launch_q8<true>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);
