@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP4_PEAK_TFLOPS = 10100.0   # dense FP4/FP6 MFMA
 FP8_PEAK_TFLOPS = 5000.0
+# HBM bytes per launch of the batch-1 lm_head GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
+# reading of a plain 1 GiB copy (factors 2.000 and 1.000): 1 218 730 KiB read + 1 429 KiB written
+# (profiles/q8_gemv_b1_lm_head_163840x7168.md).  Algorithmic bytes are 1 248 489 472.
+LM_HEAD_B1_TRAFFIC_BYTES = 1249443000
 
 
 def log(*a):
@@ -310,6 +314,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run five plain 1 GiB device copies (a kernel of known traffic to scale rocprofv3 --pmc byte counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -322,6 +328,14 @@ def main():
     _lib.require_device()
     torch.cuda.set_device(0)
 
+    if args.copy_calibration:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     log("lm_head ...")
     head, tensors = bench_lm_head(torch, args.steps, args.warmup)
     cpu = None
@@ -356,7 +370,7 @@ def main():
         "config": {"workload": "config 1: q8_0 lm_head 163840x7168 (int8 + f16 scale per 32), batch 1; step = quantize_q8(x) + GEMV",
                    "rows": 163840, "cols": 7168, "batch": 1, "algorithmic_bytes": head["alg_bytes"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": LM_HEAD_B1_TRAFFIC_BYTES,
                      "kernel": "q8_gemv_b1_kernel<224, f16 scales>", "kernel_ms": head["kernel_ms"]},
         "cpu_baseline": cpu,
         "extras": extras,
