@@ -18,6 +18,8 @@
 //     contribution is (h+h) * (2^(sb-128) * dx), the reference's expression.
 //   * one butterfly reduction per row, fixed order (deterministic).
 // Generic path: one wave per row, any cols % 32 == 0.
+#include <stdlib.h>
+
 #include "mk_common.h"
 
 namespace {
@@ -75,6 +77,41 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     const int8_t *xq = a.xq + (size_t)xi * NB * 32;
     const float *xs = a.xs + (size_t)xi * NB;
 
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    // Tiles of this matrix are dealt round-robin to the matrix's resident waves
+    // (wave w takes tiles w, w + W, ...): equal work, one compact read window.
+    // U tiles form a register block; two blocks (ping, pong) are in flight.
+    constexpr int U = (T >= 4) ? 1 : 8 / T;  // about 8 KiB per register block: T=1 -> 8 tiles, T=2 -> 4, T=3 -> 2
+    const int n_tiles = (a.rows + RT - 1) / RT;
+    const int wv = blockIdx.x * 4 + wave;
+    const int wpm = gridDim.x * 4;
+    const int my_tiles = wv < n_tiles ? (n_tiles - wv + wpm - 1) / wpm : 0;
+
+    mk_i4 wa[U][T], wb[U][T];
+    uint32_t sa[U][T], sb[U][T];
+    // Loads are unconditional (a predicated load becomes a branch and a full
+    // wait): a tile past the end re-reads the wave's first tile and a lane past
+    // the last row re-reads the last block; neither result is stored.
+    const size_t last_blk = (size_t)a.rows * NB - 1;
+    auto load_block = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int k0) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int tile = wv + ((k0 + u < my_tiles) ? (k0 + u) * wpm : 0);
+            const size_t blk0 = (size_t)tile * TILE;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                size_t blk = blk0 + t * 64 + lane;
+                blk = blk < last_blk ? blk : last_blk;
+                w[u][t] = mk_ldg128(packed + blk * 16);
+                sc[u][t] = mk_ldg_u8(scales + blk);
+            }
+        }
+    };
+    // the first register block is requested before the activation is staged:
+    // the weight stream does not wait for the prologue
+    load_block(wa, sa, 0);
+
     // stage the activation: int8 -> f16 (exact), 4 values per thread per step
     for (int i = threadIdx.x; i < NB * 8; i += 256) {
         uint32_t v = reinterpret_cast<const uint32_t *>(xq)[i];
@@ -89,8 +126,6 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     for (int i = threadIdx.x; i < NB; i += 256) xsc[i] = xs[i];
     __syncthreads();
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
     mk_h2 xr[T][16];
     float cf[T];
 #pragma unroll
@@ -101,49 +136,40 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
         cf[t] = xsc[g];
     }
 
-    const int n_tiles = (a.rows + RT - 1) / RT;
-    const int tile0 = (blockIdx.x * 4 + wave) * a.tiles_per_wave;
-    const int tile1 = min(tile0 + a.tiles_per_wave, n_tiles);
-
-    mk_i4 w[T];
-    uint32_t sb[T];
-    auto load_tile = [&](int tile) {
-        const size_t blk0 = (size_t)tile * TILE;
+    auto compute_block = [&](const mk_i4(*w)[T], const uint32_t(*sc)[T], int k0) {
+        float acc[U][RT];
 #pragma unroll
-        for (int t = 0; t < T; t++) {
-            const int bi = t * 64 + lane;
-            const bool ok = tile * RT + bi / NB < a.rows;
-            w[t] = ok ? *reinterpret_cast<const mk_i4 *>(packed + (blk0 + bi) * 16) : mk_i4{0, 0, 0, 0};
-            sb[t] = ok ? (uint32_t)scales[blk0 + bi] : 0u;
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int r = 0; r < RT; r++) acc[u][r] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                float h = dot32_fp4_f16(w[u][t], xr[t]);
+                float term = (h + h) * (mk_half_scale_from_byte(sc[u][t]) * cf[t]);
+                const int rit = (t * 64 + lane) / NB;
+#pragma unroll
+                for (int r = 0; r < RT; r++) acc[u][r] += (rit == r) ? term : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int r = 0; r < RT; r++) acc[u][r] = mk_wave_sum(acc[u][r]);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (k0 + u < my_tiles && lane < RT) {
+                const int row = (wv + (k0 + u) * wpm) * RT + lane;
+                if (row < a.rows) out[row] = (RT == 2 && lane == 1) ? acc[u][RT - 1] : acc[u][0];
+            }
         }
     };
-    if (tile0 < tile1) load_tile(tile0);
-    for (int tile = tile0; tile < tile1; tile++) {
-        mk_i4 wc[T];
-        uint32_t sc[T];
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            wc[t] = w[t];
-            sc[t] = sb[t];
-        }
-        if (tile + 1 < tile1) load_tile(tile + 1);  // next tile in flight while this one is reduced
-        float acc[RT];
-#pragma unroll
-        for (int r = 0; r < RT; r++) acc[r] = 0.0f;
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            float h = dot32_fp4_f16(wc[t], xr[t]);
-            float term = (h + h) * (mk_half_scale_from_byte(sc[t]) * cf[t]);
-            const int rit = (t * 64 + lane) / NB;
-#pragma unroll
-            for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
-        }
-#pragma unroll
-        for (int r = 0; r < RT; r++) acc[r] = mk_wave_sum(acc[r]);
-        if (lane < RT) {
-            const int row = tile * RT + lane;
-            if (row < a.rows) out[row] = (RT == 2 && lane == 1) ? acc[RT - 1] : acc[0];
-        }
+    // the prefetches are unconditional (past the end they re-read a valid tile):
+    // a load under a branch forces a full wait at the join
+    for (int k0 = 0; k0 < my_tiles; k0 += 2 * U) {
+        load_block(wb, sb, k0 + U);
+        compute_block(wa, sa, k0);
+        load_block(wa, sa, k0 + 2 * U);
+        compute_block(wb, sb, k0 + U);
     }
 }
 
@@ -317,22 +343,31 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__res
     }
 }
 
+int tune(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return (e && *e) ? atoi(e) : dflt;
+}
+
 template <int NB>
 int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
     constexpr int RT = lcm_c(NB, 64) / NB;
     GemvArgs a = a0;
     const int n_tiles = (a.rows + RT - 1) / RT;
-    // enough waves to fill 256 CUs several times over, but several tiles per
-    // wave so the activation staging is amortised
+    if (q8) {
+        // a fixed, fully resident grid shared by the matrices of the launch
+        // 2 workgroups per CU where the activation registers allow 2 waves per SIMD (T >= 4), else 3
+        int per_mat = tune("MK_MXFP4_BLOCKS", lcm_c(NB, 64) / 64 >= 4 ? 512 : 768) / (int)nmat;
+        if (per_mat < 1) per_mat = 1;
+        if (per_mat * 4 > n_tiles) per_mat = (n_tiles + 3) / 4;
+        hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(per_mat, (unsigned)nmat), dim3(256), 0, st, a);
+        return mk_launch_status("mxfp4_gemv_q8");
+    }
     int tpw = 1;
     while (tpw < 16 && (size_t)n_tiles * nmat / (tpw * 2) >= 256 * 4 * 4) tpw *= 2;
     a.tiles_per_wave = tpw;
     const unsigned gx = (unsigned)((n_tiles + 4 * tpw - 1) / (4 * tpw));
-    if (q8)
-        hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a);
-    else
-        hipLaunchKernelGGL(mxfp4_gemv_f32_kernel<NB>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a);
-    return mk_launch_status("mxfp4_gemv");
+    hipLaunchKernelGGL(mxfp4_gemv_f32_kernel<NB>, dim3(gx, (unsigned)nmat), dim3(256), 0, st, a);
+    return mk_launch_status("mxfp4_gemv_f32");
 }
 
 int launch_gemv(const GemvArgs &a, bool q8, size_t nmat, size_t cols, hipStream_t st) {

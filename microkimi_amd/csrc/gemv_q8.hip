@@ -24,8 +24,8 @@ namespace {
 
 template <bool F16>
 __device__ __forceinline__ float load_scale(const void *scales, size_t idx) {
-    if (F16) return mk_f16_bits_to_f32(reinterpret_cast<const uint16_t *>(scales)[idx]);
-    return reinterpret_cast<const float *>(scales)[idx];
+    if (F16) return mk_f16_bits_to_f32(mk_ldg_u16(reinterpret_cast<const uint16_t *>(scales) + idx));
+    return mk_ldg_f32(reinterpret_cast<const float *>(scales) + idx);
 }
 
 // ------------------------------------------------------------- batch 1
@@ -51,35 +51,38 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
     }
     mk_i4 w[T];
     float ws[T];
-    auto load_row = [&](int r) {
+    // two rows in flight (ping, pong); prefetches are unconditional, past the
+    // end they re-read the last row (a load under a branch forces a full wait)
+    mk_i4 wa[T], wb[T];
+    float sa[T], sb[T];
+    auto load_row = [&](mk_i4 *w, float *ws, int r) {
+        r = min(r, rows - 1);
         const int8_t *row = q + (size_t)r * NB * 32;
 #pragma unroll
         for (int t = 0; t < T; t++) {
             const int hb = t * 64 + lane;
-            w[t] = *reinterpret_cast<const mk_i4 *>(row + hb * 16);
+            w[t] = mk_ldg128(row + hb * 16);
             ws[t] = load_scale<F16>(scales, (size_t)r * NB + (hb >> 1));
         }
     };
-    if (wave < rows) load_row(wave);
-    for (int r = wave; r < rows; r += n_waves) {
-        mk_i4 wc[T];
-        float wsc[T];
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            wc[t] = w[t];
-            wsc[t] = ws[t];
-        }
-        if (r + n_waves < rows) load_row(r + n_waves);
+    auto compute_row = [&](const mk_i4 *w, const float *ws, int r) {
         float acc = 0.0f;
 #pragma unroll
         for (int t = 0; t < T; t++) {
             int d = 0;
 #pragma unroll
-            for (int k = 0; k < 4; k++) d = __builtin_amdgcn_sdot4(wc[t][k], xr[t][k], d, false);
-            acc += (wsc[t] * cf[t]) * (float)d;
+            for (int k = 0; k < 4; k++) d = __builtin_amdgcn_sdot4(w[t][k], xr[t][k], d, false);
+            acc += (ws[t] * cf[t]) * (float)d;
         }
         acc = mk_wave_sum(acc);
-        if (lane == 0) out[r] = acc;
+        if (lane == 0 && r < rows) out[r] = acc;
+    };
+    load_row(wa, sa, wave);
+    for (int r = wave; r < rows; r += 2 * n_waves) {
+        load_row(wb, sb, r + n_waves);
+        compute_row(wa, sa, r);
+        load_row(wa, sa, r + 2 * n_waves);
+        compute_row(wb, sb, r + n_waves);
     }
 }
 
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
 #pragma unroll
             for (int j = 0; j < S; j++) {
                 const int s = min(s0 + j, steps - 1);  // past the end: a repeated, unused load
-                wv[j] = *reinterpret_cast<const mk_i4 *>(wrow + s * 64);
+                wv[j] = mk_ldg128(wrow + s * 64);
             }
         };
         auto compute_block = [&](const mk_i4 *wv, int s0) {
@@ -180,10 +183,10 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
         };
         load_block(wa, 0);
         for (int s0 = 0; s0 < steps; s0 += 2 * S) {
-            if (s0 + S < steps) load_block(wb, s0 + S);
+            load_block(wb, s0 + S);  // unconditional: past the end it repeats the last step
             compute_block(wa, s0);
-            if (s0 + 2 * S < steps) load_block(wa, s0 + 2 * S);
-            if (s0 + S < steps) compute_block(wb, s0 + S);
+            load_block(wa, s0 + 2 * S);
+            compute_block(wb, s0 + S);
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[i] += __shfl_xor(acc[i], 32, MK_WAVE);  // the two block parities

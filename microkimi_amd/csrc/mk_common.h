@@ -14,6 +14,15 @@ typedef int mk_i8v __attribute__((ext_vector_type(8)));
 typedef float mk_f4 __attribute__((ext_vector_type(4)));
 typedef float mk_f16v __attribute__((ext_vector_type(16)));
 
+// Loads that tell the compiler the pointer is global memory.  A pointer that was
+// itself loaded from memory (an expert table entry) is a generic pointer to the
+// compiler and would be read with flat_load, which also ties up the LDS counter.
+#define MK_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ mk_i4 mk_ldg128(const void *p) { return *(const MK_GLOBAL mk_i4 *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ uint32_t mk_ldg_u8(const void *p) { return *(const MK_GLOBAL uint8_t *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ uint16_t mk_ldg_u16(const void *p) { return *(const MK_GLOBAL uint16_t *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ float mk_ldg_f32(const void *p) { return *(const MK_GLOBAL float *)(const MK_GLOBAL void *)p; }
+
 // 2^(sb-127) from an e8m0 byte as an exact bit pattern; byte 0 is the
 // subnormal 2^-127 (mxfp4::scale_from_byte, src/mxfp4.rs:340-346).
 __device__ __forceinline__ float mk_scale_from_byte(uint32_t sb) {
@@ -44,16 +53,31 @@ __device__ __forceinline__ float mk_e2m1(uint32_t nib) {
     return __uint_as_float(bits | ((nib & 8u) << 28));
 }
 
+// Wave-wide reductions without LDS traffic: four DPP steps fold each row of 16
+// lanes (quad swaps, half-row mirror, row mirror), then the four row results are
+// read with v_readlane and combined.  All 64 lanes must be active.  The result
+// is the same value in every lane; the association is fixed (deterministic).
+template <int CTRL>
+__device__ __forceinline__ float mk_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float mk_readlane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float mk_wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, MK_WAVE);
-    return v;
+    v += mk_dpp<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += mk_dpp<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += mk_dpp<0x141>(v);  // row_half_mirror
+    v += mk_dpp<0x140>(v);  // row_mirror
+    return (mk_readlane(v, 0) + mk_readlane(v, 16)) + (mk_readlane(v, 32) + mk_readlane(v, 48));
 }
 
 __device__ __forceinline__ float mk_wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, MK_WAVE));
-    return v;
+    v = fmaxf(v, mk_dpp<0xB1>(v));
+    v = fmaxf(v, mk_dpp<0x4E>(v));
+    v = fmaxf(v, mk_dpp<0x141>(v));
+    v = fmaxf(v, mk_dpp<0x140>(v));
+    return fmaxf(fmaxf(mk_readlane(v, 0), mk_readlane(v, 16)), fmaxf(mk_readlane(v, 32), mk_readlane(v, 48)));
 }
 
 // sum / max over aligned groups of 32 lanes
