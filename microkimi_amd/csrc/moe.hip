@@ -2,18 +2,20 @@
 // (src/model.rs:2227-2264,2346-2351; src/deepseek.rs:1069-1106) for B tokens as
 // one grouped pass over the (token, slot) pairs.
 //
+// Fast path (q8 mode, benchmark-like shapes): two fused launches, see below.
+// Composed path (any shape, both modes):
 //   setup     pair tables (expert pointers per pair) from the router's ids
 //   quantize  x -> q8 (once per token; gate and up quantize the same input to
 //             the same bytes in the reference)
-//   gate_up   per pair and 32-row block: a = W1 x, u = W3 x with the GEMV tiling
-//             of gemv_mxfp4.hip, act = ACT(a, u) kept in lanes 0..31, then the
-//             q8 quantization of that 32-block of `act` in-wave -- exactly the
-//             block matvec_packed would form when it re-quantizes its input for W2
+//   gate, up  grouped MXFP4 GEMVs over all pairs, elementwise activation,
+//             q8 quantization of the activation
 //   down      o = W2 act: the grouped MXFP4 GEMV over all pairs
 //   combine   out_t = sum_slot w * o in slot order (+ shared expert)
 //
 // HBM traffic: every selected expert's 23.4 MB is read once per pair; the
 // intermediates (act: 2 KiB + 256 B per pair, o: 28 KiB per pair) are noise.
+#include <stdlib.h>
+
 #include "mk_common.h"
 
 // grouped MXFP4 GEMV of gemv_mxfp4.hip: q8 (xq, xs) or f32 (xf) activations, one launch over nmat matrices
@@ -118,93 +120,281 @@ __device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
     return h;
 }
 
-// gate + up + activation + q8 of the activation block.  One wave = 32 rows of
-// one pair.  NB = d / 32.
+// ------------------------------------------------------------ fused fast path
+// Two launches per layer, no setup / quantize / combine kernels:
+//
+//   gate_up  grid (inter/32, pairs).  A workgroup owns one 32-row block of one
+//            (token, slot) pair; each of its 4 waves computes 8 rows of W1 x and
+//            W3 x.  The workgroup quantizes the token's hidden row to q8 itself
+//            (thread i owns block i: the loop of src/q8.rs:57-68) while its first
+//            weight loads are already in flight; the activation's f16 form lives
+//            in LDS.  The 32 activation values of the block are then quantized
+//            to q8 (the block matvec_packed forms when it re-quantizes its input
+//            for W2) and stored with their scale.
+//   down     grid (blocks, tokens).  The rows of W2 are dealt round-robin to the
+//            token's waves; a wave walks its rows pair by pair in slot order and
+//            accumulates y += w * (W2_e act) in registers, so the weighted sum of
+//            src/model.rs:2346-2351 needs no intermediate buffer.
+struct FusedArgs {
+    mk_expert_table tab;
+    const int32_t *ids;
+    const float *weights;
+    const float *x;
+    int topk, shared, per, d, inter, act_kind, ds_rule;
+    float limit;
+    int8_t *aq;  // [P][inter]
+    float *as;   // [P][inter/32]
+    float *out;  // [B][d]
+};
+
 template <int NB>
-__global__ __launch_bounds__(256) void moe_gate_up_q8_kernel(PairTables pt, const int8_t *__restrict__ xq, const float *__restrict__ xs,
-                                                             int inter, int act_kind, float limit, int8_t *__restrict__ aq,
-                                                             float *__restrict__ as) {
+__global__ __launch_bounds__(256) void moe_gate_up_fused_kernel(FusedArgs a) {
     constexpr int TILE = lcm_c(NB, 64);
     constexpr int T = TILE / 64;
     constexpr int RT = TILE / NB;
     static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
-    // f16 pairs kept as 32-bit words: written and read through the same type
+    constexpr int RPW = 8;           // rows per wave
+    constexpr int NI = 2 * RPW / RT;  // work items of a wave: (matrix, tile), matrix fastest
+    constexpr int G0 = T >= 4 ? 1 : (T == 3 ? 2 : (T == 2 ? 4 : 8));
+    constexpr int G = G0 < NI ? G0 : NI;  // items per register block
+    // x as f16 pairs (words), laid out [4 chunks][NB blocks][4 words]: lanes that
+    // read the same chunk of consecutive blocks touch consecutive 16-byte slots
     __shared__ __attribute__((aligned(16))) uint32_t xh[NB * 16];
     __shared__ float xsc[NB];
-    const int p = blockIdx.y;
-    const uint8_t *w1p = pt.w1p[p], *w1s = pt.w1s[p], *w3p = pt.w3p[p], *w3s = pt.w3s[p];
-    const int tok = pt.xidx[p];
-    const float wgt = pt.pw[p];
-    const int8_t *xqv = xq + (size_t)tok * NB * 32;
-    const float *xsv = xs + (size_t)tok * NB;
-    for (int i = threadIdx.x; i < NB * 8; i += 256) {
-        uint32_t v = reinterpret_cast<const uint32_t *>(xqv)[i];
+    __shared__ float act_l[32];
+
+    const int p = blockIdx.x, rb = blockIdx.y;  // pairs fastest: pairs that share an expert read a row block together
+    const int tok = p / a.per, slot = p % a.per;
+    const int e = slot < a.topk ? a.ids[tok * a.topk + slot] : a.shared;
+    const float wgt = slot < a.topk ? a.weights[tok * a.topk + slot] : 1.0f;
+    const uint8_t *wp[2] = {a.tab.w1p[e], a.tab.w3p[e]};
+    const uint8_t *wsc[2] = {a.tab.w1s[e], a.tab.w3s[e]};
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row0 = (size_t)rb * 32 + wave * RPW;
+
+    mk_i4 wa[G][T], wb[G][T];
+    uint32_t sa[G][T], sb[G][T];
+    auto load_block = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int it0) {
+#pragma unroll
+        for (int j = 0; j < G; j++) {
+            const int it = it0 + j;
+            if (it < NI) {  // compile-time after unrolling
+                const size_t blk0 = (row0 + (size_t)(it >> 1) * RT) * NB;
+#pragma unroll
+                for (int t = 0; t < T; t++) {
+                    const size_t b = blk0 + t * 64 + lane;
+                    w[j][t] = mk_ldg128(wp[it & 1] + b * 16);
+                    sc[j][t] = mk_ldg_u8(wsc[it & 1] + b);
+                }
+            }
+        }
+    };
+    load_block(wa, sa, 0);  // in flight during the prologue
+
+    // q8 of the token's hidden row: thread i owns block i (NB <= 256)
+    if (threadIdx.x < NB) {
+        const mk_f4 *src = reinterpret_cast<const mk_f4 *>(a.x + (size_t)tok * NB * 32 + threadIdx.x * 32);
+        mk_f4 v[8];
+        float mx = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = src[k];
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
+        }
+        const float dx = mx / 127.0f;
+        xsc[threadIdx.x] = dx;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
+            if (dx != 0.0f) {
+                lo.x = (_Float16)(float)mk_q8_round(v[k].x, dx);
+                lo.y = (_Float16)(float)mk_q8_round(v[k].y, dx);
+                hi.x = (_Float16)(float)mk_q8_round(v[k].z, dx);
+                hi.y = (_Float16)(float)mk_q8_round(v[k].w, dx);
+            }
+            xh[((k >> 1) * NB + threadIdx.x) * 4 + 2 * (k & 1)] = __builtin_bit_cast(uint32_t, lo);
+            xh[((k >> 1) * NB + threadIdx.x) * 4 + 2 * (k & 1) + 1] = __builtin_bit_cast(uint32_t, hi);
+        }
+    }
+    __syncthreads();
+    float cf[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) cf[t] = xsc[(t * 64 + lane) % NB];
+
+    float res[2][RPW];  // [matrix][row]
+#pragma unroll
+    for (int m = 0; m < 2; m++)
+#pragma unroll
+        for (int r = 0; r < RPW; r++) res[m][r] = 0.0f;
+    auto compute_block = [&](const mk_i4(*w)[T], const uint32_t(*sc)[T], int it0) {
+#pragma unroll
+        for (int j = 0; j < G; j++) {
+            const int it = it0 + j;
+            if (it < NI) {
+                float acc[RT];
+#pragma unroll
+                for (int r = 0; r < RT; r++) acc[r] = 0.0f;
+#pragma unroll
+                for (int t = 0; t < T; t++) {
+                    const int g = (t * 64 + lane) % NB;
+                    mk_h2 xr[16];
+#pragma unroll
+                    for (int k = 0; k < 16; k++) xr[k] = __builtin_bit_cast(mk_h2, xh[((k >> 2) * NB + g) * 4 + (k & 3)]);
+                    float h = dot32_fp4_f16(w[j][t], xr);
+                    float term = (h + h) * (mk_half_scale_from_byte(sc[j][t]) * cf[t]);
+                    const int rit = (t * 64 + lane) / NB;
+#pragma unroll
+                    for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
+                }
+#pragma unroll
+                for (int r = 0; r < RT; r++) res[it & 1][(it >> 1) * RT + r] = mk_wave_sum(acc[r]);
+            }
+        }
+    };
+#pragma unroll
+    for (int it0 = 0; it0 < NI; it0 += 2 * G) {
+        load_block(wb, sb, it0 + G);
+        compute_block(wa, sa, it0);
+        load_block(wa, sa, it0 + 2 * G);
+        compute_block(wb, sb, it0 + G);
+    }
+    float mine = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RPW; r++) {
+        const float act = mk_act(a.act_kind, res[0][r], res[1][r], a.limit, wgt);
+        if (lane == r) mine = act;
+    }
+    if (lane < RPW) act_l[wave * RPW + lane] = mine;
+    __syncthreads();
+    if (wave == 0) {
+        const float v = act_l[lane & 31];
+        const float mx = mk_half_wave_max(fabsf(v));
+        const float dx = mx / 127.0f;
+        if (lane < 32) {
+            const int qi = dx != 0.0f ? mk_q8_round(v, dx) : 0;
+            a.aq[(size_t)p * a.inter + rb * 32 + lane] = (int8_t)qi;
+            if (lane == 0) a.as[(size_t)p * (a.inter / 32) + rb] = dx;
+        }
+    }
+}
+
+constexpr int MAX_PER = 32;  // pairs per token the fused down kernel keeps in LDS
+
+template <int NB, int U>  // U = tiles per register block
+__global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
+    constexpr int TILE = lcm_c(NB, 64);
+    constexpr int T = TILE / 64;
+    constexpr int RT = TILE / NB;
+    static_assert(RT <= 2 && T <= 2 && U * T <= 8, "tile shape not covered by the fused down kernel");
+    // per pair: the activation as f16 pairs, [4 chunks][NB blocks][4 words] (see
+    // the gate/up kernel); after all pairs, their block scales [per][NB]
+    extern __shared__ __attribute__((aligned(16))) uint32_t ah[];
+    __shared__ const uint8_t *wp_l[MAX_PER];
+    __shared__ const uint8_t *ws_l[MAX_PER];
+    __shared__ float pw_l[MAX_PER];
+    const int tok = blockIdx.x, per = a.per;  // tokens fastest: they walk the rows in step
+    float *asc = reinterpret_cast<float *>(ah + (size_t)per * NB * 16);
+    if (threadIdx.x < per) {
+        const int s = threadIdx.x;
+        const int e = s < a.topk ? a.ids[tok * a.topk + s] : a.shared;
+        wp_l[s] = a.tab.w2p[e];
+        ws_l[s] = a.tab.w2s[e];
+        pw_l[s] = (s < a.topk && !a.ds_rule) ? a.weights[tok * a.topk + s] : 1.0f;
+    }
+    const int8_t *aq = a.aq + (size_t)tok * per * NB * 32;
+    for (int i = threadIdx.x; i < per * NB * 8; i += 256) {
+        uint32_t v = reinterpret_cast<const uint32_t *>(aq)[i];
         mk_h2 lo, hi;
         lo.x = (_Float16)(float)(int8_t)(v & 255u);
         lo.y = (_Float16)(float)(int8_t)((v >> 8) & 255u);
         hi.x = (_Float16)(float)(int8_t)((v >> 16) & 255u);
         hi.y = (_Float16)(float)(int8_t)(v >> 24);
-        xh[i * 2] = __builtin_bit_cast(uint32_t, lo);
-        xh[i * 2 + 1] = __builtin_bit_cast(uint32_t, hi);
+        // word i covers elements 4i..4i+3 of pair s: block g, f16 words 2j, 2j+1
+        const int s = i / (NB * 8), g = (i / 8) % NB, j = i % 8;
+        uint32_t *dst = ah + (size_t)s * NB * 16 + ((j >> 1) * NB + g) * 4 + 2 * (j & 1);
+        dst[0] = __builtin_bit_cast(uint32_t, lo);
+        dst[1] = __builtin_bit_cast(uint32_t, hi);
     }
-    for (int i = threadIdx.x; i < NB; i += 256) xsc[i] = xsv[i];
+    for (int i = threadIdx.x; i < per * NB; i += 256) asc[i] = a.as[(size_t)tok * per * NB + i];
     __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int rb = blockIdx.x * 4 + (threadIdx.x >> 6);  // 32-row block of the pair
-    if (rb * 32 >= inter) return;
-    mk_h2 xr[T][16];
-    float cf[T];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_tiles = a.d / RT;
+    const int wv = blockIdx.y * 4 + wave, wpt = gridDim.y * 4;
+    const int my_tiles = wv < n_tiles ? (n_tiles - wv + wpt - 1) / wpt : 0;
+    const int groups = (my_tiles + U - 1) / U;
+    const int n_items = groups * per;  // (tile group, pair), pair fastest: slot order per row
+
+    mk_i4 wa[U][T], wb[U][T];
+    uint32_t sa[U][T], sb[U][T];
+    auto load_item = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int i) {
+        i = i < n_items ? i : 0;  // unconditional loads: past the end, item 0 again
+        const int grp = i / per, s = i - grp * per;
+        const uint8_t *wp = wp_l[s], *ws = ws_l[s];
 #pragma unroll
-    for (int t = 0; t < T; t++) {
-        const int g = (t * 64 + lane) % NB;
+        for (int u = 0; u < U; u++) {
+            const int k = grp * U + u;
+            const int tile = wv + (k < my_tiles ? k : 0) * wpt;
+            const size_t blk0 = (size_t)tile * TILE;
 #pragma unroll
-        for (int k = 0; k < 16; k++) xr[t][k] = __builtin_bit_cast(mk_h2, xh[g * 16 + k]);
-        cf[t] = xsc[g];
-    }
-    float myact = 0.0f;
-    for (int i = 0; i < 32 / RT; i++) {
-        const size_t blk0 = ((size_t)rb * 32 + (size_t)i * RT) * NB;  // first block of the tile (rows are contiguous)
-        mk_i4 wa[T], wu[T];
-        uint32_t sa[T], su[T];
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            const size_t b = blk0 + t * 64 + lane;
-            wa[t] = *reinterpret_cast<const mk_i4 *>(w1p + b * 16);
-            wu[t] = *reinterpret_cast<const mk_i4 *>(w3p + b * 16);
-            sa[t] = w1s[b];
-            su[t] = w3s[b];
-        }
-        float ga[RT], gu[RT];
-#pragma unroll
-        for (int r = 0; r < RT; r++) ga[r] = gu[r] = 0.0f;
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            float ha = dot32_fp4_f16(wa[t], xr[t]);
-            float hu = dot32_fp4_f16(wu[t], xr[t]);
-            float ta = (ha + ha) * (mk_half_scale_from_byte(sa[t]) * cf[t]);
-            float tu = (hu + hu) * (mk_half_scale_from_byte(su[t]) * cf[t]);
-            const int rit = (t * 64 + lane) / NB;
-#pragma unroll
-            for (int r = 0; r < RT; r++) {
-                ga[r] += (rit == r) ? ta : 0.0f;
-                gu[r] += (rit == r) ? tu : 0.0f;
+            for (int t = 0; t < T; t++) {
+                w[u][t] = mk_ldg128(wp + (blk0 + t * 64 + lane) * 16);
+                sc[u][t] = mk_ldg_u8(ws + blk0 + t * 64 + lane);
             }
         }
+    };
+    float y[U][RT];
 #pragma unroll
-        for (int r = 0; r < RT; r++) {
-            float a = mk_wave_sum(ga[r]);
-            float u = mk_wave_sum(gu[r]);
-            float act = mk_act(act_kind, a, u, limit, wgt);
-            if (lane == i * RT + r) myact = act;
+    for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int r = 0; r < RT; r++) y[u][r] = 0.0f;
+    auto compute_item = [&](const mk_i4(*w)[T], const uint32_t(*sc)[T], int i) {
+        const int grp = i / per, s = i - grp * per;
+        mk_h2 xr[T][16];
+        float cf[T];
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const int g = (t * 64 + lane) % NB;
+#pragma unroll
+            for (int k = 0; k < 16; k++) xr[t][k] = __builtin_bit_cast(mk_h2, ah[(size_t)s * NB * 16 + ((k >> 2) * NB + g) * 4 + (k & 3)]);
+            cf[t] = asc[s * NB + g];
         }
-    }
-    // lanes 0..31 hold act[rb*32 + lane]: q8 of this block (src/q8.rs:57-68)
-    float mx = mk_half_wave_max(fabsf(myact));
-    float dx = mx / 127.0f;
-    if (lane < 32) {
-        int qi = dx != 0.0f ? mk_q8_round(myact, dx) : 0;
-        aq[(size_t)p * inter + rb * 32 + lane] = (int8_t)qi;
-        if (lane == 0) as[(size_t)p * (inter / 32) + rb] = dx;
+        const float pw = pw_l[s];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float acc[RT];
+#pragma unroll
+            for (int r = 0; r < RT; r++) acc[r] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                float h = dot32_fp4_f16(w[u][t], xr[t]);
+                float term = (h + h) * (mk_half_scale_from_byte(sc[u][t]) * cf[t]);
+                const int rit = (t * 64 + lane) / NB;
+#pragma unroll
+                for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
+            }
+#pragma unroll
+            for (int r = 0; r < RT; r++) y[u][r] = __fadd_rn(y[u][r], __fmul_rn(pw, mk_wave_sum(acc[r])));
+        }
+        if (s == per - 1) {  // the row's last pair: store and start the next rows
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int k = grp * U + u;
+                if (k < my_tiles && lane < RT) {
+                    const int row = (wv + k * wpt) * RT + lane;
+                    a.out[(size_t)tok * a.d + row] = (RT == 2 && lane == 1) ? y[u][RT - 1] : y[u][0];
+                }
+#pragma unroll
+                for (int r = 0; r < RT; r++) y[u][r] = 0.0f;
+            }
+        }
+    };
+    load_item(wa, sa, 0);
+    for (int i = 0; i < n_items; i += 2) {
+        load_item(wb, sb, i + 1);
+        compute_item(wa, sa, i);
+        load_item(wa, sa, i + 2);
+        if (i + 1 < n_items) compute_item(wb, sb, i + 1);
     }
 }
 
@@ -238,11 +428,56 @@ extern "C" size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_s
 }
 
 namespace {
+int tune(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return (e && *e) ? atoi(e) : dflt;
+}
+
 template <int NB>
-void launch_gate_up(const Workspace &w, size_t P, size_t inter, int act_kind, float limit, hipStream_t st) {
-    const unsigned gx = (unsigned)((inter / 32 + 3) / 4);
-    hipLaunchKernelGGL(moe_gate_up_q8_kernel<NB>, dim3(gx, (unsigned)P), dim3(256), 0, st, w.pt, w.xq, w.xs, (int)inter, act_kind, limit, w.aq,
-                       w.as);
+int launch_gate_up_fused(const FusedArgs &a, size_t P, hipStream_t st) {
+    hipLaunchKernelGGL(moe_gate_up_fused_kernel<NB>, dim3((unsigned)P, (unsigned)(a.inter / 32)), dim3(256), 0, st, a);
+    return mk_launch_status("moe_gate_up_fused");
+}
+
+template <int NB, int U>
+int launch_down_u(const FusedArgs &a, size_t B, int blocks, hipStream_t st) {
+    const size_t lds = (size_t)a.per * NB * 64 + (size_t)a.per * NB * 4;
+    static bool opted = false;
+    if (!opted) {
+        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_down_fused_kernel<NB, U>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        opted = true;
+    }
+    hipLaunchKernelGGL((moe_down_fused_kernel<NB, U>), dim3((unsigned)B, blocks), dim3(256), lds, st, a);
+    return mk_launch_status("moe_down_fused");
+}
+
+// The tokens share one resident grid.  A wave streams register blocks of U tiles;
+// U is the largest of 8/T, 4/T ... 1 for which the rows still spread over at
+// least two workgroups per CU, and the block count is then set so that the tiles
+// divide evenly among the waves (a register block that is only partly filled
+// would re-read and re-compute the wave's first tile).
+template <int NB>
+int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
+    constexpr int TILE = lcm_c(NB, 64), T = TILE / 64, RT = TILE / NB;
+    const int n_tiles = a.d / RT;
+    const int target = tune("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
+    int u = 8 / T;
+    int forced = tune("MK_MOE_DOWN_U", 0);
+    auto blocks_for = [&](int uu) {
+        int groups = (int)((double)n_tiles / ((double)(target > 0 ? target : 1) * 4 * uu) + 0.5);
+        if (groups < 1) groups = 1;
+        return (n_tiles + 4 * uu * groups - 1) / (4 * uu * groups);
+    };
+    if (forced > 0) u = forced;
+    else
+        while (u > 1 && (size_t)blocks_for(u) * B < 512) u >>= 1;
+    const int blocks = blocks_for(u);
+    switch (u) {
+        case 8: if constexpr (8 * T <= 8) return launch_down_u<NB, 8>(a, B, blocks, st);
+        case 4: if constexpr (4 * T <= 8) return launch_down_u<NB, 4>(a, B, blocks, st);
+        case 2: return launch_down_u<NB, 2>(a, B, blocks, st);
+        default: return launch_down_u<NB, 1>(a, B, blocks, st);
+    }
 }
 }  // namespace
 
@@ -259,24 +494,48 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     const int per = (int)topk + (shared >= 0 ? 1 : 0);
     const size_t P = B * per;
     Workspace w = carve(workspace, B, topk, shared >= 0, d, inter);
+    const int nb = (int)(d / 32), nbi = (int)(inter / 32);
+    const bool fast = mode == MK_MODE_Q8 && (nb == 32 || nb == 64 || nb == 128 || nb == 224) && (nbi == 32 || nbi == 64 || nbi == 128) &&
+                      per <= MAX_PER && d % 2 == 0 && (size_t)per * nbi * 68 <= 150 * 1024;
+    int s;
+    if (fast) {
+        FusedArgs fa;
+        fa.tab = *table;
+        fa.ids = ids;
+        fa.weights = weights;
+        fa.x = x;
+        fa.topk = (int)topk;
+        fa.shared = shared;
+        fa.per = per;
+        fa.d = (int)d;
+        fa.inter = (int)inter;
+        fa.act_kind = act_kind;
+        fa.ds_rule = act_kind == MK_ACT_DS ? 1 : 0;
+        fa.limit = limit;
+        fa.aq = w.aq;
+        fa.as = w.as;
+        fa.out = out;
+        switch (nb) {
+            case 32: s = launch_gate_up_fused<32>(fa, P, st); break;
+            case 64: s = launch_gate_up_fused<64>(fa, P, st); break;
+            case 128: s = launch_gate_up_fused<128>(fa, P, st); break;
+            default: s = launch_gate_up_fused<224>(fa, P, st); break;
+        }
+        if (s != MK_OK) return s;
+        switch (nbi) {
+            case 32: return launch_down_fused<32>(fa, B, st);
+            case 64: return launch_down_fused<64>(fa, B, st);
+            default: return launch_down_fused<128>(fa, B, st);
+        }
+    }
     hipLaunchKernelGGL(moe_setup_kernel, dim3((unsigned)((P + 63) / 64)), dim3(64), 0, st, *table, (int)B, (int)topk, shared, ids, weights,
                        w.pt, w.o, w.g, w.u, (int)d, (int)inter);
-    int s = mk_launch_status("moe_setup");
+    s = mk_launch_status("moe_setup");
     if (s != MK_OK) return s;
-    const int nb = (int)(d / 32);
-    const bool fast = mode == MK_MODE_Q8 && (nb == 32 || nb == 64 || nb == 128 || nb == 224);
     if (mode == MK_MODE_Q8) {
         if ((s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
     }
-    if (fast) {
-        switch (nb) {
-            case 32: launch_gate_up<32>(w, P, inter, act_kind, limit, st); break;
-            case 64: launch_gate_up<64>(w, P, inter, act_kind, limit, st); break;
-            case 128: launch_gate_up<128>(w, P, inter, act_kind, limit, st); break;
-            default: launch_gate_up<224>(w, P, inter, act_kind, limit, st); break;
-        }
-        if ((s = mk_launch_status("moe_gate_up")) != MK_OK) return s;
-    } else {
+    {
         // composed path (any shape, both modes): gate and up as grouped GEMVs,
         // elementwise activation, then (q8) the activation's own quantization
         const bool q8 = mode == MK_MODE_Q8;
