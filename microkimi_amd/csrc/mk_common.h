@@ -12,6 +12,7 @@ typedef float mk_f2 __attribute__((ext_vector_type(2)));
 typedef int mk_i4 __attribute__((ext_vector_type(4)));
 typedef int mk_i8v __attribute__((ext_vector_type(8)));
 typedef float mk_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int mk_u2 __attribute__((ext_vector_type(2)));
 typedef float mk_f16v __attribute__((ext_vector_type(16)));
 
 // Loads that tell the compiler the pointer is global memory.  A pointer that was
@@ -19,6 +20,8 @@ typedef float mk_f16v __attribute__((ext_vector_type(16)));
 // compiler and would be read with flat_load, which also ties up the LDS counter.
 #define MK_GLOBAL __attribute__((address_space(1)))
 __device__ __forceinline__ mk_i4 mk_ldg128(const void *p) { return *(const MK_GLOBAL mk_i4 *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ mk_u2 mk_ldg64(const void *p) { return *(const MK_GLOBAL mk_u2 *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ uint32_t mk_ldg_u32(const void *p) { return *(const MK_GLOBAL uint32_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u8(const void *p) { return *(const MK_GLOBAL uint8_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint16_t mk_ldg_u16(const void *p) { return *(const MK_GLOBAL uint16_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ float mk_ldg_f32(const void *p) { return *(const MK_GLOBAL float *)(const MK_GLOBAL void *)p; }
@@ -78,6 +81,24 @@ __device__ __forceinline__ float mk_wave_max(float v) {
     v = fmaxf(v, mk_dpp<0x141>(v));
     v = fmaxf(v, mk_dpp<0x140>(v));
     return fmaxf(fmaxf(mk_readlane(v, 0), mk_readlane(v, 16)), fmaxf(mk_readlane(v, 32), mk_readlane(v, 48)));
+}
+
+// sum / max over the four lanes {c, c+16, c+32, c+48} without LDS traffic
+// (gfx950 lane-swap instructions: halves of the wave, then odd/even rows of 16).
+// All 64 lanes must be active; every lane gets the result.
+__device__ __forceinline__ float mk_rows_max(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    mk_u2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __builtin_bit_cast(unsigned, fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1])));
+    r = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+}
+__device__ __forceinline__ float mk_rows_sum(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    mk_u2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned w = __builtin_bit_cast(unsigned, __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]));
+    r = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
 
 // sum / max over aligned groups of 32 lanes
