@@ -222,7 +222,8 @@ __global__ __launch_bounds__(256) void mla_partial_kernel(MlaArgs a) {
 //            whole, the second block's dot is the difference.  The integer block
 //            dots are scaled by (query block scale * cache block scale) in f32,
 //            the reference's per-block term (src/model.rs:1858-1871).  Rope part:
-//            f32 MFMA (16x16x4) over the dequantized rope bytes and the f32 query.
+//            f16 MFMA in split precision (see "out"): the rope bytes times
+//            their scale as exact f16 pairs, the f32 query as hi + lo.
 //   softmax  a lane holds head l%16 and positions 4*(l/16)+r, which is the A
 //            operand layout of the next product: probabilities stay in registers.
 //   out      v_mfma_f32_16x16x32_f16 in split precision.  The cache value
@@ -230,9 +231,9 @@ __global__ __launch_bounds__(256) void mla_partial_kernel(MlaArgs a) {
 //            as an exact f16 pair: hi = rn(q*s), lo = fma(q, s, -hi) (the product
 //            has 19 significant bits and the residual is a multiple of the
 //            scale's ulp, so hi + lo == v).  The probability is split the same
-//            way (hi = rn(p), lo = rn(p - hi), error below 2^-24).  K = 32 holds
-//            the 16 positions twice, (p_hi | p_lo) against (v_hi | v_hi) and
-//            against (v_lo | v_lo); accumulation is f32.  A lane reads 4 rows x
+//            way (hi = rn(p), lo = rn(p - hi), relative error below 2^-21).  K = 32
+//            holds the 16 positions twice: (p_hi | p_hi) and (p_lo | 0) against
+//            (v_hi | v_lo); accumulation is f32.  A lane reads 4 rows x
 //            16 dims and transposes 4x4 byte blocks in registers, because the
 //            operand wants positions contiguous in a lane and the cache has dims
 //            contiguous.  Lane l keeps dims 16c..16c+15 and 256+16c.. (c = l%16)
@@ -244,6 +245,7 @@ __global__ __launch_bounds__(256) void mla_partial_kernel(MlaArgs a) {
 // barrier per tile).  With a single split the workgroup writes the normalised
 // output itself.
 constexpr int ML = 512, MR = 64;
+constexpr float MLA_TAU = 8.0f;
 constexpr int KROW = 592;      // LDS row stride in bytes: 16 rows at 16-byte granularity fall in distinct banks
 constexpr int KS_STRIDE = 68;  // f32 scale row [block][position]
 constexpr int KH_STRIDE = 72;  // f16 scale row [block][position]
@@ -357,9 +359,15 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
         qs_l[S * 64 + lane] = q4 < 2 ? mk_f2{dx, other} : mk_f2{other, dx};
     }
     const int blk0_mask = q4 < 2 ? -1 : 0;
-    float qr[16];
+    // rope part of the query (f32 in the reference), dims 16*q4.. of head c, as an f16 pair hi + lo
+    mk_h8 qrh[2], qrl[2];
 #pragma unroll
-    for (int k = 0; k < 16; k++) qr[k] = qrow[ML + 16 * q4 + k];
+    for (int k = 0; k < 16; k++) {
+        const float v = qrow[ML + 16 * q4 + k];
+        const _Float16 hi = (_Float16)v;
+        qrh[k >> 3][k & 7] = hi;
+        qrl[k >> 3][k & 7] = (_Float16)(v - (float)hi);
+    }
 
     mk_f4 o[32];
 #pragma unroll
@@ -391,11 +399,35 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
                 cf[S] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[S], qv, zero4, 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
+            // rope: bytes -> exact f16 pairs (see the output product below), 64 dims = two K=32 steps
             mk_f4 cr0 = {0.0f, 0.0f, 0.0f, 0.0f}, cr1 = cr0;
+            {
+                const _Float16 rs = (_Float16)rsc;  // exact: the scale is stored as f16
+                const mk_h2 s2 = {rs, rs};
+                const mk_h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+                mk_h8 kh8[2], kl8[2];
 #pragma unroll
-            for (int k = 0; k < 16; k += 2) {
-                cr0 = __builtin_amdgcn_mfma_f32_16x16x4f32(mk_byte_f32(kr[k >> 2], k & 3) * rsc, qr[k], cr0, 0, 0, 0);
-                cr1 = __builtin_amdgcn_mfma_f32_16x16x4f32(mk_byte_f32(kr[k >> 2], (k & 3) + 1) * rsc, qr[k + 1], cr1, 0, 0, 0);
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t d = (uint32_t)kr[k] ^ 0x80808080u;
+                    const mk_h2 v0 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, d, 0x04010400u)) - bias;
+                    const mk_h2 v1 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, d, 0x04030402u)) - bias;
+                    const mk_h2 h0 = v0 * s2, h1 = v1 * s2;
+                    const mk_h2 l0 = __builtin_elementwise_fma(v0, s2, -h0), l1 = __builtin_elementwise_fma(v1, s2, -h1);
+                    kh8[k >> 1][4 * (k & 1) + 0] = h0.x;
+                    kh8[k >> 1][4 * (k & 1) + 1] = h0.y;
+                    kh8[k >> 1][4 * (k & 1) + 2] = h1.x;
+                    kh8[k >> 1][4 * (k & 1) + 3] = h1.y;
+                    kl8[k >> 1][4 * (k & 1) + 0] = l0.x;
+                    kl8[k >> 1][4 * (k & 1) + 1] = l0.y;
+                    kl8[k >> 1][4 * (k & 1) + 2] = l1.x;
+                    kl8[k >> 1][4 * (k & 1) + 3] = l1.y;
+                }
+                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrh[0], cr0, 0, 0, 0);
+                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrh[1], cr1, 0, 0, 0);
+                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[0], qrh[0], cr0, 0, 0, 0);
+                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[1], qrh[1], cr1, 0, 0, 0);
+                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrl[0], cr0, 0, 0, 0);
+                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrl[1], cr1, 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
             mk_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -414,31 +446,45 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
         // ---- online softmax for head c over the 16 positions
         float tm = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         tm = mk_rows_max(tm);
-        const float m_new = fmaxf(m, tm);
-        const float m_ref = m_new == -INFINITY ? 0.0f : m_new;  // a wave that has seen no position yet: all weights 0
-        const float corr = expf(m - m_ref);
+        // The reference point of the exponentials moves only when the maximum has
+        // grown by more than MLA_TAU: weights stay below e^TAU and the 128
+        // accumulators are rescaled a few times per split instead of every tile.
+        const bool move = tm > m + MLA_TAU;  // false for a wave that still has no valid position (tm = -inf)
+        const float m_new = move ? tm : m;
+        const float m_ref = m_new == -INFINITY ? 0.0f : m_new;  // no position seen yet: all weights 0
+        const float corr = move ? expf(m - m_ref) : 1.0f;
         float ts = 0.0f;
-        mk_h8 pa;
+        mk_h8 pa1, pa2;  // (p_hi | p_hi) and (p_lo | 0) over this lane's 4 positions
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const float pv = expf(sc[r] - m_ref);
             ts += pv;
             const _Float16 hi = (_Float16)pv;
-            pa[r] = hi;
-            pa[4 + r] = (_Float16)(pv - (float)hi);
+            pa1[r] = hi;
+            pa1[4 + r] = hi;
+            pa2[r] = (_Float16)(pv - (float)hi);
+            pa2[4 + r] = (_Float16)0.0f;
         }
         ts = mk_rows_sum(ts);
         l = l * corr + ts;
         m = m_new;
-        if (__any(corr != 1.0f)) {
+        if (__any(move)) {
             // the accumulators hold heads 4*q4+r: fetch their corrections from the lanes that own those heads
             float oc[4];
 #pragma unroll
             for (int r = 0; r < 4; r++) oc[r] = __shfl(corr, 4 * q4 + r, MK_WAVE);
+            // The accumulators live in the MFMA accumulation registers.  The empty asm statements pin each
+            // one there on entry and exit of this rare block, so the copies through the vector registers
+            // that the multiplication needs stay inside it instead of being paid on every tile.
 #pragma unroll
-            for (int n = 0; n < 32; n++)
+            for (int n = 0; n < 32; n++) {
+                mk_f4 t = o[n];
+                asm volatile("" : "+a"(t));
 #pragma unroll
-                for (int r = 0; r < 4; r++) o[n][r] *= oc[r];
+                for (int r = 0; r < 4; r++) t[r] *= oc[r];
+                asm volatile("" : "+a"(t));
+                o[n] = t;
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         // ---- out += P V over rows prow + 4*q4 + e
@@ -470,11 +516,10 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
                     const mk_h2 v01 = __builtin_bit_cast(mk_h2, f01) - bias, v23 = __builtin_bit_cast(mk_h2, f23) - bias;
                     const mk_h2 hi01 = v01 * s01, hi23 = v23 * s23;
                     const mk_h2 lo01 = __builtin_elementwise_fma(v01, s01, -hi01), lo23 = __builtin_elementwise_fma(v23, s23, -hi23);
-                    const mk_h8 bh = {hi01.x, hi01.y, hi23.x, hi23.y, hi01.x, hi01.y, hi23.x, hi23.y};
-                    const mk_h8 bl = {lo01.x, lo01.y, lo23.x, lo23.y, lo01.x, lo01.y, lo23.x, lo23.y};
+                    const mk_h8 b = {hi01.x, hi01.y, hi23.x, hi23.y, lo01.x, lo01.y, lo23.x, lo23.y};  // (v_hi | v_lo)
                     const int n = 16 * half + 4 * k + j;
-                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, bh, o[n], 0, 0, 0);
-                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, bl, o[n], 0, 0, 0);
+                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, b, o[n], 0, 0, 0);  // p_hi v_hi + p_hi v_lo
+                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa2, b, o[n], 0, 0, 0);  // p_lo v_hi
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -511,7 +556,8 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
             for (int k = 0; k < 4; k++) {
                 const mk_f4 v = {o[16 * half + 4 * k][r] * wself, o[16 * half + 4 * k + 1][r] * wself, o[16 * half + 4 * k + 2][r] * wself,
                                  o[16 * half + 4 * k + 3][r] * wself};
-                *reinterpret_cast<mk_f4 *>(dst + 256 * half + 4 * k) = v;
+                // 16-byte chunks are swizzled within groups of four so that the 16 lanes of a row hit 16 bank groups
+                *reinterpret_cast<mk_f4 *>(dst + 256 * half + 4 * (k ^ ((c >> 2) & 3))) = v;
             }
     }
     __syncthreads();
@@ -529,10 +575,11 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
             float *dst = single ? out + (size_t)h * ML : a.po + ((size_t)split * a.nh + h) * ML;
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const int d = 4 * ((tid & 15) + 16 * i);
-                mk_f4 v = *reinterpret_cast<const mk_f4 *>(ob + (size_t)hl * ML + d);
+                const int ch = (tid & 15) + 16 * i;  // logical chunk: dims 4*ch..; written by lane c = (ch >> 2) & 15
+                const int d = 4 * ch, dp = 4 * (ch ^ ((ch >> 4) & 3));
+                mk_f4 v = *reinterpret_cast<const mk_f4 *>(ob + (size_t)hl * ML + dp);
 #pragma unroll
-                for (int w2 = 1; w2 < 4; w2++) v += *reinterpret_cast<const mk_f4 *>(ob + (size_t)(w2 * 16 + hl) * ML + d);
+                for (int w2 = 1; w2 < 4; w2++) v += *reinterpret_cast<const mk_f4 *>(ob + (size_t)(w2 * 16 + hl) * ML + dp);
                 if (single) v = mk_f4{v.x / lt, v.y / lt, v.z / lt, v.w / lt};
                 *reinterpret_cast<mk_f4 *>(dst + d) = v;
             }
