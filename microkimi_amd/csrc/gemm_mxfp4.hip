@@ -18,10 +18,12 @@
 //                 registers 4-7 (bytes 16-31): the K = 128 step is two K = 64 halves
 //   result        lane l holds column l % 16, rows 4 (l / 16) + r
 //
-// Tiling: workgroup = 4 waves = 64 weight rows of one expert; each wave owns 16
-// rows and up to 64 token rows (4 accumulator tiles), so an expert's weights are
-// streamed from HBM once for up to 64 tokens.  At the prefill shapes (about 16
-// tokens per expert) the kernel is bound by that weight stream, not by the MFMA.
+// Two kernels.  The general one (cols % 128 == 0): workgroup = 4 waves = 64
+// weight rows of one expert; each wave owns 16 rows and up to 64 token rows (4
+// accumulator tiles), so an expert's weights are streamed from HBM once for up
+// to 64 tokens.  The streaming one (cols % 512 == 0, below) is the one the
+// model shapes take.  At the prefill shapes (about 16 tokens per expert) the
+// work is bound by the weight stream, not by the MFMA.
 #include "mk_common.h"
 
 namespace {
@@ -90,6 +92,178 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
     }
 }
 
+// ---------------------------------------------------------------- streaming kernel
+// cols % 512 == 0.  A workgroup owns 256 weight rows of one expert (a wave 64 =
+// four 16-row tiles) and walks K in tiles of 512 (four MFMA steps):
+//
+//   * the group's activation tile (up to 16*MC tokens x 512 codes + 16 scale
+//     bytes each) is staged in LDS once per K tile and serves all 16 row tiles
+//     of the workgroup; the next tile is fetched into registers meanwhile;
+//   * weights go straight from global memory to registers, one unit = one row
+//     tile x four steps (256 contiguous bytes per row, 4 KB per wave) ahead, in
+//     two alternating register blocks, with unconditional (clamped) addresses so
+//     that no wait is forced.  Units that gave a row shorter runs (64 or 128
+//     bytes, more row tiles per unit) were measured slower, whatever their
+//     bytes in flight;
+//   * a row's 16 scale bytes of the K tile come as ONE 16-byte load (a lane then
+//     shifts out the byte of its step and K block) instead of a byte per step.
+//
+// Loads take the form "uniform base + 32-bit lane offset".  The K offset goes
+// through readfirstlane, which hides the loop counter from the induction
+// variable widening that would otherwise rebuild 64-bit pointers per lane.
+constexpr int KT_STEPS = 4;
+constexpr int A_STRIDE = 512 + 16;  // LDS row stride of the activation tile: 16 rows fall in distinct banks
+constexpr int a_codes_bytes(int mc) { return 16 * mc * A_STRIDE; }
+constexpr int a_buf_bytes(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }  // codes, then 16 scale bytes per token
+
+struct GemmArgs {
+    const uint8_t *const *packed_ptrs;
+    const uint8_t *const *scales_ptrs;
+    int rows, cols;
+    const uint8_t *codes;
+    const uint8_t *exps;
+    const int32_t *offsets;
+    float *out;
+};
+
+template <int MC>
+__device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, int base, int tok1, uint8_t *lds) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, kb = lane >> 4;
+    const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
+    const int row0 = blockIdx.x * 256 + wave * 64;
+    // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
+    uint32_t woff[4], soff[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; rt++) {
+        const int r = min(row0 + rt * 16 + n, a.rows - 1);
+        woff[rt] = (uint32_t)r * (uint32_t)(cols / 2) + kb * 16;
+        soff[rt] = (uint32_t)r * (uint32_t)nb;
+    }
+    mk_i4 wa[KT_STEPS], wb[KT_STEPS], sa, sb;
+    auto load_unit = [&](mk_i4 *w, mk_i4 &sc, int kt, int rt) {
+        const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
+#pragma unroll
+        for (int s = 0; s < KT_STEPS; s++) w[s] = mk_ldg128_off(packed, woff[rt] + ku * (KT_STEPS * 64) + s * 64);
+        sc = mk_ldg128_off(scales, soff[rt] + ku * 16);
+    };
+    // activation tile staging: chunk i = tid + 256 k -> token i / 32, 16-byte chunk i % 32
+    mk_i4 st[2 * MC], ste;
+    uint32_t coff[2 * MC];  // the host checks that tokens x cols stays below 2^32
+#pragma unroll
+    for (int k = 0; k < 2 * MC; k++) {
+        const int i = tid + 256 * k;
+        coff[k] = (uint32_t)min(base + (i >> 5), tok1 - 1) * (uint32_t)cols + (i & 31) * 16;
+    }
+    const uint32_t eoff = (uint32_t)min(base + (tid & (16 * MC - 1)), tok1 - 1) * (uint32_t)nb;
+    auto stage_load = [&](int kt) {
+        const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
+#pragma unroll
+        for (int k = 0; k < 2 * MC; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
+        ste = mk_ldg128_off(a.exps, eoff + ku * 16);
+    };
+    auto stage_store = [&](uint8_t *buf) {
+#pragma unroll
+        for (int k = 0; k < 2 * MC; k++) {
+            const int i = tid + 256 * k;
+            *reinterpret_cast<mk_i4 *>(buf + (i >> 5) * A_STRIDE + (i & 31) * 16) = st[k];
+        }
+        if (tid < 16 * MC) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC) + tid * 16) = ste;
+    };
+    mk_f4 acc[4][MC];
+#pragma unroll
+    for (int rt = 0; rt < 4; rt++)
+#pragma unroll
+        for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // One unit: 4 steps x MC token tiles.  The LDS reads of the activation operands do not depend on the
+    // row tile, so after inlining the four calls of a K tile share them.
+    auto compute_unit = [&](const mk_i4 *w, const mk_i4 &sc, int rt, const uint8_t *buf) {
+#pragma unroll
+        for (int c = 0; c < MC; c++) {
+            const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC) + (c * 16 + n) * 16);
+            const uint8_t *arow = buf + (c * 16 + n) * A_STRIDE + kb * 16;
+#pragma unroll
+            for (int s = 0; s < KT_STEPS; s++) {
+                const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + s * 128);
+                const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + s * 128 + 64);
+                const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                const mk_i8v bv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
+                const int asb = (int)((uint32_t)ae[s] >> (8 * kb));  // the instruction reads byte 0
+                const int wsb = (int)((uint32_t)sc[s] >> (8 * kb));
+                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*A: fp8 e4m3*/, 4 /*B: fp4 e2m1*/, 0, asb, 0, wsb);
+            }
+        }
+    };
+
+    load_unit(wa, sa, 0, 0);
+    stage_load(0);
+    __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
+    stage_store(lds);
+    __syncthreads();
+#pragma unroll 1
+    for (int kt = 0; kt < ktiles; kt++) {
+        const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
+        stage_load(kt + 1);
+        load_unit(wb, sb, kt, 1);
+        compute_unit(wa, sa, 0, buf);
+        load_unit(wa, sa, kt, 2);
+        compute_unit(wb, sb, 1, buf);
+        load_unit(wb, sb, kt, 3);
+        compute_unit(wa, sa, 2, buf);
+        load_unit(wa, sa, kt + 1, 0);
+        compute_unit(wb, sb, 3, buf);
+        stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+        __syncthreads();
+    }
+#pragma unroll
+    for (int rt = 0; rt < 4; rt++) {
+        const int row = row0 + rt * 16 + n;
+        if (row < a.rows) {
+#pragma unroll
+            for (int c = 0; c < MC; c++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int t = base + c * 16 + kb * 4 + i;
+                    if (t < tok1) a.out[(size_t)t * a.rows + row] = acc[rt][c][i];
+                }
+        }
+    }
+}
+
+// Two instantiations share the grid: groups of up to 32 tokens (the prefill
+// case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
+// workgroup whose group belongs to the other one exits.
+template <int MC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2 : 1))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int e = blockIdx.y;
+    const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
+    const int count = tok1 - tok0;
+    if (count <= 0 || (count <= 32 ? 2 : 4) != MC) return;
+    const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[e]);
+    const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[e]);
+    if (MC == 2) {
+        if (count <= 16) gemm_pass<1>(a, packed, scales, tok0, tok1, lds);
+        else gemm_pass<2>(a, packed, scales, tok0, tok1, lds);
+    } else {
+#pragma unroll 1
+        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC>(a, packed, scales, base, tok1, lds);
+    }
+}
+
+template <int MC>
+int launch_stream(const GemmArgs &a, dim3 grid, hipStream_t st) {
+    static bool opted = false;
+    if (!opted) {
+        hipFuncSetAttribute(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * a_buf_bytes(MC));
+        opted = true;
+    }
+    hipLaunchKernelGGL(mxfp4_grouped_gemm_stream_kernel<MC>, grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
+    return mk_launch_status("mxfp4_grouped_gemm_stream");
+}
+
 }  // namespace
 
 extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
@@ -100,6 +274,13 @@ extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, cons
     MK_REQUIRE(n_groups >= 1 && n_groups <= 65535 && rows >= 1 && rows <= 0x7FFFFF00u, "bad shape");
     MK_REQUIRE(((uintptr_t)codes & 15) == 0, "codes must be 16-byte aligned");
     if (m == 0) return MK_OK;
+    if (cols % 512 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0) {
+        GemmArgs a{packed_ptrs, scales_ptrs, (int)rows, (int)cols, codes, exps, offsets, out};
+        const dim3 grid((unsigned)((rows + 255) / 256), (unsigned)n_groups);
+        int st = launch_stream<2>(a, grid, (hipStream_t)stream);
+        if (st == MK_OK && m > 32) st = launch_stream<4>(a, grid, (hipStream_t)stream);
+        return st;
+    }
     hipLaunchKernelGGL(mxfp4_grouped_gemm_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)n_groups), dim3(256), 0, (hipStream_t)stream,
                        packed_ptrs, scales_ptrs, (int)rows, (int)cols, codes, exps, offsets, out);
     return mk_launch_status("mxfp4_grouped_gemm");

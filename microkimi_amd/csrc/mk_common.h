@@ -20,11 +20,26 @@ typedef float mk_f16v __attribute__((ext_vector_type(16)));
 // compiler and would be read with flat_load, which also ties up the LDS counter.
 #define MK_GLOBAL __attribute__((address_space(1)))
 __device__ __forceinline__ mk_i4 mk_ldg128(const void *p) { return *(const MK_GLOBAL mk_i4 *)(const MK_GLOBAL void *)p; }
+// base + 32-bit byte offset, with the address arithmetic done in the global address space: a uniform base
+// and a lane offset then become the scalar-base form of the load (no 64-bit address per lane)
+__device__ __forceinline__ mk_i4 mk_ldg128_off(const void *base, uint32_t off) {
+    const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
+    return *(const MK_GLOBAL mk_i4 *)(b + off);
+}
 __device__ __forceinline__ mk_u2 mk_ldg64(const void *p) { return *(const MK_GLOBAL mk_u2 *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u32(const void *p) { return *(const MK_GLOBAL uint32_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u8(const void *p) { return *(const MK_GLOBAL uint8_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint16_t mk_ldg_u16(const void *p) { return *(const MK_GLOBAL uint16_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ float mk_ldg_f32(const void *p) { return *(const MK_GLOBAL float *)(const MK_GLOBAL void *)p; }
+
+// A pointer that is the same in every lane but was loaded with a vector load (an
+// expert table entry): moving it to scalar registers lets the loads that use it
+// take the "scalar base + 32-bit lane offset" form instead of a 64-bit address per lane.
+__device__ __forceinline__ const uint8_t *mk_uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+}
 
 // 2^(sb-127) from an e8m0 byte as an exact bit pattern; byte 0 is the
 // subnormal 2^-127 (mxfp4::scale_from_byte, src/mxfp4.rs:340-346).
