@@ -70,15 +70,16 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     __shared__ float xsc[NB];
 
     const int mat = blockIdx.y;
-    const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
-    const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    // uniform pointers in scalar registers + 32-bit lane offsets: the loads take the scalar-base form
+    const uint8_t *packed = mk_uniform_ptr(a.packed ? a.packed : a.packed_ptrs[mat]);
+    const uint8_t *scales = mk_uniform_ptr(a.packed ? a.scales : a.scales_ptrs[mat]);
     float *out = a.packed ? a.out : a.out_ptrs[mat];
     const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
     const int8_t *xq = a.xq + (size_t)xi * NB * 32;
     const float *xs = a.xs + (size_t)xi * NB;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // tile arithmetic stays on the scalar unit
     // Tiles of this matrix are dealt round-robin to the matrix's resident waves
     // (wave w takes tiles w, w + W, ...): equal work, one compact read window.
     // U tiles form a register block; two blocks (ping, pong) are in flight.
@@ -92,19 +93,20 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     uint32_t sa[U][T], sb[U][T];
     // Loads are unconditional (a predicated load becomes a branch and a full
     // wait): a tile past the end re-reads the wave's first tile and a lane past
-    // the last row re-reads the last block; neither result is stored.
-    const size_t last_blk = (size_t)a.rows * NB - 1;
+    // the last row re-reads the last block; neither result is stored.  Block
+    // indices are 32-bit (the host checks rows * NB < 2^28).
+    const uint32_t last_blk = (uint32_t)a.rows * NB - 1;
     auto load_block = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int k0) {
+        k0 = __builtin_amdgcn_readfirstlane(k0);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int tile = wv + ((k0 + u < my_tiles) ? (k0 + u) * wpm : 0);
-            const size_t blk0 = (size_t)tile * TILE;
+            const uint32_t tile = (uint32_t)wv + ((k0 + u < my_tiles) ? (uint32_t)(k0 + u) * (uint32_t)wpm : 0u);
+            const uint32_t blk0 = tile * TILE + lane;
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                size_t blk = blk0 + t * 64 + lane;
-                blk = blk < last_blk ? blk : last_blk;
-                w[u][t] = mk_ldg128(packed + blk * 16);
-                sc[u][t] = mk_ldg_u8(scales + blk);
+                const uint32_t blk = min(blk0 + t * 64, last_blk);
+                w[u][t] = mk_ldg128_off(packed, blk * 16);
+                sc[u][t] = mk_ldg_u8_off(scales, blk);
             }
         }
     };
@@ -355,8 +357,8 @@ int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
     const int n_tiles = (a.rows + RT - 1) / RT;
     if (q8) {
         // a fixed, fully resident grid shared by the matrices of the launch
-        // 2 workgroups per CU where the activation registers allow 2 waves per SIMD (T >= 4), else 3
-        int per_mat = tune("MK_MXFP4_BLOCKS", lcm_c(NB, 64) / 64 >= 4 ? 512 : 768) / (int)nmat;
+        // (2 workgroups per CU measured best for every block count per row)
+        int per_mat = tune("MK_MXFP4_BLOCKS", 512) / (int)nmat;
         if (per_mat < 1) per_mat = 1;
         if (per_mat * 4 > n_tiles) per_mat = (n_tiles + 3) / 4;
         hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(per_mat, (unsigned)nmat), dim3(256), 0, st, a);
@@ -373,12 +375,14 @@ int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
 int launch_gemv(const GemvArgs &a, bool q8, size_t nmat, size_t cols, hipStream_t st) {
     const int nb = (int)(cols / 32);
     if (a.rows == 0 || nmat == 0) return MK_OK;
-    switch (nb) {
-        case 32: return launch_fast<32>(a, q8, nmat, st);
-        case 64: return launch_fast<64>(a, q8, nmat, st);
-        case 128: return launch_fast<128>(a, q8, nmat, st);
-        case 224: return launch_fast<224>(a, q8, nmat, st);
-        default: break;
+    if ((size_t)a.rows * nb < (1u << 28)) {  // the fast kernels index blocks in 32 bits (16 bytes each)
+        switch (nb) {
+            case 32: return launch_fast<32>(a, q8, nmat, st);
+            case 64: return launch_fast<64>(a, q8, nmat, st);
+            case 128: return launch_fast<128>(a, q8, nmat, st);
+            case 224: return launch_fast<224>(a, q8, nmat, st);
+            default: break;
+        }
     }
     const unsigned gx = (unsigned)((a.rows + 3) / 4);
     if (q8)

@@ -318,7 +318,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
     for (int i = threadIdx.x; i < per * NB; i += 256) asc[i] = a.as[(size_t)tok * per * NB + i];
     __syncthreads();
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_tiles = a.d / RT;
     const int wv = blockIdx.y * 4 + wave, wpt = gridDim.y * 4;
     const int my_tiles = wv < n_tiles ? (n_tiles - wv + wpt - 1) / wpt : 0;
@@ -328,18 +328,19 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
     mk_i4 wa[U][T], wb[U][T];
     uint32_t sa[U][T], sb[U][T];
     auto load_item = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int i) {
-        i = i < n_items ? i : 0;  // unconditional loads: past the end, item 0 again
+        i = __builtin_amdgcn_readfirstlane(i < n_items ? i : 0);  // unconditional loads: past the end, item 0 again
         const int grp = i / per, s = i - grp * per;
-        const uint8_t *wp = wp_l[s], *ws = ws_l[s];
+        // uniform pointers in scalar registers + 32-bit block indices: the loads take the scalar-base form
+        const uint8_t *wp = mk_uniform_ptr(wp_l[s]), *ws = mk_uniform_ptr(ws_l[s]);
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = grp * U + u;
-            const int tile = wv + (k < my_tiles ? k : 0) * wpt;
-            const size_t blk0 = (size_t)tile * TILE;
+            const uint32_t tile = (uint32_t)(wv + (k < my_tiles ? k : 0) * wpt);
+            const uint32_t blk0 = tile * TILE + lane;
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                w[u][t] = mk_ldg128(wp + (blk0 + t * 64 + lane) * 16);
-                sc[u][t] = mk_ldg_u8(ws + blk0 + t * 64 + lane);
+                w[u][t] = mk_ldg128_off(wp, (blk0 + t * 64) * 16);
+                sc[u][t] = mk_ldg_u8_off(ws, blk0 + t * 64);
             }
         }
     };
