@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
     constexpr int T = NB * 2 / 64;  // half blocks per row / 64 lanes
     static_assert(NB % 32 == 0 && T >= 1 && T <= 8, "row shape not covered by the fast path");
     const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = gridDim.x * 4;
     mk_i4 xr[T];
     float cf[T];
@@ -55,14 +55,16 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
     // end they re-read the last row (a load under a branch forces a full wait)
     mk_i4 wa[T], wb[T];
     float sa[T], sb[T];
+    // uniform base + 32-bit lane offsets (the host checks rows * cols < 2^32): scalar-base loads; the row
+    // index is uniform per wave and goes through readfirstlane so that it stays on the scalar unit
     auto load_row = [&](mk_i4 *w, float *ws, int r) {
-        r = min(r, rows - 1);
-        const int8_t *row = q + (size_t)r * NB * 32;
+        const uint32_t ru = (uint32_t)__builtin_amdgcn_readfirstlane(min(r, rows - 1));
+        const uint32_t qoff = ru * (NB * 32) + lane * 16, soff = ru * NB + (lane >> 1);
 #pragma unroll
         for (int t = 0; t < T; t++) {
-            const int hb = t * 64 + lane;
-            w[t] = mk_ldg128(row + hb * 16);
-            ws[t] = load_scale<F16>(scales, (size_t)r * NB + (hb >> 1));
+            w[t] = mk_ldg128_off(q, qoff + t * 1024);
+            if (F16) ws[t] = mk_f16_bits_to_f32(mk_ldg_u16_off(scales, (soff + t * 32) * 2));
+            else ws[t] = mk_ldg_f32_off(scales, (soff + t * 32) * 4);
         }
     };
     auto compute_row = [&](const mk_i4 *w, const float *ws, int r) {
@@ -308,7 +310,7 @@ template <bool F16>
 int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, const int8_t *xq, const float *xs, size_t batch, float *out,
               hipStream_t st) {
     const int nb = (int)(cols / 32);
-    if (batch == 1) {
+    if (batch == 1 && rows * cols < 0xFFFFFFFFull) {  // the batch-1 kernel addresses the matrix with 32-bit byte offsets
         switch (nb) {
             case 32: launch_b1<32, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");
             case 64: launch_b1<64, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");

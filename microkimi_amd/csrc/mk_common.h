@@ -30,6 +30,14 @@ __device__ __forceinline__ uint32_t mk_ldg_u8_off(const void *base, uint32_t off
     const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
     return b[off];
 }
+__device__ __forceinline__ uint16_t mk_ldg_u16_off(const void *base, uint32_t off) {
+    const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
+    return *(const MK_GLOBAL uint16_t *)(b + off);
+}
+__device__ __forceinline__ float mk_ldg_f32_off(const void *base, uint32_t off) {
+    const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
+    return *(const MK_GLOBAL float *)(b + off);
+}
 __device__ __forceinline__ mk_u2 mk_ldg64(const void *p) { return *(const MK_GLOBAL mk_u2 *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u32(const void *p) { return *(const MK_GLOBAL uint32_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u8(const void *p) { return *(const MK_GLOBAL uint8_t *)(const MK_GLOBAL void *)p; }
