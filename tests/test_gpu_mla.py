@@ -38,6 +38,26 @@ def test_small_shapes(ctx, L, R, nh):
         assert rel_l2(got, want) <= TOL
 
 
+@pytest.mark.parametrize("ctx,nh,qscale", [(1, 16, 1.0), (3, 5, 1.0), (17, 20, 1.0), (64, 16, 1.0), (65, 33, 1.0), (130, 128, 1.0),
+                                            (700, 16, 6.0), (2048, 48, 6.0), (4100, 7, 0.0)])
+def test_production_shape_matrix_core_kernel(ctx, nh, qscale):
+    # latent 512 + rope 64 takes the MFMA kernel: single split and several, partial tiles and head groups,
+    # queries scaled up so that scores spread over far more than the lazy-rescale threshold, and an all-zero
+    # query (uniform weights)
+    from microkimi_amd import model
+    L, R = 512, 64
+    lat, rope, q, lq, ls, rq, rs = make_cache(ctx, L, R, nh, 1000 + ctx)
+    q = (q * qscale).astype(np.float32)
+    cache = model.MlaCache(L, R, ctx)
+    cache.assign_q8(dev(lq), dev(ls), dev(rq), dev(rs))
+    scale = float(np.float32(L // 4 + R) ** np.float32(-0.5))
+    for pos in sorted({ctx - 1, ctx // 2, 0}):
+        got = model.mla_attn_flash_q8_mqa(cache, dev(q), pos, scale).cpu().numpy()
+        want = oracle.mla_absorbed_decode(lq, ls.astype(np.float32), rq, rs.astype(np.float32), q, nh, scale, pos=pos)
+        assert np.all(np.isfinite(got))
+        assert rel_l2(got, want) <= TOL
+
+
 def test_append_quantizes_like_the_reference():
     torch = torch_cuda()
     from microkimi_amd import model
