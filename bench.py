@@ -345,6 +345,30 @@ def bench_gemm(torch):
     fl2 = 2.0 * 8 * M * inter * d
     res["large_m"] = {"rows_per_expert": M, "experts": 8, "ms": ms2, "tflops": fl2 / (ms2 * 1e-3) / 1e12,
                       "mfma_frac_fp8_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
+    del cl, el, xl
+    # the whole expert section of the prefill layer on the device (grouping, gather + MXFP8, gate, up, activation,
+    # down, combine): mk_dev_moe_prefill.  The gate matrices above are reused as W1; W3 and W2 are drawn here.
+    w3 = [rand_mxfp4(torch, g, inter, d) for _ in range(ne)]
+    w2 = [rand_mxfp4(torch, g, d, inter) for _ in range(ne)]
+    experts = model.PackedExperts(mats, w3, w2, d, inter)
+    ids_d, wts_d = model.router_softmax_topk(torch.from_numpy(logits_h).cuda(), W.TOP_K)
+    x_d = torch.from_numpy(x_h).cuda()
+    T = int(x_d.shape[0])
+    out = torch.empty((T, d), device="cuda")
+
+    def step3():
+        model.moe_prefill(experts, ids_d, wts_d, x_d, out=out)
+
+    ms3 = time_region(torch, step3, 5, warmup=2)
+    per_expert = 3 * (inter * d // 2 + inter * d // 32)
+    fl3 = 3 * 2.0 * m * inter * d
+    # weights once per used expert; token rows in, MXFP8 gathered rows, f32 gate / up / down outputs and their re-reads
+    alg3 = used * per_expert + T * d * 4 + 2 * (m * d + m * d // 32) + 2 * 2 * m * inter * 4 + 2 * (m * inter + m * inter // 32) + 2 * m * d * 4 + T * d * 4
+    res["expert_section"] = {"workload": "512 tokens x top-8 over 256 experts: group, gather + MXFP8, gate, up, SwiGLU + MXFP8, down, combine",
+                             "ms": ms3, "tok_s": T / (ms3 * 1e-3), "tflops": fl3 / (ms3 * 1e-3) / 1e12,
+                             "mfma_frac_fp8_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, "weight_bytes": used * per_expert,
+                             "alg_bytes": alg3, "gbs": alg3 / (ms3 * 1e-3) / 1e9, "hbm_frac": alg3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                             "finite": bool(torch.isfinite(out).all().item())}
     return res
 
 

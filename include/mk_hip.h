@@ -209,6 +209,24 @@ int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *
                               size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
                               void *stream);
 
+/* Bytes of device scratch mk_dev_moe_prefill needs. */
+size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter);
+
+/* The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) for T
+ * prompt positions: the (token, slot) pairs are grouped by expert (stable in
+ * (token, slot) order), each used expert evaluates gate, up, activation and
+ * down for its rows with mk_dev_mxfp4_grouped_gemm, and per token
+ *   out_t = sum_s w[t][s] * o[t][s]   in slot order, multiply then add.
+ * The gathered hidden rows and the activation enter the matrix cores as MXFP8
+ * (deepseek::fp8_roundtrip per 32, src/deepseek.rs:312-322); the reference's own
+ * prefill is the f32 arithmetic of matvec_packed_nt (mk_dev_mxfp4_matvec_nt).
+ * table entries 0..n_experts-1 are used; ids [T][topk] int32 (a pair whose id is
+ * out of range contributes nothing), weights [T][topk], x [T][d], out [T][d].
+ * act_kind MK_ACT_SWIGLU or MK_ACT_SITU.  d, inter multiples of 128; T * topk <= 16384
+ * per call (a longer prompt is split by the caller). */
+int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
+                       const float *x, int act_kind, void *workspace, float *out, void *stream);
+
 /* ------------------------------------------------------------ host level */
 
 /* metal::gpu_matvec_fp4 (src/metal.rs:943-1017), i.e. the GPU branch of

@@ -62,6 +62,8 @@ def _load():
         "mk_dev_mla_q8_decode": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp, vp]),
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
+        "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),
+        "mk_dev_moe_prefill": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp]),
         "mk_quantize_q8": (i32, [vp, sz, vp, vp]),

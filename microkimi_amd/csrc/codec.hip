@@ -87,36 +87,19 @@ __global__ __launch_bounds__(256) void mk_quantize_q8_kernel(const float *__rest
 }
 
 // ---------------------------------------------------------------- MXFP8 activations
-// f32 -> e4m3fn, round to nearest even, saturating at 448 (src/dequant.rs:92-120).
-__device__ __forceinline__ uint32_t mk_f32_to_e4m3(float v) {
-    if (v != v) return 0x7Fu;
-    uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
-    float a = fminf(fabsf(v), 448.0f);
-    if (a < 0.015625f) {  // below the smallest normal 2^-6: m = rne(a * 2^9), 8 carries into e=1
-        return sign | (uint32_t)rintf(a * 512.0f);
-    }
-    uint32_t bits = __float_as_uint(a);
-    uint32_t r = (bits + 0x7FFFFu + ((bits >> 20) & 1u)) >> 20;  // exponent and 3 mantissa bits, RNE with carry
-    return sign | (r - (120u << 3));
-}
-
-// One half-wave per block of 32: scale exponent e = ceil(log2(max(amax,1e-4)/448))
-// clamped to [-127, 8], code = e4m3(clamp(x / 2^e)) (src/deepseek.rs:312-322).
-// The reference takes a float log2; a correctly rounded float log2 is what
-// (float)log2((double)r) gives, so the exponent matches the host libm.
+// The e4m3 encoder and the per-32 MXFP8 quantizer live in mk_common.h (the prefill
+// pipeline uses them too).
+// a lane takes 8 consecutive values, four lanes a 32-block
 __global__ __launch_bounds__(256) void mk_quantize_mxfp8_kernel(const float *__restrict__ x, size_t n_blocks, uint8_t *__restrict__ codes,
                                                                 uint8_t *__restrict__ exps) {
-    size_t g = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
-    int j = threadIdx.x & 31;
-    if (g >= n_blocks) return;
-    float v = x[g * 32 + j];
-    float amax = fmaxf(mk_half_wave_max(fabsf(v)), 1e-4f);
-    int e = (int)ceilf((float)log2((double)(amax / 448.0f)));
-    e = max(-127, min(8, e));
-    float s = mk_scale_from_byte((uint32_t)(e + 127));
-    float qv = fminf(fmaxf(v / s, -448.0f), 448.0f);
-    codes[g * 32 + j] = (uint8_t)mk_f32_to_e4m3(qv);
-    if (j == 0) exps[g] = (uint8_t)(e + 127);
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 8 values
+    if (i >= n_blocks * 4) return;
+    const mk_f4 a = reinterpret_cast<const mk_f4 *>(x)[2 * i], b = reinterpret_cast<const mk_f4 *>(x)[2 * i + 1];
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t eb, c0, c1;
+    mk_mxfp8_quantize8(v, eb, c0, c1);
+    reinterpret_cast<mk_u2 *>(codes)[i] = mk_u2{c0, c1};
+    if ((i & 3) == 0) exps[i >> 2] = (uint8_t)eb;
 }
 
 // ------------------------------------------------------------------ C ABI
@@ -169,9 +152,10 @@ extern "C" int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, 
 extern "C" int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream) {
     MK_REQUIRE(x && codes && exps, "null pointer");
     MK_REQUIRE(n % 32 == 0, "MXFP8 blocks are 32 wide");
+    MK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)codes & 7) == 0, "x must be 16-byte and codes 8-byte aligned");
     size_t n_blocks = nvec * n / 32;
     if (n_blocks == 0) return MK_OK;
-    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    unsigned grid = (unsigned)((n_blocks * 4 + 255) / 256);
     hipLaunchKernelGGL(mk_quantize_mxfp8_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, x, n_blocks, codes, exps);
     return mk_launch_status("quantize_mxfp8");
 }

@@ -161,6 +161,71 @@ __device__ __forceinline__ uint16_t mk_f32_to_f16_bits(float f) {
     return c.u;
 }
 
+// f32 -> e4m3fn, round to nearest even, saturating at 448 (src/dequant.rs:92-120).
+__device__ __forceinline__ uint32_t mk_f32_to_e4m3(float v) {
+    if (v != v) return 0x7Fu;
+    uint32_t sign = (__float_as_uint(v) >> 24) & 0x80u;
+    float a = fminf(fabsf(v), 448.0f);
+    if (a < 0.015625f) {  // below the smallest normal 2^-6: m = rne(a * 2^9), 8 carries into e=1
+        return sign | (uint32_t)rintf(a * 512.0f);
+    }
+    uint32_t bits = __float_as_uint(a);
+    uint32_t r = (bits + 0x7FFFFu + ((bits >> 20) & 1u)) >> 20;  // exponent and 3 mantissa bits, RNE with carry
+    return sign | (r - (120u << 3));
+}
+
+// ceil(log2f(r)) for a normal positive r, where log2f is the correctly rounded float logarithm the reference calls
+// (f32::log2; (float)log2((double)r) is that value).  With r = m * 2^k, 1 <= m < 2: the result is k when m == 1 and
+// k + 1 as soon as log2(m) survives the rounding of k + log2(m) to float.  For |k| <= 127 half an ulp is at most
+// 3.9e-6 and log2(m) >= 1.1e-5 once the mantissa field is 64 or more, so only mantissa fields 1..63 (one value in
+// 131072) need the real logarithm; that branch is divergent and almost never taken.
+__device__ __forceinline__ int mk_ceil_log2f(float r) {
+    const uint32_t bits = __float_as_uint(r);
+    const int k = (int)(bits >> 23) - 127;
+    const uint32_t mf = bits & 0x7FFFFFu;
+    if (mf == 0) return k;
+    if (mf >= 64) return k + 1;
+    return (int)ceilf((float)log2((double)r));
+}
+
+// MXFP8 of one value of a 32-block held by an aligned group of 32 lanes (all active): scale exponent
+// e = ceil(log2(max(amax, 1e-4) / 448)) clamped to [-127, 8], code = e4m3(clamp(x / 2^e)) (deepseek::fp8_roundtrip,
+// src/deepseek.rs:312-322).  Returns the code; exp_byte = e + 127.
+__device__ __forceinline__ uint32_t mk_mxfp8_quantize(float v, uint32_t &exp_byte) {
+    const float amax = fmaxf(mk_half_wave_max(fabsf(v)), 1e-4f);
+    int e = mk_ceil_log2f(amax / 448.0f);
+    e = max(-127, min(8, e));
+    exp_byte = (uint32_t)(e + 127);
+    const float s = mk_scale_from_byte(exp_byte);
+    return mk_f32_to_e4m3(fminf(fmaxf(v / s, -448.0f), 448.0f));
+}
+
+// The same for a 32-block held as 8 consecutive values in each lane of an aligned quad of lanes: the block maximum
+// needs two DPP steps, the division by the power-of-two scale is an exact multiplication, and the e4m3 codes come
+// from v_cvt_pk_fp8_f32 (round to nearest even on the OCP e4m3 grid; the inputs are clamped to +-448 before).
+// c0 holds the codes of v[0..3], c1 of v[4..7], lowest byte first.
+__device__ __forceinline__ void mk_mxfp8_quantize8(const float (&v)[8], uint32_t &exp_byte, uint32_t &c0, uint32_t &c1) {
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) a = fmaxf(a, fabsf(v[i]));
+    a = fmaxf(a, mk_dpp<0xB1>(a));
+    a = fmaxf(a, mk_dpp<0x4E>(a));
+    int e = mk_ceil_log2f(fmaxf(a, 1e-4f) / 448.0f);
+    e = max(-127, min(8, e));
+    exp_byte = (uint32_t)(e + 127);
+    const float inv = mk_scale_from_byte(254u - exp_byte);  // 2^-e
+    float q[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(v[i] * inv, -448.0f), 448.0f);
+    int w0 = 0, w1 = 0;
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], w0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], w1, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
+    c0 = (uint32_t)w0;
+    c1 = (uint32_t)w1;
+}
+
 // silu(x) = x / (1 + exp(-x)) (src/deepseek.rs:97-100)
 __device__ __forceinline__ float mk_silu(float x) { return x / (1.0f + expf(-x)); }
 // situ (src/model.rs:619-621)

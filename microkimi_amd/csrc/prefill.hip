@@ -1,0 +1,217 @@
+// The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) on the
+// device: (token, slot) pairs grouped by expert, the three projections as
+// grouped GEMMs on the block-scaled matrix cores, scatter, and the per-token
+// weighted sum in slot order.
+//
+//   group     counting sort of the pairs by expert id, stable in (token, slot)
+//             order inside a group as the reference fills its groups
+//   gather    MXFP8 (e4m3 + e8m0 per 32) of each pair's hidden row, in grouped order
+//   gate, up  mk_dev_mxfp4_grouped_gemm over the expert table
+//   act       ACT(gate, up) and its MXFP8 form (the input of the down projection)
+//   down      mk_dev_mxfp4_grouped_gemm
+//   combine   out_t = sum_s w[t][s] * o[pair (t, s)], multiply then add, in slot order
+//
+// The activations enter the matrix cores as MXFP8: that is the arithmetic of
+// deepseek::fp8_roundtrip (src/deepseek.rs:312-322) applied to the gathered rows
+// and to the activation, not the pure f32 of matvec_packed_nt.
+#include "mk_common.h"
+
+namespace {
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct PrefillWs {
+    int32_t *order;    // [P] grouped row -> pair index t * topk + s
+    int32_t *pos;      // [P] pair index -> grouped row (-1: expert id out of range)
+    int32_t *offsets;  // [n_experts + 1]
+    uint8_t *codes, *exps;    // [P][d], [P][d/32]
+    float *g, *u;             // [P][inter]
+    uint8_t *codes2, *exps2;  // [P][inter], [P][inter/32]
+    float *o;                 // [P][d]
+    size_t bytes;
+};
+
+PrefillWs carve(void *base, size_t P, size_t n_experts, size_t d, size_t inter) {
+    PrefillWs w;
+    uint8_t *p = (uint8_t *)base;
+    size_t off = 0;
+    auto take = [&](size_t n) {
+        uint8_t *r = p ? p + off : nullptr;
+        off += align_up(n, 256);
+        return r;
+    };
+    w.order = (int32_t *)take(P * 4);
+    w.pos = (int32_t *)take(P * 4);
+    w.offsets = (int32_t *)take((n_experts + 1) * 4);
+    w.codes = take(P * d);
+    w.exps = take(P * (d / 32));
+    w.g = (float *)take(P * inter * 4);
+    w.u = (float *)take(P * inter * 4);
+    w.codes2 = take(P * inter);
+    w.exps2 = take(P * (inter / 32));
+    w.o = (float *)take(P * d * 4);
+    w.bytes = off;
+    return w;
+}
+
+// One workgroup of 16 waves: a stable counting sort of the pairs by expert id.  Wave w owns the pairs
+// [w C, (w + 1) C).  Per-wave histograms (LDS integer atomics: counts do not depend on their order), the expert
+// offsets by an exclusive scan, each wave's start inside each expert, then every wave places its pairs in order,
+// 64 at a time: the lanes that hold the same expert id are found with a ballot and ranked by lane number.
+constexpr int GROUP_MAX_P = 16384;
+constexpr int GROUP_WAVES = 16;
+__global__ __launch_bounds__(GROUP_WAVES * 64) void prefill_group_kernel(const int32_t *__restrict__ ids, int P, int n_experts,
+                                                                         int32_t *__restrict__ order, int32_t *__restrict__ pos,
+                                                                         int32_t *__restrict__ offsets) {
+    extern __shared__ int hist[];  // [GROUP_WAVES][n_experts], then [n_experts + 1] expert offsets
+    int *eoff = hist + GROUP_WAVES * n_experts;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int C = ((P + GROUP_WAVES * 64 - 1) / (GROUP_WAVES * 64)) * 64;  // pairs per wave, a multiple of 64
+    for (int i = threadIdx.x; i < GROUP_WAVES * n_experts + n_experts + 1; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    int *mine = hist + wave * n_experts;
+    for (int i = wave * C + lane; i < min((wave + 1) * C, P); i += 64) {
+        const int e = ids[i];
+        if (e >= 0 && e < n_experts) atomicAdd(&mine[e], 1);
+    }
+    __syncthreads();
+    // per expert: total and each wave's start relative to the expert's first row
+    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+        int run = 0;
+        for (int w = 0; w < GROUP_WAVES; w++) {
+            const int c = hist[w * n_experts + e];
+            hist[w * n_experts + e] = run;
+            run += c;
+        }
+        eoff[e + 1] = run;  // counts, scanned below
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int e = 0; e < n_experts; e++) {
+            const int c = eoff[e + 1];
+            eoff[e] = run;
+            run += c;
+        }
+        eoff[n_experts] = run;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= n_experts; e += blockDim.x) offsets[e] = eoff[e];
+    for (int i0 = wave * C; i0 < min((wave + 1) * C, P); i0 += 64) {
+        const int i = i0 + lane;
+        const int e = i < P ? ids[i] : -1;
+        const bool valid = e >= 0 && e < n_experts;
+        if (i < P && !valid) pos[i] = -1;
+        unsigned long long todo = __ballot(valid);
+        while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const int key = __shfl(e, leader, MK_WAVE);
+            const unsigned long long m = __ballot(valid && e == key);
+            const int start = eoff[key] + mine[key];  // read by every lane before the leader advances it
+            if (valid && e == key) {
+                const int r = start + __popcll(m & ((1ull << lane) - 1ull));
+                order[r] = i;
+                pos[i] = r;
+            }
+            if (lane == leader) mine[key] += __popcll(m);
+            todo &= ~m;
+        }
+    }
+}
+
+// MXFP8 of the hidden row of each grouped pair: a lane takes 8 consecutive values, four lanes a 32-block
+__global__ __launch_bounds__(256) void prefill_gather_mxfp8_kernel(const float *__restrict__ x, const int32_t *__restrict__ order,
+                                                                   const int32_t *__restrict__ offsets, int n_experts, int topk, int d,
+                                                                   uint8_t *__restrict__ codes, uint8_t *__restrict__ exps) {
+    const int per_row = d / 8;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 8 values
+    const size_t rows = (size_t)offsets[n_experts];                  // pairs with a valid expert id
+    if (i >= rows * per_row) return;
+    const size_t r = i / per_row, c = i % per_row;
+    const int t = order[r] / topk;
+    const mk_f4 *src = reinterpret_cast<const mk_f4 *>(x + (size_t)t * d) + 2 * c;
+    const mk_f4 a = src[0], b = src[1];
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t eb, c0, c1;
+    mk_mxfp8_quantize8(v, eb, c0, c1);
+    reinterpret_cast<mk_u2 *>(codes)[i] = mk_u2{c0, c1};
+    if ((c & 3) == 0) exps[r * (d / 32) + (c >> 2)] = (uint8_t)eb;
+}
+
+// act = ACT(gate, up) and its MXFP8 form
+__global__ __launch_bounds__(256) void prefill_act_mxfp8_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                const int32_t *__restrict__ offsets, int n_experts, int inter, int act_kind,
+                                                                uint8_t *__restrict__ codes, uint8_t *__restrict__ exps) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 8 values
+    const size_t n = (size_t)offsets[n_experts] * (inter / 8);
+    if (i >= n) return;
+    const mk_f4 g0 = reinterpret_cast<const mk_f4 *>(g)[2 * i], g1 = reinterpret_cast<const mk_f4 *>(g)[2 * i + 1];
+    const mk_f4 u0 = reinterpret_cast<const mk_f4 *>(u)[2 * i], u1 = reinterpret_cast<const mk_f4 *>(u)[2 * i + 1];
+    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = mk_act(act_kind, gv[k], uv[k], 0.0f, 1.0f);
+    uint32_t eb, c0, c1;
+    mk_mxfp8_quantize8(v, eb, c0, c1);
+    reinterpret_cast<mk_u2 *>(codes)[i] = mk_u2{c0, c1};
+    if ((i & 3) == 0) exps[i >> 2] = (uint8_t)eb;
+}
+
+// out_t = sum_s w[t][s] * o[pos(t, s)] in slot order, multiply then add (src/model.rs:2690-2700)
+__global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ o, const int32_t *__restrict__ pos,
+                                                              const float *__restrict__ weights, int topk, int d, float *__restrict__ out) {
+    const int t = blockIdx.y;
+    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (c >= d) return;
+    mk_f4 y = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s = 0; s < topk; s++) {
+        const int r = pos[t * topk + s];
+        if (r < 0) continue;
+        const float w = weights[t * topk + s];
+        const mk_f4 v = *reinterpret_cast<const mk_f4 *>(o + (size_t)r * d + c);
+        y.x = __fadd_rn(y.x, __fmul_rn(w, v.x));
+        y.y = __fadd_rn(y.y, __fmul_rn(w, v.y));
+        y.z = __fadd_rn(y.z, __fmul_rn(w, v.z));
+        y.w = __fadd_rn(y.w, __fmul_rn(w, v.w));
+    }
+    *reinterpret_cast<mk_f4 *>(out + (size_t)t * d + c) = y;
+}
+
+}  // namespace
+
+extern "C" size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter) {
+    return carve(nullptr, T * topk, n_experts, d, inter).bytes;
+}
+
+extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                  const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
+    MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
+    const size_t d = table->d, inter = table->inter;
+    MK_REQUIRE(d % 128 == 0 && inter % 128 == 0 && d > 0 && inter > 0, "d and inter must be positive multiples of 128");
+    MK_REQUIRE(n_experts >= 1 && n_experts <= 960 && T >= 1 && topk >= 1 && T <= 65535, "bad token / expert count");
+    MK_REQUIRE(T * topk <= (size_t)GROUP_MAX_P, "at most 16384 (token, slot) pairs per call: split the prompt");
+    MK_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)out & 15) == 0, "workspace must be 256-byte and out 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const size_t P = T * topk;
+    PrefillWs w = carve(workspace, P, n_experts, d, inter);
+    const size_t group_lds = ((size_t)GROUP_WAVES * n_experts + n_experts + 1) * sizeof(int);
+    MK_REQUIRE(group_lds <= 64 * 1024, "too many experts for the grouping kernel (17 counters per expert in 64 KiB of LDS)");
+    hipLaunchKernelGGL(prefill_group_kernel, dim3(1), dim3(GROUP_WAVES * 64), group_lds, st, ids, (int)P, (int)n_experts, w.order, w.pos,
+                       w.offsets);
+    int s = mk_launch_status("prefill_group");
+    if (s != MK_OK) return s;
+    MK_REQUIRE(((uintptr_t)x & 15) == 0, "x must be 16-byte aligned");
+    hipLaunchKernelGGL(prefill_gather_mxfp8_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
+                       (int)n_experts, (int)topk, (int)d, w.codes, w.exps);
+    if ((s = mk_launch_status("prefill_gather_mxfp8")) != MK_OK) return s;
+    if ((s = mk_dev_mxfp4_grouped_gemm(table->w1p, table->w1s, n_experts, inter, d, w.codes, w.exps, w.offsets, P, w.g, stream)) != MK_OK) return s;
+    if ((s = mk_dev_mxfp4_grouped_gemm(table->w3p, table->w3s, n_experts, inter, d, w.codes, w.exps, w.offsets, P, w.u, stream)) != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_act_mxfp8_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
+                       (int)n_experts, (int)inter, act_kind, w.codes2, w.exps2);
+    if ((s = mk_launch_status("prefill_act_mxfp8")) != MK_OK) return s;
+    if ((s = mk_dev_mxfp4_grouped_gemm(table->w2p, table->w2s, n_experts, d, inter, w.codes2, w.exps2, w.offsets, P, w.o, stream)) != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
+                       (int)d, out);
+    return mk_launch_status("prefill_combine");
+}

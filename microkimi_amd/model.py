@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 
 from . import _lib, q8 as _q8
-from ._lib import ACT_SWIGLU, MODE_F32, MODE_Q8, ExpertTable, check, cur_stream, hptr, lib, ptr
+from ._lib import ACT_DS, ACT_SITU, ACT_SWIGLU, MODE_F32, MODE_Q8, ExpertTable, check, cur_stream, hptr, lib, ptr
 
 
 class Q8Head:
@@ -159,6 +159,23 @@ def moe_decode(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_S
         out = torch.empty((B, experts.d), dtype=torch.float32, device=x.device)
     check(lib.mk_dev_moe_decode(C.byref(experts.table), B, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), shared,
                                 ptr(x.contiguous()), mode, act_kind, float(limit), ptr(experts._ws), ptr(out), cur_stream()))
+    return out
+
+
+def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None):
+    """The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) for T prompt positions: pairs grouped by
+    expert, gate / up / activation / down per used expert on the block-scaled matrix cores (MXFP8 activations),
+    per-token weighted sum in slot order.  ids [T, topk] int32, weights [T, topk] f32, x [T, d] f32; returns [T, d]."""
+    import torch
+    _lib.require_device()
+    T, topk = ids.shape
+    need = lib.mk_moe_prefill_workspace_bytes(T, topk, experts.n, experts.d, experts.inter)
+    if experts._ws is None or experts._ws.numel() < need:
+        experts._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((T, experts.d), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_moe_prefill(C.byref(experts.table), experts.n, T, topk, ptr(ids.contiguous()), ptr(weights.contiguous()),
+                                 ptr(x.contiguous()), act_kind, ptr(experts._ws), ptr(out), cur_stream()))
     return out
 
 

@@ -82,9 +82,26 @@ def test_quantize_mxfp8_bit_exact():
     x[7, :64] = 0.0
     x[7, 64:96] = np.float32(448.0)  # amax / 448 is an exact power of two
     x[7, 96:128] = np.float32(0.875)
+    # every e4m3 value, every midpoint between neighbours (ties) and their float neighbours, in blocks whose scale
+    # is 1 (a 448 in each block) and in blocks scaled by 2^-3
+    grid = np.array([oracle.e4m3_to_f32(c) for c in range(0x7F)], np.float32)  # 0 .. 448 ascending
+    mids = ((grid[:-1].astype(np.float64) + grid[1:].astype(np.float64)) / 2).astype(np.float32)
+    pts = np.concatenate([grid, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9))]).astype(np.float32)
+    pts = np.concatenate([pts, -pts])
+    rows = []
+    for k in range(0, len(pts), 31):
+        blk = np.zeros(32, np.float32)
+        blk[0] = 448.0
+        blk[1:1 + len(pts[k:k + 31])] = pts[k:k + 31]
+        rows.append(blk)
+    ties = np.concatenate(rows)
+    ties = np.concatenate([ties, ties * np.float32(0.125)])
+    pad = (-len(ties)) % 2048
+    ties = np.concatenate([ties, np.zeros(pad, np.float32)]).reshape(-1, 2048)
+    x = np.concatenate([x, ties]).astype(np.float32)
     codes, exps = dequant.quantize_mxfp8(dev(x))
     codes, exps = codes.cpu().numpy(), exps.cpu().numpy()
-    for r in range(8):
+    for r in range(x.shape[0]):
         _, c, e = oracle.fp8_roundtrip(x[r], 32)
         assert np.array_equal(exps[r], e), r
         assert np.array_equal(codes[r], c), r

@@ -76,3 +76,28 @@ def test_matches_oracle_prefill_expert_section():
     # the activation is re-rounded to e4m3 after a device expf: a last-bit difference in exp can move a value across
     # a rounding boundary, so this end-to-end check is looser than the single-GEMM one
     assert rel_l2(got, want) <= 2e-3
+
+
+@pytest.mark.parametrize("T,topk,n_experts,d,inter,act", [(24, 2, 4, 256, 128, "swiglu"), (40, 3, 7, 512, 256, "situ"), (5, 1, 3, 1024, 512, "swiglu")])
+def test_moe_prefill_on_device(T, topk, n_experts, d, inter, act):
+    # grouping, gather, the three grouped GEMMs, activation and combine all on the device (mk_dev_moe_prefill) against
+    # the oracle's moe_prefill with the MXFP8 rounding switched on; the looser bound is the device expf in front of an
+    # e4m3 rounding (see the test above)
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(T * 7 + n_experts)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.uint32)
+    if n_experts > 4:
+        ids[ids == 2] = 5  # an expert nobody selects
+    wts = rng.random((T, topk)).astype(np.float32)
+    kind = oracle.ACT_SITU if act == "situ" else oracle.ACT_SWIGLU
+    want = oracle.moe_prefill(table, ids, wts, x, act_kind=kind, round_mxfp8=True)
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x),
+                            act_kind=model.ACT_SITU if act == "situ" else model.ACT_SWIGLU).cpu().numpy()
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, want) <= 2e-3
