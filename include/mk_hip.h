@@ -177,6 +177,34 @@ int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const
  * src/model.rs:2157-2173), weights renormalised.  ids [B][k] int32, weights [B][k]. */
 int mk_dev_router_softmax_topk(const float *logits, size_t B, size_t n, size_t k, int32_t *ids, float *weights, void *stream);
 
+/* The reference's three routing rules on given logits [B][n] (one call, B tokens):
+ *   MK_ROUTER_SOFTMAX       score = key = softmax(l);               w = score / sum         (benchmark MoE layer)
+ *   MK_ROUTER_SIGMOID       score = sigmoid(l), key = score + bias; w = score / (sum+1e-20) (src/model.rs:2151-2173)
+ *   MK_ROUTER_SQRTSOFTPLUS  score = sqrt(softplus(l)), key = score + bias;
+ *                           w = score / sum * route_scale                                   (src/deepseek.rs:16-58)
+ * Selection: the k largest keys, strict '>' against the current worst, stable
+ * (ties to the lowest index), in descending key order; sums run in that order.
+ * bias [n] may be NULL.  ids [B][k] int32, weights [B][k]. */
+#define MK_ROUTER_SOFTMAX 0
+#define MK_ROUTER_SIGMOID 1
+#define MK_ROUTER_SQRTSOFTPLUS 2
+int mk_dev_router_topk(const float *logits, size_t B, size_t n, size_t k, int kind, const float *bias, float route_scale, int32_t *ids,
+                       float *weights, void *stream);
+
+/* model::rmsnorm / deepseek::ds_rmsnorm (src/model.rs:599-605, src/deepseek.rs:241-248) for B rows of d floats:
+ *   ss = dot(x, x) / d;  inv = 1 / sqrt(ss + eps);  y[i] = x[i] * inv * w[i]
+ * with the reference's dot contract (src/model.rs:46-82) replayed operation for operation: y is bit-identical.
+ * out [B][d] may be NULL.  When q and scales are given (both or neither), y is also quantized as
+ * q8::quantize_q8_into does (src/q8.rs:49-69): q [B][d] i8, scales [B][d/32] f32, d % 32 == 0 -- the input the
+ * q8-mode matvecs take, so norm -> quantize -> matvec needs no pass over y in between. */
+int mk_dev_rmsnorm(const float *x, size_t B, size_t d, const float *w, float eps, float *out, int8_t *q, float *scales, void *stream);
+
+/* model::matvec_cpu (src/model.rs:214-222): out[b][r] = dot(w[r], x[b]) for a row-major f32 matrix [rows][cols]
+ * and B vectors, with the reference's dot contract replayed operation for operation (bit-identical; each lane
+ * walks a sequential chain of cols/8 additions, so this is meant for the small matrices of a layer: router
+ * gate, latent projections). */
+int mk_dev_matvec_f32(const float *w, size_t rows, size_t cols, const float *x, size_t B, float *out, void *stream);
+
 /* ------------------------------------------- device level: MLA attention */
 
 /* mla_attn_flash_q8_mqa (src/model.rs:1804-1908) in the weight-absorbed form:

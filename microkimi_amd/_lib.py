@@ -58,6 +58,9 @@ def _load():
         "mk_moe_decode_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_dev_moe_decode": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),
         "mk_dev_router_softmax_topk": (i32, [vp, sz, sz, sz, vp, vp, vp]),
+        "mk_dev_router_topk": (i32, [vp, sz, sz, sz, i32, vp, f32, vp, vp, vp]),
+        "mk_dev_rmsnorm": (i32, [vp, sz, sz, vp, f32, vp, vp, vp, vp]),
+        "mk_dev_matvec_f32": (i32, [vp, sz, sz, vp, sz, vp, vp]),
         "mk_mla_decode_workspace_bytes": (sz, [sz, sz, sz]),
         "mk_dev_mla_q8_decode": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp, vp]),
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),

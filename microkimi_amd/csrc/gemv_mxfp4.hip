@@ -228,16 +228,16 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_f32_kernel(GemvArgs a) {
                 mk_f2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 1);
                 mk_f2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 2);
                 mk_f2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 3);
-                gsum = __fadd_rn(gsum, __fmul_rn(p0.x, x0.x));
-                gsum = __fadd_rn(gsum, __fmul_rn(p0.y, x0.y));
-                gsum = __fadd_rn(gsum, __fmul_rn(p1.x, x0.z));
-                gsum = __fadd_rn(gsum, __fmul_rn(p1.y, x0.w));
-                gsum = __fadd_rn(gsum, __fmul_rn(p2.x, x1.x));
-                gsum = __fadd_rn(gsum, __fmul_rn(p2.y, x1.y));
-                gsum = __fadd_rn(gsum, __fmul_rn(p3.x, x1.z));
-                gsum = __fadd_rn(gsum, __fmul_rn(p3.y, x1.w));
+                gsum = mk_add(gsum, mk_mul(p0.x, x0.x));
+                gsum = mk_add(gsum, mk_mul(p0.y, x0.y));
+                gsum = mk_add(gsum, mk_mul(p1.x, x0.z));
+                gsum = mk_add(gsum, mk_mul(p1.y, x0.w));
+                gsum = mk_add(gsum, mk_mul(p2.x, x1.x));
+                gsum = mk_add(gsum, mk_mul(p2.y, x1.y));
+                gsum = mk_add(gsum, mk_mul(p3.x, x1.z));
+                gsum = mk_add(gsum, mk_mul(p3.y, x1.w));
             }
-            float term = __fmul_rn(gsum, mk_scale_from_byte(sb[t]));
+            float term = mk_mul(gsum, mk_scale_from_byte(sb[t]));
             const int rit = bi / NB;
 #pragma unroll
             for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
@@ -286,9 +286,9 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_generic_kernel(GemvArgs a, int
             for (int d = 0; d < 4; d++) {
                 uint32_t wd = (uint32_t)w[d];
 #pragma unroll
-                for (int k = 0; k < 8; k++) gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> (4 * k)) & 15u), x[d * 8 + k]));
+                for (int k = 0; k < 8; k++) gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> (4 * k)) & 15u), x[d * 8 + k]));
             }
-            acc += __fmul_rn(gsum, mk_scale_from_byte(sb));
+            acc += mk_mul(gsum, mk_scale_from_byte(sb));
         }
     }
     acc = mk_wave_sum(acc);
@@ -324,16 +324,16 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__res
                     for (int d = 0; d < 4; d++) {
                         uint32_t wd = (uint32_t)w[d];
                         mk_f4 x0 = xv[d * 2], x1 = xv[d * 2 + 1];
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1(wd & 15u), x0.x));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 4) & 15u), x0.y));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 8) & 15u), x0.z));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 12) & 15u), x0.w));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 16) & 15u), x1.x));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 20) & 15u), x1.y));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 24) & 15u), x1.z));
-                        gsum = __fadd_rn(gsum, __fmul_rn(mk_e2m1((wd >> 28) & 15u), x1.w));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1(wd & 15u), x0.x));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 4) & 15u), x0.y));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 8) & 15u), x0.z));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 12) & 15u), x0.w));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 16) & 15u), x1.x));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 20) & 15u), x1.y));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 24) & 15u), x1.z));
+                        gsum = mk_add(gsum, mk_mul(mk_e2m1((wd >> 28) & 15u), x1.w));
                     }
-                    acc[p] += __fmul_rn(gsum, s);
+                    acc[p] += mk_mul(gsum, s);
                 }
             }
         }

@@ -7,6 +7,15 @@
 
 #define MK_WAVE 64
 
+// The reference is Rust, which never fuses a multiplication with the addition that follows it.  Device code is
+// compiled with contraction on by default, so it is switched off for everything that includes this header
+// (a fused multiply-add is written fmaf / __builtin_elementwise_fma where one is wanted).  mk_add / mk_mul mark
+// the places where the separate roundings are part of the parity contract; HIP's __fadd_rn / __fmul_rn are plain
+// operators inside header functions compiled with contraction on, and do get fused after inlining.
+#pragma clang fp contract(off)
+__device__ __forceinline__ float mk_add(float a, float b) { return a + b; }
+__device__ __forceinline__ float mk_mul(float a, float b) { return a * b; }
+
 typedef _Float16 mk_h2 __attribute__((ext_vector_type(2)));
 typedef float mk_f2 __attribute__((ext_vector_type(2)));
 typedef int mk_i4 __attribute__((ext_vector_type(4)));

@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
                 for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
             }
 #pragma unroll
-            for (int r = 0; r < RT; r++) y[u][r] = __fadd_rn(y[u][r], __fmul_rn(pw, mk_wave_sum(acc[r])));
+            for (int r = 0; r < RT; r++) y[u][r] = mk_add(y[u][r], mk_mul(pw, mk_wave_sum(acc[r])));
         }
         if (s == per - 1) {  // the row's last pair: store and start the next rows
 #pragma unroll
@@ -416,9 +416,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     float y = 0.0f;
     for (int s = 0; s < topk; s++) {
         const float v = o[((size_t)t * per + s) * d + j];
-        y = ds_rule ? __fadd_rn(y, v) : __fadd_rn(y, __fmul_rn(pw[t * per + s], v));
+        y = ds_rule ? mk_add(y, v) : mk_add(y, mk_mul(pw[t * per + s], v));
     }
-    if (per > topk) y = __fadd_rn(y, o[((size_t)t * per + topk) * d + j]);
+    if (per > topk) y = mk_add(y, o[((size_t)t * per + topk) * d + j]);
     out[(size_t)t * d + j] = y;
 }
 
@@ -553,74 +553,4 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((d + 255) / 256), (unsigned)B), dim3(256), 0, st, w.o, w.pt.pw, per, (int)topk, (int)d,
                        act_kind == MK_ACT_DS ? 1 : 0, out);
     return mk_launch_status("moe_combine");
-}
-
-// ---------------------------------------------------------------- router
-// softmax over n logits, top-k by probability with strict '>' replacement of
-// the current worst and a stable order (ties to the lowest index), weights
-// renormalised (src/model.rs:2157-2173 selection rule on softmax scores).
-// One wave per token; n <= 4096, k <= 64.
-__global__ __launch_bounds__(64) void router_softmax_topk_kernel(const float *__restrict__ logits, int n, int k, int32_t *__restrict__ ids,
-                                                                 float *__restrict__ weights) {
-    extern __shared__ float prob[];  // [n]
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float *row = logits + (size_t)t * n;
-    float m = -INFINITY;
-    for (int i = lane; i < n; i += 64) m = fmaxf(m, row[i]);
-    m = mk_wave_max(m);
-    // the reference sums exp(l - m) sequentially; the sum is only a common
-    // normaliser, so its association does not change the selection order
-    float z = 0.0f;
-    for (int i = lane; i < n; i += 64) {
-        float e = expf(row[i] - m);
-        prob[i] = e;
-        z += e;
-    }
-    z = mk_wave_sum(z);
-    __syncthreads();
-    for (int i = lane; i < n; i += 64) prob[i] = prob[i] / z;
-    __syncthreads();
-    // k rounds of (max value, lowest index) extraction == the stable descending order
-    float sum = 0.0f;
-    float myw = 0.0f;
-    int myid = 0;
-    for (int r = 0; r < k; r++) {
-        float bv = -1.0f;
-        int bi = 0x7FFFFFFF;
-        for (int i = lane; i < n; i += 64) {
-            float v = prob[i];
-            if (v > bv || (v == bv && i < bi)) {
-                bv = v;
-                bi = i;
-            }
-        }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            float ov = __shfl_xor(bv, off, MK_WAVE);
-            int oi = __shfl_xor(bi, off, MK_WAVE);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        if (lane == r) {
-            myw = bv;
-            myid = bi;
-        }
-        sum += bv;  // slot order, as the reference sums the selected scores
-        if (lane == 0) prob[bi] = -2.0f;
-        __syncthreads();
-    }
-    if (lane < k) {
-        ids[t * k + lane] = myid;
-        weights[t * k + lane] = myw / sum;
-    }
-}
-
-extern "C" int mk_dev_router_softmax_topk(const float *logits, size_t B, size_t n, size_t k, int32_t *ids, float *weights, void *stream) {
-    MK_REQUIRE(logits && ids && weights, "null pointer");
-    MK_REQUIRE(n >= 1 && n <= 4096 && k >= 1 && k <= 64 && k <= n && B >= 1 && B <= 65535, "bad router shape");
-    hipLaunchKernelGGL(router_softmax_topk_kernel, dim3((unsigned)B), dim3(64), n * sizeof(float), (hipStream_t)stream, logits, (int)n, (int)k,
-                       ids, weights);
-    return mk_launch_status("router_softmax_topk");
 }

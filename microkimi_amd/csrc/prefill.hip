@@ -169,10 +169,10 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__res
         if (r < 0) continue;
         const float w = weights[t * topk + s];
         const mk_f4 v = *reinterpret_cast<const mk_f4 *>(o + (size_t)r * d + c);
-        y.x = __fadd_rn(y.x, __fmul_rn(w, v.x));
-        y.y = __fadd_rn(y.y, __fmul_rn(w, v.y));
-        y.z = __fadd_rn(y.z, __fmul_rn(w, v.z));
-        y.w = __fadd_rn(y.w, __fmul_rn(w, v.w));
+        y.x = mk_add(y.x, mk_mul(w, v.x));
+        y.y = mk_add(y.y, mk_mul(w, v.y));
+        y.z = mk_add(y.z, mk_mul(w, v.z));
+        y.w = mk_add(y.w, mk_mul(w, v.w));
     }
     *reinterpret_cast<mk_f4 *>(out + (size_t)t * d + c) = y;
 }

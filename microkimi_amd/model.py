@@ -179,6 +179,53 @@ def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None):
     return out
 
 
+ROUTER_SOFTMAX, ROUTER_SIGMOID, ROUTER_SQRTSOFTPLUS = 0, 1, 2
+
+
+def rmsnorm(x, w, eps, quantize=False):
+    """model::rmsnorm / ds_rmsnorm (src/model.rs:599-605, src/deepseek.rs:241-248) for rows x [B, d] (or [d]) on the
+    device, bit-identical to the reference.  With quantize=True also returns the q8 form of the normed rows
+    (q [B, d] int8, scales [B, d/32] f32: q8::quantize_q8_into), the input of the q8-mode matvecs."""
+    import torch
+    _lib.require_device()
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    B, d = x2.shape
+    out = torch.empty_like(x2)
+    q = s = None
+    if quantize:
+        q = torch.empty((B, d), dtype=torch.int8, device=x.device)
+        s = torch.empty((B, d // 32), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_rmsnorm(ptr(x2), B, d, ptr(w.contiguous()), float(eps), ptr(out), ptr(q) if quantize else None,
+                             ptr(s) if quantize else None, cur_stream()))
+    out = out.reshape(x.shape)
+    return (out, q, s) if quantize else out
+
+
+def matvec(w, x):
+    """model::matvec (src/model.rs:198-247): w [rows, cols] f32, x [cols] or [B, cols]; the reference's dot contract,
+    bit-identical.  For the small f32 matrices of a layer (router gate, latent projections)."""
+    import torch
+    _lib.require_device()
+    rows, cols = w.shape
+    x2 = x.reshape(-1, cols).contiguous()
+    out = torch.empty((x2.shape[0], rows), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_matvec_f32(ptr(w.contiguous()), rows, cols, ptr(x2), x2.shape[0], ptr(out), cur_stream()))
+    return out.reshape(x.shape[:-1] + (rows,))
+
+
+def router_topk(logits, k, kind=ROUTER_SOFTMAX, bias=None, route_scale=1.0):
+    """The reference's routing rules on logits [B, n]: softmax (benchmark layer), sigmoid + selection bias
+    (src/model.rs:2151-2173), sqrt(softplus) + selection bias with route_scale (src/deepseek.rs:16-58)."""
+    import torch
+    _lib.require_device()
+    B, n = logits.shape
+    ids = torch.empty((B, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((B, k), dtype=torch.float32, device=logits.device)
+    check(lib.mk_dev_router_topk(ptr(logits.contiguous()), B, n, k, kind, None if bias is None else ptr(bias.contiguous()),
+                                 float(route_scale), ptr(ids), ptr(w), cur_stream()))
+    return ids, w
+
+
 def router_softmax_topk(logits, k):
     """Router of the benchmark MoE layer: softmax, top-k with the reference's tie rule, renormalised weights."""
     import torch

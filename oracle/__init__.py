@@ -218,6 +218,13 @@ def dot(a, b):
     return _lib.orc_dot(_p(a, _f32p), _p(b, _f32p), n)
 
 
+def rmsnorm(x, w, eps):
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    out = np.empty(x.size, np.float32)
+    _lib.orc_rmsnorm(_p(x, _f32p), x.size, _p(w, _f32p), C.c_float(eps), _p(out, _f32p))
+    return out
+
+
 def matvec_f32(w, rows, cols, x):
     w, x = _c(w, np.float32), _c(x, np.float32)
     out = np.empty(rows, np.float32)

@@ -379,6 +379,14 @@ ORC_API void orc_matvec_f32(const float *w, size_t rows, size_t cols, const floa
     for (size_t r = 0; r < rows; r++) out[r] = orc_dot(w + r * cols, x, cols);
 }
 
+/* src/model.rs:599-605 and src/deepseek.rs:241-248: ss = dot(x, x) / n; inv = 1 / sqrt(ss + eps);
+ * out[i] = x[i] * inv * w[i] (two multiplications, left to right) */
+ORC_API void orc_rmsnorm(const float *x, size_t n, const float *w, float eps, float *out) {
+    float ss = orc_dot(x, x, n) / (float)n;
+    float inv = 1.0f / sqrtf(ss + eps);
+    for (size_t i = 0; i < n; i++) out[i] = x[i] * inv * w[i];
+}
+
 /* ------------------------------------------------------- mxfp4 matvecs */
 
 /* src/mxfp4.rs:409-418: one row of the q8-integer path */

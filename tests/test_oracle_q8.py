@@ -93,3 +93,32 @@ def test_dot_order():
         for j in range(i, n):
             s = np.float32(s + np.float32(a[j] * b[j]))
         assert np.float32(oracle.dot(a, b)).view(np.uint32) == s.view(np.uint32), n
+
+
+def test_rmsnorm_closed_forms():
+    # model::rmsnorm (src/model.rs:599-605).  Pins: (1) a constant vector of a power of two, where every operation of
+    # the chain is exact except the final 1/sqrt, which is checked against the float64 value rounded once;
+    # (2) random vectors against the float64 formula; (3) the mean square goes through dot()'s accumulation order
+    # (a permutation that changes the 8-lane sums changes the last bits, a plain sequential sum would not match).
+    n = 64
+    x = np.full(n, 0.5, np.float32)
+    w = np.arange(1, n + 1, dtype=np.float32)
+    eps = np.float32(1e-5)
+    inv = np.float32(1.0) / np.sqrt(np.float32(0.25) + eps, dtype=np.float32)
+    want = (x * inv) * w
+    got = oracle.rmsnorm(x, w, float(eps))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    rng = np.random.default_rng(3)
+    for n in (8, 33, 512, 7168):
+        x = rng.standard_normal(n).astype(np.float32)
+        w = rng.standard_normal(n).astype(np.float32)
+        got = oracle.rmsnorm(x, w, 1e-6)
+        ref = x.astype(np.float64) / np.sqrt((x.astype(np.float64) ** 2).mean() + 1e-6) * w
+        assert np.abs(got - ref).max() <= 4e-7 * np.abs(ref).max() + 1e-12
+        ss = np.float32(oracle.dot(x, x)) / np.float32(n)
+        inv = np.float32(1.0) / np.sqrt(ss + np.float32(1e-6), dtype=np.float32)
+        assert np.array_equal(got.view(np.uint32), ((x * inv) * w).view(np.uint32))
+    # scale invariance up to eps: rmsnorm(2x) == rmsnorm(x) when eps = 0 (powers of two commute with every rounding)
+    x = rng.standard_normal(256).astype(np.float32)
+    w = np.ones(256, np.float32)
+    assert np.array_equal(oracle.rmsnorm(x, w, 0.0).view(np.uint32), oracle.rmsnorm(2 * x, w, 0.0).view(np.uint32))
