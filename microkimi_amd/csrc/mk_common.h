@@ -35,6 +35,11 @@ __device__ __forceinline__ mk_i4 mk_ldg128_off(const void *base, uint32_t off) {
     const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
     return *(const MK_GLOBAL mk_i4 *)(b + off);
 }
+// the same, marked non-temporal: for data that is streamed once and should not displace what the caches hold
+__device__ __forceinline__ mk_i4 mk_ldg128_off_nt(const void *base, uint32_t off) {
+    const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
+    return __builtin_nontemporal_load((const MK_GLOBAL mk_i4 *)(b + off));
+}
 __device__ __forceinline__ uint32_t mk_ldg_u8_off(const void *base, uint32_t off) {
     const MK_GLOBAL uint8_t *b = (const MK_GLOBAL uint8_t *)base;
     return b[off];
@@ -49,6 +54,7 @@ __device__ __forceinline__ float mk_ldg_f32_off(const void *base, uint32_t off) 
 }
 __device__ __forceinline__ mk_u2 mk_ldg64(const void *p) { return *(const MK_GLOBAL mk_u2 *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint32_t mk_ldg_u32(const void *p) { return *(const MK_GLOBAL uint32_t *)(const MK_GLOBAL void *)p; }
+__device__ __forceinline__ mk_i4 mk_ldg128_nt(const void *p) { return __builtin_nontemporal_load((const MK_GLOBAL mk_i4 *)(const MK_GLOBAL void *)p); }
 __device__ __forceinline__ uint32_t mk_ldg_u8(const void *p) { return *(const MK_GLOBAL uint8_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ uint16_t mk_ldg_u16(const void *p) { return *(const MK_GLOBAL uint16_t *)(const MK_GLOBAL void *)p; }
 __device__ __forceinline__ float mk_ldg_f32(const void *p) { return *(const MK_GLOBAL float *)(const MK_GLOBAL void *)p; }
