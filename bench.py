@@ -27,9 +27,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP4_PEAK_TFLOPS = 10100.0   # dense FP4/FP6 MFMA
 FP8_PEAK_TFLOPS = 5000.0
 # HBM bytes per launch of the batch-1 lm_head GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
-# reading of a plain 1 GiB copy (factors 2.000 and 1.000): 1 218 730 KiB read + 1 429 KiB written
+# reading of a plain 1 GiB copy (factors 2.000 and 1.000): 1 218 717 KiB read + 1 285 KiB written
 # (profiles/q8_gemv_b1_lm_head_163840x7168.md).  Algorithmic bytes are 1 248 489 472.
-LM_HEAD_B1_TRAFFIC_BYTES = 1249443000
+LM_HEAD_B1_TRAFFIC_BYTES = 1249281900
 
 
 def log(*a):
