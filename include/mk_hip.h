@@ -85,7 +85,8 @@ int mk_dev_fp8_dequant(const uint8_t *w, const uint8_t *scales, size_t rows, siz
 
 /* q8::quantize_q8_into (src/q8.rs:49-69) for `nvec` vectors of `n` floats each
  * (n % 32 == 0): q [nvec][n] i8, scales [nvec][n/32] f32.  dx = max|x|/127,
- * q = round-half-away(x/dx) clamped to +-127, zero block -> scale 0. */
+ * q = round-half-away(x/dx) clamped to +-127, zero block -> scale 0.
+ * x must be 16-byte aligned, q 4-byte aligned. */
 int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *scales, void *stream);
 
 /* deepseek::fp8_roundtrip with block 32 (src/deepseek.rs:312-322) kept in coded
@@ -142,7 +143,7 @@ int mk_dev_argmax(const float *logits, size_t batch, size_t n, void *ws, int32_t
 
 /* Q8Head::from_f32 (src/model.rs:274-286) on device: row-wise q8_0 of w [rows][cols];
  * scales written as f16 (scales_f16 != 0; the rounded value is what the matvec
- * then uses) or f32. */
+ * then uses) or f32.  w must be 16-byte aligned, q 4-byte aligned. */
 int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, void *scales, int scales_f16, void *stream);
 
 /* ------------------------------------------------ device level: MoE layer */
@@ -221,7 +222,8 @@ int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *r
                          size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream);
 
 /* MlaCache::push (src/model.rs:1583-1618) for the shared-latent cache: quantize
- * one position (latent [L] f32, rope [R] f32) into row `pos` of the cache arrays. */
+ * one position (latent [L] f32, rope [R] f32) into row `pos` of the cache arrays.
+ * latent and rope must be 16-byte aligned. */
 int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, size_t R, size_t pos, int8_t *lat_q, void *lat_s,
                             int8_t *rope_q, void *rope_s, void *stream);
 

@@ -69,20 +69,28 @@ __global__ __launch_bounds__(256) void mk_fp8_dequant_kernel(const uint8_t *__re
 template <bool SCALE_F16>
 __global__ __launch_bounds__(256) void mk_quantize_q8_kernel(const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ q,
                                                              void *__restrict__ scales) {
-    size_t g = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
-    int j = threadIdx.x & 31;
-    if (g >= n_blocks) return;  // whole half-waves leave together
-    float v = x[g * 32 + j];
-    float mx = mk_half_wave_max(fabsf(v));
-    float dx = mx / 127.0f;
-    int qi = 0;
-    if (dx != 0.0f) qi = mk_q8_round(v, dx);
-    q[g * 32 + j] = (int8_t)qi;
-    if (j == 0) {
+    // 8 lanes per 32-block, four values each
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_blocks * 8) return;  // whole groups of 8 lanes leave together
+    const mk_f4 v = reinterpret_cast<const mk_f4 *>(x)[i];
+    float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+    mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+    mx = fmaxf(mx, mk_dpp<0x141>(mx));
+    const float dx = mx / 127.0f;
+    uint32_t packed = 0;
+    if (dx != 0.0f) {
+        float qf[4];
+        mk_q8_round4(v, dx, qf);
+        packed = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                 ((uint32_t)(int)qf[3] << 24);
+    }
+    reinterpret_cast<uint32_t *>(q)[i] = packed;
+    if ((i & 7) == 0) {
         if (SCALE_F16)
-            reinterpret_cast<uint16_t *>(scales)[g] = mk_f32_to_f16_bits(dx);
+            reinterpret_cast<uint16_t *>(scales)[i >> 3] = mk_f32_to_f16_bits(dx);
         else
-            reinterpret_cast<float *>(scales)[g] = dx;
+            reinterpret_cast<float *>(scales)[i >> 3] = dx;
     }
 }
 
@@ -129,9 +137,10 @@ extern "C" int mk_dev_fp8_dequant(const uint8_t *w, const uint8_t *scales, size_
 extern "C" int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *scales, void *stream) {
     MK_REQUIRE(x && q && scales, "null pointer");
     MK_REQUIRE(n % 32 == 0, "q8 blocks are 32 wide");
+    MK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 3) == 0, "x must be 16-byte and q 4-byte aligned");
     size_t n_blocks = nvec * n / 32;
     if (n_blocks == 0) return MK_OK;
-    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    unsigned grid = (unsigned)((n_blocks + 31) / 32);
     hipLaunchKernelGGL(mk_quantize_q8_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, x, n_blocks, q, (void *)scales);
     return mk_launch_status("quantize_q8");
 }
@@ -139,9 +148,10 @@ extern "C" int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t 
 extern "C" int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, void *scales, int scales_f16, void *stream) {
     MK_REQUIRE(w && q && scales, "null pointer");
     MK_REQUIRE(cols % 32 == 0, "q8 blocks are 32 wide");
+    MK_REQUIRE(((uintptr_t)w & 15) == 0 && ((uintptr_t)q & 3) == 0, "w must be 16-byte and q 4-byte aligned");
     size_t n_blocks = rows * cols / 32;
     if (n_blocks == 0) return MK_OK;
-    unsigned grid = (unsigned)((n_blocks + 7) / 8);
+    unsigned grid = (unsigned)((n_blocks + 31) / 32);
     if (scales_f16)
         hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, n_blocks, q, scales);
     else
@@ -164,7 +174,9 @@ extern "C" int mk_dev_mla_cache_append(const float *latent, const float *rope, s
                                        int8_t *rope_q, void *rope_s, void *stream) {
     MK_REQUIRE(latent && rope && lat_q && lat_s && rope_q && rope_s, "null pointer");
     MK_REQUIRE(L % 32 == 0 && R % 32 == 0, "q8 blocks are 32 wide");
-    unsigned g1 = (unsigned)((L / 32 + 7) / 8), g2 = (unsigned)((R / 32 + 7) / 8);
+    MK_REQUIRE(((uintptr_t)latent & 15) == 0 && ((uintptr_t)rope & 15) == 0 && ((uintptr_t)lat_q & 3) == 0 && ((uintptr_t)rope_q & 3) == 0,
+               "latent and rope must be 16-byte, the cache rows 4-byte aligned");
+    unsigned g1 = (unsigned)((L / 32 + 31) / 32), g2 = (unsigned)((R / 32 + 31) / 32);
     hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(g1), dim3(256), 0, (hipStream_t)stream, latent, L / 32, lat_q + pos * L,
                        (void *)((uint16_t *)lat_s + pos * (L / 32)));
     hipLaunchKernelGGL(mk_quantize_q8_kernel<true>, dim3(g2), dim3(256), 0, (hipStream_t)stream, rope, R / 32, rope_q + pos * R,

@@ -123,18 +123,20 @@ __device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
 // ------------------------------------------------------------ fused fast path
 // Two launches per layer, no setup / quantize / combine kernels:
 //
-//   gate_up  grid (inter/32, pairs).  A workgroup owns one 32-row block of one
-//            (token, slot) pair; each of its 4 waves computes 8 rows of W1 x and
-//            W3 x.  The workgroup quantizes the token's hidden row to q8 itself
-//            (thread i owns block i: the loop of src/q8.rs:57-68) while its first
-//            weight loads are already in flight; the activation's f16 form lives
-//            in LDS.  The 32 activation values of the block are then quantized
-//            to q8 (the block matvec_packed forms when it re-quantizes its input
-//            for W2) and stored with their scale.
-//   down     grid (blocks, tokens).  The rows of W2 are dealt round-robin to the
-//            token's waves; a wave walks its rows pair by pair in slot order and
-//            accumulates y += w * (W2_e act) in registers, so the weighted sum of
-//            src/model.rs:2346-2351 needs no intermediate buffer.
+//   gate_up  one resident workgroup of 8 waves per CU.  Wave w owns the rows w,
+//            w + W, ... of W1 and W3 in every (token, slot) pair and streams them
+//            pair after pair; the workgroup quantizes the hidden rows to q8
+//            itself (src/q8.rs:57-68) while its first weight loads are in
+//            flight, and a lane keeps the activation blocks it owns in registers.
+//            Every wave has the same number of rows: no tail.  The activation
+//            value ACT(W1 x, W3 x) goes out in f32.
+//   down     grid (tokens, blocks).  The workgroup forms the q8 blocks of the
+//            token's activation rows in LDS (the block matvec_packed forms when
+//            it re-quantizes its input for W2).  The rows of W2 are dealt
+//            round-robin to the token's waves; a wave walks its rows pair by
+//            pair in slot order and accumulates y += w * (W2_e act) in registers,
+//            so the weighted sum of src/model.rs:2346-2351 needs no intermediate
+//            buffer.
 struct FusedArgs {
     mk_expert_table tab;
     const int32_t *ids;
@@ -142,146 +144,163 @@ struct FusedArgs {
     const float *x;
     int topk, shared, per, d, inter, act_kind, ds_rule;
     float limit;
-    int8_t *aq;  // [P][inter]
-    float *as;   // [P][inter/32]
+    float *af;   // [P][inter]  activation values in f32 (the down kernel forms their q8 blocks)
     float *out;  // [B][d]
 };
 
+// Row-owner gate/up: wave w owns the rows w, w + W, ... of W1 and W3 in every pair
+// (three units = 3 x 2 rows in flight per wave).  Tokens are taken in groups
+// that fit LDS (q8 of the hidden rows as f16 pairs); a lane keeps the activation
+// blocks it owns in registers and re-reads them from LDS only when the token
+// changes.  Walking the pairs in expert order instead, so that a repeated expert
+// finds its rows in the XCD's L2, was measured and gave nothing (B = 16: 577 us
+// against 569 us in token order): at 8 tokens and more the kernel is bound by the
+// vector unit's work per pair, not by where the bytes come from.
+struct RowUnit4 {
+    mk_i4 w1[4], w3[4];
+    uint32_t s1[4], s3[4];
+};
+
 template <int NB>
-__global__ __launch_bounds__(256) void moe_gate_up_fused_kernel(FusedArgs a) {
-    constexpr int TILE = lcm_c(NB, 64);
-    constexpr int T = TILE / 64;
-    constexpr int RT = TILE / NB;
-    static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
-    constexpr int RPW = 8;           // rows per wave
-    constexpr int NI = 2 * RPW / RT;  // work items of a wave: (matrix, tile), matrix fastest
-    constexpr int G0 = T >= 4 ? 1 : (T == 3 ? 2 : (T == 2 ? 4 : 8));
-    constexpr int G = G0 < NI ? G0 : NI;  // items per register block
-    // x as f16 pairs (words), laid out [4 chunks][NB blocks][4 words]: lanes that
-    // read the same chunk of consecutive blocks touch consecutive 16-byte slots
-    __shared__ __attribute__((aligned(16))) uint32_t xh[NB * 16];
-    __shared__ float xsc[NB];
-    __shared__ float act_l[32];
+__global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int B, int tg) {
+    constexpr int T = (NB + 63) / 64;  // loads per row
+    constexpr int LW = NB / T;         // lanes that carry a row (56 at NB = 224)
+    static_assert(NB % T == 0 && T <= 4, "row shape not covered");
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    const int per = a.per, gp_max = tg * per;
+    uint32_t *xh = lds;                                                   // [tg][NB * 16] f16 pairs, [4 chunks][NB][4 words]
+    float *xsc = reinterpret_cast<float *>(xh + (size_t)tg * NB * 16);   // [tg][NB]
+    const uint8_t **wp1 = reinterpret_cast<const uint8_t **>(xsc + (size_t)tg * NB);
+    const uint8_t **wp3 = wp1 + gp_max, **ws1 = wp3 + gp_max, **ws3 = ws1 + gp_max;
+    float *wgt_l = reinterpret_cast<float *>(ws3 + gp_max);
 
-    const int p = blockIdx.x, rb = blockIdx.y;  // pairs fastest: pairs that share an expert read a row block together
-    const int tok = p / a.per, slot = p % a.per;
-    const int e = slot < a.topk ? a.ids[tok * a.topk + slot] : a.shared;
-    const float wgt = slot < a.topk ? a.weights[tok * a.topk + slot] : 1.0f;
-    const uint8_t *wp[2] = {a.tab.w1p[e], a.tab.w3p[e]};
-    const uint8_t *wsc[2] = {a.tab.w1s[e], a.tab.w3s[e]};
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const size_t row0 = (size_t)rb * 32 + wave * RPW;
+    const int lane = threadIdx.x & 63, lane_c = lane < LW ? lane : LW - 1;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nw = gridDim.x * 8, w = blockIdx.x * 8 + wave;
+    // rows of this wave; a wave beyond the last row (inter not a multiple of 8) walks row inter - 1 and stores nothing:
+    // loads under a condition would make every later wait a full one
+    const bool live = w < a.inter;
+    const int J = live ? (a.inter - w + nw - 1) / nw : 1;
 
-    mk_i4 wa[G][T], wb[G][T];
-    uint32_t sa[G][T], sb[G][T];
-    auto load_block = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int it0) {
+    for (int t0 = 0; t0 < B; t0 += tg) {
+        const int nt = min(tg, B - t0), gp = nt * per;
+        // q8 of the group's hidden rows (src/q8.rs:57-68): 8 lanes per 32-block, one 16-byte load each.  The first batch
+        // of loads is issued before anything else, so that it returns ahead of the first weight loads.
+        constexpr int SB = 4;
+        const mk_f4 *xsrc = reinterpret_cast<const mk_f4 *>(a.x + (size_t)t0 * NB * 32);
+        const int n_x = nt * NB * 8;
+        mk_f4 xv[SB];
+        auto stage_load = [&](mk_f4 *v, int i0) {
 #pragma unroll
-        for (int j = 0; j < G; j++) {
-            const int it = it0 + j;
-            if (it < NI) {  // compile-time after unrolling
-                const size_t blk0 = (row0 + (size_t)(it >> 1) * RT) * NB;
+            for (int b = 0; b < SB; b++) v[b] = xsrc[min(i0 + b * 512, n_x - 1)];
+        };
+        auto stage_store = [&](const mk_f4 *v, int i0) {
 #pragma unroll
-                for (int t = 0; t < T; t++) {
-                    const size_t b = blk0 + t * 64 + lane;
-                    w[j][t] = mk_ldg128(wp[it & 1] + b * 16);
-                    sc[j][t] = mk_ldg_u8(wsc[it & 1] + b);
+            for (int b = 0; b < SB; b++) {
+                const int i = i0 + b * 512;
+                float mx = fmaxf(fmaxf(fabsf(v[b].x), fabsf(v[b].y)), fmaxf(fabsf(v[b].z), fabsf(v[b].w)));
+                mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+                mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+                mx = fmaxf(mx, mk_dpp<0x141>(mx));
+                const float dx = mx / 127.0f;
+                mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
+                if (dx != 0.0f) mk_q8_round4_f16(v[b], dx, lo, hi);
+                if (i < n_x) {
+                    const int tl = i / (NB * 8), g = (i / 8) % NB, j = i % 8;
+                    uint32_t *dst = xh + (size_t)tl * NB * 16 + ((j >> 1) * NB + g) * 4 + 2 * (j & 1);
+                    dst[0] = __builtin_bit_cast(uint32_t, lo);
+                    dst[1] = __builtin_bit_cast(uint32_t, hi);
+                    if (j == 0) xsc[tl * NB + g] = dx;
                 }
             }
+        };
+        stage_load(xv, threadIdx.x);
+        if (t0) __syncthreads();  // the previous group's LDS is still being read
+        if (threadIdx.x < gp) {
+            const int q = threadIdx.x, tok = t0 + q / per, slot = q % per;
+            const int e = slot < a.topk ? a.ids[tok * a.topk + slot] : a.shared;
+            wp1[q] = a.tab.w1p[e];
+            wp3[q] = a.tab.w3p[e];
+            ws1[q] = a.tab.w1s[e];
+            ws3[q] = a.tab.w3s[e];
+            wgt_l[q] = slot < a.topk ? a.weights[tok * a.topk + slot] : 1.0f;
         }
-    };
-    load_block(wa, sa, 0);  // in flight during the prologue
+        __syncthreads();
 
-    // q8 of the token's hidden row: thread i owns block i (NB <= 256)
-    if (threadIdx.x < NB) {
-        const mk_f4 *src = reinterpret_cast<const mk_f4 *>(a.x + (size_t)tok * NB * 32 + threadIdx.x * 32);
-        mk_f4 v[8];
-        float mx = 0.0f;
+        const int n_units = gp * J;
+        RowUnit4 ua, ub, uc;
+        auto load_unit = [&](RowUnit4 &U, int u) {
+            u = __builtin_amdgcn_readfirstlane(min(u, n_units - 1));  // past the end: the last unit again (not used)
+            const int k = u / J, j = u - k * J;
+            const int q = k;  // pairs in (token, slot) order
+            const uint8_t *p1 = mk_uniform_ptr(wp1[q]), *p3 = mk_uniform_ptr(wp3[q]);
+            const uint8_t *c1 = mk_uniform_ptr(ws1[q]), *c3 = mk_uniform_ptr(ws3[q]);
+            const uint32_t boff = (uint32_t)min(w + j * nw, a.inter - 1) * NB + lane_c;
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            v[k] = src[k];
-            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
-        }
-        const float dx = mx / 127.0f;
-        xsc[threadIdx.x] = dx;
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
-            if (dx != 0.0f) {
-                lo.x = (_Float16)(float)mk_q8_round(v[k].x, dx);
-                lo.y = (_Float16)(float)mk_q8_round(v[k].y, dx);
-                hi.x = (_Float16)(float)mk_q8_round(v[k].z, dx);
-                hi.y = (_Float16)(float)mk_q8_round(v[k].w, dx);
+            for (int t = 0; t < T; t++) {
+                U.w1[t] = mk_ldg128_off(p1, (boff + t * LW) * 16);
+                U.w3[t] = mk_ldg128_off(p3, (boff + t * LW) * 16);
+                U.s1[t] = mk_ldg_u8_off(c1, boff + t * LW);
+                U.s3[t] = mk_ldg_u8_off(c3, boff + t * LW);
             }
-            xh[((k >> 1) * NB + threadIdx.x) * 4 + 2 * (k & 1)] = __builtin_bit_cast(uint32_t, lo);
-            xh[((k >> 1) * NB + threadIdx.x) * 4 + 2 * (k & 1) + 1] = __builtin_bit_cast(uint32_t, hi);
-        }
-    }
-    __syncthreads();
-    float cf[T];
-#pragma unroll
-    for (int t = 0; t < T; t++) cf[t] = xsc[(t * 64 + lane) % NB];
+        };
+        load_unit(ua, 0);  // in flight while the hidden rows are quantized (a third unit here spills registers)
+        load_unit(ub, 1);
 
-    float res[2][RPW];  // [matrix][row]
+        stage_store(xv, threadIdx.x);
+        for (int i0 = threadIdx.x + 512 * SB; i0 < n_x; i0 += 512 * SB) {
+            stage_load(xv, i0);
+            stage_store(xv, i0);
+        }
+        __syncthreads();
+
+        {
+            mk_h2 xr[T][16];
+            float cf[T];
+            int cur_tok = -1;
+            auto compute_unit = [&](const RowUnit4 &U, int u) {
+                const int k = u / J, j = u - k * J;
+                const int q = k;  // pairs in (token, slot) order
+                const int tl = q / per;
+                if (tl != cur_tok) {
+                    cur_tok = tl;
+                    const uint32_t *src = xh + (size_t)tl * NB * 16;
 #pragma unroll
-    for (int m = 0; m < 2; m++)
+                    for (int t = 0; t < T; t++) {
+                        const int g = t * LW + lane_c;
 #pragma unroll
-        for (int r = 0; r < RPW; r++) res[m][r] = 0.0f;
-    auto compute_block = [&](const mk_i4(*w)[T], const uint32_t(*sc)[T], int it0) {
-#pragma unroll
-        for (int j = 0; j < G; j++) {
-            const int it = it0 + j;
-            if (it < NI) {
-                float acc[RT];
-#pragma unroll
-                for (int r = 0; r < RT; r++) acc[r] = 0.0f;
+                        for (int kk = 0; kk < 16; kk++) xr[t][kk] = __builtin_bit_cast(mk_h2, src[((kk >> 2) * NB + g) * 4 + (kk & 3)]);
+                        cf[t] = xsc[tl * NB + g];
+                    }
+                }
+                float s1 = 0.0f, s3 = 0.0f;
 #pragma unroll
                 for (int t = 0; t < T; t++) {
-                    const int g = (t * 64 + lane) % NB;
-                    mk_h2 xr[16];
-#pragma unroll
-                    for (int k = 0; k < 16; k++) xr[k] = __builtin_bit_cast(mk_h2, xh[((k >> 2) * NB + g) * 4 + (k & 3)]);
-                    float h = dot32_fp4_f16(w[j][t], xr);
-                    float term = (h + h) * (mk_half_scale_from_byte(sc[j][t]) * cf[t]);
-                    const int rit = (t * 64 + lane) / NB;
-#pragma unroll
-                    for (int r = 0; r < RT; r++) acc[r] += (rit == r) ? term : 0.0f;
+                    const float h1 = dot32_fp4_f16(U.w1[t], xr[t]), h3 = dot32_fp4_f16(U.w3[t], xr[t]);
+                    s1 += (h1 + h1) * (mk_half_scale_from_byte(U.s1[t]) * cf[t]);
+                    s3 += (h3 + h3) * (mk_half_scale_from_byte(U.s3[t]) * cf[t]);
                 }
-#pragma unroll
-                for (int r = 0; r < RT; r++) res[it & 1][(it >> 1) * RT + r] = mk_wave_sum(acc[r]);
+                if (lane >= LW) s1 = s3 = 0.0f;
+                const float gsum = mk_wave_sum(s1), usum = mk_wave_sum(s3);
+                const float act = mk_act(a.act_kind, gsum, usum, a.limit, wgt_l[q]);
+                if (lane == 0 && live) a.af[(size_t)(t0 * per + q) * a.inter + (w + j * nw)] = act;
+            };
+            for (int u = 0; u < n_units; u += 3) {
+                load_unit(uc, u + 2);
+                compute_unit(ua, u);
+                load_unit(ua, u + 3);
+                if (u + 1 < n_units) compute_unit(ub, u + 1);
+                load_unit(ub, u + 4);
+                if (u + 2 < n_units) compute_unit(uc, u + 2);
             }
-        }
-    };
-#pragma unroll
-    for (int it0 = 0; it0 < NI; it0 += 2 * G) {
-        load_block(wb, sb, it0 + G);
-        compute_block(wa, sa, it0);
-        load_block(wa, sa, it0 + 2 * G);
-        compute_block(wb, sb, it0 + G);
-    }
-    float mine = 0.0f;
-#pragma unroll
-    for (int r = 0; r < RPW; r++) {
-        const float act = mk_act(a.act_kind, res[0][r], res[1][r], a.limit, wgt);
-        if (lane == r) mine = act;
-    }
-    if (lane < RPW) act_l[wave * RPW + lane] = mine;
-    __syncthreads();
-    if (wave == 0) {
-        const float v = act_l[lane & 31];
-        const float mx = mk_half_wave_max(fabsf(v));
-        const float dx = mx / 127.0f;
-        if (lane < 32) {
-            const int qi = dx != 0.0f ? mk_q8_round(v, dx) : 0;
-            a.aq[(size_t)p * a.inter + rb * 32 + lane] = (int8_t)qi;
-            if (lane == 0) a.as[(size_t)p * (a.inter / 32) + rb] = dx;
         }
     }
 }
 
 constexpr int MAX_PER = 32;  // pairs per token the fused down kernel keeps in LDS
 
-template <int NB, int U>  // U = tiles per register block
-__global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
+template <int NB, int U, int WAVES>  // U = tiles per register block
+__global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a) {
     constexpr int TILE = lcm_c(NB, 64);
     constexpr int T = TILE / 64;
     constexpr int RT = TILE / NB;
@@ -294,6 +313,37 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
     __shared__ float pw_l[MAX_PER];
     const int tok = blockIdx.x, per = a.per;  // tokens fastest: they walk the rows in step
     float *asc = reinterpret_cast<float *>(ah + (size_t)per * NB * 16);
+    // q8 of the activation rows (what matvec_packed does to its input, src/q8.rs:49-69): 8 lanes per 32-block, one
+    // 16-byte load each; the first batch of loads is issued before anything else
+    constexpr int SB = 6;
+    const mk_f4 *af = reinterpret_cast<const mk_f4 *>(a.af + (size_t)tok * per * NB * 32);
+    const int n_a = per * NB * 8;
+    mk_f4 av[SB];
+    auto stage_load = [&](mk_f4 *v, int i0) {
+#pragma unroll
+        for (int b = 0; b < SB; b++) v[b] = af[min(i0 + b * WAVES * 64, n_a - 1)];
+    };
+    auto stage_store = [&](const mk_f4 *v, int i0) {
+#pragma unroll
+        for (int b = 0; b < SB; b++) {
+            const int i = i0 + b * WAVES * 64;
+            float mx = fmaxf(fmaxf(fabsf(v[b].x), fabsf(v[b].y)), fmaxf(fabsf(v[b].z), fabsf(v[b].w)));
+            mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+            mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+            mx = fmaxf(mx, mk_dpp<0x141>(mx));
+            const float dx = mx / 127.0f;
+            mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
+            if (dx != 0.0f) mk_q8_round4_f16(v[b], dx, lo, hi);
+            if (i < n_a) {
+                const int s = i / (NB * 8), g = (i / 8) % NB, j = i % 8;
+                uint32_t *dst = ah + (size_t)s * NB * 16 + ((j >> 1) * NB + g) * 4 + 2 * (j & 1);
+                dst[0] = __builtin_bit_cast(uint32_t, lo);
+                dst[1] = __builtin_bit_cast(uint32_t, hi);
+                if (j == 0) asc[s * NB + g] = dx;
+            }
+        }
+    };
+    stage_load(av, threadIdx.x);
     if (threadIdx.x < per) {
         const int s = threadIdx.x;
         const int e = s < a.topk ? a.ids[tok * a.topk + s] : a.shared;
@@ -301,26 +351,11 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
         ws_l[s] = a.tab.w2s[e];
         pw_l[s] = (s < a.topk && !a.ds_rule) ? a.weights[tok * a.topk + s] : 1.0f;
     }
-    const int8_t *aq = a.aq + (size_t)tok * per * NB * 32;
-    for (int i = threadIdx.x; i < per * NB * 8; i += 256) {
-        uint32_t v = reinterpret_cast<const uint32_t *>(aq)[i];
-        mk_h2 lo, hi;
-        lo.x = (_Float16)(float)(int8_t)(v & 255u);
-        lo.y = (_Float16)(float)(int8_t)((v >> 8) & 255u);
-        hi.x = (_Float16)(float)(int8_t)((v >> 16) & 255u);
-        hi.y = (_Float16)(float)(int8_t)(v >> 24);
-        // word i covers elements 4i..4i+3 of pair s: block g, f16 words 2j, 2j+1
-        const int s = i / (NB * 8), g = (i / 8) % NB, j = i % 8;
-        uint32_t *dst = ah + (size_t)s * NB * 16 + ((j >> 1) * NB + g) * 4 + 2 * (j & 1);
-        dst[0] = __builtin_bit_cast(uint32_t, lo);
-        dst[1] = __builtin_bit_cast(uint32_t, hi);
-    }
-    for (int i = threadIdx.x; i < per * NB; i += 256) asc[i] = a.as[(size_t)tok * per * NB + i];
-    __syncthreads();
+    __syncthreads();  // the pair tables: the first weight loads need them
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_tiles = a.d / RT;
-    const int wv = blockIdx.y * 4 + wave, wpt = gridDim.y * 4;
+    const int wv = blockIdx.y * WAVES + wave, wpt = gridDim.y * WAVES;
     const int my_tiles = wv < n_tiles ? (n_tiles - wv + wpt - 1) / wpt : 0;
     const int groups = (my_tiles + U - 1) / U;
     const int n_items = groups * per;  // (tile group, pair), pair fastest: slot order per row
@@ -335,7 +370,7 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = grp * U + u;
-            const uint32_t tile = (uint32_t)(wv + (k < my_tiles ? k : 0) * wpt);
+            const uint32_t tile = min((uint32_t)(wv + (k < my_tiles ? k : 0) * wpt), (uint32_t)(n_tiles - 1));  // idle waves re-read the last tile
             const uint32_t blk0 = tile * TILE + lane;
 #pragma unroll
             for (int t = 0; t < T; t++) {
@@ -390,12 +425,23 @@ __global__ __launch_bounds__(256) void moe_down_fused_kernel(FusedArgs a) {
             }
         }
     };
+    constexpr bool PRE2 = U * T <= 4;  // small register blocks: both in flight while the activation is staged
     load_item(wa, sa, 0);
+    if constexpr (PRE2) load_item(wb, sb, 1);
+
+    stage_store(av, threadIdx.x);
+    for (int i0 = threadIdx.x + WAVES * 64 * SB; i0 < n_a; i0 += WAVES * 64 * SB) {
+        stage_load(av, i0);
+        stage_store(av, i0);
+    }
+    __syncthreads();
+
     for (int i = 0; i < n_items; i += 2) {
-        load_item(wb, sb, i + 1);
+        if constexpr (!PRE2) load_item(wb, sb, i + 1);
         compute_item(wa, sa, i);
         load_item(wa, sa, i + 2);
         if (i + 1 < n_items) compute_item(wb, sb, i + 1);
+        if constexpr (PRE2) load_item(wb, sb, i + 3);
     }
 }
 
@@ -435,20 +481,34 @@ int tune(const char *name, int dflt) {
 }
 
 template <int NB>
-int launch_gate_up_fused(const FusedArgs &a, size_t P, hipStream_t st) {
-    hipLaunchKernelGGL(moe_gate_up_fused_kernel<NB>, dim3((unsigned)P, (unsigned)(a.inter / 32)), dim3(256), 0, st, a);
-    return mk_launch_status("moe_gate_up_fused");
+int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
+    // token group: as many hidden rows (f16 pairs + scales) and pair tables as fit 150 KiB of LDS, at most 8
+    const size_t per_tok = (size_t)NB * 68 + (size_t)a.per * 48;
+    int tg = (int)((150 * 1024) / per_tok);
+    if (tg > 8) tg = 8;
+    if (tg > (int)B) tg = (int)B;
+    const size_t lds = (size_t)tg * per_tok;
+    static bool opted = false;
+    if (!opted) {
+        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_gate_up_rows_kernel<NB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        opted = true;
+    }
+    int blocks = tune("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
+    if (blocks * 8 > a.inter) blocks = (a.inter + 7) / 8;
+    hipLaunchKernelGGL(moe_gate_up_rows_kernel<NB>, dim3(blocks), dim3(512), lds, st, a, (int)B, tg);
+    return mk_launch_status("moe_gate_up_rows");
 }
 
-template <int NB, int U>
+template <int NB, int U, int WAVES = 4>
 int launch_down_u(const FusedArgs &a, size_t B, int blocks, hipStream_t st) {
     const size_t lds = (size_t)a.per * NB * 64 + (size_t)a.per * NB * 4;
     static bool opted = false;
     if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_down_fused_kernel<NB, U>), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_down_fused_kernel<NB, U, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            150 * 1024);
         opted = true;
     }
-    hipLaunchKernelGGL((moe_down_fused_kernel<NB, U>), dim3((unsigned)B, blocks), dim3(256), lds, st, a);
+    hipLaunchKernelGGL((moe_down_fused_kernel<NB, U, WAVES>), dim3((unsigned)B, blocks), dim3(WAVES * 64), lds, st, a);
     return mk_launch_status("moe_down_fused");
 }
 
@@ -461,6 +521,17 @@ template <int NB>
 int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
     constexpr int TILE = lcm_c(NB, 64), T = TILE / 64, RT = TILE / NB;
     const int n_tiles = a.d / RT;
+    if constexpr (T == 1) {
+        // One workgroup of 14 waves per CU when the rows then divide evenly (7168 = 2^10 x 7): the activation is
+        // quantized once per CU instead of once per small workgroup, and every wave has the same number of tiles.
+        const int bpt = 256 / (int)B;  // workgroups per token
+        if (bpt >= 1 && !tune("MK_MOE_DOWN_SMALL", 0) && n_tiles % (bpt * 14) == 0) {
+            const int tiles = n_tiles / (bpt * 14);  // per wave
+            if (tiles % 8 == 0) return launch_down_u<NB, 8, 14>(a, B, bpt, st);
+            if (tiles % 4 == 0) return launch_down_u<NB, 4, 14>(a, B, bpt, st);
+            if (tiles % 2 == 0) return launch_down_u<NB, 2, 14>(a, B, bpt, st);
+        }
+    }
     const int target = tune("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
     int u = 8 / T;
     int forced = tune("MK_MOE_DOWN_U", 0);
@@ -513,14 +584,13 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
         fa.act_kind = act_kind;
         fa.ds_rule = act_kind == MK_ACT_DS ? 1 : 0;
         fa.limit = limit;
-        fa.aq = w.aq;
-        fa.as = w.as;
+        fa.af = w.af;
         fa.out = out;
         switch (nb) {
-            case 32: s = launch_gate_up_fused<32>(fa, P, st); break;
-            case 64: s = launch_gate_up_fused<64>(fa, P, st); break;
-            case 128: s = launch_gate_up_fused<128>(fa, P, st); break;
-            default: s = launch_gate_up_fused<224>(fa, P, st); break;
+            case 32: s = launch_gate_up_rows<32>(fa, B, st); break;
+            case 64: s = launch_gate_up_rows<64>(fa, B, st); break;
+            case 128: s = launch_gate_up_rows<128>(fa, B, st); break;
+            default: s = launch_gate_up_rows<224>(fa, B, st); break;
         }
         if (s != MK_OK) return s;
         switch (nbi) {

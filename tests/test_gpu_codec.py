@@ -70,6 +70,23 @@ def test_quantize_q8_bit_exact():
         qo, so = oracle.quantize_q8(x[r])
         assert np.array_equal(q[r], qo), r
         assert np.array_equal(bits(s[r]), bits(so)), r
+    # values on and next to rounding ties: block maximum 127 makes the scale exactly 1, so k + 0.5 is a tie and its
+    # float neighbours are not; other maxima put quotients within an ulp of a tie
+    n = 4096
+    y = np.zeros((n, 32), dtype=np.float32)
+    k = rng.integers(0, 126, size=(n, 31)).astype(np.float32) + 0.5
+    step = rng.integers(-2, 3, size=(n, 31))
+    near = k.copy()
+    for _ in range(2):
+        near = np.where(step > 0, np.nextafter(near, np.float32(200)), np.where(step < 0, np.nextafter(near, np.float32(-200)), near))
+        step = step - np.sign(step)
+    y[:, 1:] = near * rng.choice([-1.0, 1.0], size=(n, 31)).astype(np.float32)
+    y[:, 0] = 127.0
+    y[n // 2:] *= rng.uniform(0.01, 100.0, size=(n - n // 2, 1)).astype(np.float32)   # scales that are not a power of two
+    vt = q8.quantize_q8(dev(y.reshape(1, -1)))
+    qo, so = oracle.quantize_q8(y.reshape(-1))
+    assert np.array_equal(vt.q.cpu().numpy().reshape(-1), qo)
+    assert np.array_equal(bits(vt.scales.cpu().numpy().reshape(-1)), bits(so))
     # host-level entry point
     hv = q8.quantize_q8(x[0])
     assert np.array_equal(hv.q, q[0]) and np.array_equal(hv.scales, s[0])

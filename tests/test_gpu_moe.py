@@ -28,6 +28,8 @@ def build(n_experts, d, inter, cfg=2):
     (2048, 1024, 6, 3, 2, -1, 1),     # SiTU (K3 rule), no shared expert
     (4096, 2048, 5, 2, 3, 4, 2),      # DeepSeek rule: clamp, weight before W2, plain sum
     (1024, 512, 4, 16, 2, 3, 0),      # batch 16
+    (7168, 2048, 12, 9, 8, 11, 0),    # benchmark shapes, two token groups in the gate/up kernel (8 + 1)
+    (1024, 4096, 4, 5, 2, 3, 0),      # two rows of W1/W3 per wave
     (96, 64, 4, 2, 2, -1, 0),         # shape off the fast path (composed kernels)
 ])
 def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
