@@ -7,6 +7,8 @@
 //           t*64+l of the row (perfectly coalesced 1 KiB wave loads, no repack)
 //           and keeps the matching 16 activation bytes and block scale in
 //           registers for the whole kernel; 4 x v_dot4_i32_i8 per load.
+// batch 2-4 at 7168 columns: the batch-1 streaming pattern with the activation in
+//           LDS and two rows per LDS read (see q8_gemv_bn_kernel).
 // batch 2-8 matrix-core path.  One v_mfma_i32_16x16x64_i8 per 16 rows x 64
 //           columns.  The MFMA sums over K = 64 = two q8 blocks, whose scales
 //           differ, so the activation operand is laid out as 16 "columns" =
@@ -85,6 +87,101 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
         compute_row(wa, sa, r);
         load_row(wa, sa, r + 2 * n_waves);
         compute_row(wb, sb, r + n_waves);
+    }
+}
+
+// -------------------------------------------------- batch 2..4, long rows
+// The batch-1 streaming pattern (a wave reads whole rows, 1 KiB per load, non-
+// temporal, rows dealt round-robin to a resident grid) with the batch's
+// activation bytes and block scales in LDS: two rows are in the registers at a
+// time, so that every 16 activation bytes read from LDS meet two weight rows.
+// 4 x v_dot4_i32_i8 per (half block, batch column), the per-block term in f32 as
+// the reference writes it.  At 7168 columns this reads the matrix at the batch-1
+// rate; the matrix-core kernel below, whose lanes take 64 bytes of a row per
+// load, stays for the other row lengths.
+template <int NB, bool F16, int BATCH>
+__global__ __launch_bounds__(256, 2) void q8_gemv_bn_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows,
+                                                         const int8_t *__restrict__ xq, const float *__restrict__ xs,
+                                                         float *__restrict__ out) {
+    constexpr int T = NB * 2 / 64;
+    static_assert(NB % 32 == 0 && T >= 1 && T <= 8, "row shape not covered");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    mk_i4 *xl = reinterpret_cast<mk_i4 *>(lds);                            // [BATCH][NB * 2] half blocks
+    float *xsl = reinterpret_cast<float *>(lds + (size_t)BATCH * NB * 32);  // [BATCH][NB]
+    for (int i = threadIdx.x; i < BATCH * NB * 2; i += 256) xl[i] = reinterpret_cast<const mk_i4 *>(xq)[i];
+    for (int i = threadIdx.x; i < BATCH * NB; i += 256) xsl[i] = xs[i];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n_waves = gridDim.x * 4;
+    struct Row {
+        mk_i4 w[T];
+        float s[T];
+    };
+    auto load_row = [&](Row &R, int r) {
+        const uint32_t ru = (uint32_t)__builtin_amdgcn_readfirstlane(min(r, rows - 1));  // past the end: the last row again
+        const uint32_t qoff = ru * (NB * 32) + lane * 16, soff = ru * NB + (lane >> 1);
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            R.w[t] = mk_ldg128_off_nt(q, qoff + t * 1024);
+            if (F16) R.s[t] = mk_f16_bits_to_f32(mk_ldg_u16_off(scales, (soff + t * 32) * 2));
+            else R.s[t] = mk_ldg_f32_off(scales, (soff + t * 32) * 4);
+        }
+    };
+    auto compute_rows = [&](const Row &A, const Row &Bq, int r0, int r1) {
+        float acc0[BATCH], acc1[BATCH];
+#pragma unroll
+        for (int b = 0; b < BATCH; b++) acc0[b] = acc1[b] = 0.0f;
+        // (t, b) steps with the next step's LDS operands requested one step ahead
+        // the activation does not change from row to row: without an opaque index the compiler keeps all of it in
+        // registers (408 at batch 8) instead of reading LDS
+        int z = lane;
+        asm volatile("" : "+v"(z));
+        mk_i4 xv = xl[z];
+        float cf = xsl[z >> 1];
+#pragma unroll
+        for (int i = 0; i < T * BATCH; i++) {
+            const int t = i / BATCH, b = i % BATCH;
+            const int tn = (i + 1) / BATCH, bn = (i + 1) % BATCH;
+            mk_i4 xn = xv;
+            float cn = cf;
+            if (i + 1 < T * BATCH) {
+                xn = xl[bn * NB * 2 + tn * 64 + z];
+                cn = xsl[bn * NB + ((tn * 64 + z) >> 1)];
+            }
+            int d0 = 0, d1 = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                d0 = __builtin_amdgcn_sdot4(A.w[t][k], xv[k], d0, false);
+                d1 = __builtin_amdgcn_sdot4(Bq.w[t][k], xv[k], d1, false);
+            }
+            acc0[b] += (A.s[t] * cf) * (float)d0;
+            acc1[b] += (Bq.s[t] * cf) * (float)d1;
+            xv = xn;
+            cf = cn;
+            // the index of the following reads is made to depend on this step's dots: one step of operands in flight
+            asm volatile("" : "+v"(z) : "v"(d0), "v"(d1));
+        }
+#pragma unroll
+        for (int b = 0; b < BATCH; b++) {
+            const float v0 = mk_wave_sum(acc0[b]), v1 = mk_wave_sum(acc1[b]);
+            if (lane == 0) {
+                if (r0 < rows) out[(size_t)b * rows + r0] = v0;
+                if (r1 < rows) out[(size_t)b * rows + r1] = v1;
+            }
+        }
+    };
+    Row a0, a1, b0, b1;
+    load_row(a0, wave);
+    load_row(a1, wave + n_waves);
+    __syncthreads();
+    for (int r = wave; r < rows; r += 4 * n_waves) {
+        load_row(b0, r + 2 * n_waves);
+        load_row(b1, r + 3 * n_waves);
+        compute_rows(a0, a1, r, r + n_waves);
+        load_row(a0, r + 4 * n_waves);
+        load_row(a1, r + 5 * n_waves);
+        if (r + 2 * n_waves < rows) compute_rows(b0, b1, r + 2 * n_waves, r + 3 * n_waves);
     }
 }
 
@@ -306,10 +403,34 @@ void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, 
     hipLaunchKernelGGL((q8_gemv_b1_kernel<NB, F16>), dim3(blocks), dim3(256), 0, st, q, scales, rows, xq, xs, out);
 }
 
+template <bool F16, int BATCH>
+void launch_bn(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
+    constexpr int NB = 224;
+    int blocks = tune("MK_Q8_BN_BLOCKS", 512);
+    if (blocks * 4 > rows) blocks = (rows + 3) / 4;
+    const size_t lds = (size_t)BATCH * NB * 36;
+    static bool opted = false;
+    if (!opted) {
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_bn_kernel<NB, F16, BATCH>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+        opted = true;
+    }
+    hipLaunchKernelGGL((q8_gemv_bn_kernel<NB, F16, BATCH>), dim3(blocks), dim3(256), lds, st, q, scales, rows, xq, xs, out);
+}
+
 template <bool F16>
 int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, const int8_t *xq, const float *xs, size_t batch, float *out,
               hipStream_t st) {
     const int nb = (int)(cols / 32);
+    // measured on the 163840 x 7168 head: streaming kernel 188 / 198 / 201 us at batch 2 / 3 / 4 against 215-222 us for the
+    // matrix-core kernel; from batch 5 its vector work per row costs more than the matrix-core kernel's 64-byte runs
+    if (batch >= 2 && batch <= 4 && nb == 224 && rows * cols < 0xFFFFFFFFull && !tune("MK_Q8_NO_BN", 0)) {
+        switch (batch) {
+            case 2: launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st); break;
+            case 3: launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st); break;
+            default: launch_bn<F16, 4>(q, scales, (int)rows, xq, xs, out, st); break;
+        }
+        return mk_launch_status("q8_gemv_bn");
+    }
     if (batch == 1 && rows * cols < 0xFFFFFFFFull) {  // the batch-1 kernel addresses the matrix with 32-bit byte offsets
         switch (nb) {
             case 32: launch_b1<32, F16>(q, scales, (int)rows, xq, xs, out, st); return mk_launch_status("q8_gemv_b1");

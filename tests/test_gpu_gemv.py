@@ -109,7 +109,10 @@ def test_matvec_packed_nt(rows, cols, m):
 
 @pytest.mark.parametrize("rows,cols,batch,f16", [(512, 1024, 1, True), (512, 1024, 8, True), (512, 1024, 3, False), (100, 7168, 1, True),
                                                   (100, 7168, 8, True), (37, 96, 2, True), (37, 96, 1, False), (64, 2048, 5, True),
-                                                  (1000, 4096, 1, False)])
+                                                  (1000, 4096, 1, False),
+                                                  # streaming batch kernel (7168 columns, batch 2-4): ragged row counts
+                                                  (4099, 7168, 2, True), (2050, 7168, 3, False), (3, 7168, 4, True),
+                                                  (5000, 7168, 4, True)])
 def test_q8head_shapes(rows, cols, batch, f16):
     torch = torch_cuda()
     from microkimi_amd import model
