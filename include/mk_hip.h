@@ -257,6 +257,59 @@ size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, s
 int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                        const float *x, int act_kind, void *workspace, float *out, void *stream);
 
+/* ------------------------------------------- MKIM weight files -> device */
+
+/* Tensor dtypes of the file format (src/weights.rs:25-29). */
+#define MK_DTYPE_F32 0
+#define MK_DTYPE_MXFP4 1
+#define MK_DTYPE_I32 2
+#define MK_DTYPE_VQ1 3
+#define MK_DTYPE_MXFP4SQ 4
+#define MK_BIN_MAX_DIMS 8
+
+/* weights::Entry (src/weights.rs:31-37): one directory entry. */
+typedef struct mk_bin_entry {
+    uint8_t dtype, n_dims;
+    uint32_t dims[MK_BIN_MAX_DIMS];
+    uint64_t offset, size; /* bytes from the start of the file */
+} mk_bin_entry;
+
+typedef struct mk_binfile mk_binfile;
+
+/* BinFile::open / read_directory (src/weights.rs:424-500): parses "MKIM0001" or "MKIM0002"
+ * (+ JSON config block) and the tensor directory, and maps the whole file read-only.  Every
+ * entry is checked against blob_size (src/weights.rs:40-66) and the file length; a malformed
+ * file gives MK_ERR_INVALID where the reference panics.  No GPU is touched. */
+int mk_bin_open(const char *path, mk_binfile **out);
+void mk_bin_close(mk_binfile *f);
+size_t mk_bin_n_tensors(const mk_binfile *f);
+/* Entry i in directory order; `name` points into the handle. */
+int mk_bin_entry_at(const mk_binfile *f, size_t i, const char **name, mk_bin_entry *e);
+/* entries.get(name) (src/weights.rs:601): MK_ERR_INVALID "missing tensor" when absent. */
+int mk_bin_find(const mk_binfile *f, const char *name, mk_bin_entry *e);
+/* BinFile::blob: pointer to the tensor's bytes inside the mapping (valid until mk_bin_close), or NULL. */
+const void *mk_bin_blob(const mk_binfile *f, const char *name, size_t *size);
+/* The MKIM0002 config block (not NUL-terminated inside the file; the returned copy is), or NULL for MKIM0001. */
+const char *mk_bin_config_json(const mk_binfile *f, size_t *len);
+/* BinFile::mxfp4_parts (src/weights.rs:619-627): packed [R][C/2] then scales [R][C/32] of one blob. */
+int mk_bin_mxfp4_parts(const mk_binfile *f, const char *name, const uint8_t **packed, const uint8_t **scales, size_t *rows, size_t *cols);
+
+typedef struct mk_expert_set mk_expert_set;
+
+/* The routed experts of one MoE layer made resident on the current device: the tensors
+ * "<layer_prefix>block_sparse_moe.experts.<e>.w1|w2|w3" for e < n_experts (the names resolved in
+ * src/model.rs:979-989), each MXFP4 blob copied as stored (256-byte aligned; scales = packed +
+ * R*C/2), plus the device pointer arrays of an mk_expert_table.  w1 of expert 0 fixes
+ * [inter, d]; every other tensor is checked against it.  Experts of another dtype (VQ1,
+ * MXFP4SQ) give MK_ERR_UNSUPPORTED: such a layer stays on the caller's CPU path, as dtype 3/4
+ * blobs do for the reference's GPU entry points.  This replaces the pointer-keyed upload cache
+ * of src/metal.rs:874-936 for callers that load whole layers. */
+int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix, size_t n_experts, mk_expert_set **out);
+const mk_expert_table *mk_expert_set_table(const mk_expert_set *s);
+size_t mk_expert_set_count(const mk_expert_set *s);
+size_t mk_expert_set_bytes(const mk_expert_set *s); /* device bytes held */
+void mk_expert_set_free(mk_expert_set *s);
+
 /* ------------------------------------------------------------ host level */
 
 /* metal::gpu_matvec_fp4 (src/metal.rs:943-1017), i.e. the GPU branch of

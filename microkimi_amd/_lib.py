@@ -20,6 +20,10 @@ class MkError(RuntimeError):
         self.status = status
 
 
+class BinEntry(C.Structure):
+    _fields_ = [("dtype", C.c_uint8), ("n_dims", C.c_uint8), ("dims", C.c_uint32 * 8), ("offset", C.c_uint64), ("size", C.c_uint64)]
+
+
 class ExpertTable(C.Structure):
     _fields_ = [("w1p", C.c_void_p), ("w1s", C.c_void_p), ("w3p", C.c_void_p), ("w3s", C.c_void_p), ("w2p", C.c_void_p),
                 ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t)]
@@ -80,6 +84,19 @@ def _load():
         "mk_mla_cache_to_f32": (i32, [vp, vp, vp]),
         "mk_mla_attn": (i32, [vp, vp, f32, vp]),
         "mk_mla_cache_free": (None, [vp]),
+        "mk_bin_open": (i32, [C.c_char_p, C.POINTER(vp)]),
+        "mk_bin_close": (None, [vp]),
+        "mk_bin_n_tensors": (sz, [vp]),
+        "mk_bin_entry_at": (i32, [vp, sz, C.POINTER(C.c_char_p), C.POINTER(BinEntry)]),
+        "mk_bin_find": (i32, [vp, C.c_char_p, C.POINTER(BinEntry)]),
+        "mk_bin_blob": (vp, [vp, C.c_char_p, C.POINTER(sz)]),
+        "mk_bin_config_json": (vp, [vp, C.POINTER(sz)]),
+        "mk_bin_mxfp4_parts": (i32, [vp, C.c_char_p, C.POINTER(vp), C.POINTER(vp), C.POINTER(sz), C.POINTER(sz)]),
+        "mk_bin_load_experts": (i32, [vp, C.c_char_p, sz, C.POINTER(vp)]),
+        "mk_expert_set_table": (C.POINTER(ExpertTable), [vp]),
+        "mk_expert_set_count": (sz, [vp]),
+        "mk_expert_set_bytes": (sz, [vp]),
+        "mk_expert_set_free": (None, [vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)  # AttributeError here = the library does not export a declared symbol

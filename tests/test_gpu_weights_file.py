@@ -1,0 +1,82 @@
+"""GPU: experts loaded from an MKIM file (mk_bin_load_experts) drive the MoE kernels like tables built from tensors."""
+import numpy as np
+import pytest
+
+import mkim_writer as W
+import oracle
+from gpu_util import dev, rel_l2, torch_cuda
+
+pytestmark = pytest.mark.gpu
+
+
+def make_file(path, n_experts, d, inter, bad_dtype_at=None, bad_shape_at=None):
+    from microkimi_amd import workloads
+    rng = np.random.default_rng(7)
+    tensors = [("model.embed_tokens.weight", W.F32, (16, d), rng.standard_normal((16, d)).astype(np.float32))]
+    host = []
+    for e in range(n_experts):
+        w1 = workloads.mxfp4_matrix(2, "w1", inter, d, e)
+        w3 = workloads.mxfp4_matrix(2, "w3", inter, d, e)
+        w2 = workloads.mxfp4_matrix(2, "w2", d, inter, e)
+        host.append((w1, w3, w2))
+        for k, m, dims in (("w1", w1, (inter, d)), ("w2", w2, (d, inter)), ("w3", w3, (inter, d))):   # file order of the reference
+            name = f"model.layers.2.block_sparse_moe.experts.{e}.{k}"
+            if bad_dtype_at == (e, k):
+                tensors.append((name, W.VQ1, dims, bytes(dims[0] * dims[1] // 16)))
+            elif bad_shape_at == (e, k):
+                tensors.append((name, W.MXFP4, (dims[0], dims[1] // 2), (m[0][:, : dims[1] // 4], m[1][:, : dims[1] // 64])))
+            else:
+                tensors.append((name, W.MXFP4, dims, m))
+        tensors.append((f"model.layers.2.note.{e}", W.I32, (3,), np.array([e, 1, 2], np.int32)))   # unaligned filler between experts
+    W.write(path, tensors, config={"d_model": d})
+    return host
+
+
+def test_loaded_experts_match_tables_built_from_tensors(tmp_path):
+    torch = torch_cuda()
+    from microkimi_amd import model, weights
+    n, d, inter, B, topk = 6, 1024, 512, 5, 2
+    host = make_file(tmp_path / "m.bin", n, d, inter)
+    f = weights.BinFile.open(tmp_path / "m.bin")
+    ex = f.load_experts("model.layers.2.", n)
+    assert (ex.n, ex.d, ex.inter) == (n, d, inter)
+    assert ex.bytes >= sum(m[0].size + m[1].size for h in host for m in h)
+    todev = lambda lst: [(dev(p), dev(s)) for p, s in lst]
+    ref = model.PackedExperts(todev([h[0] for h in host]), todev([h[1] for h in host]), todev([h[2] for h in host]), d, inter)
+    rng = np.random.default_rng(3)
+    ids = np.stack([rng.permutation(n - 1)[:topk] for _ in range(B)]).astype(np.int32)
+    wts = rng.random((B, topk)).astype(np.float32)
+    x = (rng.standard_normal((B, d)) * 0.05).astype(np.float32)
+    got = model.moe_decode(ex, dev(ids), dev(wts), dev(x), shared=n - 1).cpu().numpy()
+    same = model.moe_decode(ref, dev(ids), dev(wts), dev(x), shared=n - 1).cpu().numpy()
+    assert np.array_equal(got, same)   # same kernels, same bytes: identical
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=n - 1, mode=1, threads=8)
+    assert rel_l2(got, want) <= 1e-5
+    # the prefill path reads the same table
+    T = 24
+    idp = np.stack([rng.permutation(n)[:topk] for _ in range(T)]).astype(np.int32)
+    wp = rng.random((T, topk)).astype(np.float32)
+    xp = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    a = model.moe_prefill(ex, dev(idp), dev(wp), dev(xp)).cpu().numpy()
+    b = model.moe_prefill(ref, dev(idp), dev(wp), dev(xp)).cpu().numpy()
+    assert np.array_equal(a, b)
+    ex.close()
+    f.close()
+
+
+def test_unsupported_dtype_and_shape_mismatch(tmp_path):
+    torch_cuda()
+    from microkimi_amd import weights
+    from microkimi_amd._lib import MkError
+    make_file(tmp_path / "vq.bin", 3, 256, 128, bad_dtype_at=(1, "w3"))
+    with pytest.raises(MkError) as e:
+        weights.BinFile.open(tmp_path / "vq.bin").load_experts("model.layers.2.", 3)
+    assert e.value.status == -4 and "dtype 3" in str(e.value)
+    make_file(tmp_path / "shape.bin", 3, 256, 128, bad_shape_at=(2, "w2"))
+    with pytest.raises(MkError) as e:
+        weights.BinFile.open(tmp_path / "shape.bin").load_experts("model.layers.2.", 3)
+    assert e.value.status == -1 and "expected [256, 128]" in str(e.value)
+    with pytest.raises(MkError) as e:
+        weights.BinFile.open(tmp_path / "shape.bin").load_experts("model.layers.9.", 3)
+    assert "missing tensor" in str(e.value)
