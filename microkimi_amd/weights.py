@@ -4,7 +4,7 @@
     f.entries[name]                   # Entry(dtype, dims, offset, size)
     f.config                          # dict from the MKIM0002 JSON block, None for MKIM0001
     f.blob(name) / f.f32_vec(name) / f.i32_vec(name) / f.mxfp4_parts(name)
-    experts = f.load_experts("model.layers.3.", n_experts)    # one layer's routed experts, resident on the device
+    experts = f.load_experts("layers.3.", n_experts)    # one layer's routed experts, resident on the device
 
 `load_experts` returns an object that model.moe_decode / model.moe_prefill accept in place of PackedExperts.
 """

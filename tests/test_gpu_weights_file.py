@@ -20,14 +20,14 @@ def make_file(path, n_experts, d, inter, bad_dtype_at=None, bad_shape_at=None):
         w2 = workloads.mxfp4_matrix(2, "w2", d, inter, e)
         host.append((w1, w3, w2))
         for k, m, dims in (("w1", w1, (inter, d)), ("w2", w2, (d, inter)), ("w3", w3, (inter, d))):   # file order of the reference
-            name = f"model.layers.2.block_sparse_moe.experts.{e}.{k}"
+            name = f"layers.2.block_sparse_moe.experts.{e}.{k}"
             if bad_dtype_at == (e, k):
                 tensors.append((name, W.VQ1, dims, bytes(dims[0] * dims[1] // 16)))
             elif bad_shape_at == (e, k):
                 tensors.append((name, W.MXFP4, (dims[0], dims[1] // 2), (m[0][:, : dims[1] // 4], m[1][:, : dims[1] // 64])))
             else:
                 tensors.append((name, W.MXFP4, dims, m))
-        tensors.append((f"model.layers.2.note.{e}", W.I32, (3,), np.array([e, 1, 2], np.int32)))   # unaligned filler between experts
+        tensors.append((f"layers.2.note.{e}", W.I32, (3,), np.array([e, 1, 2], np.int32)))   # unaligned filler between experts
     W.write(path, tensors, config={"d_model": d})
     return host
 
@@ -38,7 +38,7 @@ def test_loaded_experts_match_tables_built_from_tensors(tmp_path):
     n, d, inter, B, topk = 6, 1024, 512, 5, 2
     host = make_file(tmp_path / "m.bin", n, d, inter)
     f = weights.BinFile.open(tmp_path / "m.bin")
-    ex = f.load_experts("model.layers.2.", n)
+    ex = f.load_experts("layers.2.", n)
     assert (ex.n, ex.d, ex.inter) == (n, d, inter)
     assert ex.bytes >= sum(m[0].size + m[1].size for h in host for m in h)
     todev = lambda lst: [(dev(p), dev(s)) for p, s in lst]
@@ -71,12 +71,12 @@ def test_unsupported_dtype_and_shape_mismatch(tmp_path):
     from microkimi_amd._lib import MkError
     make_file(tmp_path / "vq.bin", 3, 256, 128, bad_dtype_at=(1, "w3"))
     with pytest.raises(MkError) as e:
-        weights.BinFile.open(tmp_path / "vq.bin").load_experts("model.layers.2.", 3)
+        weights.BinFile.open(tmp_path / "vq.bin").load_experts("layers.2.", 3)
     assert e.value.status == -4 and "dtype 3" in str(e.value)
     make_file(tmp_path / "shape.bin", 3, 256, 128, bad_shape_at=(2, "w2"))
     with pytest.raises(MkError) as e:
-        weights.BinFile.open(tmp_path / "shape.bin").load_experts("model.layers.2.", 3)
+        weights.BinFile.open(tmp_path / "shape.bin").load_experts("layers.2.", 3)
     assert e.value.status == -1 and "expected [256, 128]" in str(e.value)
     with pytest.raises(MkError) as e:
-        weights.BinFile.open(tmp_path / "shape.bin").load_experts("model.layers.9.", 3)
+        weights.BinFile.open(tmp_path / "shape.bin").load_experts("layers.9.", 3)
     assert "missing tensor" in str(e.value)

@@ -13,7 +13,7 @@ import mkim_writer as W
 from microkimi_amd import weights
 from microkimi_amd._lib import MkError
 
-EXP = "model.layers.0.block_sparse_moe.experts.0.w1"
+EXP = "layers.0.block_sparse_moe.experts.0.w1"
 
 
 def hand_made(tmp_path):
@@ -55,9 +55,9 @@ def test_writer_layout_and_config(tmp_path):
                ("ids", W.I32, (5,), np.arange(5, dtype=np.int32) - 2)]
     for e in range(2):
         for k, (r, c) in (("w1", (32, 64)), ("w2", (64, 32)), ("w3", (32, 64))):
-            tensors.append((f"model.layers.1.block_sparse_moe.experts.{e}.{k}", W.MXFP4, (r, c),
+            tensors.append((f"layers.1.block_sparse_moe.experts.{e}.{k}", W.MXFP4, (r, c),
                             (rng.integers(0, 256, (r, c // 2), dtype=np.uint8), rng.integers(118, 131, (r, c // 32), dtype=np.uint8))))
-    tensors.append(("model.layers.1.block_sparse_moe.gate.weight", W.F32, (2, 64), rng.standard_normal((2, 64)).astype(np.float32)))
+    tensors.append(("layers.1.block_sparse_moe.gate.weight", W.F32, (2, 64), rng.standard_normal((2, 64)).astype(np.float32)))
     p = tmp_path / "v2.bin"
     offs = W.write(p, tensors, config=cfg)
     f = weights.BinFile.open(p)
