@@ -225,6 +225,29 @@ def bench_mxfp4_gemv(torch):
             "f32_back_to_back": {"ms": f_ms, "gbs": gbs(f_ms), "frac": gbs(f_ms) / HBM_PEAK_GBS}}
 
 
+def bench_vq1(torch):
+    """VQ1 / LUT GEMV (quant::matvec_vq) on an expert-sized matrix: 2048 x 7168 = 917 504 index bytes + the 16 KiB
+    codebook; 16 distinct matrices per timed pass.  Far too small to be HBM-bound: the line reports time per matvec."""
+    from microkimi_amd import workloads as W
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    rows, cols, nmat = 2048, W.D_MODEL, 16
+    g = torch.Generator(device="cuda").manual_seed(6)
+    cb = torch.randn((256, 16), device="cuda", generator=g) * 0.05
+    idx = [torch.randint(0, 256, (rows, cols // 16), dtype=torch.uint8, device="cuda", generator=g) for _ in range(nmat)]
+    x = torch.randn(cols, device="cuda", generator=g)
+    out = torch.empty(rows, device="cuda")
+    ws = torch.empty(lib.mk_vq1_workspace_bytes(cols), dtype=torch.uint8, device="cuda")
+    res = {"workload": "VQ1 2048x7168 (one index byte per 16 weights, 256x16 f32 codebook), batch 1", "index_bytes": rows * cols // 16}
+    for name, exact in (("fast", 0), ("exact", 1)):
+        calls = [(lambda i=i, exact=exact: check(lib.mk_dev_vq1_matvec(ptr(cb), ptr(idx[i]), rows, cols, ptr(x), exact, ptr(ws), ptr(out),
+                                                                        cur_stream()))) for i in range(nmat)]
+        ms = time_graph(torch, calls)
+        loop_ms = time_region(torch, lambda: [c() for c in calls], 5) / nmat
+        res[name] = {"us_per_matvec": (ms if ms is not None else loop_ms) * 1e3, "us_python_loop": loop_ms * 1e3,
+                     "timing": "graph replay (table + sweep kernels)" if ms is not None else "python loop"}
+    return res
+
+
 def bench_moe(torch):
     """Configuration 2: 256 routed + 1 shared MXFP4 experts (6.0 GB resident), softmax top-8 router, B in {1, 4, 16}."""
     from microkimi_amd import model, workloads as W
@@ -245,12 +268,23 @@ def bench_moe(torch):
         out = torch.empty((B, d), device="cuda")
         n_distinct = len(set(ids.cpu().numpy().reshape(-1).tolist())) + 1
         alg = n_distinct * per_expert + B * 2 * d * 4
+        # A decode step meets different experts in every layer: the timed calls rotate through 16 routings (the seeded
+        # one and 15 shifted copies of it, each with another expert in the shared role), 3.4 GB at B = 1, so that
+        # repeats are not served by the 256 MB Infinity Cache.
+        routes = []
+        for k in range(16):
+            ids_k = ((ids + 16 * k) % ne).to(torch.int32).contiguous()
+            used = set(ids_k.cpu().numpy().reshape(-1).tolist())
+            shared_k = ne if k == 0 else next(e for e in range((7 * k) % ne, ne) if e not in used)
+            routes.append((ids_k, shared_k))
+        calls = [(lambda r=r: model.moe_decode(experts, r[0], wts, x, shared=r[1], out=out)) for r in routes]
 
         def step():
-            model.moe_decode(experts, ids, wts, x, shared=ne, out=out)
+            for c in calls:
+                c()
 
-        ms_eager = time_region(torch, step, 30, warmup=5)
-        ms_graph = time_graph(torch, [step] * 8)
+        ms_eager = time_region(torch, step, 4, warmup=1) / len(calls)
+        ms_graph = time_graph(torch, calls)
         ms = ms_graph if ms_graph is not None else ms_eager
         res[f"B{B}"] = {"ms": ms, "ms_python_loop": ms_eager, "timing": "graph replay" if ms_graph is not None else "python loop",
                         "tok_s": B / (ms * 1e-3), "distinct_experts": n_distinct, "pairs": B * (W.TOP_K + 1), "alg_bytes": alg,
@@ -411,7 +445,7 @@ def main():
     torch.cuda.empty_cache()
     extras = {"lm_head_batch8": head.pop("batch8")}
     if not args.no_extras:
-        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("grouped_gemm", bench_gemm)):
+        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("grouped_gemm", bench_gemm), ("vq1_gemv", bench_vq1)):
             log(name, "...")
             try:
                 extras[name] = fn(torch)

@@ -257,6 +257,21 @@ size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, s
 int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                        const float *x, int act_kind, void *workspace, float *out, void *stream);
 
+/* ---------------------------------------- device level: VQ1 / LUT GEMV */
+
+/* Bytes of device scratch for the lookup tables of one activation: cols/16 tables of 256 f32. */
+size_t mk_vq1_workspace_bytes(size_t cols);
+
+/* quant::matvec_vq (src/quant.rs:333-346), i.e. lutgemv::matvec_vq_lut (src/lutgemv.rs:208-240):
+ * out[r] = sum_c W[r][c] x[c] with W[r][16v .. 16v+16] = codebook[indices[r][v]].
+ * codebook [256][16] f32 (the file's global "vq_codebook"), indices [rows][cols/16] u8, x [cols], out [rows].
+ * Table entries are bit-identical to the reference's (sequential multiply-add chain).  exact != 0: each row adds its
+ * table entries in ascending group order from 0 like the reference's sweep, and the result is bit-identical to
+ * matvec_vq_lut / matvec_vq_gather; exact == 0: the sum over groups is split across the 64 lanes of a wave
+ * (relative L2 error against the reference below 1e-5).  The batched matvec_vq_nt is not built. */
+int mk_dev_vq1_matvec(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *x, int exact,
+                      void *workspace, float *out, void *stream);
+
 /* ------------------------------------------- MKIM weight files -> device */
 
 /* Tensor dtypes of the file format (src/weights.rs:25-29). */

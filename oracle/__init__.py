@@ -232,6 +232,17 @@ def matvec_f32(w, rows, cols, x):
     return out
 
 
+# ------------------------------------------------------- VQ1 / LUT GEMV
+def vq1_matvec(codebook, indices, rows, cols, x, lut=True):
+    """quant::matvec_vq_gather (lut=False, src/quant.rs:313-331) or lutgemv::matvec_vq_lut (src/lutgemv.rs:208-240)."""
+    codebook, indices, x = _c(codebook, np.float32), _c(indices, np.uint8), _c(x, np.float32)
+    assert codebook.size == 256 * 16 and cols % 16 == 0 and indices.size == rows * cols // 16 and x.size == cols
+    out = np.empty(rows, np.float32)
+    fn = _lib.orc_vq1_matvec_lut if lut else _lib.orc_vq1_matvec_gather
+    fn(_p(codebook, _f32p), _p(indices, _u8p), rows, cols, _p(x, _f32p), _p(out, _f32p))
+    return out
+
+
 # ---------------------------------------------------------- mxfp4 matvecs
 def _chk_packed(packed, scales, rows, cols):
     packed, scales = _c(packed, np.uint8), _c(scales, np.uint8)

@@ -387,6 +387,54 @@ ORC_API void orc_rmsnorm(const float *x, size_t n, const float *w, float eps, fl
     for (size_t i = 0; i < n; i++) out[i] = x[i] * inv * w[i];
 }
 
+/* ------------------------------------------------ VQ1 matvec / LUT GEMV */
+
+/* src/quant.rs:313-331 (matvec_vq_gather): codebook [256][16] f32, one index byte per vector of 16 consecutive
+ * row-major weights; per row the 16-wide dots in order, each accumulated from 0 in ascending j, summed in ascending
+ * vector order */
+ORC_API void orc_vq1_matvec_gather(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *x, float *out) {
+    const size_t vpr = cols / 16;
+    for (size_t r = 0; r < rows; r++) {
+        const uint8_t *irow = indices + r * vpr;
+        float sum = 0.0f;
+        for (size_t v = 0; v < vpr; v++) {
+            const float *cb = codebook + (size_t)irow[v] * 16, *xs = x + v * 16;
+            float s = 0.0f;
+            for (int j = 0; j < 16; j++) s += cb[j] * xs[j];
+            sum += s;
+        }
+        out[r] = sum;
+    }
+}
+
+/* src/lutgemv.rs:208-240 (matvec_vq_lut) with build_vq_lut_scalar (:175-185) and sweep (:67-98): tables of 256
+ * entry-activation dots per 16-wide group, built and swept 16 groups at a time, rows inner; additions only in the sweep */
+ORC_API void orc_vq1_matvec_lut(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *x, float *out) {
+    enum { TILE = 16 };
+    const size_t vpr = cols / 16;
+    float *lut = (float *)malloc(sizeof(float) * TILE * 256);
+    for (size_t r = 0; r < rows; r++) out[r] = 0.0f;
+    for (size_t g0 = 0; g0 < vpr; g0 += TILE) {
+        const size_t groups = vpr - g0 < TILE ? vpr - g0 : TILE;
+        for (size_t g = 0; g < groups; g++) {
+            const float *xs = x + (g0 + g) * 16;
+            for (int k = 0; k < 256; k++) {
+                const float *cb = codebook + (size_t)k * 16;
+                float s = 0.0f;
+                for (int j = 0; j < 16; j++) s += cb[j] * xs[j];
+                lut[g * 256 + k] = s;
+            }
+        }
+        for (size_t r = 0; r < rows; r++) {
+            float a = out[r];
+            const uint8_t *ir = indices + r * vpr;
+            for (size_t g = 0; g < groups; g++) a += lut[g * 256 + ir[g0 + g]];
+            out[r] = a;
+        }
+    }
+    free(lut);
+}
+
 /* ------------------------------------------------------- mxfp4 matvecs */
 
 /* src/mxfp4.rs:409-418: one row of the q8-integer path */
