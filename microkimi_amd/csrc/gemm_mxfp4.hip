@@ -126,25 +126,41 @@ struct GemmArgs {
     float *out;
 };
 
-template <int MC>
+// FULL: the weight loads take whole 128-byte lines (see below); measured on 8 experts x 512 tokens 495 -> 400 us, on
+// the prefill shape (at most 32 tokens per expert) 488 -> 504 us, so only the large-group kernel uses it.
+template <int MC, bool FULL>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, int base, int tok1, uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
     const int row0 = blockIdx.x * 256 + wave * 64;
     // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
-    uint32_t woff[4], soff[4];
+    // FULL: weight loads take whole 128-byte lines: load j = 2i + h of a unit covers line i (of the K tile's two) of the
+    // rows 8h .. 8h+7 of the row tile, lane (r3 = lane / 8, c = lane % 8) reading bytes 16c .. of row 8h + r3, and the
+    // operand form is restored in registers (compute_unit).  Otherwise the operand's own mapping: load s covers 64 bytes
+    // of all 16 rows, lane (kb, n) reading bytes 16 kb .. of row n (every line is then requested by two loads).
+    static_assert(KT_STEPS == 4, "two lines of 128 bytes per row and K tile");
+    const int r3 = lane >> 3, c8 = lane & 7;
+    uint32_t woff[4][FULL ? 2 : 1], soff[4];
 #pragma unroll
     for (int rt = 0; rt < 4; rt++) {
-        const int r = min(row0 + rt * 16 + n, a.rows - 1);
-        woff[rt] = (uint32_t)r * (uint32_t)(cols / 2) + kb * 16;
-        soff[rt] = (uint32_t)r * (uint32_t)nb;
+        if constexpr (FULL) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(row0 + rt * 16 + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
+        } else {
+            woff[rt][0] = (uint32_t)min(row0 + rt * 16 + n, a.rows - 1) * (uint32_t)(cols / 2) + kb * 16;
+        }
+        soff[rt] = (uint32_t)min(row0 + rt * 16 + n, a.rows - 1) * (uint32_t)nb;
     }
+    // after the lane rotation below, lane (kg, x, r3) holds what lane (r3, x, kg) loaded
+    const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
     mk_i4 wa[KT_STEPS], wb[KT_STEPS], sa, sb;
     auto load_unit = [&](mk_i4 *w, mk_i4 &sc, int kt, int rt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
 #pragma unroll
-        for (int s = 0; s < KT_STEPS; s++) w[s] = mk_ldg128_off(packed, woff[rt] + ku * (KT_STEPS * 64) + s * 64);
+        for (int j = 0; j < KT_STEPS; j++)
+            w[j] = FULL ? mk_ldg128_off(packed, woff[rt][FULL ? (j & 1) : 0] + ku * (KT_STEPS * 64) + (j >> 1) * 128)
+                        : mk_ldg128_off(packed, woff[rt][0] + ku * (KT_STEPS * 64) + j * 64);
         sc = mk_ldg128_off(scales, soff[rt] + ku * 16);
     };
     // activation tile staging: chunk i = tid + 256 k -> token i / 32, 16-byte chunk i % 32
@@ -176,9 +192,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
         for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // One unit: 4 steps x MC token tiles.  The LDS reads of the activation operands do not depend on the
-    // row tile, so after inlining the four calls of a K tile share them.
-    auto compute_unit = [&](const mk_i4 *w, const mk_i4 &sc, int rt, const uint8_t *buf) {
+    auto mma_unit = [&](const mk_i4 *w, const mk_i4 &sc, int rt, const uint8_t *buf) {
 #pragma unroll
         for (int c = 0; c < MC; c++) {
             const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC) + (c * 16 + n) * 16);
@@ -194,6 +208,29 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*A: fp8 e4m3*/, 4 /*B: fp4 e2m1*/, 0, asb, 0, wsb);
             }
         }
+    };
+    // One unit: 4 steps x MC token tiles.  The LDS reads of the activation operands do not depend on the
+    // row tile, so after inlining the four calls of a K tile share them.
+    auto compute_unit = [&](const mk_i4 *wl, const mk_i4 &sc, int rt, const uint8_t *buf) {
+        if constexpr (!FULL) {
+            mma_unit(wl, sc, rt, buf);
+            return;
+        }
+        // Loaded: for line i, wl[2i] = rows 0-7 and wl[2i+1] = rows 8-15, lane (r3, s', kg) holding the 16 bytes of K
+        // group kg of step 2i + s'.  Wanted: step s in w[s], lane (kg, row).  A rotation of the lane index by three
+        // bits (ds_bpermute) brings (kg, s', r3); then the two registers exchange their 8-lane halves inside every
+        // 16-lane row (DPP row rotate by 8 with a bank mask), which trades the lane bit s' for the row-half bit.
+        mk_i4 w[KT_STEPS];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int ra = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * i][k]), rb = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * i + 1][k]);
+                w[2 * i][k] = __builtin_amdgcn_update_dpp(ra, rb, 0x128 /* row_ror:8 */, 0xF, 0xC, false);      // lanes 8-15 of a row <- rb
+                w[2 * i + 1][k] = __builtin_amdgcn_update_dpp(rb, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);  // lanes 0-7 of a row <- ra
+            }
+        }
+        mma_unit(w, sc, rt, buf);
     };
 
     load_unit(wa, sa, 0, 0);
@@ -244,11 +281,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[e]);
     if (MC == 2) {
-        if (count <= 16) gemm_pass<1>(a, packed, scales, tok0, tok1, lds);
-        else gemm_pass<2>(a, packed, scales, tok0, tok1, lds);
+        if (count <= 16) gemm_pass<1, false>(a, packed, scales, tok0, tok1, lds);
+        else gemm_pass<2, false>(a, packed, scales, tok0, tok1, lds);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC>(a, packed, scales, base, tok1, lds);
+        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true>(a, packed, scales, base, tok1, lds);
     }
 }
 
