@@ -9,7 +9,8 @@
 //           registers for the whole kernel; 4 x v_dot4_i32_i8 per load.
 // batch 2-4 at 7168 columns: the batch-1 streaming pattern with the activation in
 //           LDS and two rows per LDS read (see q8_gemv_bn_kernel).
-// batch 2-8 matrix-core path.  One v_mfma_i32_16x16x64_i8 per 16 rows x 64
+// batch 2-8 matrix-core path (batch 5-8 at 7168 columns, 2-8 elsewhere; 219 -> 203 us at batch 8 since the loads take
+//           whole lines).  One v_mfma_i32_16x16x64_i8 per 16 rows x 64
 //           columns.  The MFMA sums over K = 64 = two q8 blocks, whose scales
 //           differ, so the activation operand is laid out as 16 "columns" =
 //           8 batch rows x 2 block parities, each holding the activation bytes of
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void q8_gemv_bn_kernel(const int8_t *__rest
 // they are fetched with seven fully coalesced 1 KiB loads, one group ahead,
 // and read back from LDS per step -- scattered 2-byte global loads per step cost
 // a cache line each and halved the bandwidth.
-template <bool F16, int WAVES>
+template <bool F16, int WAVES, bool FULL>
 __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *__restrict__ q, const void *__restrict__ scales, int rows,
                                                                   int nb, const int8_t *__restrict__ xq, const float *__restrict__ xs,
                                                                   int batch, float *__restrict__ out) {
@@ -253,17 +254,46 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
         const int row = grp * 16 + n;
         const bool row_ok = row < rows;
         const int8_t *wrow = q + (size_t)(row_ok ? row : 0) * cols + kb * 16;
+        // FULL (cols % 128 == 0): a load takes whole 128-byte lines, 8 rows x 128 bytes (lane (r3 = lane / 8, c = lane % 8)
+        // reads bytes 16c .. of row 8h + r3; loads 2i and 2i + 1 of a block cover line i of rows 0-7 and 8-15), and the
+        // operand form (16 rows x 64 bytes per step, lane (kb, n)) is restored in registers: a rotation of the lane
+        // index by three bits, then the two registers exchange the 8-lane halves of every 16-lane row.  With the
+        // operand's own mapping every line is requested by two loads.
+        const int8_t *wline[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++) wline[h] = q + (size_t)min(grp * 16 + 8 * h + (lane >> 3), rows - 1) * cols + (lane & 7) * 16;
+        const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
         const uint8_t *srow = sl + (size_t)(n * nb + par) * SB;
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         mk_i4 wa[S], wb[S];
         auto load_block = [&](mk_i4 *wv, int s0) {
 #pragma unroll
             for (int j = 0; j < S; j++) {
-                const int s = min(s0 + j, steps - 1);  // past the end: a repeated, unused load
-                wv[j] = mk_ldg128(wrow + s * 64);  // not non-temporal: a lane group takes 64 of a line's 128 bytes per step (measured 217 -> 244 us with it)
+                if constexpr (FULL) {
+                    const int line = min(s0 / 2 + (j >> 1), steps / 2 - 1);  // past the end: a repeated, unused load
+                    wv[j] = mk_ldg128_nt(wline[j & 1] + line * 128);
+                } else {
+                    const int s = min(s0 + j, steps - 1);
+                    wv[j] = mk_ldg128(wrow + s * 64);  // not non-temporal: the second half of the line must stay cached
+                }
             }
         };
-        auto compute_block = [&](const mk_i4 *wv, int s0) {
+        auto compute_block = [&](const mk_i4 *wl, int s0) {
+            mk_i4 wv[S];
+#pragma unroll
+            for (int i = 0; i < S / 2; i++) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    if constexpr (FULL) {
+                        const int ra = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * i][k]), rb = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * i + 1][k]);
+                        wv[2 * i][k] = __builtin_amdgcn_update_dpp(ra, rb, 0x128 /* row_ror:8 */, 0xF, 0xC, false);
+                        wv[2 * i + 1][k] = __builtin_amdgcn_update_dpp(rb, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);
+                    } else {
+                        wv[2 * i][k] = wl[2 * i][k];
+                        wv[2 * i + 1][k] = wl[2 * i + 1][k];
+                    }
+                }
+            }
 #pragma unroll
             for (int j = 0; j < S; j++) {
                 const int s = s0 + j;
@@ -446,8 +476,12 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
         int blocks = tune("MK_Q8_MFMA_BLOCKS", 256);  // one per CU
         if (blocks * WAVES > n_groups) blocks = (n_groups + WAVES - 1) / WAVES;
         const size_t lds = cols * 8 + (size_t)nb * 32 + (size_t)WAVES * 16 * nb * (F16 ? 2 : 4);
-        hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq, xs,
-                           (int)batch, out);
+        if (nb % 4 == 0 && !tune("MK_Q8_MFMA_HALF_LINES", 0))  // rows are whole 128-byte lines
+            hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES, true>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq,
+                               xs, (int)batch, out);
+        else
+            hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES, false>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq,
+                               xs, (int)batch, out);
         return mk_launch_status("q8_gemv_mfma");
     }
     hipLaunchKernelGGL(q8_gemv_generic_kernel<F16>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, q, scales, (int)rows, nb, xq, xs,
@@ -468,8 +502,10 @@ extern "C" int mk_dev_q8_matvec(const int8_t *q, const void *scales, int scales_
     static bool lds_opt_in = false;
     if (!lds_opt_in) {
         // the batch kernel uses up to 136 KiB of the 160 KiB LDS
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         lds_opt_in = true;
     }
     if (scales_f16) return launch_q8<true>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);
