@@ -126,9 +126,10 @@ struct GemmArgs {
     float *out;
 };
 
-// FULL: the weight loads take whole 128-byte lines (see below); measured on 8 experts x 512 tokens 495 -> 400 us, on
-// the prefill shape (at most 32 tokens per expert) 488 -> 504 us, so only the large-group kernel uses it.
-template <int MC, bool FULL>
+// FULL: the weight loads take whole 128-byte lines (see below).  NT: they are non-temporal.  Measured: 8 experts x 512
+// tokens (eight passes over each expert's weights) 495 -> 403 us with FULL, 459 us with FULL + NT; prefill shape (one pass,
+// at most 32 tokens per expert) 488 -> 504 us with FULL alone, 451 us with FULL + NT.
+template <int MC, bool FULL, bool NT>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, int base, int tok1, uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
@@ -159,8 +160,9 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
 #pragma unroll
         for (int j = 0; j < KT_STEPS; j++)
-            w[j] = FULL ? mk_ldg128_off(packed, woff[rt][FULL ? (j & 1) : 0] + ku * (KT_STEPS * 64) + (j >> 1) * 128)
-                        : mk_ldg128_off(packed, woff[rt][0] + ku * (KT_STEPS * 64) + j * 64);
+            if constexpr (FULL && NT) w[j] = mk_ldg128_off_nt(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
+            else if constexpr (FULL) w[j] = mk_ldg128_off(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
+            else w[j] = mk_ldg128_off(packed, woff[rt][0] + ku * (KT_STEPS * 64) + j * 64);
         sc = mk_ldg128_off(scales, soff[rt] + ku * 16);
     };
     // activation tile staging: chunk i = tid + 256 k -> token i / 32, 16-byte chunk i % 32
@@ -281,11 +283,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[e]);
     if (MC == 2) {
-        if (count <= 16) gemm_pass<1, false>(a, packed, scales, tok0, tok1, lds);
-        else gemm_pass<2, false>(a, packed, scales, tok0, tok1, lds);
+        if (count <= 16) gemm_pass<1, true, true>(a, packed, scales, tok0, tok1, lds);
+        else gemm_pass<2, true, true>(a, packed, scales, tok0, tok1, lds);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true>(a, packed, scales, base, tok1, lds);
+        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false>(a, packed, scales, base, tok1, lds);
     }
 }
 
