@@ -7,9 +7,9 @@
 //           t*64+l of the row (perfectly coalesced 1 KiB wave loads, no repack)
 //           and keeps the matching 16 activation bytes and block scale in
 //           registers for the whole kernel; 4 x v_dot4_i32_i8 per load.
-// batch 2-4 at 7168 columns: the batch-1 streaming pattern with the activation in
+// batch 2-3 at 7168 columns: the batch-1 streaming pattern with the activation in
 //           LDS and two rows per LDS read (see q8_gemv_bn_kernel).
-// batch 2-8 matrix-core path (batch 5-8 at 7168 columns, 2-8 elsewhere; 219 -> 203 us at batch 8 since the loads take
+// batch 2-8 matrix-core path (batch 4-8 at 7168 columns, 2-8 elsewhere; 219 -> 197 us at batch 8 since the loads take
 //           whole lines).  One v_mfma_i32_16x16x64_i8 per 16 rows x 64
 //           columns.  The MFMA sums over K = 64 = two q8 blocks, whose scales
 //           differ, so the activation operand is laid out as 16 "columns" =
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void q8_gemv_b1_kernel(const int8_t *__restric
     }
 }
 
-// -------------------------------------------------- batch 2..4, long rows
+// -------------------------------------------------- batch 2..3, long rows
 // The batch-1 streaming pattern (a wave reads whole rows, 1 KiB per load, non-
 // temporal, rows dealt round-robin to a resident grid) with the batch's
 // activation bytes and block scales in LDS: two rows are in the registers at a
@@ -451,14 +451,11 @@ template <bool F16>
 int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, const int8_t *xq, const float *xs, size_t batch, float *out,
               hipStream_t st) {
     const int nb = (int)(cols / 32);
-    // measured on the 163840 x 7168 head: streaming kernel 188 / 198 / 201 us at batch 2 / 3 / 4 against 215-222 us for the
-    // matrix-core kernel; from batch 5 its vector work per row costs more than the matrix-core kernel's 64-byte runs
-    if (batch >= 2 && batch <= 4 && nb == 224 && rows * cols < 0xFFFFFFFFull && !tune("MK_Q8_NO_BN", 0)) {
-        switch (batch) {
-            case 2: launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st); break;
-            case 3: launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st); break;
-            default: launch_bn<F16, 4>(q, scales, (int)rows, xq, xs, out, st); break;
-        }
+    // measured on the 163840 x 7168 head: streaming kernel 188 / 198 / 203 us at batch 2 / 3 / 4 against 204 / 206 / 195 us
+    // for the matrix-core kernel, whose time (195-198 us) does not grow with the batch
+    if (batch >= 2 && batch <= 3 && nb == 224 && rows * cols < 0xFFFFFFFFull && !tune("MK_Q8_NO_BN", 0)) {
+        if (batch == 2) launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st);
+        else launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st);
         return mk_launch_status("q8_gemv_bn");
     }
     if (batch == 1 && rows * cols < 0xFFFFFFFFull) {  // the batch-1 kernel addresses the matrix with 32-bit byte offsets
