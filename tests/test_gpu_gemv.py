@@ -178,3 +178,48 @@ def test_lm_head_full_size_argmax_and_parity():
         assert int(am[b]) == oracle.argmax(want), b
         if b == 0:
             assert rel_l2(got1[0], want) <= TOL
+
+
+def test_matrices_beyond_32_bit_offsets():
+    # maximum sizes: matrices whose byte size passes 2^32 leave the kernels that address them with 32-bit offsets; the
+    # rows are independent, so a sample of rows (first, last, around the 4 GiB boundary) is checked against the oracle
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    cols = 7168
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn((8, cols), device="cuda", generator=g)
+    # q8_0 head, 600 000 rows: 4.3e9 weight bytes
+    rows = 600_000
+    q = torch.randint(-127, 128, (rows, cols), dtype=torch.int8, device="cuda", generator=g)
+    s = (torch.rand((rows, cols // 32), device="cuda", generator=g) * 1e-3 + 1e-4).to(torch.float16)
+    edge = (1 << 32) // cols
+    sample = np.unique(np.clip(np.concatenate([np.arange(0, 40), np.arange(edge - 20, edge + 20), np.arange(rows - 40, rows)]), 0, rows - 1))
+    sq, ss = q[sample].cpu().numpy(), s[sample].cpu().numpy().astype(np.float32)
+    for batch in (1, 3, 8):
+        xq = q8.quantize_q8(x[:batch].contiguous())
+        out = torch.empty((batch, rows), device="cuda")
+        check(lib.mk_dev_q8_matvec(ptr(q), ptr(s), 1, rows, cols, ptr(xq.q), ptr(xq.scales), batch, ptr(out), cur_stream()))
+        got = out[:, sample].cpu().numpy()
+        for b in range(batch):
+            want = oracle.q8head_matvec(sq, ss, len(sample), cols, x[b].cpu().numpy())
+            assert rel_l2(got[b], want) <= TOL, (batch, b)
+    del q, s, out
+    torch.cuda.empty_cache()
+    # MXFP4, 1 250 000 rows: 4.5e9 packed bytes, 2.8e8 blocks
+    rows = 1_250_000
+    packed = torch.randint(0, 256, (rows, cols // 2), dtype=torch.uint8, device="cuda", generator=g)
+    scales = torch.randint(118, 131, (rows, cols // 32), dtype=torch.uint8, device="cuda", generator=g)
+    edge = (1 << 32) // (cols // 2)
+    sample = np.unique(np.clip(np.concatenate([np.arange(0, 40), np.arange(edge - 20, edge + 20), np.arange(rows - 40, rows)]), 0, rows - 1))
+    sp, sc = packed[sample].cpu().numpy(), scales[sample].cpu().numpy()
+    x0 = x[0].contiguous()
+    for mode in (1, 0):
+        out = torch.empty(rows, device="cuda")
+        if mode == 1:
+            xq = q8.quantize_q8(x0)
+            check(lib.mk_dev_mxfp4_matvec_q8(ptr(packed), ptr(scales), rows, cols, ptr(xq.q), ptr(xq.scales), ptr(out), cur_stream()))
+        else:
+            check(lib.mk_dev_mxfp4_matvec_f32(ptr(packed), ptr(scales), rows, cols, ptr(x0), ptr(out), cur_stream()))
+        want = oracle.matvec_packed(sp, sc, len(sample), cols, x0.cpu().numpy(), mode=mode)
+        assert rel_l2(out[sample].cpu().numpy(), want) <= TOL, mode
