@@ -86,14 +86,32 @@ __global__ __launch_bounds__(GROUP_WAVES * 64) void prefill_group_kernel(const i
         eoff[e + 1] = run;  // counts, scanned below
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int e = 0; e < n_experts; e++) {
-            const int c = eoff[e + 1];
-            eoff[e] = run;
-            run += c;
+    if (wave == 0) {
+        // exclusive scan of the counts (held at eoff[e + 1]) by one wave: a lane takes `per` consecutive experts
+        constexpr int MAX_PER_LANE = 15;  // 960 experts
+        const int per = (n_experts + 63) / 64;
+        int cnt[MAX_PER_LANE];
+        int local = 0;
+#pragma unroll
+        for (int k = 0; k < MAX_PER_LANE; k++) {
+            const int e = lane * per + k;
+            cnt[k] = (k < per && e < n_experts) ? eoff[e + 1] : 0;
+            local += cnt[k];
         }
-        eoff[n_experts] = run;
+        int incl = local;
+#pragma unroll
+        for (int dlt = 1; dlt < 64; dlt <<= 1) {
+            const int t = __shfl_up(incl, dlt, MK_WAVE);
+            if (lane >= dlt) incl += t;
+        }
+        int run = incl - local;
+#pragma unroll
+        for (int k = 0; k < MAX_PER_LANE; k++) {
+            const int e = lane * per + k;
+            if (k < per && e < n_experts) eoff[e] = run;
+            run += cnt[k];
+        }
+        if (lane == 63) eoff[n_experts] = incl;
     }
     __syncthreads();
     for (int e = threadIdx.x; e <= n_experts; e += blockDim.x) offsets[e] = eoff[e];
@@ -102,19 +120,24 @@ __global__ __launch_bounds__(GROUP_WAVES * 64) void prefill_group_kernel(const i
         const int e = i < P ? ids[i] : -1;
         const bool valid = e >= 0 && e < n_experts;
         if (i < P && !valid) pos[i] = -1;
-        unsigned long long todo = __ballot(valid);
-        while (todo) {
-            const int leader = __ffsll((long long)todo) - 1;
-            const int key = __shfl(e, leader, MK_WAVE);
-            const unsigned long long m = __ballot(valid && e == key);
-            const int start = eoff[key] + mine[key];  // read by every lane before the leader advances it
-            if (valid && e == key) {
-                const int r = start + __popcll(m & ((1ull << lane) - 1ull));
-                order[r] = i;
-                pos[i] = r;
-            }
-            if (lane == leader) mine[key] += __popcll(m);
-            todo &= ~m;
+        // rank of the lane among the lanes of this chunk that hold the same expert, and the size of that group:
+        // one pass over the 64 lanes (scalar broadcast of each lane's key), no serial walk over the distinct keys
+        int rank = 0, same = 0;
+        const int key = valid ? e : -1 - lane;  // invalid lanes match nobody
+#pragma unroll 8
+        for (int j = 0; j < 64; j++) {
+            const int kj = __builtin_amdgcn_readlane(key, j);
+            const int eq = kj == key ? 1 : 0;
+            same += eq;
+            rank += (j < lane) ? eq : 0;
+        }
+        int start = 0;
+        if (valid) start = eoff[e] + mine[e];  // every lane reads before any lane of this wave advances the counter
+        if (valid) {
+            const int r = start + rank;
+            order[r] = i;
+            pos[i] = r;
+            if (rank == 0) mine[e] = mine[e] + same;  // one lane per distinct key
         }
     }
 }
