@@ -126,10 +126,17 @@ struct GemmArgs {
     float *out;
 };
 
+// PIN: the loads and the matrix instructions stay where the source puts them.  Left alone, instruction selection places
+// all of a K tile's matrix instructions at its end (nothing orders them against the loads), every unit's operands stay
+// live until then, and the scheduler, out of registers, moves loads down to their first use -- one of them to the end
+// of the K tile, behind a wait for every load in flight.  An empty volatile statement that takes a unit's accumulators
+// keeps its matrix instructions in front of the next unit's loads; scheduling barriers keep the loads in place.  Prefill
+// shape: 256 -> 167 registers (three workgroups per CU), gate GEMM 450 -> 409 us, down GEMM 463 -> 403 us.  The kernel for
+// larger groups (four token tiles, accumulators in the second register file) lost by it (403 -> 474 us) and stays as it was.
 // FULL: the weight loads take whole 128-byte lines (see below).  NT: they are non-temporal.  Measured: 8 experts x 512
 // tokens (eight passes over each expert's weights) 495 -> 403 us with FULL, 459 us with FULL + NT; prefill shape (one pass,
 // at most 32 tokens per expert) 488 -> 504 us with FULL alone, 451 us with FULL + NT.
-template <int MC, bool FULL, bool NT>
+template <int MC, bool FULL, bool NT, bool PIN>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, int base, int tok1, uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
@@ -211,11 +218,18 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             }
         }
     };
+    auto pin_acc = [&](int rt) {
+        if constexpr (PIN) {
+#pragma unroll
+            for (int c = 0; c < MC; c++) asm volatile("" : "+v"(acc[rt][c]));
+        }
+    };
     // One unit: 4 steps x MC token tiles.  The LDS reads of the activation operands do not depend on the
     // row tile, so after inlining the four calls of a K tile share them.
     auto compute_unit = [&](const mk_i4 *wl, const mk_i4 &sc, int rt, const uint8_t *buf) {
         if constexpr (!FULL) {
             mma_unit(wl, sc, rt, buf);
+            pin_acc(rt);
             return;
         }
         // Loaded: for line i, wl[2i] = rows 0-7 and wl[2i+1] = rows 8-15, lane (r3, s', kg) holding the 16 bytes of K
@@ -233,6 +247,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             }
         }
         mma_unit(w, sc, rt, buf);
+        pin_acc(rt);
     };
 
     load_unit(wa, sa, 0, 0);
@@ -245,13 +260,21 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
         stage_load(kt + 1);
         load_unit(wb, sb, kt, 1);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         compute_unit(wa, sa, 0, buf);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         load_unit(wa, sa, kt, 2);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         compute_unit(wb, sb, 1, buf);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         load_unit(wb, sb, kt, 3);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         compute_unit(wa, sa, 2, buf);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         load_unit(wa, sa, kt + 1, 0);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         compute_unit(wb, sb, 3, buf);
+        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
         stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
         __syncthreads();
     }
@@ -283,11 +306,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[e]);
     if (MC == 2) {
-        if (count <= 16) gemm_pass<1, true, true>(a, packed, scales, tok0, tok1, lds);
-        else gemm_pass<2, true, true>(a, packed, scales, tok0, tok1, lds);
+        if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, tok0, tok1, lds);
+        else gemm_pass<2, true, true, true>(a, packed, scales, tok0, tok1, lds);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false>(a, packed, scales, base, tok1, lds);
+        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false, false>(a, packed, scales, base, tok1, lds);
     }
 }
 

@@ -230,12 +230,15 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
         const int n_units = gp * J;
         RowUnit4 ua, ub, uc;
         auto load_unit = [&](RowUnit4 &U, int u) {
-            u = __builtin_amdgcn_readfirstlane(min(u, n_units - 1));  // past the end: the last unit again (not used)
+            // past the end (the loads stay unconditional): every lane reads the first block of the last pair's matrices,
+            // one line per load instead of a row (the streaming loads would fetch a repeated row again)
+            const bool past = u >= n_units;
+            u = __builtin_amdgcn_readfirstlane(min(u, n_units - 1));
             const int k = u / J, j = u - k * J;
             const int q = k;  // pairs in (token, slot) order
             const uint8_t *p1 = mk_uniform_ptr(wp1[q]), *p3 = mk_uniform_ptr(wp3[q]);
             const uint8_t *c1 = mk_uniform_ptr(ws1[q]), *c3 = mk_uniform_ptr(ws3[q]);
-            const uint32_t boff = (uint32_t)min(w + j * nw, a.inter - 1) * NB + lane_c;
+            const uint32_t boff = past ? 0u : (uint32_t)min(w + j * nw, a.inter - 1) * NB + lane_c;
 #pragma unroll
             for (int t = 0; t < T; t++) {
                 U.w1[t] = mk_ldg128_off_nt(p1, (boff + t * LW) * 16);
@@ -369,7 +372,8 @@ __global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a)
     mk_i4 wa[U][T], wb[U][T];
     uint32_t sa[U][T], sb[U][T];
     auto load_item = [&](mk_i4(*w)[T], uint32_t(*sc)[T], int i) {
-        i = __builtin_amdgcn_readfirstlane(i < n_items ? i : 0);  // unconditional loads: past the end, item 0 again
+        const bool past = i >= n_items;  // unconditional loads: past the end, one line of item 0 per load
+        i = __builtin_amdgcn_readfirstlane(past ? 0 : i);
         const int grp = i / per, s = i - grp * per;
         // uniform pointers in scalar registers + 32-bit block indices: the loads take the scalar-base form
         const uint8_t *wp = mk_uniform_ptr(wp_l[s]), *ws = mk_uniform_ptr(ws_l[s]);
@@ -377,7 +381,7 @@ __global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a)
         for (int u = 0; u < U; u++) {
             const int k = grp * U + u;
             const uint32_t tile = min((uint32_t)(wv + (k < my_tiles ? k : 0) * wpt), (uint32_t)(n_tiles - 1));  // idle waves re-read the last tile
-            const uint32_t blk0 = tile * TILE + lane;
+            const uint32_t blk0 = past ? 0u : tile * TILE + lane;
 #pragma unroll
             for (int t = 0; t < T; t++) {
                 w[u][t] = mk_ldg128_off_nt(wp, (blk0 + t * 64) * 16);
