@@ -116,14 +116,17 @@ constexpr int A_STRIDE = 512 + 16;  // LDS row stride of the activation tile: 16
 constexpr int a_codes_bytes(int mc) { return 16 * mc * A_STRIDE; }
 constexpr int a_buf_bytes(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }  // codes, then 16 scale bytes per token
 
+// One launch covers n_mats (1 or 2) weight matrices per group that share the activation rows (gate and up): matrix m
+// of group e is packed_ptrs[m][e], its result goes to out[m].
 struct GemmArgs {
-    const uint8_t *const *packed_ptrs;
-    const uint8_t *const *scales_ptrs;
+    const uint8_t *const *packed_ptrs[2];
+    const uint8_t *const *scales_ptrs[2];
     int rows, cols;
     const uint8_t *codes;
     const uint8_t *exps;
     const int32_t *offsets;
-    float *out;
+    float *out[2];
+    int n_groups, n_mats, row_blocks;
 };
 
 // PIN: the loads and the matrix instructions stay where the source puts them.  Left alone, instruction selection places
@@ -137,11 +140,12 @@ struct GemmArgs {
 // tokens (eight passes over each expert's weights) 495 -> 403 us with FULL, 459 us with FULL + NT; prefill shape (one pass,
 // at most 32 tokens per expert) 488 -> 504 us with FULL alone, 451 us with FULL + NT.
 template <int MC, bool FULL, bool NT, bool PIN>
-__device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, int base, int tok1, uint8_t *lds) {
+__device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
+                                          uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
-    const int row0 = blockIdx.x * 256 + wave * 64;
+    const int row0 = rb * 256 + wave * 64;
     // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
     // FULL: weight loads take whole 128-byte lines: load j = 2i + h of a unit covers line i (of the K tile's two) of the
     // rows 8h .. 8h+7 of the row tile, lane (r3 = lane / 8, c = lane % 8) reading bytes 16c .. of row 8h + r3, and the
@@ -287,7 +291,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int t = base + c * 16 + kb * 4 + i;
-                    if (t < tok1) a.out[(size_t)t * a.rows + row] = acc[rt][c][i];
+                    if (t < tok1) out[(size_t)t * a.rows + row] = acc[rt][c][i];
                 }
         }
     }
@@ -299,23 +303,39 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 template <int MC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2 : 1))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int e = blockIdx.y;
+    // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
+    // the plain order the workgroups of one group land on all of them and each fetches the group's activation rows for
+    // itself (prefill gate GEMM: 235 MB of 2.45 GB).  When the group count allows it, XCD x takes the groups x, x + 8, ...
+    // and runs all workgroups of a group itself.
+    const int per_group = a.n_mats * a.row_blocks;
+    int e, r;
+    if (a.n_groups % 8 == 0) {
+        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        e = x + 8 * (j / per_group);
+        r = j % per_group;
+    } else {
+        e = blockIdx.x / per_group;
+        r = blockIdx.x % per_group;
+    }
+    const int m = r / a.row_blocks, rb = r % a.row_blocks;
     const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
     const int count = tok1 - tok0;
     if (count <= 0 || (count <= 32 ? 2 : 4) != MC) return;
-    const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[e]);
-    const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[e]);
+    const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
+    const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
+    float *out = a.out[m];
     if (MC == 2) {
-        if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, tok0, tok1, lds);
-        else gemm_pass<2, true, true, true>(a, packed, scales, tok0, tok1, lds);
+        if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
+        else gemm_pass<2, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false, false>(a, packed, scales, base, tok1, lds);
+        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false, false>(a, packed, scales, out, rb, base, tok1, lds);
     }
 }
 
 template <int MC>
-int launch_stream(const GemmArgs &a, dim3 grid, hipStream_t st) {
+int launch_stream(const GemmArgs &a, hipStream_t st) {
+    const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks));
     static bool opted = false;
     if (!opted) {
         hipFuncSetAttribute(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -328,22 +348,50 @@ int launch_stream(const GemmArgs &a, dim3 grid, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
-                                         size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
-                                         void *stream) {
-    MK_REQUIRE(packed_ptrs && scales_ptrs && codes && exps && offsets && out, "null pointer");
+// gate and up of the prefill section in one launch (the matrices share the token rows); see mk_common.h
+int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
+                            size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
+                            float *const *out, void *stream) {
+    MK_REQUIRE(n_mats == 1 || n_mats == 2, "one or two matrices per group");
+    for (int k = 0; k < n_mats; k++) MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k], "null pointer");
+    MK_REQUIRE(codes && exps && offsets, "null pointer");
     MK_REQUIRE(cols % 128 == 0 && cols > 0, "cols must be a positive multiple of 128");
     MK_REQUIRE(n_groups >= 1 && n_groups <= 65535 && rows >= 1 && rows <= 0x7FFFFF00u, "bad shape");
     MK_REQUIRE(((uintptr_t)codes & 15) == 0, "codes must be 16-byte aligned");
     if (m == 0) return MK_OK;
-    if (cols % 512 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0) {
-        GemmArgs a{packed_ptrs, scales_ptrs, (int)rows, (int)cols, codes, exps, offsets, out};
-        const dim3 grid((unsigned)((rows + 255) / 256), (unsigned)n_groups);
-        int st = launch_stream<2>(a, grid, (hipStream_t)stream);
-        if (st == MK_OK && m > 32) st = launch_stream<4>(a, grid, (hipStream_t)stream);
+    const size_t row_blocks = (rows + 255) / 256;
+    if (cols % 512 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0 &&
+        n_groups * n_mats * row_blocks < 0x7FFFFFFFull) {
+        GemmArgs a{};
+        for (int k = 0; k < n_mats; k++) {
+            a.packed_ptrs[k] = packed_ptrs[k];
+            a.scales_ptrs[k] = scales_ptrs[k];
+            a.out[k] = out[k];
+        }
+        a.rows = (int)rows;
+        a.cols = (int)cols;
+        a.codes = codes;
+        a.exps = exps;
+        a.offsets = offsets;
+        a.n_groups = (int)n_groups;
+        a.n_mats = n_mats;
+        a.row_blocks = (int)row_blocks;
+        int st = launch_stream<2>(a, (hipStream_t)stream);
+        if (st == MK_OK && m > 32) st = launch_stream<4>(a, (hipStream_t)stream);
         return st;
     }
-    hipLaunchKernelGGL(mxfp4_grouped_gemm_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)n_groups), dim3(256), 0, (hipStream_t)stream,
-                       packed_ptrs, scales_ptrs, (int)rows, (int)cols, codes, exps, offsets, out);
-    return mk_launch_status("mxfp4_grouped_gemm");
+    for (int k = 0; k < n_mats; k++) {
+        hipLaunchKernelGGL(mxfp4_grouped_gemm_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)n_groups), dim3(256), 0, (hipStream_t)stream,
+                           packed_ptrs[k], scales_ptrs[k], (int)rows, (int)cols, codes, exps, offsets, out[k]);
+        const int st = mk_launch_status("mxfp4_grouped_gemm");
+        if (st != MK_OK) return st;
+    }
+    return MK_OK;
+}
+
+extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                         size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
+                                         void *stream) {
+    MK_REQUIRE(packed_ptrs && scales_ptrs && codes && exps && offsets && out, "null pointer");
+    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream);
 }

@@ -307,3 +307,9 @@ int mk_check_hip(hipError_t e, const char *what);
         }                                               \
     } while (0)
 int mk_launch_status(const char *kernel);
+
+// mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
+// (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].
+int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
+                            size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
+                            float *const *out, void *stream);

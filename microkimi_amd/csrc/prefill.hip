@@ -6,7 +6,7 @@
 //   group     counting sort of the pairs by expert id, stable in (token, slot)
 //             order inside a group as the reference fills its groups
 //   gather    MXFP8 (e4m3 + e8m0 per 32) of each pair's hidden row, in grouped order
-//   gate, up  mk_dev_mxfp4_grouped_gemm over the expert table
+//   gate, up  the grouped GEMM over the expert table, both matrices in one launch
 //   act       ACT(gate, up) and its MXFP8 form (the input of the down projection)
 //   down      mk_dev_mxfp4_grouped_gemm
 //   combine   out_t = sum_s w[t][s] * o[pair (t, s)], multiply then add, in slot order
@@ -228,8 +228,12 @@ extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts
     hipLaunchKernelGGL(prefill_gather_mxfp8_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
                        (int)n_experts, (int)topk, (int)d, w.codes, w.exps);
     if ((s = mk_launch_status("prefill_gather_mxfp8")) != MK_OK) return s;
-    if ((s = mk_dev_mxfp4_grouped_gemm(table->w1p, table->w1s, n_experts, inter, d, w.codes, w.exps, w.offsets, P, w.g, stream)) != MK_OK) return s;
-    if ((s = mk_dev_mxfp4_grouped_gemm(table->w3p, table->w3s, n_experts, inter, d, w.codes, w.exps, w.offsets, P, w.u, stream)) != MK_OK) return s;
+    {
+        const uint8_t *const *pp[2] = {table->w1p, table->w3p};
+        const uint8_t *const *sp[2] = {table->w1s, table->w3s};
+        float *gu[2] = {w.g, w.u};
+        if ((s = mk_mxfp4_grouped_gemm_n(2, pp, sp, n_experts, inter, d, w.codes, w.exps, w.offsets, P, gu, stream)) != MK_OK) return s;
+    }
     hipLaunchKernelGGL(prefill_act_mxfp8_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
                        (int)n_experts, (int)inter, act_kind, w.codes2, w.exps2);
     if ((s = mk_launch_status("prefill_act_mxfp8")) != MK_OK) return s;
