@@ -216,11 +216,8 @@ extern "C" int mk_dev_rmsnorm(const float *x, size_t B, size_t d, const float *w
     MK_REQUIRE(!q || d % 32 == 0, "q8 blocks are 32 wide");
     MK_REQUIRE(((uintptr_t)x & 15) == 0 && (d % 4 == 0 || B == 1) && (!q || ((uintptr_t)q & 7) == 0), "x must be 16-byte aligned rows");
     const size_t lds = (d + 4) * sizeof(float);
-    static bool opted = false;
-    if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(rmsnorm_q8_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 132 * 1024);
-        opted = true;
-    }
+    int st = mk_lds_opt_in(reinterpret_cast<const void *>(rmsnorm_q8_kernel), 132 * 1024);
+    if (st != MK_OK) return st;
     hipLaunchKernelGGL(rmsnorm_q8_kernel, dim3((unsigned)B), dim3(256), lds, (hipStream_t)stream, x, (int)d, w, eps, out, q, scales);
     return mk_launch_status("rmsnorm_q8");
 }

@@ -336,12 +336,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2
 template <int MC>
 int launch_stream(const GemmArgs &a, hipStream_t st) {
     const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks));
-    static bool opted = false;
-    if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * a_buf_bytes(MC));
-        opted = true;
-    }
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), 2 * a_buf_bytes(MC));
+    if (s != MK_OK) return s;
     hipLaunchKernelGGL(mxfp4_grouped_gemm_stream_kernel<MC>, grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
 }

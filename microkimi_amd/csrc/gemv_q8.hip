@@ -434,17 +434,15 @@ void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, 
 }
 
 template <bool F16, int BATCH>
-void launch_bn(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
+int launch_bn(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
     constexpr int NB = 224;
     int blocks = tune("MK_Q8_BN_BLOCKS", 512);
     if (blocks * 4 > rows) blocks = (rows + 3) / 4;
     const size_t lds = (size_t)BATCH * NB * 36;
-    static bool opted = false;
-    if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_bn_kernel<NB, F16, BATCH>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-        opted = true;
-    }
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8_gemv_bn_kernel<NB, F16, BATCH>), 80 * 1024);
+    if (s != MK_OK) return s;
     hipLaunchKernelGGL((q8_gemv_bn_kernel<NB, F16, BATCH>), dim3(blocks), dim3(256), lds, st, q, scales, rows, xq, xs, out);
+    return mk_launch_status("q8_gemv_bn");
 }
 
 template <bool F16>
@@ -454,9 +452,8 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
     // measured on the 163840 x 7168 head: streaming kernel 188 / 198 / 203 us at batch 2 / 3 / 4 against 204 / 206 / 195 us
     // for the matrix-core kernel, whose time (195-198 us) does not grow with the batch
     if (batch >= 2 && batch <= 3 && nb == 224 && rows * cols < 0xFFFFFFFFull && !tune("MK_Q8_NO_BN", 0)) {
-        if (batch == 2) launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st);
-        else launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st);
-        return mk_launch_status("q8_gemv_bn");
+        if (batch == 2) return launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st);
+        return launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st);
     }
     if (batch == 1 && rows * cols < 0xFFFFFFFFull) {  // the batch-1 kernel addresses the matrix with 32-bit byte offsets
         switch (nb) {
@@ -496,14 +493,14 @@ extern "C" int mk_dev_q8_matvec(const int8_t *q, const void *scales, int scales_
     MK_REQUIRE(rows <= 0x7FFFFFF0u && cols <= (1u << 24), "shape too large");
     MK_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)xq & 15) == 0, "q and xq must be 16-byte aligned");
     if (rows == 0) return MK_OK;
-    static bool lds_opt_in = false;
-    if (!lds_opt_in) {
-        // the batch kernel uses up to 136 KiB of the 160 KiB LDS
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        hipFuncSetAttribute(reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        lds_opt_in = true;
+    // the batch kernel uses up to 136 KiB of the 160 KiB LDS
+    const void *batch_kernels[4] = {reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, true>),
+                                    reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, true>),
+                                    reinterpret_cast<const void *>(q8_gemv_mfma_kernel<true, 8, false>),
+                                    reinterpret_cast<const void *>(q8_gemv_mfma_kernel<false, 4, false>)};
+    for (const void *k : batch_kernels) {
+        const int s = mk_lds_opt_in(k, 160 * 1024);
+        if (s != MK_OK) return s;
     }
     if (scales_f16) return launch_q8<true>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);
     return launch_q8<false>(q, scales, rows, cols, xq, xs, batch, out, (hipStream_t)stream);

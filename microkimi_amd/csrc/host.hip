@@ -8,6 +8,7 @@
 
 #include <map>
 #include <mutex>
+#include <set>
 #include <tuple>
 #include <vector>
 
@@ -77,6 +78,18 @@ int mk_launch_status(const char *kernel) {
     if (e == hipSuccess) return MK_OK;
     mk_set_error("launch of %s failed: %d (%s)", kernel, (int)e, hipGetErrorString(e));
     return MK_ERR_HIP;
+}
+
+int mk_lds_opt_in(const void *kernel, int bytes) {
+    static std::mutex mu;
+    static std::set<std::pair<const void *, int>> done;
+    int dev = 0;
+    MK_HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(mu);
+    if (done.count({kernel, dev})) return MK_OK;
+    MK_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    done.insert({kernel, dev});
+    return MK_OK;
 }
 
 extern "C" const char *mk_last_error(void) { return g_err; }

@@ -307,6 +307,9 @@ int mk_check_hip(hipError_t e, const char *what);
         }                                               \
     } while (0)
 int mk_launch_status(const char *kernel);
+// Raises a kernel's dynamic LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) once per kernel and device; checked,
+// safe to call from several threads.  Launch sites call it before every launch: after the first it is a set lookup.
+int mk_lds_opt_in(const void *kernel, int bytes);
 
 // mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].

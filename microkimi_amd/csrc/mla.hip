@@ -690,11 +690,7 @@ extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, cons
     int s;
     if (mfma) {
         MK_REQUIRE(n_pos <= (1 << 22), "the MFMA kernel addresses the cache with 32-bit byte offsets: at most 4 Mi positions");
-        static bool opt_in = false;
-        if (!opt_in) {
-            hipFuncSetAttribute(reinterpret_cast<const void *>(mla_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, MLA_LDS_BYTES);
-            opt_in = true;
-        }
+        if ((s = mk_lds_opt_in(reinterpret_cast<const void *>(mla_mfma_kernel), MLA_LDS_BYTES)) != MK_OK) return s;
         hipLaunchKernelGGL(mla_mfma_kernel, dim3(a.n_splits, head_groups), dim3(256), MLA_LDS_BYTES, st, a, out);
         if ((s = mk_launch_status("mla_mfma")) != MK_OK) return s;
         if (a.n_splits == 1) return MK_OK;
@@ -703,11 +699,7 @@ extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, cons
         hipLaunchKernelGGL(mla_q_prep_kernel, dim3((nblk + 7) / 8), dim3(256), 0, st, q, (int)nh, (int)L, (int)R, qq, qs);
         if ((s = mk_launch_status("mla_q_prep")) != MK_OK) return s;
         const size_t lds = (size_t)TJ * L + (size_t)TJ * (L / 32) * 4 + (size_t)TJ * R * 4 + (size_t)HPG * TJ * 4;
-        static bool lds_opt_in = false;
-        if (!lds_opt_in) {
-            hipFuncSetAttribute(reinterpret_cast<const void *>(mla_partial_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-            lds_opt_in = true;
-        }
+        if ((s = mk_lds_opt_in(reinterpret_cast<const void *>(mla_partial_kernel), 96 * 1024)) != MK_OK) return s;
         hipLaunchKernelGGL(mla_partial_kernel, dim3(a.n_splits, head_groups), dim3(256), lds, st, a);
         if ((s = mk_launch_status("mla_partial")) != MK_OK) return s;
     }

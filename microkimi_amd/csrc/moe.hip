@@ -508,11 +508,8 @@ int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
     if (tg > 8) tg = 8;
     if (tg > (int)B) tg = (int)B;
     const size_t lds = (size_t)tg * per_tok;
-    static bool opted = false;
-    if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_gate_up_rows_kernel<NB>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        opted = true;
-    }
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(moe_gate_up_rows_kernel<NB>), 160 * 1024);
+    if (s != MK_OK) return s;
     int blocks = tune("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
     if (blocks * 8 > a.inter) blocks = (a.inter + 7) / 8;
     hipLaunchKernelGGL(moe_gate_up_rows_kernel<NB>, dim3(blocks), dim3(512), lds, st, a, (int)B, tg);
@@ -522,12 +519,8 @@ int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
 template <int NB, int U, int WAVES = 4>
 int launch_down_u(const FusedArgs &a, size_t B, int blocks, hipStream_t st) {
     const size_t lds = (size_t)a.per * NB * 64 + (size_t)a.per * NB * 4;
-    static bool opted = false;
-    if (!opted) {
-        hipFuncSetAttribute(reinterpret_cast<const void *>(moe_down_fused_kernel<NB, U, WAVES>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            150 * 1024);
-        opted = true;
-    }
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(moe_down_fused_kernel<NB, U, WAVES>), 150 * 1024);
+    if (s != MK_OK) return s;
     hipLaunchKernelGGL((moe_down_fused_kernel<NB, U, WAVES>), dim3((unsigned)B, blocks), dim3(WAVES * 64), lds, st, a);
     return mk_launch_status("moe_down_fused");
 }
