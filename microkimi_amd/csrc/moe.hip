@@ -155,7 +155,13 @@ struct FusedArgs {
 // changes.  Walking the pairs in expert order instead, so that a repeated expert
 // finds its rows in the XCD's L2, was measured and gave nothing (B = 16: 577 us
 // against 569 us in token order): at 8 tokens and more the kernel is bound by the
-// vector unit's work per pair, not by where the bytes come from.
+// vector unit's work per pair, not by where the bytes come from.  The stronger
+// form was measured too: pairs sorted by expert inside the token group and one
+// pass over an expert's rows for all pairs of its run (72 pairs of a group meet
+// about 59 distinct experts; the shared expert is then read once per group, not
+// once per token).  The fetched bytes went down, the time did not (B = 4: 150 ->
+// 154 us, B = 16: 535 -> 532 us, B = 1 unchanged), so the kernel keeps the
+// simpler (token, slot) order.
 struct RowUnit4 {
     mk_i4 w1[4], w3[4];
     uint32_t s1[4], s3[4];
