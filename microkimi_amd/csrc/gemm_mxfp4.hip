@@ -129,6 +129,50 @@ struct GemmArgs {
     int n_groups, n_mats, row_blocks;
 };
 
+// Small groups (PIN): the weights are the instruction's M operand and the token rows its N operand, so a lane of the
+// 16 x 16 result holds four consecutive weight rows of one token row: one 16-byte store.  The kernel for large groups
+// keeps the token rows as M (the other way round it lost a tenth: 400 -> 441 us on 8 experts x 512 tokens).  (With the roles the other way round a lane holds
+// one weight row of four tokens and every value is a store of its own; on the down projection of the prefill shape those
+// stores took 100 of the kernel's 400 us.)
+template <bool NT>
+__device__ __forceinline__ void store_tile(float *out, int rows, int t, int tok1, int row, const mk_f4 &v) {
+    if (t >= tok1) return;
+    float *dst = out + (size_t)t * rows + row;
+    if (row + 3 < rows && ((reinterpret_cast<uintptr_t>(dst) & 15) == 0)) {
+        if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<mk_f4 *>(dst));
+        else *reinterpret_cast<mk_f4 *>(dst) = v;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (row + i < rows) dst[i] = v[i];
+    }
+}
+
+// Two neighbouring 16-row tiles of 16 tokens as full 128-byte lines: the lanes of tokens 8-15 hand their half of the
+// second tile to the lanes of tokens 0-7 and take those lanes' half of the first (a rotation by 8 inside every 16-lane row),
+// so that one store instruction writes the whole line (32 rows) of 8 tokens instead of half a line of 16.
+// x: rows row .. row + 15, y: rows row + 16 .. row + 31 (this lane: token t0 + n, rows + 4 kb .. + 4 kb + 3 of each).
+template <bool NT>
+__device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, int tok1, int row, int n, int kb, const mk_f4 &x, const mk_f4 &y) {
+    const bool up = n >= 8;
+    // tokens 0-7: own first tile | second tile of the lane 8 below;  tokens 8-15: first tile of the lane 8 above | own second tile
+    // (written component by component: the same exchange in a loop over a vector index gave all four lanes' values of
+    // component 0 on the device)
+    const mk_i4 xi = __builtin_bit_cast(mk_i4, x), yi = __builtin_bit_cast(mk_i4, y);
+    mk_i4 fi, si;
+    fi.x = __builtin_amdgcn_update_dpp(xi.x, yi.x, 0x128 /* row_ror:8 */, 0xF, 0xC, false);
+    fi.y = __builtin_amdgcn_update_dpp(xi.y, yi.y, 0x128, 0xF, 0xC, false);
+    fi.z = __builtin_amdgcn_update_dpp(xi.z, yi.z, 0x128, 0xF, 0xC, false);
+    fi.w = __builtin_amdgcn_update_dpp(xi.w, yi.w, 0x128, 0xF, 0xC, false);
+    si.x = __builtin_amdgcn_update_dpp(yi.x, xi.x, 0x128, 0xF, 0x3, false);
+    si.y = __builtin_amdgcn_update_dpp(yi.y, xi.y, 0x128, 0xF, 0x3, false);
+    si.z = __builtin_amdgcn_update_dpp(yi.z, xi.z, 0x128, 0xF, 0x3, false);
+    si.w = __builtin_amdgcn_update_dpp(yi.w, xi.w, 0x128, 0xF, 0x3, false);
+    const mk_f4 first = __builtin_bit_cast(mk_f4, fi), second = __builtin_bit_cast(mk_f4, si);
+    store_tile<NT>(out, rows, t0 + (n & 7), tok1, row + (up ? 16 : 0) + kb * 4, first);
+    store_tile<NT>(out, rows, t0 + 8 + (n & 7), tok1, row + (up ? 16 : 0) + kb * 4, second);
+}
+
 // PIN: the loads and the matrix instructions stay where the source puts them.  Left alone, instruction selection places
 // all of a K tile's matrix instructions at its end (nothing orders them against the loads), every unit's operands stay
 // live until then, and the scheduler, out of registers, moves loads down to their first use -- one of them to the end
@@ -218,7 +262,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 const mk_i8v bv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
                 const int asb = (int)((uint32_t)ae[s] >> (8 * kb));  // the instruction reads byte 0
                 const int wsb = (int)((uint32_t)sc[s] >> (8 * kb));
-                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*A: fp8 e4m3*/, 4 /*B: fp4 e2m1*/, 0, asb, 0, wsb);
+                if constexpr (PIN)
+                    acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[rt][c], 4 /*M: fp4 weights*/, 0 /*N: fp8 rows*/, 0, wsb, 0, asb);
+                else
+                    acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*M: fp8 rows*/, 4 /*N: fp4 weights*/, 0, asb, 0, wsb);
             }
         }
     };
@@ -283,16 +330,25 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
     }
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++) {
-        const int row = row0 + rt * 16 + n;
-        if (row < a.rows) {
+    for (int rt = 0; rt < 4; rt += 2) {
+        if constexpr (PIN) {
 #pragma unroll
-            for (int c = 0; c < MC; c++)
+            for (int c = 0; c < MC; c++) store_tile_pair<NT>(out, a.rows, base + c * 16, tok1, row0 + rt * 16, n, kb, acc[rt][c], acc[rt + 1][c]);
+        } else {
+            // token rows as the M operand: a lane holds one weight row of four tokens
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int t = base + c * 16 + kb * 4 + i;
-                    if (t < tok1) out[(size_t)t * a.rows + row] = acc[rt][c][i];
+            for (int h = 0; h < 2; h++) {
+                const int row = row0 + (rt + h) * 16 + n;
+                if (row < a.rows) {
+#pragma unroll
+                    for (int c = 0; c < MC; c++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int t = base + c * 16 + kb * 4 + i;
+                            if (t < tok1) out[(size_t)t * a.rows + row] = acc[rt + h][c][i];
+                        }
                 }
+            }
         }
     }
 }

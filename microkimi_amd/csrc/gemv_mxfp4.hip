@@ -347,10 +347,6 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__res
     }
 }
 
-int tune(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return (e && *e) ? atoi(e) : dflt;
-}
 
 template <int NB>
 int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
@@ -360,7 +356,7 @@ int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
     if (q8) {
         // a fixed, fully resident grid shared by the matrices of the launch
         // (2 workgroups per CU measured best for every block count per row)
-        int per_mat = tune("MK_MXFP4_BLOCKS", 512) / (int)nmat;
+        int per_mat = mk_env_int("MK_MXFP4_BLOCKS", 512) / (int)nmat;
         if (per_mat < 1) per_mat = 1;
         if (per_mat * 4 > n_tiles) per_mat = (n_tiles + 3) / 4;
         hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(per_mat, (unsigned)nmat), dim3(256), 0, st, a);

@@ -80,6 +80,11 @@ int mk_launch_status(const char *kernel) {
     return MK_ERR_HIP;
 }
 
+int mk_env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return (e && *e) ? atoi(e) : dflt;
+}
+
 int mk_lds_opt_in(const void *kernel, int bytes) {
     static std::mutex mu;
     static std::set<std::pair<const void *, int>> done;

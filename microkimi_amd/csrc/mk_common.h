@@ -310,6 +310,8 @@ int mk_launch_status(const char *kernel);
 // Raises a kernel's dynamic LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) once per kernel and device; checked,
 // safe to call from several threads.  Launch sites call it before every launch: after the first it is a set lookup.
 int mk_lds_opt_in(const void *kernel, int bytes);
+// integer value of an environment variable (tuning and A/B switches of the launchers), dflt when unset or empty
+int mk_env_int(const char *name, int dflt);
 
 // mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].

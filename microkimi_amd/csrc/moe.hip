@@ -501,10 +501,6 @@ extern "C" size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_s
 }
 
 namespace {
-int tune(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return (e && *e) ? atoi(e) : dflt;
-}
 
 template <int NB>
 int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
@@ -516,7 +512,7 @@ int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
     const size_t lds = (size_t)tg * per_tok;
     const int s = mk_lds_opt_in(reinterpret_cast<const void *>(moe_gate_up_rows_kernel<NB>), 160 * 1024);
     if (s != MK_OK) return s;
-    int blocks = tune("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
+    int blocks = mk_env_int("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
     if (blocks * 8 > a.inter) blocks = (a.inter + 7) / 8;
     hipLaunchKernelGGL(moe_gate_up_rows_kernel<NB>, dim3(blocks), dim3(512), lds, st, a, (int)B, tg);
     return mk_launch_status("moe_gate_up_rows");
@@ -544,16 +540,16 @@ int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
         // One workgroup of 14 waves per CU when the rows then divide evenly (7168 = 2^10 x 7): the activation is
         // quantized once per CU instead of once per small workgroup, and every wave has the same number of tiles.
         const int bpt = 256 / (int)B;  // workgroups per token
-        if (bpt >= 1 && !tune("MK_MOE_DOWN_SMALL", 0) && n_tiles % (bpt * 14) == 0) {
+        if (bpt >= 1 && !mk_env_int("MK_MOE_DOWN_SMALL", 0) && n_tiles % (bpt * 14) == 0) {
             const int tiles = n_tiles / (bpt * 14);  // per wave
             if (tiles % 8 == 0) return launch_down_u<NB, 8, 14>(a, B, bpt, st);
             if (tiles % 4 == 0) return launch_down_u<NB, 4, 14>(a, B, bpt, st);
             if (tiles % 2 == 0) return launch_down_u<NB, 2, 14>(a, B, bpt, st);
         }
     }
-    const int target = tune("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
+    const int target = mk_env_int("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
     int u = 8 / T;
-    int forced = tune("MK_MOE_DOWN_U", 0);
+    int forced = mk_env_int("MK_MOE_DOWN_U", 0);
     auto blocks_for = [&](int uu) {
         int groups = (int)((double)n_tiles / ((double)(target > 0 ? target : 1) * 4 * uu) + 0.5);
         if (groups < 1) groups = 1;
