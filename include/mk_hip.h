@@ -268,9 +268,15 @@ size_t mk_vq1_workspace_bytes(size_t cols);
  * Table entries are bit-identical to the reference's (sequential multiply-add chain).  exact != 0: each row adds its
  * table entries in ascending group order from 0 like the reference's sweep, and the result is bit-identical to
  * matvec_vq_lut / matvec_vq_gather; exact == 0: the sum over groups is split across the 64 lanes of a wave
- * (relative L2 error against the reference below 1e-5).  The batched matvec_vq_nt is not built. */
+ * (relative L2 error against the reference below 1e-5). */
 int mk_dev_vq1_matvec(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *x, int exact,
                       void *workspace, float *out, void *stream);
+
+/* quant::matvec_vq_nt (src/quant.rs:353-376), the batched form for prefill: xt [cols][m] (m inputs, transposed, m a
+ * multiple of 8), out [m][rows] position-major.  Every product is added to its position's running sum in (vector, j)
+ * order, multiply then add: bit-identical to the reference.  xt must be 16-byte aligned. */
+int mk_dev_vq1_matvec_nt(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *xt, size_t m, float *out,
+                         void *stream);
 
 /* ------------------------------------------- MKIM weight files -> device */
 

@@ -86,6 +86,7 @@ def _load():
         "mk_mla_cache_free": (None, [vp]),
         "mk_vq1_workspace_bytes": (sz, [sz]),
         "mk_dev_vq1_matvec": (i32, [vp, vp, sz, sz, vp, i32, vp, vp, vp]),
+        "mk_dev_vq1_matvec_nt": (i32, [vp, vp, sz, sz, vp, sz, vp, vp]),
         "mk_bin_open": (i32, [C.c_char_p, C.POINTER(vp)]),
         "mk_bin_close": (None, [vp]),
         "mk_bin_n_tensors": (sz, [vp]),

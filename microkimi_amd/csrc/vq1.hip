@@ -13,6 +13,7 @@
 //           bit-identical to the reference, which is itself bit-identical to matvec_vq_gather.
 //
 // The table (cols/16 KiB) and the index rows stay in the L2; the kernels are latency- and launch-bound, not HBM-bound.
+// The batched form for prefill, matvec_vq_nt, is the last kernel of this file.
 #include "mk_common.h"
 
 namespace {
@@ -76,7 +77,77 @@ __global__ __launch_bounds__(64) void vq1_sweep_exact_kernel(const float *__rest
     out[r] = a;
 }
 
+// quant::matvec_vq_nt (src/quant.rs:353-376): m positions at once, every product added to its position's running sum in
+// (vector, j) order -- one sequential chain of cols multiply-adds per (row, position), not the per-vector partial sums of
+// matvec_vq.  A lane owns a row and 8 positions (the reference's block of 8): the codebook entry is gathered from LDS
+// (entries 20 floats apart, so that the 16-byte reads of different entries spread over the banks), the 8 activations of
+// a (vector, j) are the same for every lane (uniform loads).  Multiply, then add, never fused: bit-identical.
+constexpr int CB_STRIDE = 20;
+template <bool QUAD>  // QUAD: cols / 16 is a multiple of 4 and the index rows are 4-byte aligned: four index bytes per load
+__global__ __launch_bounds__(256) void vq1_nt_kernel(const float *__restrict__ codebook, const uint8_t *__restrict__ indices, int rows, int vpr,
+                                                     const float *__restrict__ xt, int m, float *__restrict__ out) {
+    __shared__ __attribute__((aligned(16))) float cb[256 * CB_STRIDE];
+    for (int i = threadIdx.x; i < 256 * 4; i += 256)
+        *reinterpret_cast<mk_f4 *>(cb + (i >> 2) * CB_STRIDE + (i & 3) * 4) = reinterpret_cast<const mk_f4 *>(codebook)[i];
+    __syncthreads();
+    const int r = blockIdx.x * 256 + threadIdx.x, t0 = blockIdx.y * 8;
+    const uint8_t *ir = indices + (size_t)min(r, rows - 1) * vpr;
+    float sum[8];
+#pragma unroll
+    for (int p = 0; p < 8; p++) sum[p] = 0.0f;
+    auto vec = [&](int v, int idx) {
+        const float *e = cb + idx * CB_STRIDE;
+        const mk_f4 c0 = *reinterpret_cast<const mk_f4 *>(e), c1 = *reinterpret_cast<const mk_f4 *>(e + 4);
+        const mk_f4 c2 = *reinterpret_cast<const mk_f4 *>(e + 8), c3 = *reinterpret_cast<const mk_f4 *>(e + 12);
+        const float c[16] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w, c2.x, c2.y, c2.z, c2.w, c3.x, c3.y, c3.z, c3.w};
+        const float *xv = xt + (size_t)v * 16 * m + t0;  // the same address in every lane
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const mk_f4 xa = *reinterpret_cast<const mk_f4 *>(xv + (size_t)j * m), xb = *reinterpret_cast<const mk_f4 *>(xv + (size_t)j * m + 4);
+            sum[0] = mk_add(sum[0], mk_mul(c[j], xa.x));
+            sum[1] = mk_add(sum[1], mk_mul(c[j], xa.y));
+            sum[2] = mk_add(sum[2], mk_mul(c[j], xa.z));
+            sum[3] = mk_add(sum[3], mk_mul(c[j], xa.w));
+            sum[4] = mk_add(sum[4], mk_mul(c[j], xb.x));
+            sum[5] = mk_add(sum[5], mk_mul(c[j], xb.y));
+            sum[6] = mk_add(sum[6], mk_mul(c[j], xb.z));
+            sum[7] = mk_add(sum[7], mk_mul(c[j], xb.w));
+        }
+    };
+    if constexpr (QUAD) {
+        uint32_t nxt = *reinterpret_cast<const uint32_t *>(ir);
+        for (int v = 0; v < vpr; v += 4) {
+            const uint32_t cur = nxt;
+            nxt = *reinterpret_cast<const uint32_t *>(ir + min(v + 4, vpr - 4));  // one load ahead
+#pragma unroll
+            for (int k = 0; k < 4; k++) vec(v + k, (int)((cur >> (8 * k)) & 0xFF));
+        }
+    } else {
+        for (int v = 0; v < vpr; v++) vec(v, (int)ir[v]);
+    }
+    if (r < rows) {
+#pragma unroll
+        for (int p = 0; p < 8; p++) out[(size_t)(t0 + p) * rows + r] = sum[p];
+    }
+}
+
 }  // namespace
+
+extern "C" int mk_dev_vq1_matvec_nt(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *xt, size_t m, float *out,
+                                    void *stream) {
+    MK_REQUIRE(codebook && indices && xt && out, "null pointer");
+    MK_REQUIRE(cols % 16 == 0 && cols > 0, "cols must be a positive multiple of 16");
+    MK_REQUIRE(m % 8 == 0, "m must be a multiple of 8 (the reference's position blocks)");
+    MK_REQUIRE(rows <= 0x7FFFFF00u && cols <= (1u << 24) && m / 8 <= 65535, "shape too large");
+    MK_REQUIRE(((uintptr_t)codebook & 15) == 0 && ((uintptr_t)xt & 15) == 0, "codebook and xt must be 16-byte aligned");
+    if (rows == 0 || m == 0) return MK_OK;
+    const dim3 grid((unsigned)((rows + 255) / 256), (unsigned)(m / 8));
+    if ((cols / 16) % 4 == 0 && ((uintptr_t)indices & 3) == 0)
+        hipLaunchKernelGGL(vq1_nt_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, codebook, indices, (int)rows, (int)(cols / 16), xt, (int)m, out);
+    else
+        hipLaunchKernelGGL(vq1_nt_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, codebook, indices, (int)rows, (int)(cols / 16), xt, (int)m, out);
+    return mk_launch_status("vq1_nt");
+}
 
 extern "C" size_t mk_vq1_workspace_bytes(size_t cols) { return cols / 16 * 256 * sizeof(float); }
 

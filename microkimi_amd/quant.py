@@ -21,3 +21,17 @@ def matvec_vq(codebook, indices, rows, cols, x, out=None, exact=False):
     check(lib.mk_dev_vq1_matvec(ptr(codebook.contiguous()), ptr(indices.contiguous()), rows, cols, ptr(x.contiguous()), int(exact),
                                 ptr(ws), ptr(out), cur_stream()))
     return out
+
+
+def matvec_vq_nt(codebook, indices, rows, cols, xt, m, out=None):
+    """quant::matvec_vq_nt (src/quant.rs:353-376): xt [cols, m] f32 (m inputs transposed, m % 8 == 0) -> out [m, rows],
+    bit-identical to the reference (one sequential multiply-add chain per row and position)."""
+    import torch
+    _lib.require_device()
+    if cols % VQ_DIM or m % 8 or codebook.numel() != VQ_K * VQ_DIM or indices.numel() != rows * cols // VQ_DIM or xt.numel() != cols * m:
+        raise ValueError("vq1 shapes: codebook [256,16], indices [rows, cols/16], xt [cols, m] with m a multiple of 8")
+    if out is None:
+        out = torch.empty((m, rows), dtype=torch.float32, device=xt.device)
+    check(lib.mk_dev_vq1_matvec_nt(ptr(codebook.contiguous()), ptr(indices.contiguous()), rows, cols, ptr(xt.contiguous()), m, ptr(out),
+                                   cur_stream()))
+    return out

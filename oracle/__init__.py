@@ -107,6 +107,9 @@ _lib.orc_moe_prefill.argtypes = [_PP, _PP, _PP, _PP, _PP, _PP, _sz, _sz, _sz, _s
 _lib.orc_rng_u8.argtypes = [C.POINTER(C.c_uint64), _u8p, _sz]
 _lib.orc_rng_f32.argtypes = [C.POINTER(C.c_uint64), _f32p, _sz]
 _lib.orc_pattern.argtypes = [_sz, _f32p, _sz]
+_lib.orc_vq1_matvec_gather.argtypes = [_f32p, _u8p, _sz, _sz, _f32p, _f32p]
+_lib.orc_vq1_matvec_lut.argtypes = [_f32p, _u8p, _sz, _sz, _f32p, _f32p]
+_lib.orc_vq1_matvec_nt.argtypes = [_f32p, _u8p, _sz, _sz, _f32p, _sz, _f32p]
 
 # ---------------------------------------------------------------- scalars
 exp2_i = _lib.orc_exp2_i
@@ -240,6 +243,15 @@ def vq1_matvec(codebook, indices, rows, cols, x, lut=True):
     out = np.empty(rows, np.float32)
     fn = _lib.orc_vq1_matvec_lut if lut else _lib.orc_vq1_matvec_gather
     fn(_p(codebook, _f32p), _p(indices, _u8p), rows, cols, _p(x, _f32p), _p(out, _f32p))
+    return out
+
+
+def vq1_matvec_nt(codebook, indices, rows, cols, xt, m):
+    """quant::matvec_vq_nt (src/quant.rs:353-376): xt [cols, m] -> out [m, rows]."""
+    codebook, indices, xt = _c(codebook, np.float32), _c(indices, np.uint8), _c(xt, np.float32)
+    assert codebook.size == 256 * 16 and cols % 16 == 0 and m % 8 == 0 and indices.size == rows * cols // 16 and xt.size == cols * m
+    out = np.empty((m, rows), np.float32)
+    _lib.orc_vq1_matvec_nt(_p(codebook, _f32p), _p(indices, _u8p), rows, cols, _p(xt, _f32p), m, _p(out, _f32p))
     return out
 
 

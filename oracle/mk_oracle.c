@@ -435,6 +435,27 @@ ORC_API void orc_vq1_matvec_lut(const float *codebook, const uint8_t *indices, s
     free(lut);
 }
 
+/* src/quant.rs:353-376 (matvec_vq_nt): m inputs transposed in xt [cols][m], blocks of 8 positions, rows inner; every
+ * product goes straight into its position's sum, in (vector, j) order; out [m][rows] */
+ORC_API void orc_vq1_matvec_nt(const float *codebook, const uint8_t *indices, size_t rows, size_t cols, const float *xt, size_t m, float *out) {
+    const size_t vpr = cols / 16;
+    for (size_t t0 = 0; t0 < m; t0 += 8) {
+        for (size_t r = 0; r < rows; r++) {
+            const uint8_t *irow = indices + r * vpr;
+            float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (size_t v = 0; v < vpr; v++) {
+                const float *cb = codebook + (size_t)irow[v] * 16;
+                for (int j = 0; j < 16; j++) {
+                    const float wv = cb[j];
+                    const float *xc = xt + (v * 16 + j) * m + t0;
+                    for (int p = 0; p < 8; p++) sum[p] += wv * xc[p];
+                }
+            }
+            for (int p = 0; p < 8; p++) out[(t0 + p) * rows + r] = sum[p];
+        }
+    }
+}
+
 /* ------------------------------------------------------- mxfp4 matvecs */
 
 /* src/mxfp4.rs:409-418: one row of the q8-integer path */

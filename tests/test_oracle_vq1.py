@@ -64,3 +64,36 @@ def test_closed_form_and_explicit_replay():
     x1[37] = 2.0
     one = oracle.vq1_matvec(cb, idx, 64, 256, x1)
     assert np.array_equal(one, cb[idx[:, 2], 5] * np.float32(2.0))
+
+
+def nt_case(rows, cols, m, seed):
+    cb, idx, _ = case(rows, cols, Rng(seed))
+    xt = np.random.default_rng(seed).standard_normal((cols, m)).astype(np.float32)
+    return cb, idx, xt
+
+
+def test_batched_form_closed_form_and_explicit_replay():
+    """matvec_vq_nt (src/quant.rs:353-376): one running sum per (row, position) over all cols products, in (vector, j) order."""
+    rows, cols, m = 24, 96, 16
+    cb, idx, xt = nt_case(rows, cols, m, 11)
+    got = oracle.vq1_matvec_nt(cb, idx, rows, cols, xt, m)
+    assert got.shape == (m, rows)
+    w = cb[idx].reshape(rows, cols)
+    want = (w.astype(np.float64) @ xt.astype(np.float64)).T
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+    # explicit f32 replay of a few (row, position) pairs: a single chain over the columns, multiply then add
+    for r, p in ((0, 0), (5, 9), (23, 15)):
+        s = np.float32(0)
+        for c in range(cols):
+            s = np.float32(s + np.float32(w[r, c] * xt[c, p]))
+        assert got[p, r].view(np.uint32) == s.view(np.uint32)
+    # the chain is not the per-vector sum of matvec_vq: same value to rounding, position by position
+    for p in (0, 7, 8):
+        one = oracle.vq1_matvec(cb, idx, rows, cols, np.ascontiguousarray(xt[:, p]))
+        assert np.max(np.abs(one - got[p])) <= 1e-5 * np.max(np.abs(one))
+    # a one-hot column of xt picks single codebook values, for its position only
+    x1 = np.zeros((cols, 8), np.float32)
+    x1[37, 3] = 2.0
+    o = oracle.vq1_matvec_nt(cb, idx, rows, cols, x1, 8)
+    assert np.array_equal(o[3], cb[idx[:, 2], 5] * np.float32(2.0))
+    assert not o[[0, 1, 2, 4, 5, 6, 7]].any()
