@@ -11,7 +11,8 @@
 //     perfectly coalesced 1 KiB requests.
 //   * the block index a lane owns repeats from tile to tile, so the lane keeps
 //     "its" 32 activations (as f16 pairs) and block scale in registers for the
-//     whole kernel: the activation is staged once per workgroup through LDS.
+//     whole kernel; they are loaded straight from global memory (no LDS, no
+//     barrier) behind the first two blocks of weight loads.
 //   * q8 mode: nibbles -> f16 by v_cvt_scalef32_pk_f16_fp4, activation bytes as
 //     f16 integers, v_dot2_f32_f16 accumulation.  Every term is a multiple of 0.5
 //     below 2^15, so the f32 accumulation is exact: h = idot/2 and the block
@@ -65,10 +66,6 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     constexpr int T = TILE / 64;
     constexpr int RT = TILE / NB;
     static_assert(RT <= 2 && T <= 8, "tile shape not covered by the fast path");
-    // f16 pairs kept as 32-bit words: written and read through the same type
-    __shared__ __attribute__((aligned(16))) uint32_t xh[NB * 16];
-    __shared__ float xsc[NB];
-
     const int mat = blockIdx.y;
     // uniform pointers in scalar registers + 32-bit lane offsets: the loads take the scalar-base form
     const uint8_t *packed = mk_uniform_ptr(a.packed ? a.packed : a.packed_ptrs[mat]);
@@ -112,32 +109,31 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
             }
         }
     };
-    // the first register block is requested before the activation is staged:
-    // the weight stream does not wait for the prologue
+    // both register blocks are requested before the activation is fetched: the
+    // weight stream does not wait for the prologue
     load_block(wa, sa, 0);
+    load_block(wb, sb, U);
 
-    // stage the activation: int8 -> f16 (exact), 4 values per thread per step
-    for (int i = threadIdx.x; i < NB * 8; i += 256) {
-        uint32_t v = reinterpret_cast<const uint32_t *>(xq)[i];
-        mk_h2 lo, hi;
-        lo.x = (_Float16)(float)(int8_t)(v & 255u);
-        lo.y = (_Float16)(float)(int8_t)((v >> 8) & 255u);
-        hi.x = (_Float16)(float)(int8_t)((v >> 16) & 255u);
-        hi.y = (_Float16)(float)(int8_t)(v >> 24);
-        xh[i * 2] = __builtin_bit_cast(uint32_t, lo);
-        xh[i * 2 + 1] = __builtin_bit_cast(uint32_t, hi);
-    }
-    for (int i = threadIdx.x; i < NB; i += 256) xsc[i] = xs[i];
-    __syncthreads();
-
+    // The lane's activation blocks go straight from global memory (7 KiB, cache
+    // resident) to registers, no LDS and no barrier: int8 -> f16 exactly, two
+    // values per v_perm: byte b ^ 0x80 in the mantissa of 1024.0 is 1152 + b.
     mk_h2 xr[T][16];
     float cf[T];
+    {
+        mk_h2 bias;
+        bias.x = bias.y = (_Float16)1152.0f;
 #pragma unroll
-    for (int t = 0; t < T; t++) {
-        const int g = (t * 64 + lane) % NB;
+        for (int t = 0; t < T; t++) {
+            const int g = (t * 64 + lane) % NB;
+            const mk_i4 v0 = mk_ldg128(xq + g * 32), v1 = mk_ldg128(xq + g * 32 + 16);
+            cf[t] = xs[g];
 #pragma unroll
-        for (int k = 0; k < 16; k++) xr[t][k] = __builtin_bit_cast(mk_h2, xh[g * 16 + k]);
-        cf[t] = xsc[g];
+            for (int j = 0; j < 8; j++) {
+                const uint32_t u = (uint32_t)(j < 4 ? v0[j] : v1[j - 4]) ^ 0x80808080u;
+                xr[t][2 * j] = __builtin_bit_cast(mk_h2, __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u)) - bias;
+                xr[t][2 * j + 1] = __builtin_bit_cast(mk_h2, __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u)) - bias;
+            }
+        }
     }
 
     auto compute_block = [&](const mk_i4(*w)[T], const uint32_t(*sc)[T], int k0) {
@@ -170,10 +166,10 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     // the prefetches are unconditional (past the end they re-read a valid tile):
     // a load under a branch forces a full wait at the join
     for (int k0 = 0; k0 < my_tiles; k0 += 2 * U) {
-        load_block(wb, sb, k0 + U);
         compute_block(wa, sa, k0);
         load_block(wa, sa, k0 + 2 * U);
         compute_block(wb, sb, k0 + U);
+        load_block(wb, sb, k0 + 3 * U);
     }
 }
 
