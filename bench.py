@@ -354,8 +354,15 @@ def bench_gemm(torch):
     pl, sl = [m[0] for m in mats], [m[1] for m in mats]
     m = int(xg.shape[0])
 
+    # the expert pointer tables and the result buffer are built once (a resident expert table, as mk_bin_load_experts
+    # gives): the timed step is the C-ABI call alone
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    mkp = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device="cuda")
+    pp, sp = mkp(pl), mkp(sl)
+    out_g = torch.empty((m, inter), dtype=torch.float32, device="cuda")
+
     def step():
-        model.grouped_gemm_mxfp8(pl, sl, inter, d, codes, exps, offsets)
+        check(lib.mk_dev_mxfp4_grouped_gemm(ptr(pp), ptr(sp), ne, inter, d, ptr(codes), ptr(exps), ptr(offsets), m, ptr(out_g), cur_stream()))
 
     ms = time_region(torch, step, 10, warmup=2)
     used = int((counts > 0).sum())
@@ -372,14 +379,16 @@ def bench_gemm(torch):
     cl, el = dequant.quantize_mxfp8(xl)
     off2 = torch.arange(0, 9, dtype=torch.int32, device="cuda") * M
 
-    def step2():
-        model.grouped_gemm_mxfp8(pl[:8], sl[:8], inter, d, cl, el, off2)
+    out_l = torch.empty((8 * M, inter), dtype=torch.float32, device="cuda")
 
-    ms2 = time_region(torch, step2, 5, warmup=1)
+    def step2():
+        check(lib.mk_dev_mxfp4_grouped_gemm(ptr(pp), ptr(sp), 8, inter, d, ptr(cl), ptr(el), ptr(off2), 8 * M, ptr(out_l), cur_stream()))
+
+    ms2 = time_region(torch, step2, 20, warmup=3)
     fl2 = 2.0 * 8 * M * inter * d
     res["large_m"] = {"rows_per_expert": M, "experts": 8, "ms": ms2, "tflops": fl2 / (ms2 * 1e-3) / 1e12,
                       "mfma_frac_fp8_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
-    del cl, el, xl
+    del cl, el, xl, out_l
     # the whole expert section of the prefill layer on the device (grouping, gather + MXFP8, gate, up, activation,
     # down, combine): mk_dev_moe_prefill.  The gate matrices above are reused as W1; W3 and W2 are drawn here.
     w3 = [rand_mxfp4(torch, g, inter, d) for _ in range(ne)]

@@ -24,6 +24,8 @@
 // to 64 tokens.  The streaming one (cols % 512 == 0, below) is the one the
 // model shapes take.  At the prefill shapes (about 16 tokens per expert) the
 // work is bound by the weight stream, not by the MFMA.
+#include <algorithm>
+
 #include "mk_common.h"
 
 namespace {
@@ -183,7 +185,7 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // FULL: the weight loads take whole 128-byte lines (see below).  NT: they are non-temporal.  Measured: 8 experts x 512
 // tokens (eight passes over each expert's weights) 495 -> 403 us with FULL, 459 us with FULL + NT; prefill shape (one pass,
 // at most 32 tokens per expert) 488 -> 504 us with FULL alone, 451 us with FULL + NT.
-template <int MC, bool FULL, bool NT, bool PIN>
+template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -301,33 +303,60 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         pin_acc(rt);
     };
 
-    load_unit(wa, sa, 0, 0);
-    stage_load(0);
-    __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
-    stage_store(lds);
-    __syncthreads();
-#pragma unroll 1
-    for (int kt = 0; kt < ktiles; kt++) {
-        const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
-        stage_load(kt + 1);
-        load_unit(wb, sb, kt, 1);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        compute_unit(wa, sa, 0, buf);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        load_unit(wa, sa, kt, 2);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        compute_unit(wb, sb, 1, buf);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        load_unit(wb, sb, kt, 3);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        compute_unit(wa, sa, 2, buf);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        load_unit(wa, sa, kt + 1, 0);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        compute_unit(wb, sb, 3, buf);
-        if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-        stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+    if constexpr (DEEP) {
+        // Four register blocks, one per row tile: the unit of row tile rt for K tile kt + 1 is requested as soon as the
+        // unit of K tile kt has been used, three units of matrix work ahead of its use.
+        mk_i4 w4[4][KT_STEPS], s4[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; rt++) load_unit(w4[rt], s4[rt], 0, rt);
+        stage_load(0);
+        __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
+        stage_store(lds);
         __syncthreads();
+#pragma unroll 1
+        for (int kt = 0; kt < ktiles; kt++) {
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
+            stage_load(kt + 1);
+#pragma unroll
+            for (int rt = 0; rt < 4; rt++) {
+                if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+                compute_unit(w4[rt], s4[rt], rt, buf);
+                if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+                load_unit(w4[rt], s4[rt], kt + 1, rt);
+            }
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+            __syncthreads();
+        }
+    } else {
+        load_unit(wa, sa, 0, 0);
+        stage_load(0);
+        __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
+        stage_store(lds);
+        __syncthreads();
+#pragma unroll 1
+        for (int kt = 0; kt < ktiles; kt++) {
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
+            stage_load(kt + 1);
+            load_unit(wb, sb, kt, 1);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            compute_unit(wa, sa, 0, buf);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            load_unit(wa, sa, kt, 2);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            compute_unit(wb, sb, 1, buf);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            load_unit(wb, sb, kt, 3);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            compute_unit(wa, sa, 2, buf);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            load_unit(wa, sa, kt + 1, 0);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            compute_unit(wb, sb, 3, buf);
+            if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+            __syncthreads();
+        }
     }
 #pragma unroll
     for (int rt = 0; rt < 4; rt += 2) {
@@ -356,8 +385,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 // Two instantiations share the grid: groups of up to 32 tokens (the prefill
 // case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
 // workgroup whose group belongs to the other one exits.
-template <int MC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2 : 1))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
+// VAR (large groups only): bit 0 = pinned instruction order with the weights as the M operand, bit 1 = four register
+// blocks of weights in flight, bit 2 = two waves per SIMD.
+template <int MC, int VAR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((MC == 2 || (VAR & 4)) ? 2 : 1))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
     // the plain order the workgroups of one group land on all of them and each fetches the group's activation rows for
@@ -384,18 +415,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MC == 2 ? 2
         if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
         else gemm_pass<2, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
     } else {
+        // the 64-token passes of a group are dealt to gridDim.y workgroups: a few large groups still fill the chip
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 16 * MC) gemm_pass<MC, true, false, false>(a, packed, scales, out, rb, base, tok1, lds);
+        for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
+            gemm_pass<MC, true, false, (VAR & 1) != 0, (VAR & 2) != 0>(a, packed, scales, out, rb, base, tok1, lds);
     }
 }
 
-template <int MC>
-int launch_stream(const GemmArgs &a, hipStream_t st) {
-    const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks));
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), 2 * a_buf_bytes(MC));
+template <int MC, int VAR>
+int launch_stream_var(const GemmArgs &a, size_t m, hipStream_t st) {
+    // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
+    // average group size (one per 64 tokens, at most 16); a workgroup without a pass exits at once.
+    unsigned passes = 1;
+    if (MC == 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
+    const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, VAR>), 2 * a_buf_bytes(MC));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL(mxfp4_grouped_gemm_stream_kernel<MC>, grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
+    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, VAR>), grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
+}
+
+template <int MC>
+int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
+    if (MC == 2) return launch_stream_var<2, 0>(a, m, st);
+    switch (mk_env_int("MK_GEMM_LARGE_VAR", 7)) {
+        case 1: return launch_stream_var<4, 1>(a, m, st);
+        case 2: return launch_stream_var<4, 2>(a, m, st);
+        case 3: return launch_stream_var<4, 3>(a, m, st);
+        case 5: return launch_stream_var<4, 5>(a, m, st);
+        case 7: return launch_stream_var<4, 7>(a, m, st);
+        default: return launch_stream_var<4, 0>(a, m, st);
+    }
 }
 
 }  // namespace
@@ -428,8 +478,8 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         a.n_groups = (int)n_groups;
         a.n_mats = n_mats;
         a.row_blocks = (int)row_blocks;
-        int st = launch_stream<2>(a, (hipStream_t)stream);
-        if (st == MK_OK && m > 32) st = launch_stream<4>(a, (hipStream_t)stream);
+        int st = launch_stream<2>(a, m, (hipStream_t)stream);
+        if (st == MK_OK && m > 32) st = launch_stream<4>(a, m, (hipStream_t)stream);
         return st;
     }
     for (int k = 0; k < n_mats; k++) {

@@ -36,7 +36,9 @@ def run_case(rows, cols, counts, seed):
 
 
 @pytest.mark.parametrize("rows,cols,counts", [(64, 128, [16]), (128, 256, [3, 0, 17, 1]), (200, 1024, [70, 5]), (2048, 7168, [9, 24]),
-                                              (7168, 2048, [16, 1, 40]), (300, 512, [0, 33, 32, 17, 64, 65])])
+                                              (7168, 2048, [16, 1, 40]), (300, 512, [0, 33, 32, 17, 64, 65]),
+                                              # large groups: their 64-token passes are dealt to several workgroups
+                                              (512, 1024, [300, 2, 130, 64]), (256, 512, [700])])
 def test_grouped_gemm(rows, cols, counts):
     got, want, plain = run_case(rows, cols, counts, len(counts) + rows)
     assert rel_l2(got, want) <= 1e-5
