@@ -131,11 +131,10 @@ struct GemmArgs {
     int n_groups, n_mats, row_blocks;
 };
 
-// Small groups (PIN): the weights are the instruction's M operand and the token rows its N operand, so a lane of the
-// 16 x 16 result holds four consecutive weight rows of one token row: one 16-byte store.  The kernel for large groups
-// keeps the token rows as M (the other way round it lost a tenth: 400 -> 441 us on 8 experts x 512 tokens).  (With the roles the other way round a lane holds
-// one weight row of four tokens and every value is a store of its own; on the down projection of the prefill shape those
-// stores took 100 of the kernel's 400 us.)
+// PIN: the weights are the instruction's M operand and the token rows its N operand, so a lane of the 16 x 16 result
+// holds four consecutive weight rows of one token row: one 16-byte store.  (With the roles the other way round a lane
+// holds one weight row of four tokens and every value is a store of its own; on the down projection of the prefill
+// shape those stores took 100 of the kernel's 400 us.)
 template <bool NT>
 __device__ __forceinline__ void store_tile(float *out, int rows, int t, int tok1, int row, const mk_f4 &v) {
     if (t >= tok1) return;
@@ -181,10 +180,24 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // of the K tile, behind a wait for every load in flight.  An empty volatile statement that takes a unit's accumulators
 // keeps its matrix instructions in front of the next unit's loads; scheduling barriers keep the loads in place.  Prefill
 // shape: 256 -> 167 registers (three workgroups per CU), gate GEMM 450 -> 409 us, down GEMM 463 -> 403 us.  The kernel for
-// larger groups (four token tiles, accumulators in the second register file) lost by it (403 -> 474 us) and stays as it was.
+// larger groups lost by it while a group's passes ran one after the other on 64 workgroups (403 -> 474 us); with the
+// passes dealt to the whole chip it runs pinned too (DEEP below).
 // FULL: the weight loads take whole 128-byte lines (see below).  NT: they are non-temporal.  Measured: 8 experts x 512
 // tokens (eight passes over each expert's weights) 495 -> 403 us with FULL, 459 us with FULL + NT; prefill shape (one pass,
 // at most 32 tokens per expert) 488 -> 504 us with FULL alone, 451 us with FULL + NT.
+// DEEP: four register blocks of weights, one per row tile, each re-requested for the next K tile as soon as it has
+// been used (three units of matrix work between issue and use) instead of two alternating blocks.
+// Large groups (8 experts x 512 tokens, 120 GFLOP): 403 us while the eight 64-token passes of a group ran one after the
+// other on 64 workgroups; 93 us (1.29 PFLOP/s) with the passes dealt to 512 workgroups, pinned order, DEEP and two
+// workgroups per CU.  Counters on that shape: the matrix cores are busy 27 us; waves spend half of their time waiting
+// for loads although the L2 answers in 270 cycles on average -- the vector cache handles 94k accesses per CU, about a
+// cycle each.  Per K tile a workgroup moves 64 KB of weights, 33 KB of activations and 16 KB of scale bytes through it
+// for 16.8 MFLOP: at this tile (256 rows x 64 tokens) the vector cache saturates at about the rate measured.  A
+// step-major pass (the K tile walked step by step with all four row tiles' weights in registers, activation operands
+// read from LDS once per step for all of them, exchange of the whole-line loads under the matrix instructions, the
+// barrier passed before the last step) was built and measured at 84-100 us -- the same; so was the operand's own load
+// mapping (a lane per row: 53 cache accesses per load instruction).  What would help is a larger tile per workgroup
+// (256 x 128: 256 FLOP per byte through the cache) and scale bytes fetched once per row instead of by four lanes.
 template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds) {
@@ -385,10 +398,8 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 // Two instantiations share the grid: groups of up to 32 tokens (the prefill
 // case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
 // workgroup whose group belongs to the other one exits.
-// VAR (large groups only): bit 0 = pinned instruction order with the weights as the M operand, bit 1 = four register
-// blocks of weights in flight, bit 2 = two waves per SIMD.
-template <int MC, int VAR>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((MC == 2 || (VAR & 4)) ? 2 : 1))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
+template <int MC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
     // the plain order the workgroups of one group land on all of them and each fetches the group's activation rows for
@@ -418,34 +429,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((MC == 2 ||
         // the 64-token passes of a group are dealt to gridDim.y workgroups: a few large groups still fill the chip
 #pragma unroll 1
         for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
-            gemm_pass<MC, true, false, (VAR & 1) != 0, (VAR & 2) != 0>(a, packed, scales, out, rb, base, tok1, lds);
+            gemm_pass<MC, true, false, true, true>(a, packed, scales, out, rb, base, tok1, lds);
     }
 }
 
-template <int MC, int VAR>
-int launch_stream_var(const GemmArgs &a, size_t m, hipStream_t st) {
+template <int MC>
+int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
     // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
     // average group size (one per 64 tokens, at most 16); a workgroup without a pass exits at once.
     unsigned passes = 1;
     if (MC == 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
     const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, VAR>), 2 * a_buf_bytes(MC));
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), 2 * a_buf_bytes(MC));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, VAR>), grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
+    hipLaunchKernelGGL(mxfp4_grouped_gemm_stream_kernel<MC>, grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
-}
-
-template <int MC>
-int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
-    if (MC == 2) return launch_stream_var<2, 0>(a, m, st);
-    switch (mk_env_int("MK_GEMM_LARGE_VAR", 7)) {
-        case 1: return launch_stream_var<4, 1>(a, m, st);
-        case 2: return launch_stream_var<4, 2>(a, m, st);
-        case 3: return launch_stream_var<4, 3>(a, m, st);
-        case 5: return launch_stream_var<4, 5>(a, m, st);
-        case 7: return launch_stream_var<4, 7>(a, m, st);
-        default: return launch_stream_var<4, 0>(a, m, st);
-    }
 }
 
 }  // namespace
