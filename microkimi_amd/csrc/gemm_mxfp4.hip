@@ -107,8 +107,10 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 //     that no wait is forced.  Units that gave a row shorter runs (64 or 128
 //     bytes, more row tiles per unit) were measured slower, whatever their
 //     bytes in flight;
-//   * a row's 16 scale bytes of the K tile come as ONE 16-byte load (a lane then
-//     shifts out the byte of its step and K block) instead of a byte per step.
+//   * the 16 scale bytes per weight row and K tile are fetched once per
+//     workgroup (thread i: row i, one 16-byte load) and staged in LDS with the
+//     activation tile; a lane reads its row's 16 bytes from there and shifts out
+//     the byte of its step and K block.
 //
 // Loads take the form "uniform base + 32-bit lane offset".  The K offset goes
 // through readfirstlane, which hides the loop counter from the induction
@@ -116,7 +118,8 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 constexpr int KT_STEPS = 4;
 constexpr int A_STRIDE = 512 + 16;  // LDS row stride of the activation tile: 16 rows fall in distinct banks
 constexpr int a_codes_bytes(int mc) { return 16 * mc * A_STRIDE; }
-constexpr int a_buf_bytes(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }  // codes, then 16 scale bytes per token
+constexpr int a_wsc_off(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }      // codes, then 16 scale bytes per token,
+constexpr int a_buf_bytes(int mc) { return a_wsc_off(mc) + 256 * 16; }            // then the K tile's 16 scale bytes of the 256 weight rows
 
 // One launch covers n_mats (1 or 2) weight matrices per group that share the activation rows (gate and up): matrix m
 // of group e is packed_ptrs[m][e], its result goes to out[m].
@@ -212,7 +215,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // of all 16 rows, lane (kb, n) reading bytes 16 kb .. of row n (every line is then requested by two loads).
     static_assert(KT_STEPS == 4, "two lines of 128 bytes per row and K tile");
     const int r3 = lane >> 3, c8 = lane & 7;
-    uint32_t woff[4][FULL ? 2 : 1], soff[4];
+    uint32_t woff[4][FULL ? 2 : 1];
 #pragma unroll
     for (int rt = 0; rt < 4; rt++) {
         if constexpr (FULL) {
@@ -221,22 +224,25 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         } else {
             woff[rt][0] = (uint32_t)min(row0 + rt * 16 + n, a.rows - 1) * (uint32_t)(cols / 2) + kb * 16;
         }
-        soff[rt] = (uint32_t)min(row0 + rt * 16 + n, a.rows - 1) * (uint32_t)nb;
     }
     // after the lane rotation below, lane (kg, x, r3) holds what lane (r3, x, kg) loaded
     const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
-    mk_i4 wa[KT_STEPS], wb[KT_STEPS], sa, sb;
-    auto load_unit = [&](mk_i4 *w, mk_i4 &sc, int kt, int rt) {
+    mk_i4 wa[KT_STEPS], wb[KT_STEPS];
+    auto load_unit = [&](mk_i4 *w, int kt, int rt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
 #pragma unroll
         for (int j = 0; j < KT_STEPS; j++)
             if constexpr (FULL && NT) w[j] = mk_ldg128_off_nt(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
             else if constexpr (FULL) w[j] = mk_ldg128_off(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
             else w[j] = mk_ldg128_off(packed, woff[rt][0] + ku * (KT_STEPS * 64) + j * 64);
-        sc = mk_ldg128_off(scales, soff[rt] + ku * 16);
     };
     // activation tile staging: chunk i = tid + 256 k -> token i / 32, 16-byte chunk i % 32
-    mk_i4 st[2 * MC], ste;
+    // The K tile's scale bytes of the workgroup's 256 weight rows (16 per row) go through LDS with the activation
+    // tile: thread i fetches row i's once.  Fetched by the lanes that use them (a lane per row, four lanes of a
+    // row the same 16 bytes) they were 4 of a wave's 29 loads per K tile and about half of its vector-cache
+    // accesses: a 16-byte load whose lanes sit in 16 different lines is looked up once per lane and pass.
+    mk_i4 st[2 * MC], ste, stw;
+    const uint32_t wsoff = (uint32_t)min(rb * 256 + tid, a.rows - 1) * (uint32_t)nb;
     uint32_t coff[2 * MC];  // the host checks that tokens x cols stays below 2^32
 #pragma unroll
     for (int k = 0; k < 2 * MC; k++) {
@@ -249,6 +255,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
         for (int k = 0; k < 2 * MC; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
         ste = mk_ldg128_off(a.exps, eoff + ku * 16);
+        stw = mk_ldg128_off(scales, wsoff + ku * 16);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
@@ -257,6 +264,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             *reinterpret_cast<mk_i4 *>(buf + (i >> 5) * A_STRIDE + (i & 31) * 16) = st[k];
         }
         if (tid < 16 * MC) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC) + tid * 16) = ste;
+        *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC) + tid * 16) = stw;
     };
     mk_f4 acc[4][MC];
 #pragma unroll
@@ -264,7 +272,8 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
         for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto mma_unit = [&](const mk_i4 *w, const mk_i4 &sc, int rt, const uint8_t *buf) {
+    auto mma_unit = [&](const mk_i4 *w, int rt, const uint8_t *buf) {
+        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC) + (wave * 64 + rt * 16 + n) * 16);
 #pragma unroll
         for (int c = 0; c < MC; c++) {
             const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC) + (c * 16 + n) * 16);
@@ -292,9 +301,9 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     };
     // One unit: 4 steps x MC token tiles.  The LDS reads of the activation operands do not depend on the
     // row tile, so after inlining the four calls of a K tile share them.
-    auto compute_unit = [&](const mk_i4 *wl, const mk_i4 &sc, int rt, const uint8_t *buf) {
+    auto compute_unit = [&](const mk_i4 *wl, int rt, const uint8_t *buf) {
         if constexpr (!FULL) {
-            mma_unit(wl, sc, rt, buf);
+            mma_unit(wl, rt, buf);
             pin_acc(rt);
             return;
         }
@@ -312,16 +321,16 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 w[2 * i + 1][k] = __builtin_amdgcn_update_dpp(rb, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);  // lanes 0-7 of a row <- ra
             }
         }
-        mma_unit(w, sc, rt, buf);
+        mma_unit(w, rt, buf);
         pin_acc(rt);
     };
 
     if constexpr (DEEP) {
         // Four register blocks, one per row tile: the unit of row tile rt for K tile kt + 1 is requested as soon as the
         // unit of K tile kt has been used, three units of matrix work ahead of its use.
-        mk_i4 w4[4][KT_STEPS], s4[4];
+        mk_i4 w4[4][KT_STEPS];
 #pragma unroll
-        for (int rt = 0; rt < 4; rt++) load_unit(w4[rt], s4[rt], 0, rt);
+        for (int rt = 0; rt < 4; rt++) load_unit(w4[rt], 0, rt);
         stage_load(0);
         __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
         stage_store(lds);
@@ -333,16 +342,16 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
             for (int rt = 0; rt < 4; rt++) {
                 if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-                compute_unit(w4[rt], s4[rt], rt, buf);
+                compute_unit(w4[rt], rt, buf);
                 if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-                load_unit(w4[rt], s4[rt], kt + 1, rt);
+                load_unit(w4[rt], kt + 1, rt);
             }
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
             __syncthreads();
         }
     } else {
-        load_unit(wa, sa, 0, 0);
+        load_unit(wa, 0, 0);
         stage_load(0);
         __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
         stage_store(lds);
@@ -351,21 +360,21 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         for (int kt = 0; kt < ktiles; kt++) {
             const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
             stage_load(kt + 1);
-            load_unit(wb, sb, kt, 1);
+            load_unit(wb, kt, 1);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            compute_unit(wa, sa, 0, buf);
+            compute_unit(wa, 0, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            load_unit(wa, sa, kt, 2);
+            load_unit(wa, kt, 2);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            compute_unit(wb, sb, 1, buf);
+            compute_unit(wb, 1, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            load_unit(wb, sb, kt, 3);
+            load_unit(wb, kt, 3);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            compute_unit(wa, sa, 2, buf);
+            compute_unit(wa, 2, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            load_unit(wa, sa, kt + 1, 0);
+            load_unit(wa, kt + 1, 0);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            compute_unit(wb, sb, 3, buf);
+            compute_unit(wb, 3, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
             __syncthreads();
