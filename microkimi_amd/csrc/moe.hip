@@ -23,6 +23,10 @@ int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const u
                              size_t cols, const int8_t *xq, const float *xs, const float *xf, const int32_t *x_index, float *const *out_ptrs,
                              hipStream_t st);
 
+int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t rows, size_t cols,
+                   const int8_t *xq, const float *xs, const int32_t *arow, const int32_t *goff, const int32_t *gexp, const int32_t *ngroups,
+                   const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream);
+
 namespace {
 
 constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
@@ -47,6 +51,13 @@ struct Workspace {
     float *g;     // [P][inter]   (composed path)
     float *u;     // [P][inter]
     float *o;     // [P][d]
+    // batched path: the pairs grouped by expert
+    int32_t *order;    // [P] grouped row -> pair
+    int32_t *pos;      // [P] pair -> grouped row
+    int32_t *rtok;     // [P] grouped row -> token
+    int32_t *goff;     // [P + 1] first grouped row of every group
+    int32_t *gexp;     // [P] expert of every group
+    int32_t *ngroups;  // [2]: number of groups, index of the largest group
     size_t bytes;
 };
 
@@ -82,6 +93,12 @@ Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, siz
     w.g = (float *)take(P * inter * 4);
     w.u = (float *)take(P * inter * 4);
     w.o = (float *)take(P * d * 4);
+    w.order = (int32_t *)take(P * 4);
+    w.pos = (int32_t *)take(P * 4);
+    w.rtok = (int32_t *)take(P * 4);
+    w.goff = (int32_t *)take((P + 1) * 4);
+    w.gexp = (int32_t *)take(P * 4);
+    w.ngroups = (int32_t *)take(8);
     w.bytes = off;
     return w;
 }
@@ -494,6 +511,115 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     out[(size_t)t * d + j] = y;
 }
 
+// ------------------------------------------------------------ batched path
+// From 8 tokens the layer is taken expert by expert: the (token, slot) pairs are grouped by expert (stable: inside a
+// group in (token, slot) order), every group's rows go through the expert's matrices together on the matrix cores
+// with the exact q8 arithmetic (gemm_q8x.hip), so an expert that several tokens selected -- the shared expert: all of
+// them -- is read once.  Kernels: this grouping, quantize_q8 of the hidden rows, gate + up, activation with the q8 form
+// of the activation rows (matvec_packed's own step), down, and the weighted sum per token in slot order.
+constexpr int BATCHED_MAX_P = 1024;
+
+__global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, int shared, const int32_t *__restrict__ ids,
+                                                               const float *__restrict__ weights, int32_t *order, int32_t *pos, int32_t *rtok,
+                                                               int32_t *goff, int32_t *gexp, int32_t *ngroups, float *pw) {
+    __shared__ int e_l[BATCHED_MAX_P], se_l[BATCHED_MAX_P], start_l[BATCHED_MAX_P];
+    const int per = topk + (shared >= 0 ? 1 : 0), P = B * per, p = threadIdx.x;
+    int e = 0;
+    if (p < P) {
+        const int t = p / per, s = p % per;
+        e = s < topk ? ids[t * topk + s] : shared;
+        e_l[p] = e;
+        pw[p] = s < topk ? weights[t * topk + s] : 1.0f;
+    }
+    __syncthreads();
+    if (p < P) {
+        // stable rank of the pair among all pairs by expert id
+        int rank = 0;
+        for (int q = 0; q < P; q++) rank += (e_l[q] < e || (e_l[q] == e && q < p)) ? 1 : 0;
+        order[rank] = p;
+        pos[p] = rank;
+        rtok[rank] = p / per;
+        se_l[rank] = e;
+    }
+    __syncthreads();
+    if (p < P) start_l[p] = (p == 0 || se_l[p] != se_l[p - 1]) ? 1 : 0;
+    __syncthreads();
+    if (p < P) {
+        int g = 0;  // groups that start at or before grouped row p
+        for (int q = 0; q <= p; q++) g += start_l[q];
+        if (start_l[p]) {
+            goff[g - 1] = p;
+            gexp[g - 1] = se_l[p];
+        }
+        if (p == P - 1) {
+            goff[g] = P;
+            ngroups[0] = g;
+        }
+    }
+    __syncthreads();
+    // the largest group (ties: the first): thread p looks at the group that starts at grouped row p
+    __shared__ int best_l;
+    if (p == 0) best_l = 0;
+    __syncthreads();
+    int len = 0;
+    if (p < P && start_l[p]) {
+        int q = p + 1;
+        while (q < P && !start_l[q]) q++;
+        len = q - p;
+        atomicMax(&best_l, (len << 12) | (BATCHED_MAX_P - 1 - p));  // longest, then lowest start
+    }
+    __syncthreads();
+    if (p < P && start_l[p] && best_l == ((len << 12) | (BATCHED_MAX_P - 1 - p))) {
+        int g = 0;
+        for (int q = 0; q <= p; q++) g += start_l[q];
+        ngroups[1] = g - 1;
+    }
+}
+
+// The activation of the grouped rows and its q8 form in one kernel (the block matvec_packed forms when it re-quantizes
+// its input for W2, src/q8.rs:57-68): 8 lanes per 32-block, four values each.
+__global__ __launch_bounds__(256) void moe_act_q8_grouped_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                                 const float *__restrict__ pw, const int32_t *__restrict__ order, int inter,
+                                                                 size_t n_blocks, int act_kind, float limit, int8_t *__restrict__ q,
+                                                                 float *__restrict__ scales) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_blocks * 8) return;  // whole groups of 8 lanes leave together
+    const mk_f4 gv = reinterpret_cast<const mk_f4 *>(g)[i], uv = reinterpret_cast<const mk_f4 *>(u)[i];
+    const float wgt = pw[order[(i * 4) / (size_t)inter]];
+    const mk_f4 v = {mk_act(act_kind, gv.x, uv.x, limit, wgt), mk_act(act_kind, gv.y, uv.y, limit, wgt), mk_act(act_kind, gv.z, uv.z, limit, wgt),
+                     mk_act(act_kind, gv.w, uv.w, limit, wgt)};
+    float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+    mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+    mx = fmaxf(mx, mk_dpp<0x141>(mx));
+    const float dx = mx / 127.0f;
+    uint32_t packed = 0;
+    if (dx != 0.0f) {
+        float qf[4];
+        mk_q8_round4(v, dx, qf);
+        packed = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                 ((uint32_t)(int)qf[3] << 24);
+    }
+    reinterpret_cast<uint32_t *>(q)[i] = packed;
+    if ((i & 7) == 0) scales[i >> 3] = dx;
+}
+
+// out[t][j] = sum_s w * o[pos(t, s)][j] in slot order (+ shared, unweighted)
+__global__ __launch_bounds__(256) void moe_combine_grouped_kernel(const float *__restrict__ o, const float *__restrict__ pw,
+                                                                  const int32_t *__restrict__ pos, int per, int topk, int d, int ds_rule,
+                                                                  float *__restrict__ out) {
+    const int t = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= d) return;
+    float y = 0.0f;
+    for (int s = 0; s < topk; s++) {
+        const float v = o[(size_t)pos[t * per + s] * d + j];
+        y = ds_rule ? mk_add(y, v) : mk_add(y, mk_mul(pw[t * per + s], v));
+    }
+    if (per > topk) y = mk_add(y, o[(size_t)pos[t * per + topk] * d + j]);
+    out[(size_t)t * d + j] = y;
+}
+
 }  // namespace
 
 extern "C" size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter) {
@@ -585,6 +711,36 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     const bool fast = mode == MK_MODE_Q8 && (nb == 32 || nb == 64 || nb == 128 || nb == 224) && (nbi == 32 || nbi == 64 || nbi == 128) &&
                       per <= MAX_PER && d % 2 == 0 && (size_t)per * nbi * 68 <= 150 * 1024;
     int s;
+    // batched path: q8 mode, both projections in K tiles of 512, enough tokens for experts to repeat
+    const bool batched = mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
+                         (int)B >= mk_env_int("MK_MOE_BATCHED_MIN", 8) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
+    if (batched) {
+        hipLaunchKernelGGL(moe_group_pairs_kernel, dim3(1), dim3(1024), 0, st, (int)B, (int)topk, shared, ids, weights, w.order, w.pos, w.rtok,
+                           w.goff, w.gexp, w.ngroups, w.pt.pw);
+        if ((s = mk_launch_status("moe_group_pairs")) != MK_OK) return s;
+        if ((s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
+        {
+            const uint8_t *const *pp[2] = {table->w1p, table->w3p};
+            const uint8_t *const *sp[2] = {table->w1s, table->w3s};
+            float *gu[2] = {w.g, w.u};
+            if ((s = mk_q8x_grouped(2, pp, sp, inter, d, w.xq, w.xs, w.rtok, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, gu, stream)) != MK_OK) return s;
+        }
+        {
+            const size_t n_blocks = P * inter / 32;
+            hipLaunchKernelGGL(moe_act_q8_grouped_kernel, dim3((unsigned)((n_blocks + 31) / 32)), dim3(256), 0, st, w.g, w.u, w.pt.pw, w.order,
+                               (int)inter, n_blocks, act_kind, limit, w.aq, w.as);
+            if ((s = mk_launch_status("moe_act_q8_grouped")) != MK_OK) return s;
+        }
+        {
+            const uint8_t *const *pp[1] = {table->w2p};
+            const uint8_t *const *sp[1] = {table->w2s};
+            float *oo[1] = {w.o};
+            if ((s = mk_q8x_grouped(1, pp, sp, d, inter, w.aq, w.as, nullptr, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, oo, stream)) != MK_OK) return s;
+        }
+        hipLaunchKernelGGL(moe_combine_grouped_kernel, dim3((unsigned)((d + 255) / 256), (unsigned)B), dim3(256), 0, st, w.o, w.pt.pw, w.pos, per,
+                           (int)topk, (int)d, act_kind == MK_ACT_DS ? 1 : 0, out);
+        return mk_launch_status("moe_combine_grouped");
+    }
     if (fast) {
         FusedArgs fa;
         fa.tab = *table;

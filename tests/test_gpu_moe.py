@@ -9,6 +9,36 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-5
 
 
+def rows_match_up_to_q8_flips(got, want, w2_of_token, d, inter, max_flips=2):
+    """The layer re-quantizes the f32 activation to q8 before W2 (matvec_packed's own step, src/mxfp4.rs:476-479), a
+    step function of its input: the gate/up sums here differ from the CPU's in their last bits (the order of the sum
+    over blocks, expf), so an activation that lies within a few ulp of a rounding boundary takes the other int8 value
+    (about one activation in 60 000).  Such a flip changes the token's row by exactly one column of that expert's W2
+    times one quantization step (4e-5 .. 4e-4 of the row).  Returns the number of such single-column differences
+    removed; asserts that a row needs at most max_flips of them and agrees to TOL otherwise."""
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4
+    flips = 0
+    for t in range(got.shape[0]):
+        diff = torch.from_numpy(got[t].astype(np.float64) - want[t].astype(np.float64)).cuda()
+        wn = float(np.linalg.norm(want[t]))
+        for _ in range(max_flips):
+            if float(diff.norm()) / wn <= TOL:
+                break
+            best = None
+            for p, sc in w2_of_token(t):
+                Wd = mxfp4.dequant(p, sc, d, inter).double()
+                c = (Wd.T @ diff) / (Wd.norm(dim=0) * diff.norm())
+                j = int(c.abs().argmax())
+                if best is None or abs(float(c[j])) > abs(best[0]):
+                    best = (float(c[j]), Wd[:, j].clone())
+            assert abs(best[0]) > 0.7, f"token {t}: a difference of {float(diff.norm()) / wn:.2e} that is not a q8 step of one activation"
+            diff = diff - best[1] * (best[1] @ diff) / (best[1] @ best[1])
+            flips += 1
+        assert float(diff.norm()) / wn <= TOL, f"token {t}: {float(diff.norm()) / wn:.2e}"
+    return flips
+
+
 def build(n_experts, d, inter, cfg=2):
     from microkimi_amd import model, workloads
     host = [(workloads.mxfp4_matrix(cfg, "w1", inter, d, e), workloads.mxfp4_matrix(cfg, "w3", inter, d, e),
@@ -31,6 +61,9 @@ def build(n_experts, d, inter, cfg=2):
     (7168, 2048, 12, 9, 8, 11, 0),    # benchmark shapes, two token groups in the gate/up kernel (8 + 1)
     (1024, 4096, 4, 5, 2, 3, 0),      # two rows of W1/W3 per wave
     (96, 64, 4, 2, 2, -1, 0),         # shape off the fast path (composed kernels)
+    (2048, 1024, 6, 8, 2, -1, 1),     # batched path (8 tokens and more: pairs grouped by expert), SiTU, no shared expert
+    (4096, 2048, 5, 11, 3, 4, 2),     # batched path, DeepSeek rule, groups of more than four tokens (several passes)
+    (7168, 2048, 12, 16, 8, 11, 0),   # batched path at the benchmark layer's shapes, batch 16
 ])
 def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
     torch = torch_cuda()
@@ -47,7 +80,10 @@ def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
     got = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
     want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=shared, mode=1, act_kind=act, limit=limit, threads=8)
     assert np.isfinite(want).all()
-    assert rel_l2(got, want) <= TOL
+    w2_dev = experts._keep[2]
+    used = lambda t: [w2_dev[int(e)] for e in ids[t]] + ([w2_dev[shared]] if shared >= 0 else [])
+    flips = rows_match_up_to_q8_flips(got, want, used, d, inter)
+    assert flips <= max(1, B // 3)
 
 
 def test_moe_decode_f32_mode():
@@ -80,7 +116,7 @@ def test_router_softmax_topk():
 def test_full_layer_257_experts_sampled_tokens():
     """Configuration 2 at its full size (256 routed + 1 shared expert at 2048 x 7168, 6 GB of MXFP4 drawn on the
     device, batch 16 routed by the seeded logits): the rows of sampled tokens against the oracle, which gets only the
-    nine experts of that token copied to the host.  Also: a token's row does not depend on its batch.
+    nine experts of that token copied to the host, at batch 16 (batched path) and at batch 1 (two-kernel path).
 
     The layer re-quantizes the f32 activation to q8 before W2 (matvec_packed's own step, src/mxfp4.rs:476-479), which
     is a step function of its input: the gate/up sums here differ from the CPU's in their last bits (the order of
@@ -114,25 +150,9 @@ def test_full_layer_257_experts_sampled_tokens():
         used = [int(e) for e in ids_h[tok]] + [ne]
         table = oracle.ExpertTable([host(w1[e]) for e in used], [host(w3[e]) for e in used], [host(w2[e]) for e in used], d, inter)
         local_ids = np.arange(topk, dtype=np.uint32)[None, :]
-        want = oracle.moe_decode(table, local_ids, wts_h[tok:tok + 1], (hidden[tok:tok + 1] * 0.02).astype(np.float32), shared=topk, mode=1, threads=8)[0]
-        diff = torch.from_numpy(got16[tok].astype(np.float64) - want).cuda()
-        wn = float(np.linalg.norm(want))
-        for _ in range(2):
-            if float(diff.norm()) / wn <= TOL:
-                break
-            # the single column of one of the token's W2 matrices that explains the difference
-            best = None
-            for e in used:
-                Wd = mxfp4.dequant(w2[e][0], w2[e][1], d, inter).double()
-                c = (Wd.T @ diff) / (Wd.norm(dim=0) * diff.norm())
-                j = int(c.abs().argmax())
-                if best is None or abs(float(c[j])) > abs(best[0]):
-                    best = (float(c[j]), Wd[:, j].clone())
-            assert abs(best[0]) > 0.7, f"token {tok}: a difference of {float(diff.norm()) / wn:.2e} that is not a q8 step of one activation"
-            col = best[1]
-            diff = diff - col * (col @ diff) / (col @ col)
-            flips += 1
-        assert float(diff.norm()) / wn <= TOL, f"token {tok}"
+        want = oracle.moe_decode(table, local_ids, wts_h[tok:tok + 1], (hidden[tok:tok + 1] * 0.02).astype(np.float32), shared=topk, mode=1, threads=8)
+        flips += rows_match_up_to_q8_flips(got16[tok:tok + 1], want, lambda t: [w2[e] for e in used], d, inter)
+        # batch 1 takes the two-kernel path, batch 16 the batched one: the same arithmetic per block, another order of the sum
         got1 = model.moe_decode(experts, ids[tok:tok + 1].contiguous(), wts[tok:tok + 1].contiguous(), x[tok:tok + 1].contiguous(), shared=ne, mode=1).cpu().numpy()
-        assert np.array_equal(got1[0], got16[tok])  # same kernels, same order of operations per token
-    assert flips <= 5
+        flips += rows_match_up_to_q8_flips(got1, want, lambda t: [w2[e] for e in used], d, inter)
+    assert flips <= 8
