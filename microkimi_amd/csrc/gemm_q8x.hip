@@ -23,7 +23,8 @@
 namespace {
 
 constexpr int QX_STEPS = 4;          // matrix instructions per K tile and row tile (K tile = 512 columns)
-constexpr int QX_TOK = 4;            // tokens per pass (two pairs: their accumulators and the weight blocks fit two waves per SIMD)
+constexpr int QX_TOK = 4;            // tokens per pass: two pairs (one pair per pass ran batch 16 at 508 us against 467: groups of three
+                                     // and four tokens then take a second pass over the weights)
 constexpr int QX_ROW = 528;          // LDS bytes of one code row (512 + 16: the a and b rows of a token 4 banks apart)
 constexpr int QX_TOK_STRIDE = 1152;  // LDS bytes between tokens (32 banks apart)
 constexpr int QX_DX_OFF = QX_TOK * QX_TOK_STRIDE;  // then 16 f32 block scales per token
@@ -62,13 +63,13 @@ __device__ __forceinline__ void qx_split(uint32_t q4, uint32_t &a_codes, uint32_
 }
 
 // One pass: up to QX_TOK tokens (NP pairs) of a group against the workgroup's 256 rows.
-template <int NP>
+template <int NP, int WAVES>
 __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                          uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
-    const int row0 = rb * 256 + wave * 64;
+    const int row0 = rb * (64 * WAVES) + wave * 64;
     // weight loads: whole 128-byte lines (8 rows x 128 bytes per load), see gemm_mxfp4.hip
     const int r3 = lane >> 3, c8 = lane & 7;
     uint32_t woff[4][2];
@@ -77,7 +78,7 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 #pragma unroll
         for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(row0 + rt * 16 + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
     const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
-    const uint32_t wsoff = (uint32_t)min(rb * 256 + tid, a.rows - 1) * (uint32_t)nb;
+    const uint32_t wsoff = (uint32_t)min(rb * (64 * WAVES) + tid, a.rows - 1) * (uint32_t)nb;
 
     // this lane as a column of the instruction: token t2 of the pair, phase p, part (0: a codes, 1: b codes)
     const int t2 = n >> 3, ph = (n >> 1) & 3, part = n & 1;
@@ -219,7 +220,9 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
         }
 }
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void q8x_grouped_kernel(Q8xArgs a) {
+// WAVES: 4 (a workgroup owns 256 rows) or 2 (128 rows: twice as many, shorter workgroups).
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2))) void q8x_grouped_kernel(Q8xArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int per_group = a.n_mats * a.row_blocks;
     // Regular workgroups: (group, matrix, row block), all passes of the group one after the other -- except for the
@@ -249,7 +252,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void q
     float *out = a.out[m];
 #pragma unroll 1
     for (int pass = first_pass; tok0 + QX_TOK * pass < tok1; pass += pass_step)
-        q8x_pass<QX_TOK / 2>(a, packed, scales, out, rb, tok0 + QX_TOK * pass, tok1, lds);
+        q8x_pass<QX_TOK / 2, WAVES>(a, packed, scales, out, rb, tok0 + QX_TOK * pass, tok1, lds);
 }
 
 }  // namespace
@@ -277,13 +280,22 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     a.ngroups = ngroups;
     a.gbig = gbig;
     a.n_mats = n_mats;
-    a.row_blocks = (int)((rows + 255) / 256);
+    // 128-row workgroups (twice as many, shorter) measured the same as 256-row ones on the benchmark layer (472 / 466 us)
+    const int waves = mk_env_int("MK_Q8X_WAVES", 4);
+    const size_t wg_rows = 64 * (size_t)waves;
+    a.row_blocks = (int)((rows + wg_rows - 1) / wg_rows);
     const size_t passes = (max_group_rows + QX_TOK - 1) / QX_TOK;
     const size_t regular = max_groups * n_mats * a.row_blocks, grid = regular + (passes - 1) * n_mats * a.row_blocks;
     MK_REQUIRE(passes >= 1 && grid < 0x7FFFFFFFull, "too many workgroups");
     a.regular = (int)regular;
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel), 2 * QX_BUF);
-    if (s != MK_OK) return s;
-    hipLaunchKernelGGL(q8x_grouped_kernel, dim3((unsigned)grid), dim3(256), 2 * QX_BUF, (hipStream_t)stream, a);
+    if (waves == 2) {
+        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<2>), 2 * QX_BUF);
+        if (s != MK_OK) return s;
+        hipLaunchKernelGGL(q8x_grouped_kernel<2>, dim3((unsigned)grid), dim3(128), 2 * QX_BUF, (hipStream_t)stream, a);
+    } else {
+        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<4>), 2 * QX_BUF);
+        if (s != MK_OK) return s;
+        hipLaunchKernelGGL(q8x_grouped_kernel<4>, dim3((unsigned)grid), dim3(256), 2 * QX_BUF, (hipStream_t)stream, a);
+    }
     return mk_launch_status("q8x_grouped");
 }

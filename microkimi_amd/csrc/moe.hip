@@ -522,7 +522,9 @@ constexpr int BATCHED_MAX_P = 1024;
 __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, int shared, const int32_t *__restrict__ ids,
                                                                const float *__restrict__ weights, int32_t *order, int32_t *pos, int32_t *rtok,
                                                                int32_t *goff, int32_t *gexp, int32_t *ngroups, float *pw) {
-    __shared__ int e_l[BATCHED_MAX_P], se_l[BATCHED_MAX_P], start_l[BATCHED_MAX_P];
+    __shared__ __attribute__((aligned(16))) int e_l[BATCHED_MAX_P], start_l[BATCHED_MAX_P];
+    __shared__ int se_l[BATCHED_MAX_P], goff_l[BATCHED_MAX_P + 1];
+    __shared__ int ng_l, best_l;
     const int per = topk + (shared >= 0 ? 1 : 0), P = B * per, p = threadIdx.x;
     int e = 0;
     if (p < P) {
@@ -530,12 +532,20 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
         e = s < topk ? ids[t * topk + s] : shared;
         e_l[p] = e;
         pw[p] = s < topk ? weights[t * topk + s] : 1.0f;
+    } else {
+        e_l[p] = 0x7FFFFFFF;  // behind every pair: the loops below read whole 16-byte groups
+        start_l[p] = 0;
     }
+    if (p == 0) best_l = 0;
     __syncthreads();
     if (p < P) {
         // stable rank of the pair among all pairs by expert id
         int rank = 0;
-        for (int q = 0; q < P; q++) rank += (e_l[q] < e || (e_l[q] == e && q < p)) ? 1 : 0;
+        for (int q = 0; q < P; q += 4) {
+            const mk_i4 v = *reinterpret_cast<const mk_i4 *>(e_l + q);
+#pragma unroll
+            for (int k = 0; k < 4; k++) rank += (v[k] < e || (v[k] == e && q + k < p)) ? 1 : 0;
+        }
         order[rank] = p;
         pos[p] = rank;
         rtok[rank] = p / per;
@@ -546,34 +556,28 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
     __syncthreads();
     if (p < P) {
         int g = 0;  // groups that start at or before grouped row p
-        for (int q = 0; q <= p; q++) g += start_l[q];
+        for (int q = 0; q <= p; q += 4) {
+            const mk_i4 v = *reinterpret_cast<const mk_i4 *>(start_l + q);
+#pragma unroll
+            for (int k = 0; k < 4; k++) g += (q + k <= p) ? v[k] : 0;
+        }
         if (start_l[p]) {
             goff[g - 1] = p;
+            goff_l[g - 1] = p;
             gexp[g - 1] = se_l[p];
         }
         if (p == P - 1) {
             goff[g] = P;
+            goff_l[g] = P;
             ngroups[0] = g;
+            ng_l = g;
         }
     }
     __syncthreads();
-    // the largest group (ties: the first): thread p looks at the group that starts at grouped row p
-    __shared__ int best_l;
-    if (p == 0) best_l = 0;
+    // the largest group (ties: the first)
+    if (p < ng_l) atomicMax(&best_l, ((goff_l[p + 1] - goff_l[p]) << 12) | (4095 - p));
     __syncthreads();
-    int len = 0;
-    if (p < P && start_l[p]) {
-        int q = p + 1;
-        while (q < P && !start_l[q]) q++;
-        len = q - p;
-        atomicMax(&best_l, (len << 12) | (BATCHED_MAX_P - 1 - p));  // longest, then lowest start
-    }
-    __syncthreads();
-    if (p < P && start_l[p] && best_l == ((len << 12) | (BATCHED_MAX_P - 1 - p))) {
-        int g = 0;
-        for (int q = 0; q <= p; q++) g += start_l[q];
-        ngroups[1] = g - 1;
-    }
+    if (p == 0) ngroups[1] = 4095 - (best_l & 4095);
 }
 
 // The activation of the grouped rows and its q8 form in one kernel (the block matvec_packed forms when it re-quantizes
