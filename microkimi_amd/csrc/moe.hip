@@ -519,54 +519,98 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
 // of the activation rows (matvec_packed's own step), down, and the weighted sum per token in slot order.
 constexpr int BATCHED_MAX_P = 1024;
 
+// Workgroup 0 groups the pairs; the others form the q8 blocks of the hidden rows (src/q8.rs:57-68, 8 lanes per
+// 32-block as mk_quantize_q8_kernel) -- one launch for the two steps in front of the gate/up GEMM.
 __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, int shared, const int32_t *__restrict__ ids,
                                                                const float *__restrict__ weights, int32_t *order, int32_t *pos, int32_t *rtok,
-                                                               int32_t *goff, int32_t *gexp, int32_t *ngroups, float *pw) {
-    __shared__ __attribute__((aligned(16))) int e_l[BATCHED_MAX_P], start_l[BATCHED_MAX_P];
-    __shared__ int se_l[BATCHED_MAX_P], goff_l[BATCHED_MAX_P + 1];
-    __shared__ int ng_l, best_l;
-    const int per = topk + (shared >= 0 ? 1 : 0), P = B * per, p = threadIdx.x;
-    int e = 0;
-    if (p < P) {
-        const int t = p / per, s = p % per;
-        e = s < topk ? ids[t * topk + s] : shared;
-        e_l[p] = e;
-        pw[p] = s < topk ? weights[t * topk + s] : 1.0f;
-    } else {
-        e_l[p] = 0x7FFFFFFF;  // behind every pair: the loops below read whole 16-byte groups
-        start_l[p] = 0;
+                                                               int32_t *goff, int32_t *gexp, int32_t *ngroups, float *pw,
+                                                               const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ xq,
+                                                               float *__restrict__ xs) {
+    if (blockIdx.x > 0) {
+        const size_t i = (size_t)(blockIdx.x - 1) * blockDim.x + threadIdx.x;
+        if (i >= n_blocks * 8) return;  // whole groups of 8 lanes leave together
+        const mk_f4 v = reinterpret_cast<const mk_f4 *>(x)[i];
+        float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+        mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+        mx = fmaxf(mx, mk_dpp<0x141>(mx));
+        const float dx = mx / 127.0f;
+        uint32_t packed = 0;
+        if (dx != 0.0f) {
+            float qf[4];
+            mk_q8_round4(v, dx, qf);
+            packed = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                     ((uint32_t)(int)qf[3] << 24);
+        }
+        reinterpret_cast<uint32_t *>(xq)[i] = packed;
+        if ((i & 7) == 0) xs[i >> 3] = dx;
+        return;
     }
-    if (p == 0) best_l = 0;
+    __shared__ __attribute__((aligned(16))) int e_l[BATCHED_MAX_P], start_l[BATCHED_MAX_P];
+    __shared__ int se_l[BATCHED_MAX_P], goff_l[BATCHED_MAX_P + 1], cnt_l[BATCHED_MAX_P];
+    __shared__ int ng_l, best_l;
+    const int per = topk + (shared >= 0 ? 1 : 0), P = B * per, tid = threadIdx.x;
+    {
+        int e = 0x7FFFFFFF;  // behind every pair: the loops below read whole 16-byte groups
+        if (tid < P) {
+            const int t = tid / per, s = tid % per;
+            e = s < topk ? ids[t * topk + s] : shared;
+            pw[tid] = s < topk ? weights[t * topk + s] : 1.0f;
+        }
+        e_l[tid] = e;
+        start_l[tid] = 0;
+        cnt_l[tid] = 0;
+    }
+    if (tid == 0) best_l = 0;
     __syncthreads();
-    if (p < P) {
+    // The P x P comparisons are spread over all 1024 threads: thread (p, part) counts over a slice of q.
+    const int parts = max(1, 1024 / P), p = tid % P, part = tid / P;
+    const int slice = ((P + parts - 1) / parts + 3) & ~3;  // a multiple of 4
+    const bool worker = part < parts;
+    const int q0 = part * slice, q1 = min(P, q0 + slice);
+    if (worker) {
         // stable rank of the pair among all pairs by expert id
+        const int e = e_l[p];
         int rank = 0;
-        for (int q = 0; q < P; q += 4) {
+        for (int q = q0; q < q1; q += 4) {
             const mk_i4 v = *reinterpret_cast<const mk_i4 *>(e_l + q);
 #pragma unroll
             for (int k = 0; k < 4; k++) rank += (v[k] < e || (v[k] == e && q + k < p)) ? 1 : 0;
         }
-        order[rank] = p;
-        pos[p] = rank;
-        rtok[rank] = p / per;
-        se_l[rank] = e;
+        if (rank) atomicAdd(&cnt_l[p], rank);
     }
     __syncthreads();
-    if (p < P) start_l[p] = (p == 0 || se_l[p] != se_l[p - 1]) ? 1 : 0;
+    if (tid < P) {
+        const int rank = cnt_l[tid];
+        order[rank] = tid;
+        pos[tid] = rank;
+        rtok[rank] = tid / per;
+        se_l[rank] = e_l[tid];
+    }
     __syncthreads();
-    if (p < P) {
-        int g = 0;  // groups that start at or before grouped row p
-        for (int q = 0; q <= p; q += 4) {
+    if (tid < P) {
+        start_l[tid] = (tid == 0 || se_l[tid] != se_l[tid - 1]) ? 1 : 0;
+        cnt_l[tid] = 0;
+    }
+    __syncthreads();
+    if (worker) {
+        int g = 0;  // groups that start at or before grouped row p, this thread's slice of them
+        for (int q = q0; q < q1 && q <= p; q += 4) {
             const mk_i4 v = *reinterpret_cast<const mk_i4 *>(start_l + q);
 #pragma unroll
             for (int k = 0; k < 4; k++) g += (q + k <= p) ? v[k] : 0;
         }
-        if (start_l[p]) {
-            goff[g - 1] = p;
-            goff_l[g - 1] = p;
-            gexp[g - 1] = se_l[p];
+        if (g) atomicAdd(&cnt_l[p], g);
+    }
+    __syncthreads();
+    if (tid < P) {
+        const int g = cnt_l[tid];
+        if (start_l[tid]) {
+            goff[g - 1] = tid;
+            goff_l[g - 1] = tid;
+            gexp[g - 1] = se_l[tid];
         }
-        if (p == P - 1) {
+        if (tid == P - 1) {
             goff[g] = P;
             goff_l[g] = P;
             ngroups[0] = g;
@@ -575,9 +619,9 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
     }
     __syncthreads();
     // the largest group (ties: the first)
-    if (p < ng_l) atomicMax(&best_l, ((goff_l[p + 1] - goff_l[p]) << 12) | (4095 - p));
+    if (tid < ng_l) atomicMax(&best_l, ((goff_l[tid + 1] - goff_l[tid]) << 12) | (4095 - tid));
     __syncthreads();
-    if (p == 0) ngroups[1] = 4095 - (best_l & 4095);
+    if (tid == 0) ngroups[1] = 4095 - (best_l & 4095);
 }
 
 // The activation of the grouped rows and its q8 form in one kernel (the block matvec_packed forms when it re-quantizes
@@ -719,10 +763,13 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     const bool batched = mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
                          (int)B >= mk_env_int("MK_MOE_BATCHED_MIN", 8) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
     if (batched) {
-        hipLaunchKernelGGL(moe_group_pairs_kernel, dim3(1), dim3(1024), 0, st, (int)B, (int)topk, shared, ids, weights, w.order, w.pos, w.rtok,
-                           w.goff, w.gexp, w.ngroups, w.pt.pw);
-        if ((s = mk_launch_status("moe_group_pairs")) != MK_OK) return s;
-        if ((s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
+        {
+            MK_REQUIRE(((uintptr_t)x & 15) == 0, "x must be 16-byte aligned");
+            const size_t n_blocks = B * d / 32;
+            hipLaunchKernelGGL(moe_group_pairs_kernel, dim3(1 + (unsigned)((n_blocks * 8 + 1023) / 1024)), dim3(1024), 0, st, (int)B, (int)topk,
+                               shared, ids, weights, w.order, w.pos, w.rtok, w.goff, w.gexp, w.ngroups, w.pt.pw, x, n_blocks, w.xq, w.xs);
+            if ((s = mk_launch_status("moe_group_pairs")) != MK_OK) return s;
+        }
         {
             const uint8_t *const *pp[2] = {table->w1p, table->w3p};
             const uint8_t *const *sp[2] = {table->w1s, table->w3s};
