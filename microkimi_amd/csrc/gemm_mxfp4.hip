@@ -199,7 +199,9 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // step-major pass (the K tile walked step by step with all four row tiles' weights in registers, activation operands
 // read from LDS once per step for all of them, exchange of the whole-line loads under the matrix instructions, the
 // barrier passed before the last step) was built and measured at 84-100 us -- the same; so was the operand's own load
-// mapping (a lane per row: 53 cache accesses per load instruction).  What would help is a larger tile per workgroup
+// mapping (a lane per row: 53 cache accesses per load instruction), and a form in which two row tiles share one read of
+// the activation operands (half the LDS reads: 101-111 us).  None of LDS reads, prefetch depth, waves per SIMD or the
+// load mapping is what holds this shape.  What would help is a larger tile per workgroup
 // (256 x 128: 256 FLOP per byte through the cache) and scale bytes fetched once per row instead of by four lanes.
 template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
