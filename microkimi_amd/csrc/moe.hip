@@ -512,7 +512,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
 }
 
 // ------------------------------------------------------------ batched path
-// From 8 tokens the layer is taken expert by expert: the (token, slot) pairs are grouped by expert (stable: inside a
+// From 4 tokens (the measured crossover: batch 3 140 / 154 us, batch 4 148 / 142 us, batch 5 229 / 216 us, two-kernel
+// path / this one) the layer is taken expert by expert: the (token, slot) pairs are grouped by expert (stable: inside a
 // group in (token, slot) order), every group's rows go through the expert's matrices together on the matrix cores
 // with the exact q8 arithmetic (gemm_q8x.hip), so an expert that several tokens selected -- the shared expert: all of
 // them -- is read once.  Kernels: this grouping, quantize_q8 of the hidden rows, gate + up, activation with the q8 form
@@ -761,7 +762,7 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     int s;
     // batched path: q8 mode, both projections in K tiles of 512, enough tokens for experts to repeat
     const bool batched = mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
-                         (int)B >= mk_env_int("MK_MOE_BATCHED_MIN", 8) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
+                         (int)B >= mk_env_int("MK_MOE_BATCHED_MIN", 4) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
     if (batched) {
         {
             MK_REQUIRE(((uintptr_t)x & 15) == 0, "x must be 16-byte aligned");

@@ -54,14 +54,15 @@ def build(n_experts, d, inter, cfg=2):
 
 @pytest.mark.parametrize("d,inter,n_experts,B,topk,shared,act", [
     (7168, 2048, 12, 1, 8, 11, 0),    # benchmark layer shapes, batch 1, shared expert
-    (7168, 2048, 12, 4, 8, 11, 0),    # batch 4
+    (7168, 2048, 12, 4, 8, 11, 0),    # batch 4 (the smallest batch on the batched path)
+    (7168, 2048, 12, 3, 8, 11, 0),    # batch 3 (two-kernel path)
     (2048, 1024, 6, 3, 2, -1, 1),     # SiTU (K3 rule), no shared expert
     (4096, 2048, 5, 2, 3, 4, 2),      # DeepSeek rule: clamp, weight before W2, plain sum
     (1024, 512, 4, 16, 2, 3, 0),      # batch 16
     (7168, 2048, 12, 9, 8, 11, 0),    # benchmark shapes, two token groups in the gate/up kernel (8 + 1)
     (1024, 4096, 4, 5, 2, 3, 0),      # two rows of W1/W3 per wave
     (96, 64, 4, 2, 2, -1, 0),         # shape off the fast path (composed kernels)
-    (2048, 1024, 6, 8, 2, -1, 1),     # batched path (8 tokens and more: pairs grouped by expert), SiTU, no shared expert
+    (2048, 1024, 6, 8, 2, -1, 1),     # batched path (4 tokens and more: pairs grouped by expert), SiTU, no shared expert
     (4096, 2048, 5, 11, 3, 4, 2),     # batched path, DeepSeek rule, groups of more than four tokens (several passes)
     (7168, 2048, 12, 16, 8, 11, 0),   # batched path at the benchmark layer's shapes, batch 16
 ])
