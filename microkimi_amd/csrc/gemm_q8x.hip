@@ -30,6 +30,10 @@ constexpr int QX_TOK_STRIDE = 1152;  // LDS bytes between tokens (32 banks apart
 constexpr int QX_DX_OFF = QX_TOK * QX_TOK_STRIDE;  // then 16 f32 block scales per token
 constexpr int QX_WSC_OFF = QX_DX_OFF + QX_TOK * 64;  // then 16 weight scale bytes for each of the 256 rows
 constexpr int QX_BUF = QX_WSC_OFF + 256 * 16;
+// behind the two buffers: zeros, as far as the largest constant offset of an operand read reaches (see q8x_pass)
+constexpr int QX_ZERO_OFF = 2 * QX_BUF;
+constexpr int QX_ZERO_BYTES = (QX_TOK / 2 - 1) * 2 * QX_TOK_STRIDE + (QX_STEPS - 1) * 128 + 16;
+constexpr int QX_LDS = QX_ZERO_OFF + ((QX_ZERO_BYTES + 255) / 256) * 256;
 
 struct Q8xArgs {
     const uint8_t *const *packed_ptrs[2];  // by expert id
@@ -84,8 +88,11 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
     const int t2 = n >> 3, ph = (n >> 1) & 3, part = n & 1;
     // 8-bit operand layout: lane group kb holds K bytes 16 kb .. (registers 0-3) and 64 + 16 kb .. (registers 4-7), so
     // K block ph lives in registers (ph >> 1) of the lane groups 2 (ph & 1), 2 (ph & 1) + 1
+    // A lane whose register half holds none of its column's block reads that half from a region of zeros instead
+    // (all such lanes the same address: a broadcast), which saves masking the operand: 8 instructions per matrix
+    // instruction.
     const bool active = (ph & 1) == (kb >> 1);
-    const uint32_t mlo = (active && ph < 2) ? 0xFFFFFFFFu : 0u, mhi = (active && ph >= 2) ? 0xFFFFFFFFu : 0u;
+    const bool has_lo = active && ph < 2, has_hi = active && ph >= 2;
     const int bscale = part ? 127 : 131;  // e8m0 of the column's blocks: 2^0 for the b codes, 2^4 for the a codes
     const uint32_t a_lane_off = (uint32_t)(t2 * QX_TOK_STRIDE + part * QX_ROW + ph * 32 + (kb & 1) * 16);
     const uint32_t dx_lane_off = (uint32_t)(QX_DX_OFF + t2 * 64 + ph * 4);
@@ -136,8 +143,7 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 #pragma unroll
         for (int c = 0; c < NP; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute_unit = [&](const mk_i4 *wl, int rt, const uint8_t *buf0) __attribute__((always_inline)) {
-        const uint8_t *buf = buf0;
+    auto compute_unit = [&](const mk_i4 *wl, int rt, const uint8_t *buf, const uint8_t *plo, const uint8_t *phi) __attribute__((always_inline)) {
         // operand form of the unit's two lines (see gemm_mxfp4.hip): lane rotation, then the half-row exchange
         mk_i4 w[QX_STEPS];
 #pragma unroll
@@ -156,10 +162,10 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 #pragma unroll
             for (int c = 0; c < NP; c++) {
                 if (c < npair) {
-                    const mk_i4 dq = *reinterpret_cast<const mk_i4 *>(buf + a_lane_off + c * 2 * QX_TOK_STRIDE + s * 128);
+                    const mk_i4 dl = *reinterpret_cast<const mk_i4 *>(plo + c * 2 * QX_TOK_STRIDE + s * 128);
+                    const mk_i4 dh = *reinterpret_cast<const mk_i4 *>(phi + c * 2 * QX_TOK_STRIDE + s * 128);
                     const float dxv = *reinterpret_cast<const float *>(buf + dx_lane_off + c * 128 + s * 16);
-                    const mk_i8v av = {(int)((uint32_t)dq[0] & mlo), (int)((uint32_t)dq[1] & mlo), (int)((uint32_t)dq[2] & mlo), (int)((uint32_t)dq[3] & mlo),
-                                       (int)((uint32_t)dq[0] & mhi), (int)((uint32_t)dq[1] & mhi), (int)((uint32_t)dq[2] & mhi), (int)((uint32_t)dq[3] & mhi)};
+                    const mk_i8v av = {dl[0], dl[1], dl[2], dl[3], dh[0], dh[1], dh[2], dh[3]};
                     mk_f4 t = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, mk_f4{0.0f, 0.0f, 0.0f, 0.0f}, 4 /*M: fp4 weights*/,
                                                                             0 /*N: e4m3 codes*/, 0, wsb, 0, bscale);
 #pragma unroll
@@ -181,15 +187,16 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 #pragma unroll 1
     for (int kt = 0; kt < ktiles; kt++) {
         const uint8_t *buf = lds + (kt & 1) * QX_BUF;
+        const uint8_t *plo = has_lo ? buf + a_lane_off : lds + QX_ZERO_OFF, *phi = has_hi ? buf + a_lane_off : lds + QX_ZERO_OFF;
         stage_load(kt + 1);
         load_unit(wb, kt, 1);
-        compute_unit(wa, 0, buf);
+        compute_unit(wa, 0, buf, plo, phi);
         load_unit(wa, kt, 2);
-        compute_unit(wb, 1, buf);
+        compute_unit(wb, 1, buf, plo, phi);
         load_unit(wb, kt, 3);
-        compute_unit(wa, 2, buf);
+        compute_unit(wa, 2, buf, plo, phi);
         load_unit(wa, kt + 1, 0);
-        compute_unit(wb, 3, buf);
+        compute_unit(wb, 3, buf, plo, phi);
         stage_store(lds + ((kt + 1) & 1) * QX_BUF);
         __syncthreads();
     }
@@ -222,7 +229,7 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 
 // WAVES: 4 (a workgroup owns 256 rows) or 2 (128 rows: twice as many, shorter workgroups).
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2))) void q8x_grouped_kernel(Q8xArgs a) {
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4))) void q8x_grouped_kernel(Q8xArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int per_group = a.n_mats * a.row_blocks;
     // Regular workgroups: (group, matrix, row block), all passes of the group one after the other -- except for the
@@ -250,6 +257,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2)))
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
     float *out = a.out[m];
+    for (int i = threadIdx.x * 16; i < QX_LDS - QX_ZERO_OFF; i += 64 * WAVES * 16) *reinterpret_cast<mk_i4 *>(lds + QX_ZERO_OFF + i) = mk_i4{0, 0, 0, 0};
 #pragma unroll 1
     for (int pass = first_pass; tok0 + QX_TOK * pass < tok1; pass += pass_step)
         q8x_pass<QX_TOK / 2, WAVES>(a, packed, scales, out, rb, tok0 + QX_TOK * pass, tok1, lds);
@@ -289,13 +297,13 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     MK_REQUIRE(passes >= 1 && grid < 0x7FFFFFFFull, "too many workgroups");
     a.regular = (int)regular;
     if (waves == 2) {
-        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<2>), 2 * QX_BUF);
+        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<2>), QX_LDS);
         if (s != MK_OK) return s;
-        hipLaunchKernelGGL(q8x_grouped_kernel<2>, dim3((unsigned)grid), dim3(128), 2 * QX_BUF, (hipStream_t)stream, a);
+        hipLaunchKernelGGL(q8x_grouped_kernel<2>, dim3((unsigned)grid), dim3(128), QX_LDS, (hipStream_t)stream, a);
     } else {
-        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<4>), 2 * QX_BUF);
+        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<4>), QX_LDS);
         if (s != MK_OK) return s;
-        hipLaunchKernelGGL(q8x_grouped_kernel<4>, dim3((unsigned)grid), dim3(256), 2 * QX_BUF, (hipStream_t)stream, a);
+        hipLaunchKernelGGL(q8x_grouped_kernel<4>, dim3((unsigned)grid), dim3(256), QX_LDS, (hipStream_t)stream, a);
     }
     return mk_launch_status("q8x_grouped");
 }
