@@ -155,25 +155,36 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
                 w[2 * i + 1][k] = __builtin_amdgcn_update_dpp(rb2, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);
             }
         const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + QX_WSC_OFF + (wave * 64 + rt * 16 + n) * 16);
+        // A matrix instruction's result is taken out after the next one has been issued, so that its latency is covered.
+        mk_f4 tp[NP];
+        float dp[NP];
 #pragma unroll
-        for (int s = 0; s < QX_STEPS; s++) {
-            const mk_i8v wv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
-            const int wsb = (int)((uint32_t)sc[s] >> (8 * kb));
+        for (int s = 0; s <= QX_STEPS; s++) {
 #pragma unroll
             for (int c = 0; c < NP; c++) {
                 if (c < npair) {
-                    const mk_i4 dl = *reinterpret_cast<const mk_i4 *>(plo + c * 2 * QX_TOK_STRIDE + s * 128);
-                    const mk_i4 dh = *reinterpret_cast<const mk_i4 *>(phi + c * 2 * QX_TOK_STRIDE + s * 128);
-                    const float dxv = *reinterpret_cast<const float *>(buf + dx_lane_off + c * 128 + s * 16);
-                    const mk_i8v av = {dl[0], dl[1], dl[2], dl[3], dh[0], dh[1], dh[2], dh[3]};
-                    mk_f4 t = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, mk_f4{0.0f, 0.0f, 0.0f, 0.0f}, 4 /*M: fp4 weights*/,
-                                                                            0 /*N: e4m3 codes*/, 0, wsb, 0, bscale);
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        // the a and the b part of the block sit in neighbouring lanes: exact sum, then the block term
-                        const float both = t[r] + mk_dpp<0xB1>(t[r]);  // quad_perm [1, 0, 3, 2]
-                        acc[rt][c][r] += both * dxv;
+                    mk_f4 tc = {0.0f, 0.0f, 0.0f, 0.0f};
+                    float dc = 0.0f;
+                    if (s < QX_STEPS) {
+                        const mk_i8v wv = {w[s & 3][0], w[s & 3][1], w[s & 3][2], w[s & 3][3], 0, 0, 0, 0};
+                        const int wsb = (int)((uint32_t)sc[s & 3] >> (8 * kb));
+                        const mk_i4 dl = *reinterpret_cast<const mk_i4 *>(plo + c * 2 * QX_TOK_STRIDE + (s & 3) * 128);
+                        const mk_i4 dh = *reinterpret_cast<const mk_i4 *>(phi + c * 2 * QX_TOK_STRIDE + (s & 3) * 128);
+                        dc = *reinterpret_cast<const float *>(buf + dx_lane_off + c * 128 + (s & 3) * 16);
+                        const mk_i8v av = {dl[0], dl[1], dl[2], dl[3], dh[0], dh[1], dh[2], dh[3]};
+                        tc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, av, mk_f4{0.0f, 0.0f, 0.0f, 0.0f}, 4 /*M: fp4 weights*/,
+                                                                              0 /*N: e4m3 codes*/, 0, wsb, 0, bscale);
                     }
+                    if (s > 0) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            // the a and the b part of the block sit in neighbouring lanes: exact sum, then the block term
+                            const float both = tp[c][r] + mk_dpp<0xB1>(tp[c][r]);  // quad_perm [1, 0, 3, 2]
+                            acc[rt][c][r] += both * dp[c];
+                        }
+                    }
+                    tp[c] = tc;
+                    dp[c] = dc;
                 }
             }
         }
@@ -229,7 +240,7 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 
 // WAVES: 4 (a workgroup owns 256 rows) or 2 (128 rows: twice as many, shorter workgroups).
 template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(4))) void q8x_grouped_kernel(Q8xArgs a) {
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3))) void q8x_grouped_kernel(Q8xArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int per_group = a.n_mats * a.row_blocks;
     // Regular workgroups: (group, matrix, row block), all passes of the group one after the other -- except for the
