@@ -511,9 +511,10 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const uint32_t p01 = j < 2 ? t01l : t01h, p23 = j < 2 ? t23l : t23h;
-                    // two bytes -> two f16: 0x6400 | u is 1024 + u exactly; minus 1152 gives the signed byte
-                    const uint32_t sel = (j & 1) ? 0x0C030C02u : 0x0C010C00u;
-                    const uint32_t f01 = mk_perm(0u, p01, sel) | 0x64006400u, f23 = mk_perm(0u, p23, sel) | 0x64006400u;
+                    // two bytes -> two f16: 0x6400 | u is 1024 + u exactly (the 0x64 bytes come out of the same v_perm);
+                    // minus 1152 gives the signed byte
+                    const uint32_t sel = (j & 1) ? 0x04030402u : 0x04010400u;
+                    const uint32_t f01 = mk_perm(0x64646464u, p01, sel), f23 = mk_perm(0x64646464u, p23, sel);
                     const mk_h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
                     const mk_h2 v01 = __builtin_bit_cast(mk_h2, f01) - bias, v23 = __builtin_bit_cast(mk_h2, f23) - bias;
                     const mk_h2 hi01 = v01 * s01, hi23 = v23 * s23;
