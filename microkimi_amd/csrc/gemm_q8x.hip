@@ -47,6 +47,7 @@ struct Q8xArgs {
     const int32_t *ngroups; // number of groups (device)
     const int32_t *gbig;    // the group with the most rows (device): its passes beyond the first get workgroups of their own
     int regular;            // workgroups of the regular part of the grid (groups x matrices x row blocks)
+    int extra_sets;         // sets of workgroups behind it that take the later passes of the largest group in turn
     float *out[2];          // [grouped rows][rows]
     int n_mats, row_blocks;
 };
@@ -254,13 +255,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
         r0 = blockIdx.x % per_group;
         if (gi >= *a.ngroups) return;
         first_pass = 0;
-        pass_step = gi == big ? 0x10000 : 1;
+        pass_step = (gi == big && a.extra_sets > 0) ? 0x10000 : 1;
     } else {
         const int x = blockIdx.x - a.regular;
         gi = big;
         r0 = x % per_group;
         first_pass = 1 + x / per_group;
-        pass_step = 0x10000;
+        pass_step = a.extra_sets;  // whatever the group's size, every pass is taken by exactly one workgroup
     }
     const int m = r0 / a.row_blocks, rb = r0 % a.row_blocks;
     const int tok0 = a.goff[gi], tok1 = a.goff[gi + 1];
@@ -307,6 +308,7 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     const size_t regular = max_groups * n_mats * a.row_blocks, grid = regular + (passes - 1) * n_mats * a.row_blocks;
     MK_REQUIRE(passes >= 1 && grid < 0x7FFFFFFFull, "too many workgroups");
     a.regular = (int)regular;
+    a.extra_sets = (int)(passes - 1);
     if (waves == 2) {
         const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8x_grouped_kernel<2>), QX_LDS);
         if (s != MK_OK) return s;

@@ -65,6 +65,7 @@ def build(n_experts, d, inter, cfg=2):
     (2048, 1024, 6, 8, 2, -1, 1),     # batched path (4 tokens and more: pairs grouped by expert), SiTU, no shared expert
     (4096, 2048, 5, 11, 3, 4, 2),     # batched path, DeepSeek rule, groups of more than four tokens (several passes)
     (7168, 2048, 12, 16, 8, 11, 0),   # batched path at the benchmark layer's shapes, batch 16
+    (1024, 512, 4, 5, 3, -1, 0),      # batched path, an odd number of pairs
 ])
 def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
     torch = torch_cuda()
@@ -85,6 +86,22 @@ def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
     used = lambda t: [w2_dev[int(e)] for e in ids[t]] + ([w2_dev[shared]] if shared >= 0 else [])
     flips = rows_match_up_to_q8_flips(got, want, used, d, inter)
     assert flips <= max(1, B // 3)
+
+
+def test_batched_path_all_tokens_on_the_same_experts():
+    """Every token selects the same two experts (and the shared one): three groups of 13 rows, each several passes of
+    four tokens -- the largest group's later passes run on workgroups of their own, the others' one after the other."""
+    from microkimi_amd import model
+    d, inter, n_experts, B, topk, shared = 1024, 512, 4, 13, 2, 3
+    table, experts = build(n_experts, d, inter)
+    rng = np.random.default_rng(77)
+    ids = np.tile(np.array([[2, 0]], dtype=np.int32), (B, 1))
+    wts = rng.random((B, topk)).astype(np.float32)
+    x = (rng.standard_normal((B, d)) * 0.02).astype(np.float32)
+    got = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1).cpu().numpy()
+    want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=shared, mode=1, threads=8)
+    w2_dev = experts._keep[2]
+    rows_match_up_to_q8_flips(got, want, lambda t: [w2_dev[2], w2_dev[0], w2_dev[shared]], d, inter)
 
 
 def test_moe_decode_f32_mode():
