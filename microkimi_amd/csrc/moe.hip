@@ -196,15 +196,15 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
     const uint8_t **wp1 = reinterpret_cast<const uint8_t **>(xsc + (size_t)tg * NB);
     const uint8_t **wp3 = wp1 + gp_max, **ws1 = wp3 + gp_max, **ws3 = ws1 + gp_max;
     float *wgt_l = reinterpret_cast<float *>(ws3 + gp_max);
+    int *next_l = reinterpret_cast<int *>(wgt_l + gp_max);  // the workgroup's unit counter (units are taken, not owned)
 
     const int lane = threadIdx.x & 63, lane_c = lane < LW ? lane : LW - 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nw = gridDim.x * 8, w = blockIdx.x * 8 + wave;
-    // rows of this wave; a wave beyond the last row (inter not a multiple of 8) walks row inter - 1 and stores nothing:
-    // loads under a condition would make every later wait a full one
-    const bool live = w < a.inter;
-    const int J = live ? (a.inter - w + nw - 1) / nw : 1;
-
+    // rows of this workgroup: 8 b + i + j nw for i < 8, j < J (the same J for all its waves); a row beyond the last one
+    // is read as row inter - 1 and stored nowhere: loads under a condition would make every later wait a full one
+    const int wg_row0 = (int)blockIdx.x * 8;
+    const int J = wg_row0 < a.inter ? (a.inter - wg_row0 + nw - 1) / nw : 1;
     for (int t0 = 0; t0 < B; t0 += tg) {
         const int nt = min(tg, B - t0), gp = nt * per;
         // q8 of the group's hidden rows (src/q8.rs:57-68): 8 lanes per 32-block, one 16-byte load each.  The first batch
@@ -250,18 +250,20 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
         }
         __syncthreads();
 
-        const int n_units = gp * J;
+        // The workgroup's units -- (pair, one of its 8 J rows) -- are taken by its waves from a counter in LDS instead of
+        // being dealt in advance: the waves of a workgroup are served unevenly by the memory system (with equal shares
+        // they finished up to 5 us apart), so the faster ones take more.  The first three units of a wave are fixed.
+        const int upw = 8 * J, n_units = gp * upw;
         RowUnit4 ua, ub, uc;
         auto load_unit = [&](RowUnit4 &U, int u) {
             // past the end (the loads stay unconditional): every lane reads the first block of the last pair's matrices,
             // one line per load instead of a row (the streaming loads would fetch a repeated row again)
             const bool past = u >= n_units;
             u = __builtin_amdgcn_readfirstlane(min(u, n_units - 1));
-            const int k = u / J, j = u - k * J;
-            const int q = k;  // pairs in (token, slot) order
+            const int q = u / upw, r = u - q * upw;  // pairs in (token, slot) order
             const uint8_t *p1 = mk_uniform_ptr(wp1[q]), *p3 = mk_uniform_ptr(wp3[q]);
             const uint8_t *c1 = mk_uniform_ptr(ws1[q]), *c3 = mk_uniform_ptr(ws3[q]);
-            const uint32_t boff = past ? 0u : (uint32_t)min(w + j * nw, a.inter - 1) * NB + lane_c;
+            const uint32_t boff = past ? 0u : (uint32_t)min((int)blockIdx.x * 8 + (r & 7) + (r >> 3) * nw, a.inter - 1) * NB + lane_c;
 #pragma unroll
             for (int t = 0; t < T; t++) {
                 U.w1[t] = mk_ldg128_off_nt(p1, (boff + t * LW) * 16);
@@ -270,8 +272,10 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
                 U.s3[t] = mk_ldg_u8_off(c3, boff + t * LW);
             }
         };
-        load_unit(ua, 0);  // in flight while the hidden rows are quantized (a third unit here spills registers)
-        load_unit(ub, 1);
+        int ia = wave, ib = wave + 8, ic = wave + 16;
+        if (threadIdx.x == 0) *next_l = 24;
+        load_unit(ua, ia);  // in flight while the hidden rows are quantized (a third unit here spills registers)
+        load_unit(ub, ib);
 
         stage_store(xv, threadIdx.x);
         for (int i0 = threadIdx.x + 512 * SB; i0 < n_x; i0 += 512 * SB) {
@@ -291,8 +295,8 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
                 // the kernel itself gains little (B = 4: 172 -> 166 us), the younger waves end when they did before.
                 if ((u + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1);
                 else __builtin_amdgcn_s_setprio(0);
-                const int k = u / J, j = u - k * J;
-                const int q = k;  // pairs in (token, slot) order
+                const int q = u / upw, r = u - q * upw;  // pairs in (token, slot) order
+                const int row = (int)blockIdx.x * 8 + (r & 7) + (r >> 3) * nw;
                 const int tl = q / per;
                 if (tl != cur_tok) {
                     cur_tok = tl;
@@ -315,15 +319,27 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
                 if (lane >= LW) s1 = s3 = 0.0f;
                 const float gsum = mk_wave_sum(s1), usum = mk_wave_sum(s3);
                 const float act = mk_act(a.act_kind, gsum, usum, a.limit, wgt_l[q]);
-                if (lane == 0 && live) a.af[(size_t)(t0 * per + q) * a.inter + (w + j * nw)] = act;
+                if (lane == 0 && row < a.inter) a.af[(size_t)(t0 * per + q) * a.inter + row] = act;
             };
-            for (int u = 0; u < n_units; u += 3) {
-                load_unit(uc, u + 2);
-                compute_unit(ua, u);
-                load_unit(ua, u + 3);
-                if (u + 1 < n_units) compute_unit(ub, u + 1);
-                load_unit(ub, u + 4);
-                if (u + 2 < n_units) compute_unit(uc, u + 2);
+            auto take = [&]() {
+                int v = 0;
+                if (lane == 0) v = atomicAdd(next_l, 1);
+                return __builtin_amdgcn_readfirstlane(v);
+            };
+            // unit ids grow along a wave's sequence: once one is past the end, so are the later ones
+            while (ia < n_units) {
+                load_unit(uc, ic);
+                const int na = take();
+                compute_unit(ua, ia);
+                ia = na;
+                load_unit(ua, ia);
+                const int nb2 = take();
+                if (ib < n_units) compute_unit(ub, ib);
+                ib = nb2;
+                load_unit(ub, ib);
+                const int nc = take();
+                if (ic < n_units) compute_unit(uc, ic);
+                ic = nc;
             }
         }
     }
