@@ -200,13 +200,26 @@ def cpu_baseline_lm_head(torch, tensors, sample_rows=16384, budget_s=12.0):
             "gpu_vs_cpu_rel_l2_on_sample": rel}
 
 
+def time_cpu(fn, budget_s=4.0, max_calls=50):
+    """Median seconds per call of a CPU function over a bounded sample (one untimed call first)."""
+    fn()
+    ts = []
+    t_end = time.perf_counter() + budget_s
+    while (time.perf_counter() < t_end and len(ts) < max_calls) or not ts:
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2], len(ts)
+
+
 def rand_mxfp4(torch, g, rows, cols):
     p = torch.randint(0, 256, (rows, cols // 2), dtype=torch.uint8, device="cuda", generator=g)
     s = torch.randint(118, 131, (rows, cols // 32), dtype=torch.uint8, device="cuda", generator=g)
     return p, s
 
 
-def bench_mxfp4_gemv(torch):
+def bench_mxfp4_gemv(torch, cpu=True):
     """Configuration 0 as a stream over 64 distinct matrices (7.8 MB each, 500 MB in all: more than the 256 MB
     Infinity Cache), as one grouped launch and as 64 back-to-back launches."""
     from microkimi_amd import mxfp4, q8, workloads as W
@@ -239,7 +252,14 @@ def bench_mxfp4_gemv(torch):
 
     f_ms = time_region(torch, singles_f32, 5)
     gbs = lambda ms: per * nmat / (ms * 1e-3) / 1e9
-    return {"workload": "64 distinct 2048x7168 MXFP4 matrices, batch 1", "alg_bytes_per_matrix": per,
+    cpu_port = None
+    if cpu:
+        # the CPU oracle's matvec_packed (q8 mode, one thread: what an expert job of the reference runs) on the first matrix
+        import oracle
+        ph, sh, xh = mats[0][0].cpu().numpy(), mats[0][1].cpu().numpy(), x.cpu().numpy()
+        sec, n = time_cpu(lambda: oracle.matvec_packed(ph, sh, rows, cols, xh, mode=1))
+        cpu_port = {"gbs": per / sec / 1e9, "us_per_gemv": sec * 1e6, "cores": 1, "kind": "port", "sample": f"one 2048x7168 matrix, median of {n} calls"}
+    return {"workload": "64 distinct 2048x7168 MXFP4 matrices, batch 1", "alg_bytes_per_matrix": per, "cpu_port": cpu_port,
             "q8_grouped_launch": {"ms": r_ms, "gbs": gbs(r_ms), "frac": gbs(r_ms) / HBM_PEAK_GBS,
                                   "timing": "30 launches back to back between one pair of events, median of 5",
                                   "ms_with_events_around_each_launch": g_ms},
@@ -270,7 +290,7 @@ def bench_vq1(torch):
     return res
 
 
-def bench_moe(torch):
+def bench_moe(torch, cpu=True):
     """Configuration 2: 256 routed + 1 shared MXFP4 experts (6.0 GB resident), softmax top-8 router, B in {1, 4, 16}."""
     from microkimi_amd import model, workloads as W
     d, inter, ne = W.D_MODEL, W.D_INTER, W.N_EXPERTS
@@ -312,10 +332,22 @@ def bench_moe(torch):
                         "tok_s": B / (ms * 1e-3), "distinct_experts": n_distinct, "pairs": B * (W.TOP_K + 1), "alg_bytes": alg,
                         "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "finite": bool(torch.isfinite(out).all().item())}
+        if cpu and B == 1:
+            # the CPU oracle on the same token: one job per selected expert, as the reference's pool runs them
+            import numpy as np
+            import oracle
+            used = [int(e) for e in ids.cpu().numpy()[0]] + [ne]
+            host = lambda pr: (pr[0].cpu().numpy(), pr[1].cpu().numpy())
+            table = oracle.ExpertTable([host(w1[e]) for e in used], [host(w3[e]) for e in used], [host(w2[e]) for e in used], d, inter)
+            wts_h, x_h = wts.cpu().numpy(), x.cpu().numpy()
+            lid = np.arange(W.TOP_K, dtype=np.uint32)[None, :]
+            sec, n = time_cpu(lambda: oracle.moe_decode(table, lid, wts_h, x_h, shared=W.TOP_K, mode=1, threads=len(used)))
+            res["B1"]["cpu_port"] = {"ms": sec * 1e3, "tok_s": 1.0 / sec, "cores": len(used), "kind": "port",
+                                     "sample": f"the same token and experts, one thread per expert, median of {n} calls"}
     return res
 
 
-def bench_mla(torch):
+def bench_mla(torch, cpu=True):
     """Configuration 3: 128 heads over a shared q8_0 latent cache; 32 distinct caches are rotated at every context
     length (a model has 24 MLA layers) so repeats are not served by the Infinity Cache."""
     from microkimi_amd import model, workloads as W
@@ -353,6 +385,15 @@ def bench_mla(torch):
         res[f"ctx{ctx}"] = {"us": ms * 1e3, "us_python_loop": ms_eager * 1e3, "timing": "graph replay" if ms_graph is not None else "python loop",
                             "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                             "tflops": flops / (ms * 1e-3) / 1e12}
+        if cpu and ctx == 1024:
+            # the CPU oracle's mla_attn_flash_q8_mqa (one thread, as the reference runs it) on the first cache
+            import oracle
+            c0 = caches[0]
+            lq, ls = c0.lat_q.cpu().numpy(), c0.lat_s.float().cpu().numpy()
+            rq, rs = c0.rope_q.cpu().numpy(), c0.rope_s.float().cpu().numpy()
+            qh = q.cpu().numpy()
+            sec, n = time_cpu(lambda: oracle.mla_absorbed_decode(lq, ls, rq, rs, qh, nh, W.MLA_SCALE), budget_s=4.0, max_calls=10)
+            res[f"ctx{ctx}"]["cpu_port"] = {"ms": sec * 1e3, "cores": 1, "kind": "port", "sample": f"the first cache, median of {n} calls"}
         del caches
     return res
 
@@ -479,7 +520,7 @@ def main():
         for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("grouped_gemm", bench_gemm), ("vq1_gemv", bench_vq1)):
             log(name, "...")
             try:
-                extras[name] = fn(torch)
+                extras[name] = fn(torch, not args.no_cpu) if name in ("mxfp4_gemv", "moe_decode", "mla_decode") else fn(torch)
             except Exception as e:  # an extra must not hide the headline
                 extras[name] = {"error": repr(e)}
             torch.cuda.empty_cache()
