@@ -112,6 +112,15 @@ int mk_dev_mxfp4_matvec_f32(const uint8_t *packed, const uint8_t *scales, size_t
 int mk_dev_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out, int mode,
                         int8_t *xq_ws, float *xs_ws, void *stream);
 
+/* matvec_packed_q8 (src/mxfp4.rs:405-443) for m activation rows against ONE matrix, the weights read once for all of
+ * them, on the block-scaled matrix cores with the reference's block terms bit for bit:
+ *   out[i][r] = sum_g (idot_g as f32) * (2^(sb_g - 128) * xs[i][g])      (only the order of the sum over g differs)
+ * xq [m][cols] int8 and xs [m][cols/32] f32 as quantize_q8 gives them, out [m][rows]; cols % 512 == 0.
+ * workspace: 256 bytes of device memory, 256-byte aligned (the one-group description the grouped kernel reads).
+ * The MoE decode layer uses the same kernel for the tokens that share an expert (from 4 tokens per call). */
+int mk_dev_mxfp4_matvec_q8_batched(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const int8_t *xq,
+                                   const float *xs, size_t m, void *workspace, float *out, void *stream);
+
 /* The same q8 matvec over `nmat` matrices of one shape in ONE launch: the
  * grouped-expert form.  packed_ptrs / scales_ptrs / out_ptrs: device arrays of
  * nmat device pointers; xq [nx][cols], xs [nx][cols/32]; x_index[nmat] (device,

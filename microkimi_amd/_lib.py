@@ -1,7 +1,7 @@
 """ctypes binding of libmk_hip.so (the C ABI declared in include/mk_hip.h).
 
 The library is the product: there is no Python or CPU stand-in for it.  If it
-has not been built (python -m microkimi_amd.build) loading fails with an error.
+has not been built (python microkimi_amd/build.py) loading fails with an error.
 """
 import ctypes as C
 import os
@@ -35,7 +35,7 @@ def _load():
     # and the second one finds no device.
     import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
-        raise ImportError(f"{LIB_PATH} is missing: build it with `python -m microkimi_amd.build` (needs hipcc); "
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python microkimi_amd/build.py` (needs hipcc); "
                           "there is no fallback implementation")
     lib = C.CDLL(LIB_PATH)
     vp, sz, i32, f32 = C.c_void_p, C.c_size_t, C.c_int, C.c_float
@@ -55,6 +55,7 @@ def _load():
         "mk_dev_mxfp4_matvec_f32": (i32, [vp, vp, sz, sz, vp, vp, vp]),
         "mk_dev_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp, i32, vp, vp, vp]),
         "mk_dev_mxfp4_matvec_q8_grouped": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
+        "mk_dev_mxfp4_matvec_q8_batched": (i32, [vp, vp, sz, sz, vp, vp, sz, vp, vp, vp]),
         "mk_dev_mxfp4_matvec_nt": (i32, [vp, vp, sz, sz, vp, sz, vp, vp]),
         "mk_dev_q8_matvec": (i32, [vp, vp, i32, sz, sz, vp, vp, sz, vp, vp]),
         "mk_dev_argmax": (i32, [vp, sz, sz, vp, vp, vp]),

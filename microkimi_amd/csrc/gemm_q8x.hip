@@ -320,3 +320,36 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     }
     return mk_launch_status("q8x_grouped");
 }
+
+namespace {
+// the description of one group of m rows on expert 0, written where the grouped kernel expects device arrays
+__global__ void q8x_one_group_kernel(const uint8_t *packed, const uint8_t *scales, int m, uint8_t *ws) {
+    if (threadIdx.x != 0) return;
+    *reinterpret_cast<const uint8_t **>(ws) = packed;
+    *reinterpret_cast<const uint8_t **>(ws + 8) = scales;
+    int32_t *w = reinterpret_cast<int32_t *>(ws + 16);
+    w[0] = 0;  // goff[0]
+    w[1] = m;  // goff[1]
+    w[2] = 0;  // gexp[0]
+    w[3] = 1;  // ngroups
+    w[4] = 0;  // the largest group
+}
+}  // namespace
+
+extern "C" int mk_dev_mxfp4_matvec_q8_batched(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const int8_t *xq,
+                                              const float *xs, size_t m, void *workspace, float *out, void *stream) {
+    MK_REQUIRE(packed && scales && xq && xs && workspace && out, "null pointer");
+    MK_REQUIRE(cols % 512 == 0 && cols > 0 && rows >= 1 && rows <= 0x7FFFFF00u, "cols must be a positive multiple of 512");
+    MK_REQUIRE(m <= 65535 && m * cols < 0xFFFFFFFFull, "too many activation rows");
+    MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)xq & 15) == 0 && ((uintptr_t)scales & 15) == 0 && ((uintptr_t)workspace & 255) == 0,
+               "packed, scales and xq must be 16-byte aligned, the workspace 256-byte aligned");
+    if (m == 0) return MK_OK;
+    uint8_t *ws = (uint8_t *)workspace;
+    hipLaunchKernelGGL(q8x_one_group_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, packed, scales, (int)m, ws);
+    const int s = mk_launch_status("q8x_one_group");
+    if (s != MK_OK) return s;
+    const uint8_t *const *pp = reinterpret_cast<const uint8_t *const *>(ws);
+    const uint8_t *const *sp = reinterpret_cast<const uint8_t *const *>(ws + 8);
+    const int32_t *w = reinterpret_cast<const int32_t *>(ws + 16);
+    return mk_q8x_grouped(1, &pp, &sp, rows, cols, xq, xs, nullptr, w, w + 2, w + 3, w + 4, 1, m, &out, stream);
+}

@@ -67,6 +67,19 @@ def matvec_packed(packed, scales, rows, cols, x, out, n_threads=1):
         check(lib.mk_dev_mxfp4_matvec(ptr(packed), ptr(scales), rows, cols, ptr(x), ptr(out), MODE_F32, None, None, cur_stream()))
 
 
+def matvec_packed_q8_batched(packed, scales, rows, cols, xq, out=None):
+    """matvec_packed_q8 (src/mxfp4.rs:405-443) for the m rows of the Q8Vec xq ([m, cols] int8 + [m, cols/32] scales)
+    against one matrix on the matrix cores, with the reference's block terms bit for bit; returns [m, rows]."""
+    import torch
+    _lib.require_device()
+    m = xq.q.shape[0] if xq.q.dim() == 2 else 1
+    if out is None:
+        out = torch.empty((m, rows), dtype=torch.float32, device=packed.device)
+    ws = torch.empty(256, dtype=torch.uint8, device=packed.device)
+    check(lib.mk_dev_mxfp4_matvec_q8_batched(ptr(packed), ptr(scales), rows, cols, ptr(xq.q), ptr(xq.scales), m, ptr(ws), ptr(out), cur_stream()))
+    return out
+
+
 def matvec_packed_grouped_q8(packed_list, scales_list, rows, cols, xq, x_index, outs):
     """One launch over many matrices of one shape (the grouped-expert form): packed_list / scales_list / outs are
     lists of device tensors, xq a Q8Vec holding [nx, cols] activations, x_index an int32 device tensor or None."""

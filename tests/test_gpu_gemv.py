@@ -223,3 +223,37 @@ def test_matrices_beyond_32_bit_offsets():
             check(lib.mk_dev_mxfp4_matvec_f32(ptr(packed), ptr(scales), rows, cols, ptr(x0), ptr(out), cur_stream()))
         want = oracle.matvec_packed(sp, sc, len(sample), cols, x0.cpu().numpy(), mode=mode)
         assert rel_l2(out[sample].cpu().numpy(), want) <= TOL, mode
+
+
+def test_batched_q8_matvec_on_the_matrix_cores():
+    """mk_dev_mxfp4_matvec_q8_batched (the kernel of the batched MoE decode): m activation rows against one matrix.
+    (1) With a single non-zero block per weight row the output IS one block term: bit-identical to the oracle's
+    matvec_packed_q8 -- the int8 = 16 a + b split on the FP8 matrix cores is exact and the term is rounded once, as the
+    reference's.  (2) Dense weights: the sum over blocks in another order, rel. L2 <= 1e-5, for 1 to 9 rows (one pass
+    with one or two token pairs, several passes)."""
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8
+    rng = np.random.default_rng(11)
+    rows, cols = 300, 1024
+    nb = cols // 32
+    for m in (1, 2, 3, 4, 9):
+        x = rng.standard_normal((m, cols)).astype(np.float32) * rng.uniform(0.01, 30.0, (m, 1)).astype(np.float32)
+        xq = q8.quantize_q8(dev(x))
+        xq_h, xs_h = xq.q.cpu().numpy(), xq.scales.cpu().numpy()
+        # (1) one block per row
+        packed = np.zeros((rows, cols // 2), np.uint8)
+        scales = rng.integers(100, 150, (rows, nb)).astype(np.uint8)
+        blk = rng.integers(0, nb, rows)
+        for r in range(rows):
+            packed[r, blk[r] * 16:(blk[r] + 1) * 16] = rng.integers(0, 256, 16)
+        got = mxfp4.matvec_packed_q8_batched(dev(packed), dev(scales), rows, cols, xq).cpu().numpy()
+        for i in range(m):
+            want = oracle.matvec_packed_q8(packed, scales, rows, cols, xq_h[i], xs_h[i])
+            assert np.array_equal(got[i].view(np.uint32), want.view(np.uint32)), (m, i)
+        # (2) dense
+        packed = rng.integers(0, 256, (rows, cols // 2)).astype(np.uint8)
+        scales = rng.integers(118, 131, (rows, nb)).astype(np.uint8)
+        got = mxfp4.matvec_packed_q8_batched(dev(packed), dev(scales), rows, cols, xq).cpu().numpy()
+        for i in range(m):
+            want = oracle.matvec_packed_q8(packed, scales, rows, cols, xq_h[i], xs_h[i])
+            assert rel_l2(got[i], want) <= 1e-5
