@@ -92,6 +92,22 @@ def test_grouped_launch_matches_per_matrix():
         want = oracle.matvec_packed(mats[i][0], mats[i][1], rows, cols, xs[idx[i]], mode=1)
         assert rel_l2(outs[i].cpu().numpy(), want) <= TOL
     del keep
+    # all matrices against one activation (no index); the results are bit-identical to the per-matrix launches (same
+    # tiles, same per-tile arithmetic, whatever the number of workgroups per matrix)
+    for r2, n2 in ((256, 5), (301, 3), (2048, 7)):
+        mats2 = [workloads.mxfp4_matrix(9, "h", r2, cols, i) for i in range(n2)]
+        pd2, sd2 = [dev(m[0]) for m in mats2], [dev(m[1]) for m in mats2]
+        outs2 = [torch.empty(r2, device="cuda") for _ in range(n2)]
+        x1 = q8.quantize_q8(dev(xs[:1]))
+        keep = mxfp4.matvec_packed_grouped_q8(pd2, sd2, r2, cols, x1, None, outs2)
+        torch.cuda.synchronize()
+        for i in range(n2):
+            want = oracle.matvec_packed(mats2[i][0], mats2[i][1], r2, cols, xs[0], mode=1)
+            assert rel_l2(outs2[i].cpu().numpy(), want) <= TOL
+            single = torch.empty(r2, device="cuda")
+            mxfp4.matvec_packed(pd2[i], sd2[i], r2, cols, dev(xs[0]), single)
+            assert torch.equal(single, outs2[i])
+        del keep
 
 
 @pytest.mark.parametrize("rows,cols,m", [(64, 128, 8), (33, 64, 5), (128, 512, 24), (40, 7168, 3)])
