@@ -192,17 +192,18 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // been used (three units of matrix work between issue and use) instead of two alternating blocks.
 // Large groups (8 experts x 512 tokens, 120 GFLOP): 403 us while the eight 64-token passes of a group ran one after the
 // other on 64 workgroups; 93 us (1.29 PFLOP/s) with the passes dealt to 512 workgroups, pinned order, DEEP and two
-// workgroups per CU.  Counters on that shape: the matrix cores are busy 27 us; waves spend half of their time waiting
-// for loads although the L2 answers in 270 cycles on average -- the vector cache handles 94k accesses per CU, about a
-// cycle each.  Per K tile a workgroup moves 64 KB of weights, 33 KB of activations and 16 KB of scale bytes through it
-// for 16.8 MFLOP: at this tile (256 rows x 64 tokens) the vector cache saturates at about the rate measured.  A
+// workgroups per CU.  Counters on that shape: the matrix cores are busy 27 us of the 93; waves spend half of their time
+// waiting for loads although the L2 hit rate is 83 % and it answers in 270 cycles on average; the vector cache handles
+// 94k accesses per CU.  Per K tile a workgroup moves 64 KB of weights and 33 KB of activations through it for 16.8
+// MFLOP.  Measured since, each passing the tests and none changing the time by more than the run-to-run spread: a
 // step-major pass (the K tile walked step by step with all four row tiles' weights in registers, activation operands
 // read from LDS once per step for all of them, exchange of the whole-line loads under the matrix instructions, the
-// barrier passed before the last step) was built and measured at 84-100 us -- the same; so was the operand's own load
-// mapping (a lane per row: 53 cache accesses per load instruction), and a form in which two row tiles share one read of
-// the activation operands (half the LDS reads: 101-111 us).  None of LDS reads, prefetch depth, waves per SIMD or the
-// load mapping is what holds this shape.  What would help is a larger tile per workgroup
-// (256 x 128: 256 FLOP per byte through the cache) and scale bytes fetched once per row instead of by four lanes.
+// barrier passed before the last step) 84-100 us; the operand's own load mapping (a lane per row: 53 cache accesses per
+// load instruction instead of 26); two row tiles sharing one read of the activation operands (half the LDS reads)
+// 101-111 us; the scale bytes fetched once per row and K tile through LDS (a third fewer cache accesses; kept).  So
+// neither LDS reads, prefetch depth, waves per SIMD, the load mapping nor the number of cache accesses alone is what
+// holds this shape at 1.1-1.3 PFLOP/s; what does has not been identified.  The next thing to measure is a larger tile
+// per workgroup (256 x 128 tokens: half the bytes through the cache per FLOP) with a per-step timeline of one wave.
 template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds) {
