@@ -199,10 +199,11 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // step-major pass (the K tile walked step by step with all four row tiles' weights in registers, activation operands
 // read from LDS once per step for all of them, exchange of the whole-line loads under the matrix instructions, the
 // barrier passed before the last step) 84-100 us; the operand's own load mapping (a lane per row: 53 cache accesses per
-// load instruction instead of 26); two row tiles sharing one read of the activation operands (half the LDS reads)
-// 101-111 us; the scale bytes fetched once per row and K tile through LDS (a third fewer cache accesses; kept).  So
-// neither LDS reads, prefetch depth, waves per SIMD, the load mapping nor the number of cache accesses alone is what
-// holds this shape at 1.1-1.3 PFLOP/s; what does has not been identified.  The next thing to measure is a larger tile
+// load instruction instead of 26); the scale bytes fetched once per row and K tile through LDS (a third fewer cache
+// accesses; kept).  What did help: two row tiles sharing one read of the activation operands (half the LDS reads) with
+// the line exchange done in place, so that it still fits two waves per SIMD: 93-109 -> 82-95 us (1.3-1.5 PFLOP/s; the
+// same form with a second copy of the units in registers ran at one wave per SIMD and 101-111 us).  All four row tiles
+// per read (step-major, in place) needs 43 registers more than two waves per SIMD allow.  The next thing to measure is a larger tile
 // per workgroup (256 x 128 tokens: half the bytes through the cache per FLOP) with a per-step timeline of one wave.
 template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
@@ -296,6 +297,40 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             }
         }
     };
+    // Two row tiles against one read of the activation operands (large groups: with four token tiles the LDS reads of a
+    // unit, 32 KB per wave, take longer than its 16 matrix instructions; shared by two units they take half)
+    auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf) {
+        // the scale bytes are read one at a time where they are used: held as 16-byte rows they cost the registers that
+        // make the difference between two waves per SIMD with and without a spill
+        const uint8_t *sc0 = buf + a_wsc_off(MC) + (wave * 64 + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
+#pragma unroll
+        for (int c = 0; c < MC; c++) {
+            const uint8_t *ae = buf + a_codes_bytes(MC) + (c * 16 + n) * 16 + kb;
+            const uint8_t *arow = buf + (c * 16 + n) * A_STRIDE + kb * 16;
+#pragma unroll
+            for (int s = 0; s < KT_STEPS; s++) {
+                const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + s * 128);
+                const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + s * 128 + 64);
+                const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                const int asb = ae[s * 4];
+                const mk_i8v b0 = {w0[s][0], w0[s][1], w0[s][2], w0[s][3], 0, 0, 0, 0}, b1 = {w1[s][0], w1[s][1], w1[s][2], w1[s][3], 0, 0, 0, 0};
+                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b0, av, acc[rt][c], 4, 0, 0, (int)sc0[s * 4], 0, asb);
+                acc[rt + 1][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b1, av, acc[rt + 1][c], 4, 0, 0, (int)sc1[s * 4], 0, asb);
+            }
+        }
+    };
+    // the line exchange of compute_unit, in place (no second copy of the unit in registers)
+    auto exchange_in_place = [&](mk_i4 *w) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int ra = __builtin_amdgcn_ds_bpermute(rot_idx, w[2 * i][k]), rb2 = __builtin_amdgcn_ds_bpermute(rot_idx, w[2 * i + 1][k]);
+                w[2 * i][k] = __builtin_amdgcn_update_dpp(ra, rb2, 0x128 /* row_ror:8 */, 0xF, 0xC, false);
+                w[2 * i + 1][k] = __builtin_amdgcn_update_dpp(rb2, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);
+            }
+        }
+    };
     auto pin_acc = [&](int rt) {
         if constexpr (PIN) {
 #pragma unroll
@@ -342,12 +377,28 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         for (int kt = 0; kt < ktiles; kt++) {
             const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
             stage_load(kt + 1);
+            if constexpr (PIN && FULL && MC >= 4) {
+                // large groups: two row tiles per read of the activation operands (93-109 -> 82-95 us on 8 experts x 512 tokens)
 #pragma unroll
-            for (int rt = 0; rt < 4; rt++) {
-                if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-                compute_unit(w4[rt], rt, buf);
-                if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-                load_unit(w4[rt], kt + 1, rt);
+                for (int rt = 0; rt < 4; rt += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    exchange_in_place(w4[rt]);
+                    exchange_in_place(w4[rt + 1]);
+                    mma_unit2(w4[rt], w4[rt + 1], rt, buf);
+                    pin_acc(rt);
+                    pin_acc(rt + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_unit(w4[rt], kt + 1, rt);
+                    load_unit(w4[rt + 1], kt + 1, rt + 1);
+                }
+            } else {
+#pragma unroll
+                for (int rt = 0; rt < 4; rt++) {
+                    if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+                    compute_unit(w4[rt], rt, buf);
+                    if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
+                    load_unit(w4[rt], kt + 1, rt);
+                }
             }
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
