@@ -159,12 +159,15 @@ int mk_dev_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, 
 
 /* Expert table: device arrays of per-expert device pointers, indexed by expert
  * id.  w1, w3: [inter][d] (gate, up); w2: [d][inter] (down); each MXFP4 as
- * (packed, scales) in the reference layout. */
+ * (packed, scales) in the reference layout.  n_experts: entries per array; when
+ * it is not 0 a routed id outside [0, n_experts) selects nothing (the pair adds
+ * nothing to its token's row), with 0 the ids are trusted. */
 typedef struct {
     const uint8_t *const *w1p, *const *w1s;
     const uint8_t *const *w3p, *const *w3s;
     const uint8_t *const *w2p, *const *w2s;
     size_t d, inter;
+    size_t n_experts;
 } mk_expert_table;
 
 /* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
@@ -181,6 +184,18 @@ size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size
  * each call. */
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
+
+/* The two halves of mk_dev_moe_decode on their own, for callers that keep the reference's call structure (two
+ * matvec_packed calls, the activation, then the third matvec_packed: src/model.rs:2246-2259, src/deepseek.rs:1080-1089)
+ * and for stage-wise checks.  Arguments as mk_dev_moe_decode; the same kernels run.
+ *   _act       act[(t * per + s)][inter] = ACT(W1_e x_t, W3_e x_t) for slot s of token t, per = topk (+ 1: the shared
+ *              expert is the last slot); f32, before matvec_packed's own q8 step.
+ *   _from_act  out_t from given activation rows in that layout (the q8 mode re-quantizes them per 32 exactly as
+ *              matvec_packed does for W2), weighted sum in slot order. */
+int mk_dev_moe_decode_act(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
+                          const float *x, int mode, int act_kind, float limit, void *workspace, float *act, void *stream);
+int mk_dev_moe_decode_from_act(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
+                               const float *act, int mode, int act_kind, void *workspace, float *out, void *stream);
 
 /* Router of the benchmark MoE layer on device: softmax over logits [B][n], top-k
  * with the reference's rule (strict '>' insertion: ties to the lowest index;
@@ -251,14 +266,30 @@ int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *
 /* Bytes of device scratch mk_dev_moe_prefill needs. */
 size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter);
 
+/* Where mk_dev_moe_prefill keeps its intermediates inside the workspace (byte offsets from its start; valid after the
+ * call has run, until the next one on that workspace).  P = T * topk pairs, "grouped row" = position of a pair after the
+ * grouping by expert (src/model.rs:2539-2544).
+ *   order   [P] int32      grouped row -> pair index t * topk + s
+ *   pos     [P] int32      pair index -> grouped row, -1 for an expert id out of range
+ *   offsets [n_experts+1]  int32: expert e owns the grouped rows offsets[e] .. offsets[e+1]
+ *   g, u    [P][inter] f32 the gate and up projections per grouped row (before the activation)
+ *   o       [P][d] f32     the down projection per grouped row, before the weighted sum */
+typedef struct {
+    size_t order, pos, offsets, g, u, o;
+} mk_prefill_layout;
+int mk_moe_prefill_workspace_layout(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter, mk_prefill_layout *out);
+
 /* The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) for T
  * prompt positions: the (token, slot) pairs are grouped by expert (stable in
  * (token, slot) order), each used expert evaluates gate, up, activation and
  * down for its rows with mk_dev_mxfp4_grouped_gemm, and per token
  *   out_t = sum_s w[t][s] * o[t][s]   in slot order, multiply then add.
  * The gathered hidden rows and the activation enter the matrix cores as MXFP8
- * (deepseek::fp8_roundtrip per 32, src/deepseek.rs:312-322); the reference's own
- * prefill is the f32 arithmetic of matvec_packed_nt (mk_dev_mxfp4_matvec_nt).
+ * (deepseek::fp8_roundtrip per 32, src/deepseek.rs:312-322, with the block
+ * exponent free to use the whole e8m0 range instead of that function's clamp at
+ * 8, so that large activations do not saturate); the reference's own prefill is
+ * the f32 arithmetic of matvec_packed_nt (mk_dev_mxfp4_matvec_nt), from which
+ * this differs by the e4m3 rounding of the two inputs (2-3 % of a row's norm).
  * table entries 0..n_experts-1 are used; ids [T][topk] int32 (a pair whose id is
  * out of range contributes nothing), weights [T][topk], x [T][d], out [T][d].
  * act_kind MK_ACT_SWIGLU or MK_ACT_SITU.  d, inter multiples of 128; T * topk <= 16384

@@ -26,7 +26,11 @@ class BinEntry(C.Structure):
 
 class ExpertTable(C.Structure):
     _fields_ = [("w1p", C.c_void_p), ("w1s", C.c_void_p), ("w3p", C.c_void_p), ("w3s", C.c_void_p), ("w2p", C.c_void_p),
-                ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t)]
+                ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t), ("n_experts", C.c_size_t)]
+
+
+class PrefillLayout(C.Structure):
+    _fields_ = [("order", C.c_size_t), ("pos", C.c_size_t), ("offsets", C.c_size_t), ("g", C.c_size_t), ("u", C.c_size_t), ("o", C.c_size_t)]
 
 
 def _load():
@@ -62,6 +66,8 @@ def _load():
         "mk_dev_q8head_from_f32": (i32, [vp, sz, sz, vp, vp, i32, vp]),
         "mk_moe_decode_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_dev_moe_decode": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),
+        "mk_dev_moe_decode_act": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),
+        "mk_dev_moe_decode_from_act": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, vp, vp, vp]),
         "mk_dev_router_softmax_topk": (i32, [vp, sz, sz, sz, vp, vp, vp]),
         "mk_dev_router_topk": (i32, [vp, sz, sz, sz, i32, vp, f32, vp, vp, vp]),
         "mk_dev_rmsnorm": (i32, [vp, sz, sz, vp, f32, vp, vp, vp, vp]),
@@ -71,6 +77,7 @@ def _load():
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
         "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),
+        "mk_moe_prefill_workspace_layout": (i32, [sz, sz, sz, sz, sz, C.POINTER(PrefillLayout)]),
         "mk_dev_moe_prefill": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp]),

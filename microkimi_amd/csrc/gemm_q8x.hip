@@ -301,7 +301,7 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     a.gbig = gbig;
     a.n_mats = n_mats;
     // 128-row workgroups (twice as many, shorter) measured the same as 256-row ones on the benchmark layer (472 / 466 us)
-    const int waves = mk_env_int("MK_Q8X_WAVES", 4);
+    const int waves = MK_TUNE("MK_Q8X_WAVES", 4);
     const size_t wg_rows = 64 * (size_t)waves;
     a.row_blocks = (int)((rows + wg_rows - 1) / wg_rows);
     const size_t passes = (max_group_rows + QX_TOK - 1) / QX_TOK;

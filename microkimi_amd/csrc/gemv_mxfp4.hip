@@ -355,7 +355,7 @@ int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
     if (q8) {
         // a fixed, fully resident grid shared by the matrices of the launch
         // (2 workgroups per CU measured best for every block count per row)
-        int per_mat = mk_env_int("MK_MXFP4_BLOCKS", 512) / (int)nmat;
+        int per_mat = MK_TUNE("MK_MXFP4_BLOCKS", 512) / (int)nmat;
         if (per_mat < 1) per_mat = 1;
         if (per_mat * 4 > n_tiles) per_mat = (n_tiles + 3) / 4;
         hipLaunchKernelGGL(mxfp4_gemv_q8_kernel<NB>, dim3(per_mat, (unsigned)nmat), dim3(256), 0, st, a);

@@ -424,7 +424,7 @@ __global__ __launch_bounds__(256) void argmax_stage2_kernel(const float *__restr
 template <int NB, bool F16>
 void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
     // a fixed, fully resident grid: blocks-per-CU x 256 CUs x 4 waves
-    int blocks = mk_env_int("MK_Q8_B1_BLOCKS", 512);
+    int blocks = MK_TUNE("MK_Q8_B1_BLOCKS", 512);
     if (blocks * 4 > rows) blocks = (rows + 3) / 4;
     hipLaunchKernelGGL((q8_gemv_b1_kernel<NB, F16>), dim3(blocks), dim3(256), 0, st, q, scales, rows, xq, xs, out);
 }
@@ -432,7 +432,7 @@ void launch_b1(const int8_t *q, const void *scales, int rows, const int8_t *xq, 
 template <bool F16, int BATCH>
 int launch_bn(const int8_t *q, const void *scales, int rows, const int8_t *xq, const float *xs, float *out, hipStream_t st) {
     constexpr int NB = 224;
-    int blocks = mk_env_int("MK_Q8_BN_BLOCKS", 512);
+    int blocks = MK_TUNE("MK_Q8_BN_BLOCKS", 512);
     if (blocks * 4 > rows) blocks = (rows + 3) / 4;
     const size_t lds = (size_t)BATCH * NB * 36;
     const int s = mk_lds_opt_in(reinterpret_cast<const void *>(q8_gemv_bn_kernel<NB, F16, BATCH>), 80 * 1024);
@@ -447,7 +447,7 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
     const int nb = (int)(cols / 32);
     // measured on the 163840 x 7168 head: streaming kernel 188 / 198 / 203 us at batch 2 / 3 / 4 against 204 / 206 / 195 us
     // for the matrix-core kernel, whose time (195-198 us) does not grow with the batch
-    if (batch >= 2 && batch <= 3 && nb == 224 && rows * cols < 0xFFFFFFFFull && !mk_env_int("MK_Q8_NO_BN", 0)) {
+    if (batch >= 2 && batch <= 3 && nb == 224 && rows * cols < 0xFFFFFFFFull && !MK_TUNE("MK_Q8_NO_BN", 0)) {
         if (batch == 2) return launch_bn<F16, 2>(q, scales, (int)rows, xq, xs, out, st);
         return launch_bn<F16, 3>(q, scales, (int)rows, xq, xs, out, st);
     }
@@ -463,10 +463,10 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
         // LDS: activations (cols * 8) + their scales (nb * 32) + one scale tile per wave (16 * nb * 2 or 4 bytes)
         constexpr int WAVES = F16 ? 8 : 4;
         const int n_groups = (int)((rows + 15) / 16);
-        int blocks = mk_env_int("MK_Q8_MFMA_BLOCKS", 256);  // one per CU
+        int blocks = MK_TUNE("MK_Q8_MFMA_BLOCKS", 256);  // one per CU
         if (blocks * WAVES > n_groups) blocks = (n_groups + WAVES - 1) / WAVES;
         const size_t lds = cols * 8 + (size_t)nb * 32 + (size_t)WAVES * 16 * nb * (F16 ? 2 : 4);
-        if (nb % 4 == 0 && !mk_env_int("MK_Q8_MFMA_HALF_LINES", 0))  // rows are whole 128-byte lines
+        if (nb % 4 == 0 && !MK_TUNE("MK_Q8_MFMA_HALF_LINES", 0))  // rows are whole 128-byte lines
             hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES, true>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq,
                                xs, (int)batch, out);
         else

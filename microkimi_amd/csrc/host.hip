@@ -88,12 +88,20 @@ int mk_env_int(const char *name, int dflt) {
 int mk_lds_opt_in(const void *kernel, int bytes) {
     static std::mutex mu;
     static std::set<std::pair<const void *, int>> done;
+    // what this thread has already seen done: the launch path takes no lock after a kernel's first launch
+    thread_local const void *seen_kernel[8] = {};
+    thread_local int seen_dev[8] = {};
     int dev = 0;
     MK_HIP_TRY(hipGetDevice(&dev));
+    const unsigned slot = (unsigned)(((uintptr_t)kernel >> 4) & 7);
+    if (seen_kernel[slot] == kernel && seen_dev[slot] == dev) return MK_OK;
     std::lock_guard<std::mutex> lk(mu);
-    if (done.count({kernel, dev})) return MK_OK;
-    MK_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-    done.insert({kernel, dev});
+    if (!done.count({kernel, dev})) {
+        MK_HIP_TRY(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+        done.insert({kernel, dev});
+    }
+    seen_kernel[slot] = kernel;
+    seen_dev[slot] = dev;
     return MK_OK;
 }
 

@@ -252,7 +252,9 @@ __device__ __forceinline__ uint32_t mk_mxfp8_quantize(float v, uint32_t &exp_byt
 // The same for a 32-block held as 8 consecutive values in each lane of an aligned quad of lanes: the block maximum
 // needs two DPP steps, the division by the power-of-two scale is an exact multiplication, and the e4m3 codes come
 // from v_cvt_pk_fp8_f32 (round to nearest even on the OCP e4m3 grid; the inputs are clamped to +-448 before).
-// c0 holds the codes of v[0..3], c1 of v[4..7], lowest byte first.
+// c0 holds the codes of v[0..3], c1 of v[4..7], lowest byte first.  EMAX: upper clamp of the scale exponent, 8 in the
+// reference's rule; 127 uses the whole e8m0 range, so that no block saturates.
+template <int EMAX = 8>
 __device__ __forceinline__ void mk_mxfp8_quantize8(const float (&v)[8], uint32_t &exp_byte, uint32_t &c0, uint32_t &c1) {
     float a = 0.0f;
 #pragma unroll
@@ -260,9 +262,10 @@ __device__ __forceinline__ void mk_mxfp8_quantize8(const float (&v)[8], uint32_t
     a = fmaxf(a, mk_dpp<0xB1>(a));
     a = fmaxf(a, mk_dpp<0x4E>(a));
     int e = mk_ceil_log2f(fmaxf(a, 1e-4f) / 448.0f);
-    e = max(-127, min(8, e));
+    e = max(-127, min(EMAX, e));
     exp_byte = (uint32_t)(e + 127);
-    const float inv = mk_scale_from_byte(254u - exp_byte);  // 2^-e
+    // 2^-e, exact: byte 254 - (e + 127) for e < 127; for e = 127 the power 2^-127 is the subnormal that byte 0 decodes to
+    const float inv = mk_scale_from_byte(254u - exp_byte);
     float q[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(v[i] * inv, -448.0f), 448.0f);
@@ -310,8 +313,11 @@ int mk_launch_status(const char *kernel);
 // Raises a kernel's dynamic LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) once per kernel and device; checked,
 // safe to call from several threads.  Launch sites call it before every launch: after the first it is a set lookup.
 int mk_lds_opt_in(const void *kernel, int bytes);
-// integer value of an environment variable (tuning and A/B switches of the launchers), dflt when unset or empty
+// integer value of an environment variable, dflt when unset or empty
 int mk_env_int(const char *name, int dflt);
+// A tuning or A/B switch of a launcher: the environment is read once per process, at the first launch that asks; after
+// that the value is a constant (no getenv on the launch path).
+#define MK_TUNE(name, dflt) ([]() -> int { static const int v = mk_env_int(name, dflt); return v; }())
 
 // mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].

@@ -643,8 +643,9 @@ extern "C" size_t mk_mla_decode_workspace_bytes(size_t nh, size_t L, size_t n_po
            2 * align_up(MAX_SPLITS * nh * 4, 256);
 }
 
-extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos,
-                                    const float *q, size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream) {
+namespace {
+int mla_decode_impl(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos, const float *q, size_t nh,
+                    size_t L, size_t R, float scale, void *workspace, float *out, void *stream) {
     MK_REQUIRE(lat_q && lat_s && q && workspace && out && (R == 0 || (rope_q && rope_s)), "null pointer");
     MK_REQUIRE(L % 64 == 0 && L >= 64 && L <= 512, "latent width must be a multiple of 64 up to 512");
     MK_REQUIRE(R % 32 == 0 && R <= 64, "rope width must be 0, 32 or 64");
@@ -678,7 +679,7 @@ extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, cons
     a.n_pos = n_pos;
     a.scale = scale;
     const int tiles = (n_pos + TJ - 1) / TJ;
-    const bool mfma = L == ML && R == MR && getenv("MK_MLA_VALU") == nullptr;
+    const bool mfma = L == ML && R == MR && !MK_TUNE("MK_MLA_VALU", 0);
     // split the context in whole tiles: one workgroup per CU for the MFMA kernel
     // (its register and LDS budget allows one), about 512 for the VALU kernel
     const int head_groups = (int)((nh + HPG - 1) / HPG);
@@ -706,4 +707,10 @@ extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, cons
     }
     hipLaunchKernelGGL(mla_merge_kernel, dim3((unsigned)nh), dim3(512), 0, st, a.po, a.pm, a.pl, (int)nh, (int)L, a.n_splits, out);
     return mk_launch_status("mla_merge");
+}
+}  // namespace
+
+extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos,
+                                    const float *q, size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream) {
+    return mla_decode_impl(lat_q, lat_s, rope_q, rope_s, pos, q, nh, L, R, scale, workspace, out, stream);
 }

@@ -103,13 +103,21 @@ Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, siz
     return w;
 }
 
+// Expert id of a routed pair.  When the table states its size, an id outside it selects entry 0 with routing weight 0:
+// the pair then adds nothing to the token's row (the pointer arrays are never read out of bounds).
+__device__ __forceinline__ int mk_checked_expert(int e, size_t n_experts, bool &ok) {
+    ok = n_experts == 0 || (unsigned)e < (unsigned)n_experts;
+    return ok ? e : 0;
+}
+
 __global__ void moe_setup_kernel(mk_expert_table tab, int B, int topk, int shared, const int32_t *__restrict__ ids,
                                  const float *__restrict__ weights, PairTables pt, float *o, float *g, float *u, int d, int inter) {
     const int per = topk + (shared >= 0 ? 1 : 0);
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= B * per) return;
     const int t = p / per, s = p % per;
-    const int e = s < topk ? ids[t * topk + s] : shared;
+    bool ok = true;
+    const int e = s < topk ? mk_checked_expert(ids[t * topk + s], tab.n_experts, ok) : shared;
     pt.w1p[p] = tab.w1p[e];
     pt.w1s[p] = tab.w1s[e];
     pt.w3p[p] = tab.w3p[e];
@@ -121,7 +129,7 @@ __global__ void moe_setup_kernel(mk_expert_table tab, int B, int topk, int share
     pt.uptr[p] = u + (size_t)p * inter;
     pt.xidx[p] = t;
     pt.aidx[p] = p;
-    pt.pw[p] = s < topk ? weights[t * topk + s] : 1.0f;
+    pt.pw[p] = s < topk ? (ok ? weights[t * topk + s] : 0.0f) : 1.0f;
 }
 
 __device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
@@ -241,12 +249,13 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
         if (t0) __syncthreads();  // the previous group's LDS is still being read
         if (threadIdx.x < gp) {
             const int q = threadIdx.x, tok = t0 + q / per, slot = q % per;
-            const int e = slot < a.topk ? a.ids[tok * a.topk + slot] : a.shared;
+            bool ok = true;
+            const int e = slot < a.topk ? mk_checked_expert(a.ids[tok * a.topk + slot], a.tab.n_experts, ok) : a.shared;
             wp1[q] = a.tab.w1p[e];
             wp3[q] = a.tab.w3p[e];
             ws1[q] = a.tab.w1s[e];
             ws3[q] = a.tab.w3s[e];
-            wgt_l[q] = slot < a.topk ? a.weights[tok * a.topk + slot] : 1.0f;
+            wgt_l[q] = slot < a.topk ? (ok ? a.weights[tok * a.topk + slot] : 0.0f) : 1.0f;
         }
         __syncthreads();
 
@@ -394,10 +403,11 @@ __global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a)
     stage_load(av, threadIdx.x);
     if (threadIdx.x < per) {
         const int s = threadIdx.x;
-        const int e = s < a.topk ? a.ids[tok * a.topk + s] : a.shared;
+        bool ok = true;
+        const int e = s < a.topk ? mk_checked_expert(a.ids[tok * a.topk + s], a.tab.n_experts, ok) : a.shared;
         wp_l[s] = a.tab.w2p[e];
         ws_l[s] = a.tab.w2s[e];
-        pw_l[s] = (s < a.topk && !a.ds_rule) ? a.weights[tok * a.topk + s] : 1.0f;
+        pw_l[s] = !ok ? 0.0f : (s < a.topk && !a.ds_rule) ? a.weights[tok * a.topk + s] : 1.0f;
     }
     __syncthreads();  // the pair tables: the first weight loads need them
 
@@ -538,7 +548,7 @@ constexpr int BATCHED_MAX_P = 1024;
 
 // Workgroup 0 groups the pairs; the others form the q8 blocks of the hidden rows (src/q8.rs:57-68, 8 lanes per
 // 32-block as mk_quantize_q8_kernel) -- one launch for the two steps in front of the gate/up GEMM.
-__global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, int shared, const int32_t *__restrict__ ids,
+__global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, int shared, size_t n_experts, const int32_t *__restrict__ ids,
                                                                const float *__restrict__ weights, int32_t *order, int32_t *pos, int32_t *rtok,
                                                                int32_t *goff, int32_t *gexp, int32_t *ngroups, float *pw,
                                                                const float *__restrict__ x, size_t n_blocks, int8_t *__restrict__ xq,
@@ -571,8 +581,9 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
         int e = 0x7FFFFFFF;  // behind every pair: the loops below read whole 16-byte groups
         if (tid < P) {
             const int t = tid / per, s = tid % per;
-            e = s < topk ? ids[t * topk + s] : shared;
-            pw[tid] = s < topk ? weights[t * topk + s] : 1.0f;
+            bool ok = true;
+            e = s < topk ? mk_checked_expert(ids[t * topk + s], n_experts, ok) : shared;
+            pw[tid] = s < topk ? (ok ? weights[t * topk + s] : 0.0f) : 1.0f;
         }
         e_l[tid] = e;
         start_l[tid] = 0;
@@ -642,17 +653,28 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
 }
 
 // The activation of the grouped rows and its q8 form in one kernel (the block matvec_packed forms when it re-quantizes
-// its input for W2, src/q8.rs:57-68): 8 lanes per 32-block, four values each.
+// its input for W2, src/q8.rs:57-68): 8 lanes per 32-block, four values each.  act_in (optional): the activation rows
+// are given, [pair][inter] in (token, slot) order, instead of being formed from g and u; act_out (optional): the f32
+// activation rows are also written there in that order.
 __global__ __launch_bounds__(256) void moe_act_q8_grouped_kernel(const float *__restrict__ g, const float *__restrict__ u,
                                                                  const float *__restrict__ pw, const int32_t *__restrict__ order, int inter,
-                                                                 size_t n_blocks, int act_kind, float limit, int8_t *__restrict__ q,
+                                                                 size_t n_blocks, int act_kind, float limit, const float *__restrict__ act_in,
+                                                                 float *__restrict__ act_out, int8_t *__restrict__ q,
                                                                  float *__restrict__ scales) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n_blocks * 8) return;  // whole groups of 8 lanes leave together
-    const mk_f4 gv = reinterpret_cast<const mk_f4 *>(g)[i], uv = reinterpret_cast<const mk_f4 *>(u)[i];
-    const float wgt = pw[order[(i * 4) / (size_t)inter]];
-    const mk_f4 v = {mk_act(act_kind, gv.x, uv.x, limit, wgt), mk_act(act_kind, gv.y, uv.y, limit, wgt), mk_act(act_kind, gv.z, uv.z, limit, wgt),
-                     mk_act(act_kind, gv.w, uv.w, limit, wgt)};
+    const size_t row = (i * 4) / (size_t)inter, col4 = i - row * (size_t)(inter / 4);
+    const int pair = order[row];
+    mk_f4 v;
+    if (act_in) {
+        v = reinterpret_cast<const mk_f4 *>(act_in + (size_t)pair * inter)[col4];
+    } else {
+        const mk_f4 gv = reinterpret_cast<const mk_f4 *>(g)[i], uv = reinterpret_cast<const mk_f4 *>(u)[i];
+        const float wgt = pw[pair];
+        v = mk_f4{mk_act(act_kind, gv.x, uv.x, limit, wgt), mk_act(act_kind, gv.y, uv.y, limit, wgt), mk_act(act_kind, gv.z, uv.z, limit, wgt),
+                  mk_act(act_kind, gv.w, uv.w, limit, wgt)};
+    }
+    if (act_out) reinterpret_cast<mk_f4 *>(act_out + (size_t)pair * inter)[col4] = v;
     float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     mx = fmaxf(mx, mk_dpp<0xB1>(mx));
     mx = fmaxf(mx, mk_dpp<0x4E>(mx));
@@ -703,7 +725,7 @@ int launch_gate_up_rows(const FusedArgs &a, size_t B, hipStream_t st) {
     const size_t lds = (size_t)tg * per_tok;
     const int s = mk_lds_opt_in(reinterpret_cast<const void *>(moe_gate_up_rows_kernel<NB>), 160 * 1024);
     if (s != MK_OK) return s;
-    int blocks = mk_env_int("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
+    int blocks = MK_TUNE("MK_MOE_ROWS_BLOCKS", 256);  // one resident workgroup per CU
     if (blocks * 8 > a.inter) blocks = (a.inter + 7) / 8;
     hipLaunchKernelGGL(moe_gate_up_rows_kernel<NB>, dim3(blocks), dim3(512), lds, st, a, (int)B, tg);
     return mk_launch_status("moe_gate_up_rows");
@@ -731,16 +753,16 @@ int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
         // One workgroup of 14 waves per CU when the rows then divide evenly (7168 = 2^10 x 7): the activation is
         // quantized once per CU instead of once per small workgroup, and every wave has the same number of tiles.
         const int bpt = 256 / (int)B;  // workgroups per token
-        if (bpt >= 1 && !mk_env_int("MK_MOE_DOWN_SMALL", 0) && n_tiles % (bpt * 14) == 0) {
+        if (bpt >= 1 && !MK_TUNE("MK_MOE_DOWN_SMALL", 0) && n_tiles % (bpt * 14) == 0) {
             const int tiles = n_tiles / (bpt * 14);  // per wave
             if (tiles % 8 == 0) return launch_down_u<NB, 8, 14>(a, B, bpt, st);
             if (tiles % 4 == 0) return launch_down_u<NB, 4, 14>(a, B, bpt, st);
             if (tiles % 2 == 0) return launch_down_u<NB, 2, 14>(a, B, bpt, st);
         }
     }
-    const int target = mk_env_int("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
+    const int target = MK_TUNE("MK_MOE_DOWN_BLOCKS", 768) / (int)B;  // blocks per token
     int u = 8 / T;
-    int forced = mk_env_int("MK_MOE_DOWN_U", 0);
+    int forced = MK_TUNE("MK_MOE_DOWN_U", 0);
     auto blocks_for = [&](int uu) {
         int groups = (int)((double)n_tiles / ((double)(target > 0 ? target : 1) * 4 * uu) + 0.5);
         if (groups < 1) groups = 1;
@@ -759,15 +781,25 @@ int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
 }
 }  // namespace
 
-extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
-                                 const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream) {
-    MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
+namespace {
+enum { STAGE_ALL = 0, STAGE_ACT = 1, STAGE_FROM_ACT = 2 };
+
+// The layer, or one of its two stages: STAGE_ACT stops after the activation rows (act_io [B * per][inter], out),
+// STAGE_FROM_ACT starts from given activation rows (act_io, in).  Both run the kernels the whole layer runs.
+int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared, const float *x,
+                    int mode, int act_kind, float limit, void *workspace, float *out, void *stream, int stage, float *act_io) {
+    MK_REQUIRE(table && ids && weights && workspace, "null pointer");
+    MK_REQUIRE(stage == STAGE_FROM_ACT || x, "null pointer");
+    MK_REQUIRE(stage == STAGE_ACT || out, "null pointer");
+    MK_REQUIRE(stage == STAGE_ALL || act_io, "null pointer");
     MK_REQUIRE(mode == MK_MODE_Q8 || mode == MK_MODE_F32, "mode must be MK_MODE_F32 or MK_MODE_Q8");
     MK_REQUIRE(act_kind >= MK_ACT_SWIGLU && act_kind <= MK_ACT_DS, "unknown activation");
     const size_t d = table->d, inter = table->inter;
     MK_REQUIRE(d % 32 == 0 && inter % 32 == 0 && d > 0 && inter > 0, "d and inter must be positive multiples of 32");
     MK_REQUIRE(B >= 1 && topk >= 1 && B * (topk + 1) <= 65535, "bad batch / top-k");
+    MK_REQUIRE(table->n_experts == 0 || shared < (long long)table->n_experts, "shared expert id beyond the table");
     MK_REQUIRE(((uintptr_t)workspace & 255) == 0, "workspace must be 256-byte aligned");
+    MK_REQUIRE(!act_io || ((uintptr_t)act_io & 15) == 0, "activation rows must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     const int per = (int)topk + (shared >= 0 ? 1 : 0);
     const size_t P = B * per;
@@ -778,16 +810,17 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
     int s;
     // batched path: q8 mode, both projections in K tiles of 512, enough tokens for experts to repeat
     const bool batched = mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
-                         (int)B >= mk_env_int("MK_MOE_BATCHED_MIN", 4) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
+                         (int)B >= MK_TUNE("MK_MOE_BATCHED_MIN", 4) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
     if (batched) {
         {
-            MK_REQUIRE(((uintptr_t)x & 15) == 0, "x must be 16-byte aligned");
-            const size_t n_blocks = B * d / 32;
+            // the grouping is needed by both stages; with given activation rows there is no hidden row to quantize
+            MK_REQUIRE(stage == STAGE_FROM_ACT || ((uintptr_t)x & 15) == 0, "x must be 16-byte aligned");
+            const size_t n_blocks = stage == STAGE_FROM_ACT ? 0 : B * d / 32;
             hipLaunchKernelGGL(moe_group_pairs_kernel, dim3(1 + (unsigned)((n_blocks * 8 + 1023) / 1024)), dim3(1024), 0, st, (int)B, (int)topk,
-                               shared, ids, weights, w.order, w.pos, w.rtok, w.goff, w.gexp, w.ngroups, w.pt.pw, x, n_blocks, w.xq, w.xs);
+                               shared, table->n_experts, ids, weights, w.order, w.pos, w.rtok, w.goff, w.gexp, w.ngroups, w.pt.pw, x, n_blocks, w.xq, w.xs);
             if ((s = mk_launch_status("moe_group_pairs")) != MK_OK) return s;
         }
-        {
+        if (stage != STAGE_FROM_ACT) {
             const uint8_t *const *pp[2] = {table->w1p, table->w3p};
             const uint8_t *const *sp[2] = {table->w1s, table->w3s};
             float *gu[2] = {w.g, w.u};
@@ -796,9 +829,11 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
         {
             const size_t n_blocks = P * inter / 32;
             hipLaunchKernelGGL(moe_act_q8_grouped_kernel, dim3((unsigned)((n_blocks + 31) / 32)), dim3(256), 0, st, w.g, w.u, w.pt.pw, w.order,
-                               (int)inter, n_blocks, act_kind, limit, w.aq, w.as);
+                               (int)inter, n_blocks, act_kind, limit, stage == STAGE_FROM_ACT ? act_io : nullptr,
+                               stage == STAGE_ACT ? act_io : nullptr, w.aq, w.as);
             if ((s = mk_launch_status("moe_act_q8_grouped")) != MK_OK) return s;
         }
+        if (stage == STAGE_ACT) return MK_OK;
         {
             const uint8_t *const *pp[1] = {table->w2p};
             const uint8_t *const *sp[1] = {table->w2s};
@@ -809,6 +844,7 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
                            (int)topk, (int)d, act_kind == MK_ACT_DS ? 1 : 0, out);
         return mk_launch_status("moe_combine_grouped");
     }
+    float *af = stage == STAGE_ALL ? w.af : act_io;  // [P][inter] activation rows in (token, slot) order
     if (fast) {
         FusedArgs fa;
         fa.tab = *table;
@@ -823,15 +859,17 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
         fa.act_kind = act_kind;
         fa.ds_rule = act_kind == MK_ACT_DS ? 1 : 0;
         fa.limit = limit;
-        fa.af = w.af;
+        fa.af = af;
         fa.out = out;
-        switch (nb) {
-            case 32: s = launch_gate_up_rows<32>(fa, B, st); break;
-            case 64: s = launch_gate_up_rows<64>(fa, B, st); break;
-            case 128: s = launch_gate_up_rows<128>(fa, B, st); break;
-            default: s = launch_gate_up_rows<224>(fa, B, st); break;
+        if (stage != STAGE_FROM_ACT) {
+            switch (nb) {
+                case 32: s = launch_gate_up_rows<32>(fa, B, st); break;
+                case 64: s = launch_gate_up_rows<64>(fa, B, st); break;
+                case 128: s = launch_gate_up_rows<128>(fa, B, st); break;
+                default: s = launch_gate_up_rows<224>(fa, B, st); break;
+            }
+            if (s != MK_OK || stage == STAGE_ACT) return s;
         }
-        if (s != MK_OK) return s;
         switch (nbi) {
             case 32: return launch_down_fused<32>(fa, B, st);
             case 64: return launch_down_fused<64>(fa, B, st);
@@ -842,24 +880,38 @@ extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t 
                        w.pt, w.o, w.g, w.u, (int)d, (int)inter);
     s = mk_launch_status("moe_setup");
     if (s != MK_OK) return s;
-    if (mode == MK_MODE_Q8) {
-        if ((s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
-    }
-    {
+    const bool q8 = mode == MK_MODE_Q8;
+    if (stage != STAGE_FROM_ACT) {
         // composed path (any shape, both modes): gate and up as grouped GEMVs,
         // elementwise activation, then (q8) the activation's own quantization
-        const bool q8 = mode == MK_MODE_Q8;
+        if (q8 && (s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
         if ((s = mk_gemv_grouped_internal(q8, w.pt.w1p, w.pt.w1s, P, inter, d, w.xq, w.xs, x, w.pt.xidx, w.pt.gptr, st)) != MK_OK) return s;
         if ((s = mk_gemv_grouped_internal(q8, w.pt.w3p, w.pt.w3s, P, inter, d, w.xq, w.xs, x, w.pt.xidx, w.pt.uptr, st)) != MK_OK) return s;
         const int n = (int)(P * inter);
         hipLaunchKernelGGL(moe_act_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.pt.pw, (int)inter, n, act_kind, limit,
-                           w.af);
-        if ((s = mk_launch_status("moe_act")) != MK_OK) return s;
-        if (q8 && (s = mk_dev_quantize_q8(w.af, P, inter, w.aq, w.as, stream)) != MK_OK) return s;
+                           af);
+        if ((s = mk_launch_status("moe_act")) != MK_OK || stage == STAGE_ACT) return s;
     }
-    if ((s = mk_gemv_grouped_internal(mode == MK_MODE_Q8, w.pt.w2p, w.pt.w2s, P, d, inter, w.aq, w.as, w.af, w.pt.aidx, w.pt.optr, st)) != MK_OK)
-        return s;
+    if (q8 && (s = mk_dev_quantize_q8(af, P, inter, w.aq, w.as, stream)) != MK_OK) return s;
+    if ((s = mk_gemv_grouped_internal(q8, w.pt.w2p, w.pt.w2s, P, d, inter, w.aq, w.as, af, w.pt.aidx, w.pt.optr, st)) != MK_OK) return s;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((d + 255) / 256), (unsigned)B), dim3(256), 0, st, w.o, w.pt.pw, per, (int)topk, (int)d,
                        act_kind == MK_ACT_DS ? 1 : 0, out);
     return mk_launch_status("moe_combine");
+}
+}  // namespace
+
+extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
+                                 const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream) {
+    return moe_decode_impl(table, B, topk, ids, weights, shared, x, mode, act_kind, limit, workspace, out, stream, STAGE_ALL, nullptr);
+}
+
+extern "C" int mk_dev_moe_decode_act(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
+                                     const float *x, int mode, int act_kind, float limit, void *workspace, float *act, void *stream) {
+    return moe_decode_impl(table, B, topk, ids, weights, shared, x, mode, act_kind, limit, workspace, nullptr, stream, STAGE_ACT, act);
+}
+
+extern "C" int mk_dev_moe_decode_from_act(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights,
+                                          int shared, const float *act, int mode, int act_kind, void *workspace, float *out, void *stream) {
+    return moe_decode_impl(table, B, topk, ids, weights, shared, nullptr, mode, act_kind, 0.0f, workspace, out, stream, STAGE_FROM_ACT,
+                           const_cast<float *>(act));
 }

@@ -293,6 +293,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->table.w2s = tab + 5 * n_experts;
     s->table.d = d;
     s->table.inter = inter;
+    s->table.n_experts = n_experts;
     *out = s;
     return MK_OK;
 }

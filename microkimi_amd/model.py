@@ -141,7 +141,7 @@ class PackedExperts:
         dev = w1[0][0].device
         arr = lambda lst, k: torch.tensor([t[k].data_ptr() for t in lst], dtype=torch.int64, device=dev)
         self._ptrs = [arr(w1, 0), arr(w1, 1), arr(w3, 0), arr(w3, 1), arr(w2, 0), arr(w2, 1)]
-        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter)
+        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n)
         self._ws = None
 
 
@@ -160,6 +160,56 @@ def moe_decode(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_S
     check(lib.mk_dev_moe_decode(C.byref(experts.table), B, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), shared,
                                 ptr(x.contiguous()), mode, act_kind, float(limit), ptr(experts._ws), ptr(out), cur_stream()))
     return out
+
+
+def _moe_ws(experts, B, topk, shared, device):
+    import torch
+    need = lib.mk_moe_decode_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    if experts._ws is None or experts._ws.numel() < need:
+        experts._ws = torch.empty(need, dtype=torch.uint8, device=device)
+    return experts._ws
+
+
+def moe_decode_act(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_SWIGLU, limit=0.0):
+    """First half of moe_decode: ACT(W1_e x_t, W3_e x_t) per (token, slot) pair (the shared expert is the last slot),
+    the f32 rows that the W2 matvec of src/model.rs:2255-2259 / src/deepseek.rs:1088-1089 takes.  Returns
+    [B, per, inter]."""
+    import torch
+    _lib.require_device()
+    B, topk = ids.shape
+    per = topk + (1 if shared >= 0 else 0)
+    act = torch.empty((B, per, experts.inter), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_moe_decode_act(C.byref(experts.table), B, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), shared,
+                                    ptr(x.contiguous()), mode, act_kind, float(limit), ptr(_moe_ws(experts, B, topk, shared, x.device)),
+                                    ptr(act), cur_stream()))
+    return act
+
+
+def moe_decode_from_act(experts, ids, weights, act, shared=-1, mode=MODE_Q8, act_kind=ACT_SWIGLU):
+    """Second half of moe_decode: the W2 matvecs on given activation rows [B, per, inter] and the weighted sum in slot
+    order (src/model.rs:2255-2259, 2346-2351).  Returns [B, d]."""
+    import torch
+    _lib.require_device()
+    B, topk = ids.shape
+    out = torch.empty((B, experts.d), dtype=torch.float32, device=act.device)
+    check(lib.mk_dev_moe_decode_from_act(C.byref(experts.table), B, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), shared,
+                                         ptr(act.contiguous()), mode, act_kind, ptr(_moe_ws(experts, B, topk, shared, act.device)), ptr(out),
+                                         cur_stream()))
+    return out
+
+
+def moe_prefill_intermediates(experts, T, topk):
+    """Views of mk_dev_moe_prefill's intermediates inside the workspace of the last moe_prefill call on `experts`
+    (grouping of src/model.rs:2539-2544 and the per-pair rows before the weighted sum): dict with order, pos,
+    offsets (int32), g and u [P, inter] and o [P, d] (f32), rows in grouped order."""
+    import torch
+    lay = _lib.PrefillLayout()
+    check(lib.mk_moe_prefill_workspace_layout(T, topk, experts.n, experts.d, experts.inter, C.byref(lay)))
+    ws, P = experts._ws, T * topk
+    i32 = lambda off, n: ws[off:off + 4 * n].view(torch.int32)
+    f32 = lambda off, r, c: ws[off:off + 4 * r * c].view(torch.float32).view(r, c)
+    return {"order": i32(lay.order, P), "pos": i32(lay.pos, P), "offsets": i32(lay.offsets, experts.n + 1),
+            "g": f32(lay.g, P, experts.inter), "u": f32(lay.u, P, experts.inter), "o": f32(lay.o, P, experts.d)}
 
 
 def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None):

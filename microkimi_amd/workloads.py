@@ -67,14 +67,16 @@ def config3_raw(ctx, L=MLA_LATENT, R=MLA_ROPE, nh=MLA_HEADS):
 
 
 def q8_0_rows(x):
-    """q8_0 of the rows of x with the reference rule (dx = max/127, round half away, clamp), scales stored as f16."""
+    """q8_0 of the rows of x with the reference rule (src/q8.rs:57-68: dx = max/127 in f32, q = roundf(x / dx) clamped
+    to +-127, zero block -> scale 0), scales stored as f16.  The f32 quotient is rounded half away from zero in f64,
+    where |r| + 0.5 is exact, so that r = 0.49999997 gives 0 as roundf does."""
     x = np.ascontiguousarray(x, np.float32)
     n, w = x.shape
     b = x.reshape(n, w // 32, 32)
     dx = (np.abs(b).max(axis=2) / np.float32(127.0)).astype(np.float32)
     safe = np.where(dx == 0, np.float32(1), dx)
-    r = b / safe[..., None]
-    q = np.clip(np.sign(r) * np.floor(np.abs(r) + np.float32(0.5)), -127, 127)
+    r = (b / safe[..., None]).astype(np.float32).astype(np.float64)
+    q = np.clip(np.sign(r) * np.floor(np.abs(r) + 0.5), -127, 127)
     q = np.where(dx[..., None] == 0, 0, q).astype(np.int8).reshape(n, w)
     return q, dx.astype(np.float16)
 

@@ -26,7 +26,8 @@ def build(force=False):
 
 
 def _load():
-    if not os.path.exists(_SO):
+    src = os.path.join(_HERE, "mk_oracle.c")
+    if not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
         build()
     return C.CDLL(_SO)
 
@@ -80,6 +81,7 @@ _lib.orc_mxfp4_quantize.argtypes = [_f32p, _sz, _sz, C.c_int, _u8p, _u8p]
 _lib.orc_dequant_fp8.argtypes = [_u8p, _u8p, _sz, _sz, _f32p]
 _lib.orc_quantize_fp8.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
 _lib.orc_fp8_roundtrip.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
+_lib.orc_fp8_roundtrip_emax.argtypes = [_f32p, _sz, _sz, C.c_int, _u8p, _u8p]
 _lib.orc_quantize_q8.argtypes = [_f32p, _sz, _i8p, _f32p]
 _lib.orc_matvec_f32.argtypes = [_f32p, _sz, _sz, _f32p, _f32p]
 _lib.orc_matvec_packed_q8.argtypes = [_u8p, _u8p, _sz, _sz, _i8p, _f32p, _f32p]
@@ -101,6 +103,7 @@ _lib.orc_router_softmax.argtypes = [_f32p, _sz, _sz, _u32p, _f32p]
 _lib.orc_expert_forward_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _sz, _sz, C.c_float, _f32p]
 _PP = C.POINTER(_u8p)
 _lib.orc_expert_packed.argtypes = [_u8p, _u8p, _u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+_lib.orc_expert_act.argtypes = [_u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
 _lib.orc_moe_decode.argtypes = [_PP, _PP, _PP, _PP, _PP, _PP, _sz, _sz, _sz, _sz, _u32p, _f32p, C.c_int, _f32p, C.c_int, C.c_int,
                                 C.c_float, _sz, _f32p]
 _lib.orc_moe_prefill.argtypes = [_PP, _PP, _PP, _PP, _PP, _PP, _sz, _sz, _sz, _sz, _sz, _u32p, _f32p, _f32p, C.c_int, C.c_int, _f32p]
@@ -184,12 +187,13 @@ def quantize_fp8(w, rows, cols):
     return qw, scales
 
 
-def fp8_roundtrip(x, block):
-    """Returns (rounded x, e4m3 codes, e8m0 exponent bytes)."""
+def fp8_roundtrip(x, block, emax=8):
+    """Returns (rounded x, e4m3 codes, e8m0 exponent bytes).  emax = 8 is the reference's clamp of the scale exponent,
+    127 the full e8m0 range."""
     x = _c(x, np.float32).copy().reshape(-1)
     codes = np.empty(x.size, np.uint8)
     exps = np.empty((x.size + block - 1) // block, np.uint8)
-    _lib.orc_fp8_roundtrip(_p(x, _f32p), x.size, block, _p(codes, _u8p), _p(exps, _u8p))
+    _lib.orc_fp8_roundtrip_emax(_p(x, _f32p), x.size, block, emax, _p(codes, _u8p), _p(exps, _u8p))
     return x, codes, exps
 
 
@@ -201,6 +205,18 @@ def quantize_q8(x):
     s = np.empty(x.size // 32, np.float32)
     _lib.orc_quantize_q8(_p(x, _f32p), x.size, _p(q, _i8p), _p(s, _f32p))
     return q, s
+
+
+def q8_0_rows(x):
+    """quantize_q8 of every row of x [n][w]; the f32 block scales are also returned rounded to f16 (the q8_0 storage
+    form of the device caches).  Returns (q [n][w] int8, scales f32 [n][w/32], scales f16 [n][w/32])."""
+    x = _c(x, np.float32)
+    n, w = x.shape
+    q = np.empty((n, w), np.int8)
+    s = np.empty((n, w // 32), np.float32)
+    for i in range(n):
+        q[i], s[i] = quantize_q8(x[i])
+    return q, s, s.astype(np.float16)
 
 
 def block_dot(packed16, x32):
@@ -493,6 +509,16 @@ def expert_packed(w1, w3, w2, d, inter, x, mode=1, act_kind=ACT_SWIGLU, limit=0.
     return out
 
 
+def expert_act(w1, w3, d, inter, x, mode=1, act_kind=ACT_SWIGLU, limit=0.0, wgt=1.0):
+    """ACT(W1 x, W3 x): the f32 vector a packed expert hands to its W2 matvec."""
+    (w1p, w1s), (w3p, w3s) = (_chk_packed(p, s, inter, d) for (p, s) in (w1, w3))
+    x = _c(x, np.float32)
+    act = np.empty(inter, np.float32)
+    _lib.orc_expert_act(_p(w1p, _u8p), _p(w1s, _u8p), _p(w3p, _u8p), _p(w3s, _u8p), d, inter, _p(x, _f32p), mode, act_kind, limit, wgt,
+                        _p(act, _f32p))
+    return act
+
+
 def moe_decode(table, ids, weights, x, shared=-1, mode=1, act_kind=ACT_SWIGLU, limit=0.0, threads=1):
     ids, weights, x = _c(ids, np.uint32), _c(weights, np.float32), _c(x, np.float32)
     B, topk = ids.shape
@@ -505,6 +531,8 @@ def moe_decode(table, ids, weights, x, shared=-1, mode=1, act_kind=ACT_SWIGLU, l
 
 
 def moe_prefill(table, ids, weights, x, act_kind=ACT_SWIGLU, round_mxfp8=False):
+    """round_mxfp8: False/0 the reference's f32 arithmetic; True/1 inputs and activation through the reference's
+    fp8_roundtrip per 32; 2 the same with the full e8m0 scale range (no saturation)."""
     ids, weights, x = _c(ids, np.uint32), _c(weights, np.float32), _c(x, np.float32)
     n, topk = ids.shape
     out = np.empty((n, table.d), np.float32)

@@ -234,7 +234,11 @@ ORC_API void orc_quantize_fp8(const float *w, size_t rows, size_t cols, uint8_t 
 /* src/deepseek.rs:312-322: act_quant round trip, pow2 scale per `block`.
  * Also returns the scale exponent bytes (e + 127) when exps != NULL: that is
  * the MXFP8 (e4m3 + e8m0) activation encoding the block-scaled GEMM consumes. */
-ORC_API void orc_fp8_roundtrip(float *x, size_t n, size_t block, uint8_t *codes, uint8_t *exps) {
+/* The same round trip with the upper clamp of the scale exponent as a parameter.  The reference clamps at 8
+ * (its rule for DeepSeek's activations); with emax = 127 the whole e8m0 range is used and no block saturates,
+ * which is how the prefill expert section of this build encodes its MXFP8 activations (a SwiGLU value of the
+ * benchmark's random experts reaches 4e5 > 448 * 2^8). */
+ORC_API void orc_fp8_roundtrip_emax(float *x, size_t n, size_t block, int emax, uint8_t *codes, uint8_t *exps) {
     for (size_t b0 = 0; b0 < n; b0 += block) {
         size_t len = (b0 + block <= n) ? block : n - b0;
         float amax = 0.0f;
@@ -242,7 +246,7 @@ ORC_API void orc_fp8_roundtrip(float *x, size_t n, size_t block, uint8_t *codes,
         amax = fmaxf(amax, 1e-4f);
         int e = (int)ceilf(log2f(amax / 448.0f));
         if (e < -127) e = -127;
-        if (e > 8) e = 8;
+        if (e > emax) e = emax;
         float s = orc_exp2_i(e);
         if (exps) exps[b0 / block] = (uint8_t)(e + 127);
         for (size_t i = 0; i < len; i++) {
@@ -251,6 +255,10 @@ ORC_API void orc_fp8_roundtrip(float *x, size_t n, size_t block, uint8_t *codes,
             x[b0 + i] = orc_e4m3_to_f32(c) * s;
         }
     }
+}
+
+ORC_API void orc_fp8_roundtrip(float *x, size_t n, size_t block, uint8_t *codes, uint8_t *exps) {
+    orc_fp8_roundtrip_emax(x, n, block, 8, codes, exps);
 }
 
 /* ------------------------------------------------------- q8 activations */
@@ -1106,15 +1114,13 @@ ORC_API void orc_expert_forward_f32(const float *w1, const float *w2, const floa
  *   ORC_ACT_DS      act = wgt * silu(min(g,L)) * clamp(u,L) (src/deepseek.rs:1083-1087; weight applied before W2) */
 enum { ORC_ACT_SWIGLU = 0, ORC_ACT_SITU = 1, ORC_ACT_DS = 2 };
 
-/* One packed expert on one input: the three matvec_packed calls of
- * src/model.rs:2246-2259 / src/deepseek.rs:1080-1089.  w1,w3: [inter][d],
- * w2: [d][inter]; each as (packed, scales).  mode as orc_matvec_packed. */
-ORC_API void orc_expert_packed(const uint8_t *w1p, const uint8_t *w1s, const uint8_t *w3p, const uint8_t *w3s, const uint8_t *w2p,
-                               const uint8_t *w2s, size_t d, size_t inter, const float *x, int mode, int act_kind, float limit,
-                               float wgt, float *out) {
+/* The first two matvec_packed calls of a packed expert and its activation
+ * (src/model.rs:2246-2252 / src/deepseek.rs:1080-1087): act[j] = ACT(W1 x, W3 x)[j],
+ * the f32 vector that the third call (W2) takes as its input. */
+ORC_API void orc_expert_act(const uint8_t *w1p, const uint8_t *w1s, const uint8_t *w3p, const uint8_t *w3s, size_t d, size_t inter,
+                            const float *x, int mode, int act_kind, float limit, float wgt, float *act) {
     float *a = (float *)malloc(sizeof(float) * inter);
     float *u = (float *)malloc(sizeof(float) * inter);
-    float *act = (float *)malloc(sizeof(float) * inter);
     orc_matvec_packed(w1p, w1s, inter, d, x, a, mode);
     orc_matvec_packed(w3p, w3s, inter, d, x, u, mode);
     for (size_t j = 0; j < inter; j++) {
@@ -1128,9 +1134,19 @@ ORC_API void orc_expert_packed(const uint8_t *w1p, const uint8_t *w1s, const uin
             act[j] = (a[j] / (1.0f + expf(-a[j]))) * u[j];
         }
     }
-    orc_matvec_packed(w2p, w2s, d, inter, act, out, mode);
     free(a);
     free(u);
+}
+
+/* One packed expert on one input: the three matvec_packed calls of
+ * src/model.rs:2246-2259 / src/deepseek.rs:1080-1089.  w1,w3: [inter][d],
+ * w2: [d][inter]; each as (packed, scales).  mode as orc_matvec_packed. */
+ORC_API void orc_expert_packed(const uint8_t *w1p, const uint8_t *w1s, const uint8_t *w3p, const uint8_t *w3s, const uint8_t *w2p,
+                               const uint8_t *w2s, size_t d, size_t inter, const float *x, int mode, int act_kind, float limit,
+                               float wgt, float *out) {
+    float *act = (float *)malloc(sizeof(float) * inter);
+    orc_expert_act(w1p, w1s, w3p, w3s, d, inter, x, mode, act_kind, limit, wgt, act);
+    orc_matvec_packed(w2p, w2s, d, inter, act, out, mode);
     free(act);
 }
 
@@ -1216,9 +1232,11 @@ ORC_API void orc_moe_decode(const uint8_t *const *w1p, const uint8_t *const *w1s
  * (token, slot), then per token the weighted sum in slot order.  Always the
  * f32 arithmetic of matvec_packed_nt.  act_kind SWIGLU or SITU.
  * When round_mxfp8 != 0 the gathered inputs and the activation are first
- * passed through the e4m3 + e8m0/32 round trip (orc_fp8_roundtrip, block 32
- * along K): that is the input precision of the block-scaled MFMA GEMM, and the
- * oracle it is compared against tightly. */
+ * passed through the e4m3 + e8m0/32 round trip (block 32 along K): that is the
+ * input precision of the block-scaled MFMA GEMM, and the oracle it is compared
+ * against tightly.  1: the reference's orc_fp8_roundtrip (scale exponent
+ * clamped at 8); 2: the full e8m0 range (orc_fp8_roundtrip_emax with 127), the
+ * encoding of the device's prefill section. */
 ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                              const uint8_t *const *w2p, const uint8_t *const *w2s, size_t n_experts, size_t d, size_t inter, size_t n,
                              size_t topk, const uint32_t *ids, const float *weights, const float *x, int act_kind, int round_mxfp8,
@@ -1240,7 +1258,7 @@ ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1
         for (size_t i = 0; i < m; i++) {
             size_t t = pairs[i] / topk;
             memcpy(tmp, x + t * d, sizeof(float) * d);
-            if (round_mxfp8) orc_fp8_roundtrip(tmp, d, 32, NULL, NULL);
+            if (round_mxfp8) orc_fp8_roundtrip_emax(tmp, d, 32, round_mxfp8 == 2 ? 127 : 8, NULL, NULL);
             for (size_t c = 0; c < d; c++) ht[c * m8 + i] = tmp[c];
         }
         float *a = (float *)malloc(sizeof(float) * m8 * inter);
@@ -1253,7 +1271,7 @@ ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1
                 float g = a[i * inter + j], uu = u[i * inter + j];
                 tmp[j] = (act_kind == ORC_ACT_SITU) ? orc_situ(g, uu) : (g / (1.0f + expf(-g))) * uu;
             }
-            if (round_mxfp8) orc_fp8_roundtrip(tmp, inter, 32, NULL, NULL);
+            if (round_mxfp8) orc_fp8_roundtrip_emax(tmp, inter, 32, round_mxfp8 == 2 ? 127 : 8, NULL, NULL);
             for (size_t j = 0; j < inter; j++) act_t[j * m8 + i] = tmp[j];
         }
         float *o = (float *)malloc(sizeof(float) * m8 * d);

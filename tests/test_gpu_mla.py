@@ -59,12 +59,21 @@ def test_production_shape_matrix_core_kernel(ctx, nh, qscale):
 
 
 def test_append_quantizes_like_the_reference():
+    # MlaCache::push (src/model.rs:1583-1618) against the oracle's quantize_q8 (src/q8.rs:49-69), the f32 block scale
+    # then stored as f16; with a zero block, exact ties (round half away), a value just below a tie and tiny values
     torch = torch_cuda()
     from microkimi_amd import model
     L, R, n = 512, 64, 40
-    lat, rope, q, lq, ls, rq, rs = make_cache(n, L, R, 4, 77)
+    lat, rope, q, _, _, _, _ = make_cache(n, L, R, 4, 77)
     lat[3, :32] = 0.0
-    lq, ls = __import__("microkimi_amd").workloads.q8_0_rows(lat)
+    lat[5, :32] = 0.0
+    lat[5, 0], lat[5, 1], lat[5, 2], lat[5, 3], lat[5, 4], lat[5, 5] = 127.0, 0.5, -0.5, 2.5, np.float32(0.49999997), -126.5
+    rope[6, :32] = 0.0
+    rope[6, 0], rope[6, 1], rope[6, 2] = -127.0, 1.5, np.float32(-0.49999997)
+    lat[7, 32:64] *= np.float32(1e-30)
+    lq, _, ls = oracle.q8_0_rows(lat)
+    rq, _, rs = oracle.q8_0_rows(rope)
+    assert list(lq[5, :6]) == [127, 1, -1, 3, 0, -127] and list(rq[6, :3]) == [-127, 2, 0]
     cache = model.MlaCache(L, R, n)
     for j in range(n):
         cache.push(dev(lat[j]), dev(rope[j]))

@@ -42,6 +42,30 @@ def test_quantize_bound_and_ties():
     assert s[0] == 1.0 and list(q[:5]) == [127, 1, -1, 2, 3]
 
 
+def test_quantize_just_below_a_tie_rounds_down():
+    # roundf, not floor(|r| + 0.5) in f32: 0.49999997 + 0.5 rounds to 1.0 in f32, roundf(0.49999997) is 0
+    x = np.zeros(32, np.float32)
+    x[0], x[1], x[2] = 127.0, np.float32(0.49999997), np.float32(-0.49999997)
+    q, s = oracle.quantize_q8(x)
+    assert s[0] == 1.0 and list(q[:3]) == [127, 0, 0]
+
+
+def test_workloads_q8_0_rows_equals_the_oracle():
+    # the benchmark's cache builder (numpy) against quantize_q8, including ties and the case above
+    from microkimi_amd import workloads
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((50, 576)).astype(np.float32)
+    x[0, :32] = 0.0
+    x[1, :32] = 0.0
+    x[1, 0], x[1, 1], x[1, 2], x[1, 3], x[1, 4] = 127.0, 0.5, -1.5, np.float32(0.49999997), 126.5
+    x[2, 32:64] = np.float32(1e-30)
+    q, s16 = workloads.q8_0_rows(x)
+    oq, os32, os16 = oracle.q8_0_rows(x)
+    assert np.array_equal(q, oq)
+    assert np.array_equal(s16.view(np.uint16), os16.view(np.uint16))
+    assert list(q[1, :5]) == [127, 1, -2, 0, 127]
+
+
 def test_block_dot_matches_brute_force_on_reference_stream():
     # src/q8.rs:283-296: seed 0xDEADBEEF, 2000 cases, x = (u8 % 255) as i8
     for scalar in (0, 1):
