@@ -485,6 +485,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", default="",
+                    help="comma-separated names of extras (mxfp4_gemv, moe_decode, mla_decode, grouped_gemm, vq1_gemv): run only "
+                         "those and print their figures as one JSON object (a development aid; the contract line needs a full run)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain 1 GiB device copies (a kernel of known traffic to scale rocprofv3 --pmc byte counters by)")
     args = ap.parse_args()
@@ -507,6 +510,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    if args.only:
+        table = {"mxfp4_gemv": bench_mxfp4_gemv, "moe_decode": bench_moe, "mla_decode": bench_mla, "grouped_gemm": bench_gemm, "vq1_gemv": bench_vq1}
+        res = {}
+        for name in args.only.split(","):
+            log(name, "...")
+            fn = table[name]
+            res[name] = fn(torch, not args.no_cpu) if name in ("mxfp4_gemv", "moe_decode", "mla_decode") else fn(torch)
+            torch.cuda.empty_cache()
+        print(json.dumps(res))
+        return
     log("lm_head ...")
     head, tensors = bench_lm_head(torch, args.steps, args.warmup)
     cpu = None
