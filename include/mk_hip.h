@@ -245,6 +245,20 @@ size_t mk_mla_decode_workspace_bytes(size_t nh, size_t L, size_t n_pos);
 int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos, const float *q,
                          size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream);
 
+/* mk_dev_mla_q8_decode for callers that cannot allocate or carry a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments without
+ * the workspace: the kernels' scratch (quantized query, the context splits' partial outputs and their softmax
+ * statistics) lives in a device array inside the library, 16 916 480 bytes that every GPU the library runs on holds
+ * until the process ends.  Limits: nh <= 128 (mk_mla_decode_static_max_heads) and L <= 512; beyond them the call
+ * returns MK_ERR_UNSUPPORTED and writes nothing.  It calls no hipMalloc / hipFree and no allocating library routine.
+ * All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race -- issue them
+ * on one stream or order them with events.  Nothing in the array needs clearing between calls (every word a call
+ * reads was written by that call).  mk_init resolves the array's device address; without mk_init the first call on a
+ * device does, so make that first call outside a graph capture. */
+size_t mk_mla_decode_static_max_heads(void);
+int mk_dev_mla_q8_decode_static(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos, const float *q,
+                                size_t nh, size_t L, size_t R, float scale, float *out, void *stream);
+
 /* MlaCache::push (src/model.rs:1583-1618) for the shared-latent cache: quantize
  * one position (latent [L] f32, rope [R] f32) into row `pos` of the cache arrays.
  * latent and rope must be 16-byte aligned. */

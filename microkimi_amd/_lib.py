@@ -74,6 +74,8 @@ def _load():
         "mk_dev_matvec_f32": (i32, [vp, sz, sz, vp, sz, vp, vp]),
         "mk_mla_decode_workspace_bytes": (sz, [sz, sz, sz]),
         "mk_dev_mla_q8_decode": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp, vp]),
+        "mk_mla_decode_static_max_heads": (sz, []),
+        "mk_dev_mla_q8_decode_static": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp]),
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
         "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),

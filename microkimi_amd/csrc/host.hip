@@ -128,6 +128,7 @@ extern "C" int mk_init(int device) {
     }
     if (mk_check_hip(hipSetDevice(device), "hipSetDevice") != MK_OK) return g_ctx.status = MK_ERR_HIP;
     if (mk_check_hip(hipStreamCreate(&g_ctx.stream), "hipStreamCreate") != MK_OK) return g_ctx.status = MK_ERR_HIP;
+    if (mk_mla_static_init(nullptr) != MK_OK) return g_ctx.status = MK_ERR_HIP;
     const char *mb = getenv("MK_GPU_CACHE_MB");
     if (mb && *mb) g_ctx.cache_cap = (size_t)strtoull(mb, nullptr, 10) << 20;
     g_ctx.device = device;

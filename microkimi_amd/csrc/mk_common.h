@@ -319,6 +319,10 @@ int mk_env_int(const char *name, int dflt);
 // that the value is a constant (no getenv on the launch path).
 #define MK_TUNE(name, dflt) ([]() -> int { static const int v = mk_env_int(name, dflt); return v; }())
 
+// mla.hip: resolves the device address of the static scratch of mk_dev_mla_q8_decode_static on the current device
+// (once per device); out_ptr may be null.
+int mk_mla_static_init(void **out_ptr);
+
 // mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,

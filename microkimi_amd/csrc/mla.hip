@@ -17,6 +17,8 @@
 // (src/selftest.rs:648-704, 1e-5).
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "mk_common.h"
 
 namespace {
@@ -713,4 +715,57 @@ int mla_decode_impl(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q
 extern "C" int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos,
                                     const float *q, size_t nh, size_t L, size_t R, float scale, void *workspace, float *out, void *stream) {
     return mla_decode_impl(lat_q, lat_s, rope_q, rope_s, pos, q, nh, L, R, scale, workspace, out, stream);
+}
+
+// ------------------------------------------------ the entry point that allocates nothing
+// mk_dev_mla_q8_decode_static: the same kernels with their scratch (the quantized query, the splits' partial outputs
+// and their (max, normaliser) pairs) in a file-scope device array instead of a caller's workspace.  Sized for the
+// largest supported call: 128 heads, latent 512, MAX_SPLITS splits.
+constexpr size_t MLA_STATIC_MAX_NH = 128, MLA_STATIC_MAX_L = 512;
+constexpr size_t MLA_STATIC_BYTES = 128 * 512 + 128 * 16 * 4 + (size_t)MAX_SPLITS * 128 * 512 * 4 + 2 * (size_t)MAX_SPLITS * 128 * 4;
+static __device__ __align__(256) uint8_t mla_static_scratch[MLA_STATIC_BYTES];
+
+namespace {
+constexpr int MLA_STATIC_MAX_DEVICES = 64;
+std::mutex g_static_mu;
+void *g_static_ptr[MLA_STATIC_MAX_DEVICES] = {};  // device address of mla_static_scratch on each device (every GPU holds its own copy)
+}  // namespace
+
+// Resolves the scratch array's address on the current device, once per device.  mk_init calls it, so a caller that
+// initialises the library before it starts a graph capture never reaches the runtime query from inside the capture.
+int mk_mla_static_init(void **out_ptr) {
+    int dev = 0;
+    MK_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MLA_STATIC_MAX_DEVICES) {
+        mk_set_error("device index %d beyond the %d this entry point keeps scratch addresses for", dev, MLA_STATIC_MAX_DEVICES);
+        return MK_ERR_UNSUPPORTED;
+    }
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void *p = nullptr;
+        MK_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(mla_static_scratch)));
+        if (!p || ((uintptr_t)p & 255) != 0) {
+            mk_set_error("hipGetSymbolAddress(mla_static_scratch) gave %p", p);
+            return MK_ERR_HIP;
+        }
+        g_static_ptr[dev] = p;
+    }
+    if (out_ptr) *out_ptr = g_static_ptr[dev];
+    return MK_OK;
+}
+
+extern "C" size_t mk_mla_decode_static_max_heads(void) { return MLA_STATIC_MAX_NH; }
+
+extern "C" int mk_dev_mla_q8_decode_static(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos,
+                                           const float *q, size_t nh, size_t L, size_t R, float scale, float *out, void *stream) {
+    if (nh > MLA_STATIC_MAX_NH || L > MLA_STATIC_MAX_L || mk_mla_decode_workspace_bytes(nh, L, pos + 1) > MLA_STATIC_BYTES) {
+        mk_set_error("mk_dev_mla_q8_decode_static holds scratch for at most %zu heads of latent width %zu (%zu bytes); got %zu heads, width %zu: "
+                     "use mk_dev_mla_q8_decode with a workspace",
+                     MLA_STATIC_MAX_NH, MLA_STATIC_MAX_L, MLA_STATIC_BYTES, nh, L);
+        return MK_ERR_UNSUPPORTED;
+    }
+    void *scratch = nullptr;  // the array's device address: never the array's name, which is a host-side stand-in here
+    const int s = mk_mla_static_init(&scratch);
+    if (s != MK_OK) return s;
+    return mla_decode_impl(lat_q, lat_s, rope_q, rope_s, pos, q, nh, L, R, scale, scratch, out, stream);
 }
