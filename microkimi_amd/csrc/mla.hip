@@ -210,58 +210,19 @@ __global__ __launch_bounds__(256) void mla_partial_kernel(MlaArgs a) {
 }
 
 // ---------------------------------------------------------------- MFMA kernel
-// Latent 512 + rope 64 (the shape of the production models).  A workgroup serves
-// 16 heads over one split of the context; its 4 waves share each 64-position
-// tile in LDS and take 16 positions each, every wave with its own running
-// (max, normaliser, output) that are merged through LDS at the end -- so a
-// split costs one partial result per 16 heads, not one per wave.  Per tile and
-// wave:
-//
-//   scores^T [pos][head]  latent part: v_mfma_i32_16x16x64_i8, cache bytes as the
-//            A operand (lane l: row l%16, bytes 16*(l/16).. of the 64-byte step),
-//            q8 query as B.  One instruction spans two scale blocks: it is
-//            issued once with the query masked to the first block and once
-//            whole, the second block's dot is the difference.  The integer block
-//            dots are scaled by (query block scale * cache block scale) in f32,
-//            the reference's per-block term (src/model.rs:1858-1871).  Rope part:
-//            f16 MFMA in split precision (see "out"): the rope bytes times
-//            their scale as exact f16 pairs, the f32 query as hi + lo.
-//   softmax  a lane holds head l%16 and positions 4*(l/16)+r, which is the A
-//            operand layout of the next product: probabilities stay in registers.
-//   out      v_mfma_f32_16x16x32_f16 in split precision.  The cache value
-//            v = q * s (int8 times f16 scale, src/model.rs:1641-1646) is formed
-//            as an exact f16 pair: hi = rn(q*s), lo = fma(q, s, -hi) (the product
-//            has 19 significant bits and the residual is a multiple of the
-//            scale's ulp, so hi + lo == v).  The probability is split the same
-//            way (hi = rn(p), lo = rn(p - hi), relative error below 2^-21).  K = 32
-//            holds the 16 positions twice: (p_hi | p_hi) and (p_lo | 0) against
-//            (v_hi | v_lo); accumulation is f32.  A lane reads 4 rows x
-//            16 dims and transposes 4x4 byte blocks in registers, because the
-//            operand wants positions contiguous in a lane and the cache has dims
-//            contiguous.  Lane l keeps dims 16c..16c+15 and 256+16c.. (c = l%16)
-//            of heads 4*(l/16)+r.
-//
-// The query's latent part is quantized in the prologue, in registers
-// (src/model.rs:1812-1821).  The next tile is fetched into registers while the
-// current one is computed and written to the other LDS buffer afterwards (one
-// barrier per tile).  With a single split the workgroup writes the normalised
-// output itself.
+// Latent 512 + rope 64 (the shape of the production models).
 constexpr int ML = 512, MR = 64;
-constexpr float MLA_TAU = 8.0f;
 constexpr int KROW = 592;      // LDS row stride in bytes: 16 rows at 16-byte granularity fall in distinct banks
 constexpr int KS_STRIDE = 68;  // f32 scale row [block][position]
 constexpr int KH_STRIDE = 72;  // f16 scale row [block][position]
 constexpr int KS_OFF = TJ * KROW;
 constexpr int KH_OFF = KS_OFF + 18 * KS_STRIDE * 4;
 constexpr int MLA_TILE_BYTES = KH_OFF + 16 * KH_STRIDE * 2;
-constexpr int MLA_Q_OFF = 2 * MLA_TILE_BYTES;              // the quantized query, exchanged between the waves in the prologue
-constexpr int MLA_Q_BYTES = 8 * 64 * 16 + 8 * 64 * 8;
-constexpr int MLA_O_OFF = 1024;                            // epilogue: after the waves' (m, l), four [16 heads][512] f32 outputs
-constexpr int MLA_LDS_BYTES = MLA_O_OFF + 4 * 16 * ML * 4;
-static_assert(MLA_Q_OFF + MLA_Q_BYTES <= MLA_LDS_BYTES, "LDS layout");
+constexpr int P_STRIDE = 72;   // f16 per probability row: 64 positions + 8 of padding
 
 typedef _Float16 mk_h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 mk_h8 __attribute__((ext_vector_type(8)));
+typedef int mk_i2 __attribute__((ext_vector_type(2)));
 
 struct MlaStage {
     mk_i4 lat[8];
@@ -270,19 +231,79 @@ struct MlaStage {
     uint32_t rs;
 };
 
-__device__ __forceinline__ float mk_byte_f32(int w, int k) { return (float)(int8_t)((uint32_t)w >> (8 * k)); }
 __device__ __forceinline__ uint32_t mk_perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
 
-__global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restrict__ out) {
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for every global load
+// in flight (s_waitcnt vmcnt(0)), which would put the latency of the next tile's prefetch into each barrier.
+__device__ __forceinline__ void mk_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// e^x for x <= 0 through the hardware 2^x (v_exp_f32, about 1 ulp): the rounding of x * log2(e) adds |x| * 2^-24
+// relative, 2e-6 at x = -30, where the weight itself is 1e-13.  exp(-inf) = 0.
+__device__ __forceinline__ float mk_exp_neg(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
+// A workgroup of four waves serves 16 heads over one split of the context, 64 positions (a tile) at a time, from ONE
+// tile buffer: 180 registers and 62 KiB of LDS, so two workgroups share a compute unit.
+//
+//   scores   wave w: positions 16 w .. 16 w + 15 against the 16 heads.  Latent part: v_mfma_i32_16x16x64_i8, cache bytes
+//            as the A operand (lane l: row l%16, bytes 16*(l/16).. of the 64-byte step), q8 query as B.  One
+//            instruction spans two scale blocks: it is issued with the second block's query bytes zeroed and whole,
+//            the second block's dot is the difference.  The integer block dots are scaled by (query block scale *
+//            cache block scale) in f32, the reference's per-block term (src/model.rs:1858-1871).  Rope part:
+//            v_mfma_f32_16x16x32_f16 in split precision: the rope bytes times their scale as exact f16 pairs (see
+//            "out"), the f32 query as hi + lo.
+//   softmax  one reference point per head and tile: the four waves exchange maxima and sums through LDS and write the
+//            probabilities as f16 pairs into a [head][position] tile
+//   out      wave w owns the output dims 128 w .. 128 w + 127 of all heads over all 64 positions: each cache byte is
+//            converted once per workgroup.  v_mfma_f32_16x16x32_f16 in split precision: the cache value v = q * s (int8
+//            times f16 scale, src/model.rs:1641-1646) is formed as an exact f16 pair, hi = rn(q*s), lo = fma(q, s, -hi)
+//            (the product has 19 significant bits and the residual is a multiple of the scale's ulp, so hi + lo == v);
+//            the probability is split the same way (hi = rn(p), lo = rn(p - hi), relative error below 2^-21); the
+//            products p_hi v_hi, p_hi v_lo, p_lo v_hi are accumulated in f32.  The B operand (K = 32 positions x N = 16
+//            dims) wants the 8 positions of a lane contiguous while the cache has dims contiguous:
+//            ds_read_b64_tr_b8 delivers that transpose (a group of 16 lanes reads 8 rows x 16 bytes, lanes 2k and 2k+1
+//            giving the two halves of row k, and lane i receives byte i of every row; measured with byte-valued LDS
+//            contents).  Bytes -> f16 with v_perm: 0x6400 | (b ^ 0x80) is 1152 + b.  Two operand tiles are converted
+//            and multiplied at a time.
+//   refill   barrier, the prefetched next tile goes from registers into the one buffer, barrier
+//
+// A split's partial result is one [16][512] block per workgroup; with a single split the workgroup writes the
+// normalised output itself.  Where the time goes at 16k context (64 splits x 8 head groups, 31 us; measured by
+// compiling parts out): launch, first tile and exit 5 us, query quantization 2 us, the partial results' stores 5.5 us,
+// rope scores + softmax + refill 1.5 us per tile, latent scores 1.35 us per tile, output product 1.85 us per tile; the
+// barriers cost 1.2 us in all and the prefetch loads nothing.  Two other forms were built, passed the parity tests and
+// measured the same 30-31 us: eight waves serving 32 heads (half the byte conversions per head, but lock-stepped
+// phases and one workgroup per CU), and four waves serving 32 heads with one wave per SIMD.
+constexpr int NHG = 1;  // 16-head groups per workgroup
+struct M4 {
+    static constexpr int HEADS = 16 * NHG;
+    static constexpr int Q_OFF = MLA_TILE_BYTES;                // [NHG][8 S][64 lanes] 16-byte query operands
+    static constexpr int Z_OFF = Q_OFF + NHG * 8 * 64 * 16;     // 64 zero bytes: the "masked" query operand of lanes 32-63
+    static constexpr int QS_OFF = Z_OFF + 64;                   // [NHG][8][64] scale pairs
+    static constexpr int P_OFF = QS_OFF + NHG * 8 * 64 * 8;     // P hi [HEADS][P_STRIDE] f16, then P lo
+    static constexpr int ST_OFF = P_OFF + 2 * HEADS * P_STRIDE * 2;
+    static constexpr int LDS_BYTES = ST_OFF + (4 * HEADS + 4 * HEADS + 3 * HEADS) * 4;  // wmax, wsum, corr, final m, final l
+};
+
+__global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__restrict__ out) {
+    using C4 = M4;
+    constexpr int HEADS = C4::HEADS;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int q4 = lane >> 4, c = lane & 15;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int split = blockIdx.x;
-    const int hbase = blockIdx.y * 16;
+    const int hbase = blockIdx.y * HEADS;
     const int p_begin = split * a.split_len;
     const int p_end = min(p_begin + a.split_len, a.n_pos);
     const int ntiles = (p_end - p_begin + TJ - 1) / TJ;
     const int last_pos = a.n_pos - 1;
+
+    float *wmax_l = reinterpret_cast<float *>(lds + C4::ST_OFF);  // [4 waves][HEADS]
+    float *wsum_l = wmax_l + 4 * HEADS;
+    float *corr_l = wsum_l + 4 * HEADS;
+    float *finm_l = corr_l + HEADS, *finl_l = finm_l + HEADS;
+    _Float16 *ph_l = reinterpret_cast<_Float16 *>(lds + C4::P_OFF);
+    _Float16 *pl_l = ph_l + HEADS * P_STRIDE;
+    mk_i4 *qb_l = reinterpret_cast<mk_i4 *>(lds + C4::Q_OFF);   // [hg][S][lane]
+    mk_f2 *qs_l = reinterpret_cast<mk_f2 *>(lds + C4::QS_OFF);  // [hg][S][lane]: scales of blocks 2S, 2S+1
 
     // byte offsets stay below 2^31: the host checks the position count
     auto stage_load = [&](MlaStage &st, int t0) {
@@ -294,18 +315,18 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
         const uint32_t pr = (uint32_t)min(t0 + (tid >> 2), last_pos);
         st.rope = mk_ldg128(a.rope_q + (pr * MR + (tid & 3) * 16));
         st.ls = mk_ldg64(a.lat_s + (pr * (ML / 32) + 4 * (tid & 3)));
-        const uint32_t pr2 = (uint32_t)min(t0 + (tid & 63), last_pos);
+        const uint32_t pr2 = (uint32_t)min(t0 + lane, last_pos);
         st.rs = mk_ldg_u32(a.rope_s + pr2 * (MR / 32));
     };
-    auto stage_store = [&](const MlaStage &st, uint8_t *buf) {
-        float *ks = reinterpret_cast<float *>(buf + KS_OFF);
-        uint16_t *kh = reinterpret_cast<uint16_t *>(buf + KH_OFF);
+    auto stage_store = [&](const MlaStage &st) {
+        float *ks = reinterpret_cast<float *>(lds + KS_OFF);
+        uint16_t *kh = reinterpret_cast<uint16_t *>(lds + KH_OFF);
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const int i = tid + 256 * k;
-            *reinterpret_cast<mk_i4 *>(buf + (i >> 5) * KROW + (i & 31) * 16) = st.lat[k];  // row (tid >> 5) + 8k
+            *reinterpret_cast<mk_i4 *>(lds + (i >> 5) * KROW + (i & 31) * 16) = st.lat[k];  // row (tid >> 5) + 8k
         }
-        *reinterpret_cast<mk_i4 *>(buf + (tid >> 2) * KROW + ML + (tid & 3) * 16) = st.rope;
+        *reinterpret_cast<mk_i4 *>(lds + (tid >> 2) * KROW + ML + (tid & 3) * 16) = st.rope;
         const int pos = tid >> 2, g0 = 4 * (tid & 3);
         const uint16_t h0 = (uint16_t)(st.ls.x & 0xFFFFu), h1 = (uint16_t)(st.ls.x >> 16);
         const uint16_t h2 = (uint16_t)(st.ls.y & 0xFFFFu), h3 = (uint16_t)(st.ls.y >> 16);
@@ -317,94 +338,96 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
         kh[(g0 + 1) * KH_STRIDE + pos] = h1;
         kh[(g0 + 2) * KH_STRIDE + pos] = h2;
         kh[(g0 + 3) * KH_STRIDE + pos] = h3;
-        if (tid < 64) {
-            ks[16 * KS_STRIDE + tid] = mk_f16_bits_to_f32((uint16_t)(st.rs & 0xFFFFu));
-            ks[17 * KS_STRIDE + tid] = mk_f16_bits_to_f32((uint16_t)(st.rs >> 16));
+        if (wave == 0) {
+            ks[16 * KS_STRIDE + lane] = mk_f16_bits_to_f32((uint16_t)(st.rs & 0xFFFFu));
+            ks[17 * KS_STRIDE + lane] = mk_f16_bits_to_f32((uint16_t)(st.rs >> 16));
         }
     };
     MlaStage st;
     stage_load(st, p_begin);
 
-    // The query of head hbase + c.  Lane (c, q4) owns bytes 16*(4S+q4).. of each
-    // 64-value step S, half of scale block 2S + q4/2; its partner for the block
-    // maximum is lane ^ 16.  Each wave quantizes two of the eight steps and
-    // passes them to the others through LDS.
-    const int head = min(hbase + c, a.nh - 1);
-    const float *qrow = a.q + (size_t)head * (ML + MR);
-    mk_i4 *qb_l = reinterpret_cast<mk_i4 *>(lds + MLA_Q_OFF);            // [S][lane]
-    mk_f2 *qs_l = reinterpret_cast<mk_f2 *>(lds + MLA_Q_OFF + 8 * 64 * 16);  // [S][lane]: scales of blocks 2S, 2S+1
+    // The queries.  Lane (c, q4) owns bytes 16*(4S+q4).. of each 64-value step S of head c of a 16-head group, half of
+    // scale block 2S + q4/2; its partner for the block maximum is lane ^ 16.  Each wave quantizes two of the eight
+    // steps of every head group and passes them to the others through LDS (src/model.rs:1812-1821).
+    mk_h8 qrh[NHG][2], qrl[NHG][2];  // rope part of the query (f32 in the reference), dims 16*q4.. of head c, as f16 pairs hi + lo
+    {
+        const int q4 = lane >> 4, c = lane & 15;
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int S = 2 * wave + i;
-        const mk_f4 *src = reinterpret_cast<const mk_f4 *>(qrow + (4 * S + q4) * 16);
-        mk_f4 v[4];
-        float mx = 0.0f;
+        for (int hg = 0; hg < NHG; hg++) {
+            const float *qrow = a.q + (size_t)min(hbase + 16 * hg + c, a.nh - 1) * (ML + MR);
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            v[k] = src[k];
-            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, MK_WAVE));
-        const float dx = mx / 127.0f;
-        mk_i4 packed;
+            for (int i = 0; i < 2; i++) {
+                const int S = 2 * wave + i;
+                const mk_f4 *src = reinterpret_cast<const mk_f4 *>(qrow + (4 * S + q4) * 16);
+                mk_f4 v[4];
+                float mx = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            uint32_t w = 0;
-            if (dx != 0.0f) {
-                float qf[4];
-                mk_q8_round4(v[k], dx, qf);  // the same integers as mk_q8_round, a third of the instructions
-                w = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
-                    ((uint32_t)(int)qf[3] << 24);
+                for (int k = 0; k < 4; k++) {
+                    v[k] = src[k];
+                    mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, MK_WAVE));
+                const float dx = mx / 127.0f;
+                mk_i4 packed;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    uint32_t w = 0;
+                    if (dx != 0.0f) {
+                        float qf[4];
+                        mk_q8_round4(v[k], dx, qf);
+                        w = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                            ((uint32_t)(int)qf[3] << 24);
+                    }
+                    packed[k] = (int)w;
+                }
+                const float other = __shfl_xor(dx, 32, MK_WAVE);
+                qb_l[(hg * 8 + S) * 64 + lane] = packed;
+                qs_l[(hg * 8 + S) * 64 + lane] = q4 < 2 ? mk_f2{dx, other} : mk_f2{other, dx};
             }
-            packed[k] = (int)w;
-        }
-        const float other = __shfl_xor(dx, 32, MK_WAVE);
-        qb_l[S * 64 + lane] = packed;
-        qs_l[S * 64 + lane] = q4 < 2 ? mk_f2{dx, other} : mk_f2{other, dx};
-    }
-    const int blk0_mask = q4 < 2 ? -1 : 0;
-    // rope part of the query (f32 in the reference), dims 16*q4.. of head c, as an f16 pair hi + lo
-    mk_h8 qrh[2], qrl[2];
 #pragma unroll
-    for (int k = 0; k < 16; k++) {
-        const float v = qrow[ML + 16 * q4 + k];
-        const _Float16 hi = (_Float16)v;
-        qrh[k >> 3][k & 7] = hi;
-        qrl[k >> 3][k & 7] = (_Float16)(v - (float)hi);
+            for (int k = 0; k < 16; k++) {
+                const float v = qrow[ML + 16 * q4 + k];
+                const _Float16 hi = (_Float16)v;
+                qrh[hg][k >> 3][k & 7] = hi;
+                qrl[hg][k >> 3][k & 7] = (_Float16)(v - (float)hi);
+            }
+        }
+        if (tid < 16) reinterpret_cast<uint32_t *>(lds + C4::Z_OFF)[tid] = 0u;
     }
 
-    mk_f4 o[32];
+    mk_f4 o[NHG][8];  // heads 16 hg + 4 q4 + r, dim 128 wave + 16 n + c
 #pragma unroll
-    for (int n = 0; n < 32; n++) o[n] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
-    float m = -INFINITY, l = 0.0f;
+    for (int hg = 0; hg < NHG; hg++)
+#pragma unroll
+        for (int n = 0; n < 8; n++) o[hg][n] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m[NHG], l[NHG];  // of head 16 hg + c; the four waves keep equal copies
+#pragma unroll
+    for (int hg = 0; hg < NHG; hg++) {
+        m[hg] = -INFINITY;
+        l[hg] = 0.0f;
+    }
     const mk_i4 zero4 = {0, 0, 0, 0};
-    stage_store(st, lds);
+    stage_store(st);
     __syncthreads();
 
-    auto compute_tile = [&](const uint8_t *buf, int t0) {
-        const float *ks = reinterpret_cast<const float *>(buf + KS_OFF);
-        // ---- scores of this wave's 16 positions
+    for (int tile = 0; tile < ntiles; tile++) {
+        const int t0 = p_begin + tile * TJ;
+        const int t_next = min(t0 + TJ, last_pos);  // clamped: the last iteration's fetch is not used
+        // The lane index is made opaque once per tile: every LDS address below is then recomputed from it inside the
+        // loop (a few instructions each) instead of being kept in a register of its own across the whole kernel.
+        int lane_v = lane;
+        asm volatile("" : "+v"(lane_v));
+        const int q4 = lane_v >> 4, c = lane_v & 15;
+        const float *ks = reinterpret_cast<const float *>(lds + KS_OFF);
+        // ---- scores of this wave's 16 positions x 16 NHG heads
         const int prow = 16 * wave;
-        const uint8_t *krow = buf + (prow + c) * KROW + q4 * 16;
-        float sc[4];
+        const uint8_t *krow = lds + (prow + c) * KROW + q4 * 16;
+        float sc[NHG][4];
         {
-            // all integer block dots first (16 independent MFMAs), the rope product while
-            // they drain, then the per-block scaling: no MFMA result is waited for early
-            mk_i4 ka[8], c0[8], cf[8];
-#pragma unroll
-            for (int S = 0; S < 8; S++) ka[S] = *reinterpret_cast<const mk_i4 *>(krow + S * 64);
-            const mk_i4 kr = *reinterpret_cast<const mk_i4 *>(buf + (prow + c) * KROW + ML + q4 * 16);
+            // rope: bytes -> exact f16 pairs (see the output product below), 64 dims = two K = 32 steps
+            const mk_i4 kr = *reinterpret_cast<const mk_i4 *>(lds + (prow + c) * KROW + ML + q4 * 16);
             const float rsc = ks[(16 + (q4 >> 1)) * KS_STRIDE + prow + c];
-#pragma unroll
-            for (int S = 0; S < 8; S++) {
-                const mk_i4 qv = qb_l[S * 64 + lane];  // the query stays in LDS: registers are the scarce resource here
-                const mk_i4 qm = {qv[0] & blk0_mask, qv[1] & blk0_mask, qv[2] & blk0_mask, qv[3] & blk0_mask};
-                c0[S] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[S], qm, zero4, 0, 0, 0);
-                cf[S] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[S], qv, zero4, 0, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // rope: bytes -> exact f16 pairs (see the output product below), 64 dims = two K=32 steps
-            mk_f4 cr0 = {0.0f, 0.0f, 0.0f, 0.0f}, cr1 = cr0;
+            mk_f4 cr[NHG];
             {
                 const _Float16 rs = (_Float16)rsc;  // exact: the scale is stored as f16
                 const mk_h2 s2 = {rs, rs};
@@ -426,184 +449,237 @@ __global__ __launch_bounds__(256) void mla_mfma_kernel(MlaArgs a, float *__restr
                     kl8[k >> 1][4 * (k & 1) + 2] = l1.x;
                     kl8[k >> 1][4 * (k & 1) + 3] = l1.y;
                 }
-                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrh[0], cr0, 0, 0, 0);
-                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrh[1], cr1, 0, 0, 0);
-                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[0], qrh[0], cr0, 0, 0, 0);
-                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[1], qrh[1], cr1, 0, 0, 0);
-                cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrl[0], cr0, 0, 0, 0);
-                cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrl[1], cr1, 0, 0, 0);
+#pragma unroll
+                for (int hg = 0; hg < NHG; hg++) {
+                    mk_f4 cr0 = {0.0f, 0.0f, 0.0f, 0.0f}, cr1 = cr0;
+                    cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrh[hg][0], cr0, 0, 0, 0);
+                    cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrh[hg][1], cr1, 0, 0, 0);
+                    cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[0], qrh[hg][0], cr0, 0, 0, 0);
+                    cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kl8[1], qrh[hg][1], cr1, 0, 0, 0);
+                    cr0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[0], qrl[hg][0], cr0, 0, 0, 0);
+                    cr1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kh8[1], qrl[hg][1], cr1, 0, 0, 0);
+                    cr[hg] = cr0 + cr1;
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
-            mk_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+            // latent part in two halves of four 64-value steps.  A step spans two scale blocks: the instruction is issued
+            // with the query of lanes 32-63 (the second block) replaced by zeros, and whole; the second block's dot is
+            // the difference.  The zeroed operand is read from a zero region of LDS, one address select per step.
+            mk_f4 acc[NHG];
 #pragma unroll
-            for (int S = 0; S < 8; S++) {
-                const mk_f2 qsc = qs_l[S * 64 + lane];
-                const mk_f4 k0 = *reinterpret_cast<const mk_f4 *>(ks + (2 * S) * KS_STRIDE + prow + 4 * q4);
-                const mk_f4 k1 = *reinterpret_cast<const mk_f4 *>(ks + (2 * S + 1) * KS_STRIDE + prow + 4 * q4);
+            for (int hg = 0; hg < NHG; hg++) acc[hg] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+            const uint32_t q_addr = (uint32_t)(C4::Q_OFF + lane_v * 16), qm_addr = q4 < 2 ? q_addr : (uint32_t)C4::Z_OFF;
+            const uint32_t qm_step = q4 < 2 ? 1024u : 0u;
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[r] += (qsc.x * k0[r]) * (float)c0[S][r] + (qsc.y * k1[r]) * (float)(cf[S][r] - c0[S][r]);
-            }
+            for (int half = 0; half < 2; half++) {
+                mk_i4 ka[4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) sc[r] = (t0 + prow + 4 * q4 + r) < p_end ? (acc[r] + (cr0[r] + cr1[r])) * a.scale : -INFINITY;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- online softmax for head c over the 16 positions
-        float tm = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-        tm = mk_rows_max(tm);
-        // The reference point of the exponentials moves only when the maximum has
-        // grown by more than MLA_TAU: weights stay below e^TAU and the 128
-        // accumulators are rescaled a few times per split instead of every tile.
-        const bool move = tm > m + MLA_TAU;  // false for a wave that still has no valid position (tm = -inf)
-        const float m_new = move ? tm : m;
-        const float m_ref = m_new == -INFINITY ? 0.0f : m_new;  // no position seen yet: all weights 0
-        const float corr = move ? expf(m - m_ref) : 1.0f;
-        float ts = 0.0f;
-        mk_h8 pa1, pa2;  // (p_hi | p_hi) and (p_lo | 0) over this lane's 4 positions
+                for (int S = 0; S < 4; S++) ka[S] = *reinterpret_cast<const mk_i4 *>(krow + (4 * half + S) * 64);
+                mk_f4 k0[4], k1[4];  // the cache's block scales of this lane's 4 positions: shared by the head groups
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const float pv = expf(sc[r] - m_ref);
-            ts += pv;
-            const _Float16 hi = (_Float16)pv;
-            pa1[r] = hi;
-            pa1[4 + r] = hi;
-            pa2[r] = (_Float16)(pv - (float)hi);
-            pa2[4 + r] = (_Float16)0.0f;
-        }
-        ts = mk_rows_sum(ts);
-        l = l * corr + ts;
-        m = m_new;
-        if (__any(move)) {
-            // the accumulators hold heads 4*q4+r: fetch their corrections from the lanes that own those heads
-            float oc[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) oc[r] = __shfl(corr, 4 * q4 + r, MK_WAVE);
-            // The accumulators live in the MFMA accumulation registers.  The empty asm statements pin each
-            // one there on entry and exit of this rare block, so the copies through the vector registers
-            // that the multiplication needs stay inside it instead of being paid on every tile.
-#pragma unroll
-            for (int n = 0; n < 32; n++) {
-                mk_f4 t = o[n];
-                asm volatile("" : "+a"(t));
-#pragma unroll
-                for (int r = 0; r < 4; r++) t[r] *= oc[r];
-                asm volatile("" : "+a"(t));
-                o[n] = t;
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- out += P V over rows prow + 4*q4 + e
-        const uint8_t *vbase = buf + (prow + 4 * q4) * KROW + 16 * c;
-        const uint16_t *kh = reinterpret_cast<const uint16_t *>(buf + KH_OFF);
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            // scales of the 4 rows for this lane's block, as f16 pairs (rows 0,1) and (rows 2,3)
-            const mk_u2 sraw = *reinterpret_cast<const mk_u2 *>(kh + (8 * half + (c >> 1)) * KH_STRIDE + prow + 4 * q4);
-            const uint32_t sw0 = sraw[0], sw1 = sraw[1];  // scalars first: a bit cast straight from a vector element reads element 0
-            const mk_h2 s01 = __builtin_bit_cast(mk_h2, sw0), s23 = __builtin_bit_cast(mk_h2, sw1);
-            mk_i4 w[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) w[e] = *reinterpret_cast<const mk_i4 *>(vbase + e * KROW + 256 * half);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                // 4 rows x 4 dims of bytes, sign bit flipped (b ^ 0x80 = b + 128 as unsigned), transposed
-                const uint32_t d0 = (uint32_t)w[0][k] ^ 0x80808080u, d1 = (uint32_t)w[1][k] ^ 0x80808080u;
-                const uint32_t d2 = (uint32_t)w[2][k] ^ 0x80808080u, d3 = (uint32_t)w[3][k] ^ 0x80808080u;
-                const uint32_t t01l = mk_perm(d1, d0, 0x05010400u), t01h = mk_perm(d1, d0, 0x07030602u);  // (r0 r1) pairs of dims 0,1 / 2,3
-                const uint32_t t23l = mk_perm(d3, d2, 0x05010400u), t23h = mk_perm(d3, d2, 0x07030602u);
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint32_t p01 = j < 2 ? t01l : t01h, p23 = j < 2 ? t23l : t23h;
-                    // two bytes -> two f16: 0x6400 | u is 1024 + u exactly (the 0x64 bytes come out of the same v_perm);
-                    // minus 1152 gives the signed byte
-                    const uint32_t sel = (j & 1) ? 0x04030402u : 0x04010400u;
-                    const uint32_t f01 = mk_perm(0x64646464u, p01, sel), f23 = mk_perm(0x64646464u, p23, sel);
-                    const mk_h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-                    const mk_h2 v01 = __builtin_bit_cast(mk_h2, f01) - bias, v23 = __builtin_bit_cast(mk_h2, f23) - bias;
-                    const mk_h2 hi01 = v01 * s01, hi23 = v23 * s23;
-                    const mk_h2 lo01 = __builtin_elementwise_fma(v01, s01, -hi01), lo23 = __builtin_elementwise_fma(v23, s23, -hi23);
-                    const mk_h8 b = {hi01.x, hi01.y, hi23.x, hi23.y, lo01.x, lo01.y, lo23.x, lo23.y};  // (v_hi | v_lo)
-                    const int n = 16 * half + 4 * k + j;
-                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa1, b, o[n], 0, 0, 0);  // p_hi v_hi + p_hi v_lo
-                    o[n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa2, b, o[n], 0, 0, 0);  // p_lo v_hi
+                for (int S = 0; S < 4; S++) {
+                    const int SS = 4 * half + S;
+                    k0[S] = *reinterpret_cast<const mk_f4 *>(ks + (2 * SS) * KS_STRIDE + prow + 4 * q4);
+                    k1[S] = *reinterpret_cast<const mk_f4 *>(ks + (2 * SS + 1) * KS_STRIDE + prow + 4 * q4);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int hg = 0; hg < NHG; hg++) {
+                    mk_i4 c0[4], cf[4];
+#pragma unroll
+                    for (int S = 0; S < 4; S++) {
+                        const int SS = hg * 8 + 4 * half + S;
+                        const mk_i4 qv = *reinterpret_cast<const mk_i4 *>(lds + q_addr + SS * 1024);
+                        const mk_i4 qm = *reinterpret_cast<const mk_i4 *>(lds + qm_addr + SS * qm_step);
+                        c0[S] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[S], qm, zero4, 0, 0, 0);
+                        cf[S] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ka[S], qv, zero4, 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int S = 0; S < 4; S++) {
+                        const mk_f2 qsc = qs_l[(hg * 8 + 4 * half + S) * 64 + lane_v];
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            acc[hg][r] = fmaf(qsc.y * k1[S][r], (float)(cf[S][r] - c0[S][r]), fmaf(qsc.x * k0[S][r], (float)c0[S][r], acc[hg][r]));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int hg = 0; hg < NHG; hg++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) sc[hg][r] = (t0 + prow + 4 * q4 + r) < p_end ? (acc[hg][r] + cr[hg][r]) * a.scale : -INFINITY;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // the next tile's loads go out behind the score stage (whose registers they would otherwise share); the softmax
+        // exchange and the output product cover their latency
+        stage_load(st, t_next);
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- online softmax: one reference point per head and tile for all four waves
+#pragma unroll
+        for (int hg = 0; hg < NHG; hg++) {
+            float tm = fmaxf(fmaxf(sc[hg][0], sc[hg][1]), fmaxf(sc[hg][2], sc[hg][3]));
+            tm = mk_rows_max(tm);
+            if (q4 == 0) wmax_l[wave * HEADS + 16 * hg + c] = tm;
+        }
+        mk_lds_barrier();
+#pragma unroll
+        for (int hg = 0; hg < NHG; hg++) {
+            const int hl = 16 * hg + c;
+            const float mt4 = fmaxf(fmaxf(wmax_l[hl], wmax_l[HEADS + hl]), fmaxf(wmax_l[2 * HEADS + hl], wmax_l[3 * HEADS + hl]));  // finite
+            const float m_new = fmaxf(m[hg], mt4);
+            const float corr = mk_exp_neg(m[hg] - m_new);  // first tile: exp(-inf) = 0
+            float ts = 0.0f;
+            mk_h4 phi, plo;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float pv = mk_exp_neg(sc[hg][r] - m_new);
+                ts += pv;
+                const _Float16 hi = (_Float16)pv;
+                phi[r] = hi;
+                plo[r] = (_Float16)(pv - (float)hi);
+            }
+            ts = mk_rows_sum(ts);
+            if (q4 == 0) wsum_l[wave * HEADS + hl] = ts;
+            if (wave == 0 && q4 == 0) corr_l[hl] = corr;
+            *reinterpret_cast<mk_h4 *>(ph_l + hl * P_STRIDE + prow + 4 * q4) = phi;
+            *reinterpret_cast<mk_h4 *>(pl_l + hl * P_STRIDE + prow + 4 * q4) = plo;
+            l[hg] *= corr;
+            m[hg] = m_new;
+        }
+        mk_lds_barrier();
+#pragma unroll
+        for (int hg = 0; hg < NHG; hg++) {
+            const int hl = 16 * hg + c;
+            l[hg] += (wsum_l[hl] + wsum_l[HEADS + hl]) + (wsum_l[2 * HEADS + hl] + wsum_l[3 * HEADS + hl]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- out[heads][dims 128 wave ..] += P V over the tile's 64 positions
+#pragma unroll
+        for (int hg = 0; hg < NHG; hg++) {
+            const mk_f4 cA = *reinterpret_cast<const mk_f4 *>(corr_l + 16 * hg + 4 * q4);
+#pragma unroll
+            for (int n = 0; n < 8; n++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[hg][n][r] *= cA[r];
+        }
+        const uint16_t *kh = reinterpret_cast<const uint16_t *>(lds + KH_OFF);
+        const mk_h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+        // operand tile (kstep, n): positions 32 kstep + 8 q4 .. + 7, dims 128 wave + 16 n + c.  Transposed read: lanes
+        // 2k, 2k+1 of each 16-lane group address the two halves of row p0 + k, dims d0..d0+15; lane c receives dim
+        // d0 + c of rows p0 .. p0 + 7.  Two tiles (n, n + 1) go through conversion and the matrix cores together, so
+        // that consecutive matrix instructions accumulate into different registers; the next pair's bytes and scales
+        // are requested before the current pair is converted.
+        mk_i2 raw[2][2];
+        mk_i4 sraw[2];
+        auto fetch = [&](int j, int slot) {  // pair j = (kstep, n / 2): both tiles lie in one 32-dim block
+            const int p0 = 32 * (j >> 2) + 8 * q4;
+            const int d0 = 128 * wave + 32 * (j & 3);
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const uint8_t *src = lds + (p0 + (c >> 1)) * KROW + d0 + 16 * e + 8 * (c & 1);
+                raw[slot][e] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) mk_i2 *)src);
+            }
+            sraw[slot] = *reinterpret_cast<const mk_i4 *>(kh + (d0 >> 5) * KH_STRIDE + p0);
+        };
+        fetch(0, 0);
+        mk_h8 pah[NHG], pal[NHG];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int kstep = j >> 2, n0 = 2 * (j & 3);
+            if ((j & 3) == 0) {
+                const int p0 = 32 * kstep + 8 * q4;  // this lane's 8 positions of the K = 32 step
+#pragma unroll
+                for (int hg = 0; hg < NHG; hg++) {
+                    pah[hg] = *reinterpret_cast<const mk_h8 *>(ph_l + (16 * hg + c) * P_STRIDE + p0);
+                    pal[hg] = *reinterpret_cast<const mk_h8 *>(pl_l + (16 * hg + c) * P_STRIDE + p0);
+                }
+            }
+            if (j + 1 < 8) fetch(j + 1, (j + 1) & 1);
+            const int sl = j & 1;
+            const uint32_t s0 = (uint32_t)sraw[sl][0], s1 = (uint32_t)sraw[sl][1], s2 = (uint32_t)sraw[sl][2], s3 = (uint32_t)sraw[sl][3];
+            const mk_h2 s01 = __builtin_bit_cast(mk_h2, s0), s23 = __builtin_bit_cast(mk_h2, s1);
+            const mk_h2 s45 = __builtin_bit_cast(mk_h2, s2), s67 = __builtin_bit_cast(mk_h2, s3);
+            mk_h8 bh[2], bl[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const uint32_t w0 = (uint32_t)raw[sl][e][0] ^ 0x80808080u, w1 = (uint32_t)raw[sl][e][1] ^ 0x80808080u;
+                const mk_h2 v01 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, w0, 0x04010400u)) - bias;
+                const mk_h2 v23 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, w0, 0x04030402u)) - bias;
+                const mk_h2 v45 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, w1, 0x04010400u)) - bias;
+                const mk_h2 v67 = __builtin_bit_cast(mk_h2, mk_perm(0x64646464u, w1, 0x04030402u)) - bias;
+                const mk_h2 h01 = v01 * s01, h23 = v23 * s23, h45 = v45 * s45, h67 = v67 * s67;
+                const mk_h2 l01 = __builtin_elementwise_fma(v01, s01, -h01), l23 = __builtin_elementwise_fma(v23, s23, -h23);
+                const mk_h2 l45 = __builtin_elementwise_fma(v45, s45, -h45), l67 = __builtin_elementwise_fma(v67, s67, -h67);
+                bh[e] = mk_h8{h01.x, h01.y, h23.x, h23.y, h45.x, h45.y, h67.x, h67.y};
+                bl[e] = mk_h8{l01.x, l01.y, l23.x, l23.y, l45.x, l45.y, l67.x, l67.y};
+            }
+#pragma unroll
+            for (int hg = 0; hg < NHG; hg++) {
+                o[hg][n0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pah[hg], bh[0], o[hg][n0], 0, 0, 0);
+                o[hg][n0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pah[hg], bh[1], o[hg][n0 + 1], 0, 0, 0);
+            }
+#pragma unroll
+            for (int hg = 0; hg < NHG; hg++) {
+                o[hg][n0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pah[hg], bl[0], o[hg][n0], 0, 0, 0);
+                o[hg][n0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pah[hg], bl[1], o[hg][n0 + 1], 0, 0, 0);
+            }
+#pragma unroll
+            for (int hg = 0; hg < NHG; hg++) {
+                o[hg][n0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pal[hg], bh[0], o[hg][n0], 0, 0, 0);
+                o[hg][n0 + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pal[hg], bh[1], o[hg][n0 + 1], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // ---- refill the tile buffer: everybody is done reading it, then the prefetched rows go in
+        mk_lds_barrier();
+        stage_store(st);
+        mk_lds_barrier();
+    }
+
+    // ---- store: the split's partial [HEADS][512] block, or the normalised rows when there is one split
+    {
+        const int q4 = lane >> 4, c = lane & 15;
+        if (wave == 0 && q4 == 0) {
+#pragma unroll
+            for (int hg = 0; hg < NHG; hg++) {
+                finm_l[16 * hg + c] = m[hg];
+                finl_l[16 * hg + c] = l[hg];
             }
         }
-    };
-
-    for (int tile = 0; tile < ntiles; tile++) {
-        const int t0 = p_begin + tile * TJ;
-        stage_load(st, min(t0 + TJ, last_pos));  // next tile (clamped: the last iteration's fetch is not used)
-        compute_tile(lds + (tile & 1) * MLA_TILE_BYTES, t0);
-        stage_store(st, lds + ((tile + 1) & 1) * MLA_TILE_BYTES);
         __syncthreads();
-    }
-
-    // ---- merge the four waves (log-sum-exp), then store
-    float *ml = reinterpret_cast<float *>(lds);              // [wave][head][m, l]
-    float *ob = reinterpret_cast<float *>(lds + MLA_O_OFF);  // [wave][head][dim]
-    if (q4 == 0) {
-        ml[(wave * 16 + c) * 2] = m;
-        ml[(wave * 16 + c) * 2 + 1] = l;
-    }
-    __syncthreads();
+        const bool single = a.n_splits == 1;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int h = 4 * q4 + r;
-        float mm = -INFINITY;
+        for (int hg = 0; hg < NHG; hg++) {
+            const mk_f4 lt = *reinterpret_cast<const mk_f4 *>(finl_l + 16 * hg + 4 * q4);
 #pragma unroll
-        for (int w2 = 0; w2 < 4; w2++) mm = fmaxf(mm, ml[(w2 * 16 + h) * 2]);
-        const float wself = expf(ml[(wave * 16 + h) * 2] - mm);
-        float *dst = ob + ((size_t)(wave * 16 + h)) * ML + 16 * c;
+            for (int r = 0; r < 4; r++) {
+                const int h = hbase + 16 * hg + 4 * q4 + r;
+                if (h < a.nh) {
+                    float *dst = (single ? out + (size_t)h * ML : a.po + ((size_t)split * a.nh + h) * ML) + 128 * wave + c;
+                    if (single) {
 #pragma unroll
-        for (int half = 0; half < 2; half++)
+                        for (int n = 0; n < 8; n++) dst[16 * n] = o[hg][n][r] / lt[r];
+                    } else {
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const mk_f4 v = {o[16 * half + 4 * k][r] * wself, o[16 * half + 4 * k + 1][r] * wself, o[16 * half + 4 * k + 2][r] * wself,
-                                 o[16 * half + 4 * k + 3][r] * wself};
-                // 16-byte chunks are swizzled within groups of four so that the 16 lanes of a row hit 16 bank groups
-                *reinterpret_cast<mk_f4 *>(dst + 256 * half + 4 * (k ^ ((c >> 2) & 3))) = v;
+                        for (int n = 0; n < 8; n++) dst[16 * n] = o[hg][n][r];
+                    }
+                }
             }
-    }
-    __syncthreads();
-    {
-        // thread: head tid/16, dims 4*(tid%16 + 16*i)
-        const int hl = tid >> 4, h = hbase + hl;
-        float mm = -INFINITY;
-#pragma unroll
-        for (int w2 = 0; w2 < 4; w2++) mm = fmaxf(mm, ml[(w2 * 16 + hl) * 2]);
-        float lt = 0.0f;
-#pragma unroll
-        for (int w2 = 0; w2 < 4; w2++) lt += ml[(w2 * 16 + hl) * 2 + 1] * expf(ml[(w2 * 16 + hl) * 2] - mm);
-        if (h < a.nh) {
-            const bool single = a.n_splits == 1;
-            float *dst = single ? out + (size_t)h * ML : a.po + ((size_t)split * a.nh + h) * ML;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int ch = (tid & 15) + 16 * i;  // logical chunk: dims 4*ch..; written by lane c = (ch >> 2) & 15
-                const int d = 4 * ch, dp = 4 * (ch ^ ((ch >> 4) & 3));
-                mk_f4 v = *reinterpret_cast<const mk_f4 *>(ob + (size_t)hl * ML + dp);
-#pragma unroll
-                for (int w2 = 1; w2 < 4; w2++) v += *reinterpret_cast<const mk_f4 *>(ob + (size_t)(w2 * 16 + hl) * ML + dp);
-                if (single) v = mk_f4{v.x / lt, v.y / lt, v.z / lt, v.w / lt};
-                *reinterpret_cast<mk_f4 *>(dst + d) = v;
-            }
-            if (!single && (tid & 15) == 0) {
-                a.pm[split * a.nh + h] = mm;
-                a.pl[split * a.nh + h] = lt;
-            }
+        }
+        if (!single && tid < HEADS && hbase + tid < a.nh) {
+            a.pm[split * a.nh + hbase + tid] = finm_l[tid];
+            a.pl[split * a.nh + hbase + tid] = finl_l[tid];
         }
     }
 }
 
-// log-sum-exp merge of the splits.  A workgroup per head: thread (d4, part)
-// sums every 4th split for 4 output dims with all its loads in flight at once,
-// the four parts meet in LDS.
-__global__ __launch_bounds__(512) void mla_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
+// log-sum-exp merge of the splits.  A workgroup per (head, quarter of the output dims): thread (d4, part) sums
+// every 8th split for 4 output dims with all its loads in flight at once, the eight parts meet in LDS.
+__global__ __launch_bounds__(256) void mla_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
                                                         int nh, int L, int n_splits, float *__restrict__ out) {
     __shared__ float w_l[MAX_SPLITS];
     __shared__ float den_l;
-    __shared__ mk_f4 part_l[3][128];
+    __shared__ mk_f4 part_l[7][32];
     const int h = blockIdx.x, tid = threadIdx.x;
     if (tid < 64) {
         float mx = -INFINITY;
@@ -619,17 +695,18 @@ __global__ __launch_bounds__(512) void mla_merge_kernel(const float *__restrict_
         if (tid == 0) den_l = den;
     }
     __syncthreads();
-    const int d4 = tid & 127, part = tid >> 7;
+    const int d4 = blockIdx.y * 32 + (tid & 31), part = tid >> 5;
     const bool live = d4 * 4 < L;
     mk_f4 num = {0.0f, 0.0f, 0.0f, 0.0f};
     if (live) {
-#pragma unroll 4
-        for (int s = part; s < n_splits; s += 4) num += *reinterpret_cast<const mk_f4 *>(po + ((size_t)s * nh + h) * L + d4 * 4) * w_l[s];
+#pragma unroll 8
+        for (int s = part; s < n_splits; s += 8) num += *reinterpret_cast<const mk_f4 *>(po + ((size_t)s * nh + h) * L + d4 * 4) * w_l[s];
     }
-    if (part > 0) part_l[part - 1][d4] = num;
+    if (part > 0) part_l[part - 1][tid & 31] = num;
     __syncthreads();
     if (part == 0 && live) {
-        num += part_l[0][d4] + part_l[1][d4] + part_l[2][d4];
+#pragma unroll
+        for (int k = 0; k < 7; k++) num += part_l[k][tid & 31];
         const float den = den_l;
         *reinterpret_cast<mk_f4 *>(out + (size_t)h * L + d4 * 4) = mk_f4{num.x / den, num.y / den, num.z / den, num.w / den};
     }
@@ -682,10 +759,12 @@ int mla_decode_impl(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q
     a.scale = scale;
     const int tiles = (n_pos + TJ - 1) / TJ;
     const bool mfma = L == ML && R == MR && !MK_TUNE("MK_MLA_VALU", 0);
-    // split the context in whole tiles: one workgroup per CU for the MFMA kernel
-    // (its register and LDS budget allows one), about 512 for the VALU kernel
+    // Split the context in whole tiles.  Every split costs a partial result per head (2 KiB each way: stored here,
+    // read by the merge), every workgroup a launch slot: two workgroups per CU (512) pay from about 8k positions,
+    // below that one per CU (256).  About 512 workgroups for the VALU kernel.
     const int head_groups = (int)((nh + HPG - 1) / HPG);
-    int want = ((mfma ? 256 : 512) + head_groups - 1) / head_groups;
+    const int wgs_tune = MK_TUNE("MK_MLA_WGS", 0);
+    int want = ((wgs_tune ? wgs_tune : (mfma && n_pos < 8192 ? 256 : 512)) + head_groups - 1) / head_groups;
     if (want > MAX_SPLITS) want = MAX_SPLITS;
     if (want > tiles) want = tiles;
     const int tiles_per_split = (tiles + want - 1) / want;
@@ -694,8 +773,8 @@ int mla_decode_impl(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q
     int s;
     if (mfma) {
         MK_REQUIRE(n_pos <= (1 << 22), "the MFMA kernel addresses the cache with 32-bit byte offsets: at most 4 Mi positions");
-        if ((s = mk_lds_opt_in(reinterpret_cast<const void *>(mla_mfma_kernel), MLA_LDS_BYTES)) != MK_OK) return s;
-        hipLaunchKernelGGL(mla_mfma_kernel, dim3(a.n_splits, head_groups), dim3(256), MLA_LDS_BYTES, st, a, out);
+        if ((s = mk_lds_opt_in(reinterpret_cast<const void *>(mla_mfma_kernel), M4::LDS_BYTES)) != MK_OK) return s;
+        hipLaunchKernelGGL(mla_mfma_kernel, dim3(a.n_splits, head_groups), dim3(256), M4::LDS_BYTES, st, a, out);
         if ((s = mk_launch_status("mla_mfma")) != MK_OK) return s;
         if (a.n_splits == 1) return MK_OK;
     } else {
@@ -707,7 +786,7 @@ int mla_decode_impl(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q
         hipLaunchKernelGGL(mla_partial_kernel, dim3(a.n_splits, head_groups), dim3(256), lds, st, a);
         if ((s = mk_launch_status("mla_partial")) != MK_OK) return s;
     }
-    hipLaunchKernelGGL(mla_merge_kernel, dim3((unsigned)nh), dim3(512), 0, st, a.po, a.pm, a.pl, (int)nh, (int)L, a.n_splits, out);
+    hipLaunchKernelGGL(mla_merge_kernel, dim3((unsigned)nh, (unsigned)((L / 4 + 31) / 32)), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)L, a.n_splits, out);
     return mk_launch_status("mla_merge");
 }
 }  // namespace
