@@ -239,7 +239,7 @@ int mk_dev_matvec_f32(const float *w, size_t rows, size_t cols, const float *x, 
  *   q [nh][L+R] f32 (latent part first), out [nh][L] f32
  * score = (dot(q_rope, dequant(rope)) + sum_g (qs_g*ks_g)*idot_g) * scale over the
  * q8-quantized latent query; online softmax; out = sum p * dequant(latent) / l.
- * Positions 0..=pos are attended (pos < n).  L % 32 == 0, R % 32 == 0.
+ * Positions 0..=pos are attended (pos < n).  L a multiple of 64 up to 512; R 0, 32 or 64.
  * workspace: mk_mla_decode_workspace_bytes(nh, L, pos + 1). */
 size_t mk_mla_decode_workspace_bytes(size_t nh, size_t L, size_t n_pos);
 int mk_dev_mla_q8_decode(const int8_t *lat_q, const void *lat_s, const int8_t *rope_q, const void *rope_s, size_t pos, const float *q,
@@ -264,6 +264,30 @@ int mk_dev_mla_q8_decode_static(const int8_t *lat_q, const void *lat_s, const in
  * latent and rope must be 16-byte aligned. */
 int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, size_t R, size_t pos, int8_t *lat_q, void *lat_s,
                             int8_t *rope_q, void *rope_s, void *stream);
+
+/* The cache layout the reference keeps (MlaCache, src/model.rs:765-781): per position
+ *   kq [nh][nope] i8, ks [nh][nope/32] f32   latent part of K per head
+ *   kr [rope] f32                             rope part of K, shared by the heads, never quantized
+ *   vq [nh][vd] i8, vs [nh][vd/32] f32        V per head
+ * positions contiguous in each array.  nope a multiple of 32 up to 256, vd a multiple of 32 up to 512.  The Hadamard
+ * option (MICROKIMI_KV_HADAMARD, off by default) is not built.
+ *
+ * _append   MlaCache::push (src/model.rs:1583-1618) for n_new positions into rows pos0 .. pos0 + n_new - 1 (n_new > 1
+ *           is MlaCache::assign_f32, src/model.rs:1680-1692): k_rows [n_new][nh][nope+rope] (latent part first per
+ *           head; the rope row is taken from head 0), v_rows [n_new][nh][vd].
+ * _to_f32   MlaCache::to_f32 (src/model.rs:1623-1676): k [n][nh][nope+rope], v [n][nh][vd].
+ * _q8_attn  mla_attn_flash_q8_mqa (src/model.rs:1804-1908) for m queries q [m][nh][nope+rope]: query i attends the
+ *           positions 0 ..= pos0 + i (m = 1: the decode step of mla_forward, src/model.rs:1980-1985; m > 1: the
+ *           per-position loop of mla_prefill, src/model.rs:2080-2102).  out [m][nh][vd].
+ *           workspace: mk_mla_heads_workspace_bytes(m, nh, nope, vd). */
+int mk_dev_mla_heads_append(const float *k_rows, const float *v_rows, size_t n_new, size_t nh, size_t nope, size_t rope, size_t vd,
+                            size_t pos0, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream);
+int mk_dev_mla_heads_to_f32(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t n, size_t nh,
+                            size_t nope, size_t rope, size_t vd, float *k, float *v, void *stream);
+size_t mk_mla_heads_workspace_bytes(size_t m, size_t nh, size_t nope, size_t vd);
+int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t pos0,
+                             const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, void *workspace,
+                             float *out, void *stream);
 
 /* ---------------------------------- device level: prefill expert GEMM */
 
@@ -393,6 +417,25 @@ void mk_expert_set_free(mk_expert_set *s);
  * first 16 host bytes on every hit.  Arithmetic follows mk_q8_enabled(). */
 int mk_mxfp4_matvec(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, float *out);
 
+/* metal::gpu_matvec (src/metal.rs:750-870), the GPU branch of model::matvec (src/model.rs:199-208): y = W x for a
+ * row-major f32 matrix on host slices, the weight cached on the device like the packed ones.  The dot contract of
+ * src/model.rs:46-82 is replayed: the result is bit-identical to matvec_cpu. */
+int mk_matvec_f32(const float *w, size_t rows, size_t cols, const float *x, float *out);
+
+/* GpuProf / gpu_prof_print (src/metal.rs:667-716): accumulated over the host-level matvecs while profiling is on
+ * (MK_GPU_DEBUG=1 at mk_init, or mk_prof_enable(1)).  With profiling on the phases are separated by extra
+ * synchronisations: cache = weight lookup / upload, io = input upload, launch = kernel enqueue, wait = until the
+ * kernels are done, readback = result copy. */
+typedef struct {
+    uint64_t calls, hits, misses;
+    double t_cache_ms, t_io_ms, t_launch_ms, t_wait_ms, t_readback_ms;
+    size_t cache_tensors, cache_bytes;
+} mk_prof;
+void mk_prof_enable(int on);
+void mk_prof_reset(void);
+void mk_prof_get(mk_prof *out);
+void mk_prof_print(void);
+
 /* mxfp4::dequant on host slices (upload, kernel, download). */
 int mk_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out);
 
@@ -407,15 +450,30 @@ int mk_q8head_from_q8(const int8_t *q, const float *scales, size_t rows, size_t 
 int mk_q8head_matvec(mk_q8head *h, const float *x, size_t batch, float *out, int32_t *argmax_out);
 void mk_q8head_free(mk_q8head *h);
 
-/* Shared-latent q8 MLA cache kept on device (MlaCache, src/model.rs:765-781,1556-1618). */
+/* MlaCache (src/model.rs:765-781,1556-1692) kept on the device, in one of two layouts:
+ *   mk_mla_cache_new        shared latent: per position one q8_0 latent row (L int8, f16 scales) that is K and V of every
+ *                           head, and one q8_0 rope row (R int8, f16 scales) -- the weight-absorbed form.  L a multiple of
+ *                           64 up to 512, R 32 or 64.  A position is given as (latent [L], rope [R]).
+ *   mk_mla_cache_new_heads  the reference's own layout: per position and head a K-nope row and a V row (int8 + f32
+ *                           scales) and one shared f32 rope row.  A position is given as the reference gives it to
+ *                           MlaCache::push: (k_row [nh][nope+rope], v_row [nh][vd]).
+ * row0 / row1 below are those two rows; rows0 / rows1 are n of them, position-major. */
 typedef struct mk_mla_cache mk_mla_cache;
 int mk_mla_cache_new(size_t nh, size_t L, size_t R, size_t capacity, mk_mla_cache **out);
-int mk_mla_cache_push(mk_mla_cache *c, const float *latent, const float *rope);
+int mk_mla_cache_new_heads(size_t nh, size_t nope, size_t rope, size_t vd, size_t capacity, mk_mla_cache **out);
+/* MlaCache::push (src/model.rs:1583-1618) */
+int mk_mla_cache_push(mk_mla_cache *c, const float *row0, const float *row1);
+/* MlaCache::assign_f32 (src/model.rs:1680-1692): the cache is emptied and refilled from n f32 positions (snapshot restore) */
+int mk_mla_cache_assign_f32(mk_mla_cache *c, const float *rows0, const float *rows1, size_t n);
 size_t mk_mla_cache_positions(const mk_mla_cache *c);
-/* MlaCache::to_f32 (src/model.rs:1623-1676): dequantized rows, latent [n][L], rope [n][R] */
-int mk_mla_cache_to_f32(const mk_mla_cache *c, float *latent, float *rope);
-/* attention of all heads over positions 0..=positions-1: q [nh][L+R] host, out [nh][L] host */
+/* MlaCache::to_f32 (src/model.rs:1623-1676): the dequantized rows q * s of all positions, in the shapes push takes */
+int mk_mla_cache_to_f32(const mk_mla_cache *c, float *rows0, float *rows1);
+/* mla_attn_flash_q8_mqa (src/model.rs:1804-1908) over positions 0 ..= positions-1: q [nh][L+R] (heads layout:
+ * [nh][nope+rope]) host, out [nh][L] (heads layout: [nh][vd]) host */
 int mk_mla_attn(mk_mla_cache *c, const float *q, float scale, float *out);
+/* the attention loop of mla_prefill (src/model.rs:2080-2102) after the prompt's m positions have been pushed: query i
+ * of q [m][nh][...] attends the positions 0 ..= positions - m + i; out [m][nh][...] */
+int mk_mla_attn_prefill(mk_mla_cache *c, const float *q, size_t m, float scale, float *out);
 void mk_mla_cache_free(mk_mla_cache *c);
 
 #ifdef __cplusplus

@@ -29,6 +29,12 @@ class ExpertTable(C.Structure):
                 ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t), ("n_experts", C.c_size_t)]
 
 
+class Prof(C.Structure):
+    _fields_ = [("calls", C.c_uint64), ("hits", C.c_uint64), ("misses", C.c_uint64), ("t_cache_ms", C.c_double), ("t_io_ms", C.c_double),
+                ("t_launch_ms", C.c_double), ("t_wait_ms", C.c_double), ("t_readback_ms", C.c_double), ("cache_tensors", C.c_size_t),
+                ("cache_bytes", C.c_size_t)]
+
+
 class PrefillLayout(C.Structure):
     _fields_ = [("order", C.c_size_t), ("pos", C.c_size_t), ("offsets", C.c_size_t), ("g", C.c_size_t), ("u", C.c_size_t), ("o", C.c_size_t)]
 
@@ -77,19 +83,31 @@ def _load():
         "mk_mla_decode_static_max_heads": (sz, []),
         "mk_dev_mla_q8_decode_static": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp]),
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
+        "mk_dev_mla_heads_append": (i32, [vp, vp, sz, sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
+        "mk_dev_mla_heads_to_f32": (i32, [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp]),
+        "mk_mla_heads_workspace_bytes": (sz, [sz, sz, sz, sz]),
+        "mk_dev_mla_heads_q8_attn": (i32, [vp, vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, f32, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
         "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),
         "mk_moe_prefill_workspace_layout": (i32, [sz, sz, sz, sz, sz, C.POINTER(PrefillLayout)]),
         "mk_dev_moe_prefill": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp]),
+        "mk_matvec_f32": (i32, [vp, sz, sz, vp, vp]),
+        "mk_prof_enable": (None, [i32]),
+        "mk_prof_reset": (None, []),
+        "mk_prof_get": (None, [C.POINTER(Prof)]),
+        "mk_prof_print": (None, []),
         "mk_quantize_q8": (i32, [vp, sz, vp, vp]),
         "mk_q8head_from_f32": (i32, [vp, sz, sz, i32, C.POINTER(vp)]),
         "mk_q8head_from_q8": (i32, [vp, vp, sz, sz, i32, C.POINTER(vp)]),
         "mk_q8head_matvec": (i32, [vp, vp, sz, vp, vp]),
         "mk_q8head_free": (None, [vp]),
         "mk_mla_cache_new": (i32, [sz, sz, sz, sz, C.POINTER(vp)]),
+        "mk_mla_cache_new_heads": (i32, [sz, sz, sz, sz, sz, C.POINTER(vp)]),
         "mk_mla_cache_push": (i32, [vp, vp, vp]),
+        "mk_mla_cache_assign_f32": (i32, [vp, vp, vp, sz]),
+        "mk_mla_attn_prefill": (i32, [vp, vp, sz, f32, vp]),
         "mk_mla_cache_positions": (sz, [vp]),
         "mk_mla_cache_to_f32": (i32, [vp, vp, vp]),
         "mk_mla_attn": (i32, [vp, vp, f32, vp]),

@@ -1,0 +1,358 @@
+// q8_0 MLA attention over the cache layout the reference keeps (src/model.rs:765-781): per position and head a
+// latent K row (nope int8 + nope/32 f32 scales) and a V row (vd int8 + vd/32 f32 scales), plus ONE f32 rope row per
+// position shared by the heads.
+//
+//   append   MlaCache::push (src/model.rs:1583-1618) for one or many positions (many = assign_f32,
+//            src/model.rs:1680-1692): rope row from head 0, q8::quantize_q8_into per head for K-nope and V
+//   to_f32   MlaCache::to_f32 (src/model.rs:1623-1676)
+//   decode   mla_attn_flash_q8_mqa (src/model.rs:1804-1908) for one query per head: every head owns its K and V
+//            rows, so each cache byte is used once -- a streaming kernel, HBM-bound by construction.  Grid (split,
+//            head, query): four waves walk 64-position tiles; scores with v_dot4_i32_i8 on the raw bytes and the
+//            reference's per-block scale product, f32 rope dot, online softmax, V rows dequantized as q * s.
+//            Splits are merged by log-sum-exp.  With several queries (prefill, src/model.rs:2080-2102) query i
+//            attends positions 0 ..= pos0 + i.
+//
+// The Hadamard option (MICROKIMI_KV_HADAMARD, off by default) is not built: a cache in that mode stays on the CPU.
+#include "mk_common.h"
+
+namespace {
+
+constexpr int TJ = 64;          // positions per tile (FLASH_KV, src/model.rs:1348)
+constexpr int MAX_SPLITS = 64;
+constexpr int MAX_NB = 8;       // latent blocks per head the decode kernel holds in registers (nope <= 256)
+constexpr int MAX_VD = 512;
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// One 32-block per aligned group of 32 lanes: q8::quantize_q8_into (src/q8.rs:57-68).
+__device__ __forceinline__ void quantize_block32(float v, int8_t *q_out, float *s_out, int j) {
+    const float mx = mk_half_wave_max(fabsf(v));
+    const float dx = mx / 127.0f;
+    q_out[j] = (int8_t)(dx != 0.0f ? mk_q8_round(v, dx) : 0);
+    if (j == 0) *s_out = dx;
+}
+
+// grid: (blocks of the position's rows, position).  Blocks 0 .. nh*nope/32-1: K-nope of head h; then nh*vd/32 V blocks;
+// the last workgroups copy the rope row of head 0.
+__global__ __launch_bounds__(256) void heads_append_kernel(const float *__restrict__ k_rows, const float *__restrict__ v_rows, int nh, int nope,
+                                                           int rope, int vd, size_t pos0, int8_t *__restrict__ kq, float *__restrict__ ks,
+                                                           float *__restrict__ kr, int8_t *__restrict__ vq, float *__restrict__ vs) {
+    const int nbk = nh * nope / 32, nbv = nh * vd / 32;
+    const size_t jn = blockIdx.y, pos = pos0 + jn;
+    const int blk = (blockIdx.x * blockDim.x + threadIdx.x) >> 5, j = threadIdx.x & 31;
+    const int qh = nope + rope;
+    if (blk < nbk) {
+        const int h = blk / (nope / 32), g = blk % (nope / 32);
+        const float v = k_rows[(jn * nh + h) * qh + g * 32 + j];
+        quantize_block32(v, kq + (pos * nh + h) * nope + g * 32, ks + pos * nbk + blk, j);
+    } else if (blk < nbk + nbv) {
+        const int b = blk - nbk, h = b / (vd / 32), g = b % (vd / 32);
+        const float v = v_rows[(jn * nh + h) * vd + g * 32 + j];
+        quantize_block32(v, vq + (pos * nh + h) * vd + g * 32, vs + pos * nbv + b, j);
+    } else {
+        const int d = (blk - nbk - nbv) * 32 + j;
+        if (d < rope) kr[pos * rope + d] = k_rows[jn * nh * qh + nope + d];  // rope is shared: stored once, from head 0
+    }
+}
+
+__global__ __launch_bounds__(256) void heads_to_f32_kernel(const int8_t *__restrict__ kq, const float *__restrict__ ks,
+                                                           const float *__restrict__ kr, const int8_t *__restrict__ vq,
+                                                           const float *__restrict__ vs, int nh, int nope, int rope, int vd,
+                                                           float *__restrict__ k, float *__restrict__ v) {
+    const size_t j = blockIdx.y;
+    const int qh = nope + rope;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nh * qh; i += gridDim.x * blockDim.x) {
+        const int h = i / qh, d = i % qh;
+        k[(j * nh + h) * qh + d] = d < nope ? (float)kq[(j * nh + h) * nope + d] * ks[(j * nh + h) * (nope / 32) + d / 32] : kr[j * rope + d - nope];
+    }
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nh * vd; i += gridDim.x * blockDim.x) {
+        const int h = i / vd, d = i % vd;
+        v[(j * nh + h) * vd + d] = (float)vq[(j * nh + h) * vd + d] * vs[(j * nh + h) * (vd / 32) + d / 32];
+    }
+}
+
+// q8 of the latent part of every (query, head): (src/model.rs:1812-1821)
+__global__ __launch_bounds__(256) void heads_q_prep_kernel(const float *__restrict__ q, int rows, int nope, int rope, int8_t *__restrict__ qq,
+                                                           float *__restrict__ qs) {
+    const int nb = nope / 32;
+    const int blk = (blockIdx.x * blockDim.x + threadIdx.x) >> 5, j = threadIdx.x & 31;
+    if (blk >= rows * nb) return;
+    const int r = blk / nb, g = blk % nb;
+    quantize_block32(q[(size_t)r * (nope + rope) + g * 32 + j], qq + (size_t)r * nope + g * 32, qs + blk, j);
+}
+
+struct HeadsArgs {
+    const int8_t *kq;
+    const float *ks;
+    const float *kr;
+    const int8_t *vq;
+    const float *vs;
+    const float *q;    // [m][nh][nope+rope]
+    const int8_t *qq;  // [m][nh][nope]
+    const float *qs;   // [m][nh][nope/32]
+    int nh, nope, rope, vd, n_pos0, split_len, n_splits;
+    float scale;
+    float *po, *pm, *pl;  // split partials (one query only)
+    float *out;           // [m][nh][vd]
+};
+
+// Workgroup = (split, head, query), 256 threads.  Per 64-position tile:
+//   scores   thread (i = tid / 4, part = tid % 4): position i of the tile, blocks part, part + 4, ... of the head's latent
+//            row and every 4th rope dim; the four parts meet through two lane shuffles
+//   softmax  every wave reduces the 64 scores itself (no second barrier for the statistics)
+//   out      thread (slot = tid / 32, dq = tid % 32): positions slot, slot + 8, ... of the tile, dims 4 dq .. 4 dq + 3
+//            (+128, +256, +384 for wider V rows); the eight slots meet in LDS at the end
+__global__ __launch_bounds__(256) void heads_decode_kernel(HeadsArgs a) {
+    __shared__ float sc_l[TJ];
+    __shared__ float red_l[8][MAX_VD];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int split = blockIdx.x, h = blockIdx.y, qi = blockIdx.z;
+    const int nh = a.nh, nope = a.nope, rope = a.rope, vd = a.vd, nb = nope / 32, nbv = vd / 32;
+    const int n_pos = a.n_pos0 + qi;
+    const int p_begin = split * a.split_len;
+    const int p_end = min(p_begin + a.split_len, n_pos);
+    const size_t qrow = (size_t)qi * nh + h;
+    // this thread's share of the query: latent blocks part, part + 4, ... and rope dims part, part + 4, ...
+    const int part = tid & 3, ip = tid >> 2;
+    mk_i4 qreg[MAX_NB / 4][2];
+    float qsc[MAX_NB / 4];
+#pragma unroll
+    for (int k = 0; k < MAX_NB / 4; k++) {
+        const int g = part + 4 * k;
+        if (g < nb) {
+            const mk_i4 *src = reinterpret_cast<const mk_i4 *>(a.qq + qrow * nope + g * 32);
+            qreg[k][0] = src[0];
+            qreg[k][1] = src[1];
+            qsc[k] = a.qs[qrow * nb + g];
+        } else {
+            qreg[k][0] = qreg[k][1] = mk_i4{0, 0, 0, 0};
+            qsc[k] = 0.0f;
+        }
+    }
+    const float *qr = a.q + qrow * (nope + rope) + nope;
+    const int slot = tid >> 5, dq = tid & 31;
+    float o[MAX_VD / 128][4];
+#pragma unroll
+    for (int c = 0; c < MAX_VD / 128; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[c][e] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    for (int t0 = p_begin; t0 < p_end; t0 += TJ) {
+        const int tn = min(TJ, p_end - t0);
+        // ---- scores
+        float s = 0.0f;
+        if (ip < tn) {
+            const size_t j = (size_t)(t0 + ip);
+            const int8_t *krow = a.kq + (j * nh + h) * nope;
+            const float *ksr = a.ks + (j * nh + h) * nb;
+#pragma unroll
+            for (int k = 0; k < MAX_NB / 4; k++) {
+                const int g = part + 4 * k;
+                if (g < nb) {
+                    const mk_i4 *src = reinterpret_cast<const mk_i4 *>(krow + g * 32);
+                    const mk_i4 k0 = src[0], k1 = src[1];
+                    int idot = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) idot = __builtin_amdgcn_sdot4(k0[e], qreg[k][0][e], idot, false);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) idot = __builtin_amdgcn_sdot4(k1[e], qreg[k][1][e], idot, false);
+                    s += (qsc[k] * ksr[g]) * (float)idot;
+                }
+            }
+            const float *krr = a.kr + j * rope;
+            for (int d = part; d < rope; d += 4) s += qr[d] * krr[d];
+        }
+        s += __shfl_xor(s, 1, MK_WAVE);
+        s += __shfl_xor(s, 2, MK_WAVE);
+        __syncthreads();  // the previous tile's scores have been consumed
+        if (part == 0) sc_l[ip] = ip < tn ? s * a.scale : -INFINITY;
+        __syncthreads();
+        // ---- online softmax (every wave computes the tile's statistics for itself)
+        const float sv = sc_l[lane];
+        const float tm = mk_wave_max(sv);
+        const float m_new = fmaxf(m, tm);
+        const float corr = expf(m - m_new);
+        const float pv = expf(sv - m_new);  // -inf score (position past the end) gives 0
+        l = l * corr + mk_wave_sum(pv);
+        m = m_new;
+#pragma unroll
+        for (int c = 0; c < MAX_VD / 128; c++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[c][e] *= corr;
+        // ---- out += p V: this thread's positions slot, slot + 8, ...
+        for (int i = slot; i < tn; i += 8) {
+            const float p = expf(sc_l[i] - m_new);
+            const size_t j = (size_t)(t0 + i);
+            const int8_t *vrow = a.vq + (j * nh + h) * vd;
+            const float *vsr = a.vs + (j * nh + h) * nbv;
+#pragma unroll
+            for (int c = 0; c < MAX_VD / 128; c++) {
+                const int d0 = 128 * c + 4 * dq;
+                if (d0 < vd) {
+                    const uint32_t w = *reinterpret_cast<const uint32_t *>(vrow + d0);
+                    const float ps = p * vsr[d0 >> 5];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[c][e] += ps * (float)(int8_t)(w >> (8 * e));
+                }
+            }
+        }
+    }
+    // ---- the eight position slots meet in LDS
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < MAX_VD / 128; c++) {
+        const int d0 = 128 * c + 4 * dq;
+        if (d0 < vd)
+#pragma unroll
+            for (int e = 0; e < 4; e++) red_l[slot][d0 + e] = o[c][e];
+    }
+    __syncthreads();
+    for (int d = tid; d < vd; d += 256) {
+        float v = red_l[0][d];
+#pragma unroll
+        for (int k = 1; k < 8; k++) v += red_l[k][d];
+        if (a.n_splits == 1) {
+            a.out[qrow * vd + d] = v / l;
+        } else {
+            a.po[((size_t)split * nh + h) * vd + d] = v;
+        }
+    }
+    if (a.n_splits > 1 && tid == 0) {
+        a.pm[split * nh + h] = m;
+        a.pl[split * nh + h] = l;
+    }
+}
+
+// log-sum-exp merge of the splits of one query: a workgroup per head
+__global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
+                                                          int nh, int vd, int n_splits, float *__restrict__ out) {
+    __shared__ float w_l[MAX_SPLITS];
+    __shared__ float den_l;
+    const int h = blockIdx.x, tid = threadIdx.x;
+    if (tid < 64) {
+        float mx = -INFINITY;
+        for (int s = tid; s < n_splits; s += 64) mx = fmaxf(mx, pm[s * nh + h]);
+        mx = mk_wave_max(mx);
+        float den = 0.0f;
+        for (int s = tid; s < n_splits; s += 64) {
+            const float w = expf(pm[s * nh + h] - mx);
+            w_l[s] = w;
+            den += pl[s * nh + h] * w;
+        }
+        den = mk_wave_sum(den);
+        if (tid == 0) den_l = den;
+    }
+    __syncthreads();
+    for (int d = tid; d < vd; d += 256) {
+        float num = 0.0f;
+        for (int s = 0; s < n_splits; s++) num += po[((size_t)s * nh + h) * vd + d] * w_l[s];
+        out[(size_t)h * vd + d] = num / den_l;
+    }
+}
+
+int check_shape(size_t nh, size_t nope, size_t rope, size_t vd) {
+    MK_REQUIRE(nh >= 1 && nh <= 65535, "bad head count");
+    MK_REQUIRE(nope % 32 == 0 && nope >= 32 && nope <= 32 * MAX_NB, "latent K width must be a multiple of 32 up to 256");
+    MK_REQUIRE(vd % 32 == 0 && vd >= 32 && vd <= MAX_VD, "V width must be a multiple of 32 up to 512");
+    MK_REQUIRE(rope <= 4096, "rope width out of range");
+    return MK_OK;
+}
+
+}  // namespace
+
+extern "C" int mk_dev_mla_heads_append(const float *k_rows, const float *v_rows, size_t n_new, size_t nh, size_t nope, size_t rope, size_t vd,
+                                       size_t pos0, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream) {
+    MK_REQUIRE(k_rows && v_rows && kq && ks && vq && vs && (kr || rope == 0), "null pointer");
+    int s = check_shape(nh, nope, rope, vd);
+    if (s != MK_OK) return s;
+    if (n_new == 0) return MK_OK;
+    MK_REQUIRE(n_new <= 65535, "at most 65535 positions per call");
+    const size_t blocks32 = nh * nope / 32 + nh * vd / 32 + (rope + 31) / 32;
+    hipLaunchKernelGGL(heads_append_kernel, dim3((unsigned)((blocks32 + 7) / 8), (unsigned)n_new), dim3(256), 0, (hipStream_t)stream, k_rows, v_rows,
+                       (int)nh, (int)nope, (int)rope, (int)vd, pos0, kq, ks, kr, vq, vs);
+    return mk_launch_status("heads_append");
+}
+
+extern "C" int mk_dev_mla_heads_to_f32(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t n,
+                                       size_t nh, size_t nope, size_t rope, size_t vd, float *k, float *v, void *stream) {
+    MK_REQUIRE(kq && ks && vq && vs && k && v && (kr || rope == 0), "null pointer");
+    int s = check_shape(nh, nope, rope, vd);
+    if (s != MK_OK) return s;
+    if (n == 0) return MK_OK;
+    MK_REQUIRE(n <= 65535 * 64, "too many positions");
+    for (size_t j0 = 0; j0 < n; j0 += 65535) {
+        const size_t nj = n - j0 < 65535 ? n - j0 : 65535;
+        hipLaunchKernelGGL(heads_to_f32_kernel, dim3(8, (unsigned)nj), dim3(256), 0, (hipStream_t)stream, kq + j0 * nh * nope,
+                           ks + j0 * nh * (nope / 32), kr + j0 * rope, vq + j0 * nh * vd, vs + j0 * nh * (vd / 32), (int)nh, (int)nope, (int)rope,
+                           (int)vd, k + j0 * nh * (nope + rope), v + j0 * nh * vd);
+        if ((s = mk_launch_status("heads_to_f32")) != MK_OK) return s;
+    }
+    return MK_OK;
+}
+
+extern "C" size_t mk_mla_heads_workspace_bytes(size_t m, size_t nh, size_t nope, size_t vd) {
+    return align_up(m * nh * nope, 256) + align_up(m * nh * (nope / 32) * 4, 256) + align_up(MAX_SPLITS * nh * vd * 4, 256) +
+           2 * align_up(MAX_SPLITS * nh * 4, 256);
+}
+
+extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t pos0,
+                                        const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, void *workspace,
+                                        float *out, void *stream) {
+    MK_REQUIRE(kq && ks && vq && vs && q && workspace && out && (kr || rope == 0), "null pointer");
+    int s = check_shape(nh, nope, rope, vd);
+    if (s != MK_OK) return s;
+    MK_REQUIRE(m >= 1 && m <= 65535, "bad query count");
+    MK_REQUIRE(pos0 + m < 0x7FFFFF00u, "position out of range");
+    MK_REQUIRE(((uintptr_t)kq & 15) == 0 && ((uintptr_t)vq & 3) == 0 && ((uintptr_t)workspace & 255) == 0,
+               "K bytes must be 16-byte, V bytes 4-byte and the workspace 256-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t *w = (uint8_t *)workspace;
+    HeadsArgs a;
+    a.kq = kq;
+    a.ks = ks;
+    a.kr = kr;
+    a.vq = vq;
+    a.vs = vs;
+    a.q = q;
+    int8_t *qq = (int8_t *)w;
+    w += align_up(m * nh * nope, 256);
+    float *qs = (float *)w;
+    w += align_up(m * nh * (nope / 32) * 4, 256);
+    a.po = (float *)w;
+    w += align_up(MAX_SPLITS * nh * vd * 4, 256);
+    a.pm = (float *)w;
+    w += align_up(MAX_SPLITS * nh * 4, 256);
+    a.pl = (float *)w;
+    a.qq = qq;
+    a.qs = qs;
+    a.nh = (int)nh;
+    a.nope = (int)nope;
+    a.rope = (int)rope;
+    a.vd = (int)vd;
+    a.n_pos0 = (int)pos0 + 1;
+    a.scale = scale;
+    a.out = out;
+    const int rows = (int)(m * nh);
+    hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, qq, qs);
+    if ((s = mk_launch_status("heads_q_prep")) != MK_OK) return s;
+    // one query: split the context so that about 1024 workgroups stream the cache; several queries (prefill): the
+    // (query, head) grid is parallel enough, one split each
+    int n_splits = 1, split_len = (int)((pos0 + m + TJ - 1) / TJ) * TJ;
+    if (m == 1) {
+        const int tiles = (int)((pos0 + 1 + TJ - 1) / TJ);
+        int want = (int)((1024 + nh - 1) / nh);
+        if (want > MAX_SPLITS) want = MAX_SPLITS;
+        if (want > tiles) want = tiles;
+        const int tps = (tiles + want - 1) / want;
+        split_len = tps * TJ;
+        n_splits = (tiles + tps - 1) / tps;
+    }
+    a.split_len = split_len;
+    a.n_splits = n_splits;
+    hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);
+    if ((s = mk_launch_status("heads_decode")) != MK_OK) return s;
+    if (n_splits == 1) return MK_OK;
+    hipLaunchKernelGGL(heads_merge_kernel, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
+    return mk_launch_status("heads_merge");
+}

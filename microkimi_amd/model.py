@@ -130,6 +130,69 @@ def mla_attn_flash_q8_mqa(cache, q, pos, scale, out=None):
     return out
 
 
+class MlaHeadsCache:
+    """MlaCache in the reference's own layout (src/model.rs:765-781) on the device: per position and head a q8 K-nope
+    row and a q8 V row (int8 + f32 scales), one shared f32 rope row.  push / assign_f32 / to_f32 / attention mirror
+    MlaCache::push, ::assign_f32, ::to_f32 and mla_attn_flash_q8_mqa; attn with several queries is the attention loop
+    of mla_prefill (src/model.rs:2080-2102)."""
+
+    def __init__(self, nh, nope, rope, vd, capacity, device="cuda"):
+        import torch
+        self.nh, self.nope, self.rope, self.vd, self.cap, self.n = nh, nope, rope, vd, capacity, 0
+        self.kq = torch.zeros((capacity, nh * nope), dtype=torch.int8, device=device)
+        self.ks = torch.zeros((capacity, nh * nope // 32), dtype=torch.float32, device=device)
+        self.kr = torch.zeros((capacity, rope), dtype=torch.float32, device=device)
+        self.vq = torch.zeros((capacity, nh * vd), dtype=torch.int8, device=device)
+        self.vs = torch.zeros((capacity, nh * vd // 32), dtype=torch.float32, device=device)
+        self._ws = None
+
+    def positions(self):
+        return self.n
+
+    def push(self, k_rows, v_rows):
+        """k_rows [n_new, nh * (nope + rope)], v_rows [n_new, nh * vd] (or one row each) appended."""
+        _lib.require_device()
+        k_rows = k_rows.reshape(-1, self.nh * (self.nope + self.rope)).contiguous()
+        v_rows = v_rows.reshape(-1, self.nh * self.vd).contiguous()
+        n_new = k_rows.shape[0]
+        if self.n + n_new > self.cap:
+            raise RuntimeError("MlaCache is full")
+        check(lib.mk_dev_mla_heads_append(ptr(k_rows), ptr(v_rows), n_new, self.nh, self.nope, self.rope, self.vd, self.n, ptr(self.kq),
+                                          ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), cur_stream()))
+        self.n += n_new
+
+    def assign_f32(self, k, v):
+        """MlaCache::assign_f32 (src/model.rs:1680-1692): emptied, then refilled from f32 rows."""
+        self.n = 0
+        self.push(k, v)
+
+    def to_f32(self):
+        import torch
+        _lib.require_device()
+        k = torch.empty((self.n, self.nh * (self.nope + self.rope)), dtype=torch.float32, device=self.kq.device)
+        v = torch.empty((self.n, self.nh * self.vd), dtype=torch.float32, device=self.kq.device)
+        if self.n:
+            check(lib.mk_dev_mla_heads_to_f32(ptr(self.kq), ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), self.n, self.nh, self.nope,
+                                              self.rope, self.vd, ptr(k), ptr(v), cur_stream()))
+        return k, v
+
+    def attn(self, q, pos0, scale):
+        """q [m, nh * (nope + rope)]: query i attends the positions 0 ..= pos0 + i.  Returns [m, nh * vd]."""
+        import torch
+        _lib.require_device()
+        q = q.reshape(-1, self.nh * (self.nope + self.rope)).contiguous()
+        m = q.shape[0]
+        if pos0 + m > self.n:
+            raise ValueError("queries reach beyond the cached positions")
+        need = lib.mk_mla_heads_workspace_bytes(m, self.nh, self.nope, self.vd)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        out = torch.empty((m, self.nh * self.vd), dtype=torch.float32, device=q.device)
+        check(lib.mk_dev_mla_heads_q8_attn(ptr(self.kq), ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), pos0, ptr(q), m, self.nh,
+                                           self.nope, self.rope, self.vd, float(scale), ptr(self._ws), ptr(out), cur_stream()))
+        return out
+
+
 class PackedExperts:
     """Expert table of an MoE layer on the device: per expert w1, w3 [inter, d] and w2 [d, inter], each MXFP4
     (packed, scales) in the reference layout.  Built from lists of device tensors."""

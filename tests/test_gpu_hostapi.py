@@ -88,3 +88,91 @@ def test_invalid_arguments_write_nothing():
                                   _lib.hptr(out))
     assert st == -1 and np.all(out == 3.0)
     assert _lib.lib.mk_available() == 1
+
+
+def test_matvec_f32_host_level_is_bit_identical_and_cached():
+    # metal::gpu_matvec (src/metal.rs:750): host slices, the weight cached by (pointer, rows, cols)
+    import ctypes as C
+    from microkimi_amd._lib import Prof, check, hptr, lib
+    rng = np.random.default_rng(3)
+    rows, cols = 300, 1000
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    x = rng.standard_normal(cols).astype(np.float32)
+    y = np.empty(rows, np.float32)
+    lib.mk_prof_reset()
+    lib.mk_prof_enable(1)
+    try:
+        for _ in range(3):
+            check(lib.mk_matvec_f32(hptr(w), rows, cols, hptr(x), hptr(y)))
+        want = oracle.matvec_f32(w, rows, cols, x)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+        w[0, 0] += 1.0   # same pointer, other contents: the first 16 bytes differ, the copy is replaced
+        check(lib.mk_matvec_f32(hptr(w), rows, cols, hptr(x), hptr(y)))
+        assert np.array_equal(y.view(np.uint32), oracle.matvec_f32(w, rows, cols, x).view(np.uint32))
+        p = Prof()
+        lib.mk_prof_get(C.byref(p))
+        # GpuProf (src/metal.rs:667-716): 4 calls, 2 uploads (first use, changed contents), 2 hits, phases timed
+        assert (p.calls, p.misses, p.hits) == (4, 2, 2)
+        assert p.t_wait_ms > 0 and p.t_readback_ms > 0 and p.t_io_ms > 0 and p.cache_tensors >= 1
+        lib.mk_prof_print()
+    finally:
+        lib.mk_prof_enable(0)
+
+
+def test_host_level_matvec_from_several_threads():
+    # the reference calls matvec_packed from its pool workers, one job per selected expert (src/model.rs:2227-2264):
+    # eight threads, each with its own weight, activation and output, 20 calls each
+    import threading
+    from microkimi_amd._lib import hptr, lib
+    from microkimi_amd import workloads
+    rows, cols, nthreads = 256, 2048, 8
+    mats = [workloads.mxfp4_matrix(0, "tw", rows, cols, t) for t in range(nthreads)]
+    xs = [np.random.default_rng(t).standard_normal(cols).astype(np.float32) for t in range(nthreads)]
+    want = [oracle.matvec_packed(mats[t][0], mats[t][1], rows, cols, xs[t], mode=1) for t in range(nthreads)]
+    outs = [np.zeros(rows, np.float32) for _ in range(nthreads)]
+    errs = []
+
+    def work(t):
+        for _ in range(20):
+            st = lib.mk_mxfp4_matvec(hptr(mats[t][0]), hptr(mats[t][1]), rows, cols, hptr(xs[t]), hptr(outs[t]))
+            if st != 0:
+                errs.append((t, st))
+                return
+            if rel_l2(outs[t], want[t]) > 1e-5:
+                errs.append((t, "wrong result"))
+                return
+
+    lib.mk_force_q8(1)
+    try:
+        th = [threading.Thread(target=work, args=(t,)) for t in range(nthreads)]
+        for t in th:
+            t.start()
+        for t in th:
+            t.join()
+    finally:
+        lib.mk_force_q8(-1)
+    assert not errs, errs
+
+
+def test_shared_latent_handle_assign_f32_and_prefill():
+    # MlaCache::assign_f32 (src/model.rs:1680-1692) and the mla_prefill loop on the shared-latent handle
+    torch_cuda()
+    from microkimi_amd import _lib, workloads
+    nh, L, R, n = 8, 512, 64, 70
+    lat, rope, q = workloads.config3_raw(n, nh=nh)
+    c = ctypes.c_void_p()
+    _lib.check(_lib.lib.mk_mla_cache_new(nh, L, R, n, ctypes.byref(c)))
+    try:
+        _lib.check(_lib.lib.mk_mla_cache_push(c, _lib.hptr(lat[5]), _lib.hptr(rope[5])))   # stale: assign starts empty
+        _lib.check(_lib.lib.mk_mla_cache_assign_f32(c, _lib.hptr(lat), _lib.hptr(rope), n))
+        assert _lib.lib.mk_mla_cache_positions(c) == n
+        lq, _, ls = oracle.q8_0_rows(lat)
+        rq, _, rs = oracle.q8_0_rows(rope)
+        qs = np.stack([q, q * 0.5, -q]).astype(np.float32)
+        outs = np.zeros((3, nh, L), np.float32)
+        _lib.check(_lib.lib.mk_mla_attn_prefill(c, _lib.hptr(qs), 3, workloads.MLA_SCALE, _lib.hptr(outs)))
+        for i in range(3):
+            want = oracle.mla_absorbed_decode(lq, ls.astype(np.float32), rq, rs.astype(np.float32), qs[i], nh, workloads.MLA_SCALE, pos=n - 3 + i)
+            assert rel_l2(outs[i], want) <= 1e-5
+    finally:
+        _lib.lib.mk_mla_cache_free(c)
