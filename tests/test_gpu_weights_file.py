@@ -80,3 +80,71 @@ def test_unsupported_dtype_and_shape_mismatch(tmp_path):
     with pytest.raises(MkError) as e:
         weights.BinFile.open(tmp_path / "shape.bin").load_experts("layers.9.", 3)
     assert "missing tensor" in str(e.value)
+
+
+def test_file_written_by_the_reference_writer_dequantizes_like_the_reference_reader():
+    """The fixture of tests/golden/make_mkim_fixture.py: a file from the reference's exporter (nano/export.py), with the
+    values the reference's reader (nano/bin2pt.py dequant_mxfp4) gives for its expert tensors.  mk_bin_* blobs through
+    mk_dev_mxfp4_dequant, and the resident expert table of mk_bin_load_experts, must give those values bit for bit."""
+    import os
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, weights
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    exp = np.load(os.path.join(here, "mkim_ref_expected.npz"))
+    f = weights.BinFile.open(os.path.join(here, "mkim_ref.bin"))
+    d, inter, n = 64, 32, 3
+    for e in range(n):
+        for k, (r, c) in (("w1", (inter, d)), ("w2", (d, inter)), ("w3", (inter, d))):
+            name = f"layers.0.block_sparse_moe.experts.{e}.{k}"
+            pk, sc, rr, cc = f.mxfp4_parts(name)
+            assert (rr, cc) == (r, c)
+            got = mxfp4.dequant(dev(np.ascontiguousarray(pk)), dev(np.ascontiguousarray(sc)), r, c).cpu().numpy()
+            want = exp["dequant:" + name]
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), name
+            # the oracle agrees too (its dequant is pinned by ref/ds_golden.json)
+            assert np.array_equal(oracle.mxfp4_dequant(pk, sc, r, c).view(np.uint32), want.view(np.uint32))
+    ex = f.load_experts("layers.0.", n)
+    assert (ex.n, ex.d, ex.inter) == (n, d, inter)
+    # the resident copies give the same layer output as a table built from the file's tensors, and the oracle's
+    from microkimi_amd import model
+    parts = {k: [f.mxfp4_parts(f"layers.0.block_sparse_moe.experts.{e}.{k}")[:2] for e in range(n)] for k in ("w1", "w3", "w2")}
+    todev = lambda lst: [(dev(np.ascontiguousarray(p)), dev(np.ascontiguousarray(s))) for p, s in lst]
+    ref = model.PackedExperts(todev(parts["w1"]), todev(parts["w3"]), todev(parts["w2"]), d, inter)
+    rng = np.random.default_rng(4)
+    ids = np.stack([rng.permutation(n)[:2] for _ in range(3)]).astype(np.int32)
+    wts = rng.random((3, 2)).astype(np.float32)
+    x = rng.standard_normal((3, d)).astype(np.float32)
+    got = model.moe_decode(ex, dev(ids), dev(wts), dev(x)).cpu().numpy()
+    same = model.moe_decode(ref, dev(ids), dev(wts), dev(x)).cpu().numpy()
+    assert np.array_equal(got, same)
+    hostp = lambda k: [(np.ascontiguousarray(p), np.ascontiguousarray(s)) for p, s in parts[k]]
+    table = oracle.ExpertTable(hostp("w1"), hostp("w3"), hostp("w2"), d, inter)
+    want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, mode=1)
+    assert rel_l2(got, want) <= 1e-5
+    ex.close()
+    f.close()
+
+
+def test_mxfp4sq_expert_blobs_are_refused(tmp_path):
+    # dtype 4 (MXFP4SQ, src/mxfp4.rs:140-240) is off the runtime path in the reference too ("the runtime packed matvec
+    # still reads DTYPE_MXFP4 only", src/mxfp4.rs:150-151): such a layer stays on the caller's CPU path
+    torch_cuda()
+    from microkimi_amd import weights
+    from microkimi_amd._lib import MkError
+    d, inter = 64, 32
+    rng = np.random.default_rng(1)
+    tensors = []
+    for e in range(2):
+        for k, (r, c) in (("w1", (inter, d)), ("w2", (d, inter)), ("w3", (inter, d))):
+            name = f"layers.0.block_sparse_moe.experts.{e}.{k}"
+            if (e, k) == (1, "w2"):
+                tensors.append((name, 4, (r, c), bytes(r * c // 2 + r * c // 32 + 4)))   # packed + quadratic scale bytes + f32 smax
+            else:
+                tensors.append((name, W.MXFP4, (r, c), (rng.integers(0, 256, (r, c // 2), dtype=np.uint8), rng.integers(118, 131, (r, c // 32), dtype=np.uint8))))
+    W.write(tmp_path / "sq.bin", tensors, config={"d_model": d})
+    f = weights.BinFile.open(tmp_path / "sq.bin")
+    assert f.entries["layers.0.block_sparse_moe.experts.1.w2"].dtype == 4
+    with pytest.raises(MkError) as e:
+        f.load_experts("layers.0.", 2)
+    assert e.value.status == -4 and "dtype 4" in str(e.value)
+    f.close()

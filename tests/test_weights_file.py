@@ -105,3 +105,29 @@ def test_directory_size_must_match_dims(tmp_path):
     assert "does not match" in str(e.value)
     with pytest.raises(MkError):
         weights.BinFile.open(tmp_path / "absent.bin")
+
+
+def test_file_written_by_the_reference_writer():
+    """tests/golden/mkim_ref.bin was written by the reference's own exporter (nano/export.py write_bin, experts
+    quantized by its quantize_mxfp4) and read back by the reference's own reader (nano/bin2pt.py read_bin):
+    mk_bin_* must see the same config, directory and bytes.  (tests/golden/make_mkim_fixture.py made both files.)"""
+    import json
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    exp = np.load(os.path.join(here, "mkim_ref_expected.npz"))
+    raw = open(os.path.join(here, "mkim_ref.bin"), "rb").read()
+    f = weights.BinFile.open(os.path.join(here, "mkim_ref.bin"))
+    assert f.config == json.loads(exp["config_json"].tobytes().decode())
+    names = [str(n) for n in exp["names"]]
+    assert f.names == names
+    for i, name in enumerate(names):
+        e = f.entries[name]
+        nd = int(exp["n_dims"][i])
+        assert e.dtype == int(exp["dtypes"][i]) and e.dims == tuple(int(v) for v in exp["dims"][i][:nd])
+        assert (e.offset, e.size) == (int(exp["offsets"][i]), int(exp["sizes"][i]))
+        assert f.blob(name).tobytes() == raw[e.offset:e.offset + e.size]
+    # an expert blob splits into nibbles then scales (weights::BinFile::mxfp4_parts); the all-zero block has scale byte 0
+    pk, sc, r, c = f.mxfp4_parts("layers.0.block_sparse_moe.experts.1.w1")
+    assert (r, c) == (32, 64) and sc[3, 0] == 0 and not pk[3, :16].any()
+    assert np.array_equal(f.i32_vec("mla_layers"), np.array([0, 3, 7]))
+    f.close()
