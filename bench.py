@@ -26,10 +26,21 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 FP4_PEAK_TFLOPS = 10100.0   # dense FP4/FP6 MFMA
 FP8_PEAK_TFLOPS = 5000.0
-# HBM bytes per launch of the batch-1 lm_head GEMV from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
-# reading of a plain 1 GiB copy (factors 2.000 and 1.000): 1 218 717 KiB read + 1 285 KiB written
-# (profiles/q8_gemv_b1_lm_head_163840x7168.md).  Algorithmic bytes are 1 248 489 472.
-LM_HEAD_B1_TRAFFIC_BYTES = 1249281900
+INT8_PEAK_TOPS = 5000.0
+F16_PEAK_TFLOPS = 2500.0
+# The committed counter summary of the headline kernel: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per launch, each scaled by
+# the reading of a plain 1 GiB copy.  Its line "traffic_bytes_per_launch = N" is what `roofline.traffic` reports.
+LM_HEAD_B1_PROFILE = os.path.join(ROOT, "profiles", "q8_gemv_b1_lm_head_163840x7168.md")
+
+
+def profile_traffic(path):
+    """HBM bytes per launch as the committed counter summary states them, or None when the file or the line is absent."""
+    import re
+    try:
+        m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", open(path).read())
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
 
 
 def log(*a):
@@ -170,8 +181,19 @@ def bench_lm_head(torch, steps, warmup):
     return res, (q, s, x, out8, am)
 
 
-def cpu_baseline_lm_head(torch, tensors, sample_rows=16384, budget_s=12.0):
-    """The CPU oracle's Q8Head::matvec on the first `sample_rows` rows of the same head (same pool split rule)."""
+def host_workers():
+    """Threads for the CPU baseline: std::thread::hardware_concurrency as the reference's pool takes it, bounded by this
+    process's CPU affinity and by OMP_NUM_THREADS where the host sets one (a shared machine's CPU share)."""
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    try:
+        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    except ValueError:
+        pass
+    return max(1, cores)
+
+
+def cpu_baseline_lm_head(torch, tensors, sample_rows=163840, budget_s=12.0):
+    """The CPU oracle's Q8Head::matvec on the same head, all rows (same pool split rule as the reference)."""
     import numpy as np
     import oracle
     q, s, x, out8, am = tensors
@@ -179,8 +201,7 @@ def cpu_baseline_lm_head(torch, tensors, sample_rows=16384, budget_s=12.0):
     qh = q[:sample_rows].cpu().numpy()
     sh = s[:sample_rows].float().cpu().numpy()
     xh = x[0].cpu().numpy()
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
-    workers = max(1, min(cores, 16))
+    workers = host_workers()
     oracle.q8head_matvec(qh, sh, sample_rows, cols, xh, workers=workers)  # warm-up
     ts = []
     t_end = time.perf_counter() + budget_s
@@ -195,8 +216,8 @@ def cpu_baseline_lm_head(torch, tensors, sample_rows=16384, budget_s=12.0):
     got = out8[0, :sample_rows].cpu().numpy()
     rel = float(np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want))
     return {"value": bytes_sample / med / 1e9, "unit": "GB/s", "cores": workers, "kind": "port",
-            "sample": f"first {sample_rows} of 163840 rows x 7168, batch 1, median of {len(ts)} calls, {med * 1e3:.2f} ms/call "
-                      f"(full head would take about {med * 1e3 * 163840 / sample_rows:.1f} ms)",
+            "sample": f"{sample_rows} of 163840 rows x 7168, batch 1, median of {len(ts)} calls, {med * 1e3:.2f} ms/call, "
+                      f"{workers} threads (hardware concurrency within this process's CPU share)",
             "gpu_vs_cpu_rel_l2_on_sample": rel}
 
 
@@ -305,7 +326,7 @@ def bench_moe(torch, cpu=True):
     for B in (1, 4, 16):
         logits_h, hidden_h = W.config2_tokens(B)
         logits = torch.from_numpy(logits_h).cuda()
-        x = torch.from_numpy(hidden_h * 0.02).cuda()  # small hidden state keeps SwiGLU of random experts finite
+        x = torch.from_numpy(hidden_h).cuda()  # hidden state ~ N(0, 1)
         ids, wts = model.router_softmax_topk(logits, W.TOP_K)
         out = torch.empty((B, d), device="cuda")
         n_distinct = len(set(ids.cpu().numpy().reshape(-1).tolist())) + 1
@@ -382,9 +403,13 @@ def bench_mla(torch, cpu=True):
         ms = ms_graph if ms_graph is not None else ms_eager
         alg = ctx * 612 + nh * (L + R) * 4 + nh * L * 4
         flops = 2.0 * nh * (L + R + L) * ctx
+        # matrix-core floor of this arithmetic: the scores as one int8 pass over latent + rope, P V as three f16 passes
+        # (the exact split of an int8 x f16-scale product and of p into f16 halves)
+        floor_us = (2.0 * nh * (L + R) * ctx / (INT8_PEAK_TOPS * 1e12) + 3 * 2.0 * nh * L * ctx / (F16_PEAK_TFLOPS * 1e12)) * 1e6
         res[f"ctx{ctx}"] = {"us": ms * 1e3, "us_python_loop": ms_eager * 1e3, "timing": "graph replay" if ms_graph is not None else "python loop",
                             "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                            "tflops": flops / (ms * 1e-3) / 1e12}
+                            "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "tflops": flops / (ms * 1e-3) / 1e12,
+                            "mfma_floor_us": floor_us, "frac_of_mfma_floor": floor_us / (ms * 1e3)}
         if cpu and ctx == 1024:
             # the CPU oracle's mla_attn_flash_q8_mqa (one thread, as the reference runs it) on the first cache
             import oracle
@@ -434,7 +459,7 @@ def bench_gemm(torch):
     flops = 2.0 * m * inter * d
     res = {"workload": "gate GEMM of 512 tokens x top-8 over 256 experts (4096 rows, 2048 x 7168 per expert), MXFP8 activations",
            "prefill": {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "mfma_frac_fp8_peak": flops / (ms * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
-                       "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "mfma_frac_fp4_peak": flops / (ms * 1e-3) / 1e12 / FP4_PEAK_TFLOPS, "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                        "rows_per_expert_max": int(counts.max()), "experts_used": used}}
     # large-M variant: the kernel's own ceiling
     M = 512
@@ -450,7 +475,8 @@ def bench_gemm(torch):
     ms2 = time_region(torch, step2, 20, warmup=3)
     fl2 = 2.0 * 8 * M * inter * d
     res["large_m"] = {"rows_per_expert": M, "experts": 8, "ms": ms2, "tflops": fl2 / (ms2 * 1e-3) / 1e12,
-                      "mfma_frac_fp8_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS}
+                      "mfma_frac_fp8_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
+                      "mfma_frac_fp4_peak": fl2 / (ms2 * 1e-3) / 1e12 / FP4_PEAK_TFLOPS}
     del cl, el, xl, out_l
     # the whole expert section of the prefill layer on the device (grouping, gather + MXFP8, gate, up, activation,
     # down, combine): mk_dev_moe_prefill.  The gate matrices above are reused as W1; W3 and W2 are drawn here.
@@ -472,7 +498,8 @@ def bench_gemm(torch):
     alg3 = used * per_expert + T * d * 4 + 2 * (m * d + m * d // 32) + 2 * 2 * m * inter * 4 + 2 * (m * inter + m * inter // 32) + 2 * m * d * 4 + T * d * 4
     res["expert_section"] = {"workload": "512 tokens x top-8 over 256 experts: group, gather + MXFP8, gate, up, SwiGLU + MXFP8, down, combine",
                              "ms": ms3, "tok_s": T / (ms3 * 1e-3), "tflops": fl3 / (ms3 * 1e-3) / 1e12,
-                             "mfma_frac_fp8_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, "weight_bytes": used * per_expert,
+                             "mfma_frac_fp8_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
+                             "mfma_frac_fp4_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP4_PEAK_TFLOPS, "weight_bytes": used * per_expert,
                              "alg_bytes": alg3, "gbs": alg3 / (ms3 * 1e-3) / 1e9, "hbm_frac": alg3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS,
                              "finite": bool(torch.isfinite(out).all().item())}
     return res
@@ -554,7 +581,7 @@ def main():
         "config": {"workload": "config 1: q8_0 lm_head 163840x7168 (int8 + f16 scale per 32), batch 1; step = quantize_q8(x) + GEMV",
                    "rows": 163840, "cols": 7168, "batch": 1, "algorithmic_bytes": head["alg_bytes"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": LM_HEAD_B1_TRAFFIC_BYTES,
+                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": profile_traffic(LM_HEAD_B1_PROFILE),
                      "kernel": "q8_gemv_b1_kernel<224, f16 scales>", "kernel_ms": head["kernel_ms"]},
         "cpu_baseline": cpu,
         "extras": extras,
