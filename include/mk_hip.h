@@ -94,6 +94,18 @@ int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *
  * is the activation format of mk_dev_mxfp4_grouped_gemm. */
 int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream);
 
+/* mxfp4::quantize (search != 0) / quantize_naive (search == 0) (src/mxfp4.rs:38-138): per 32-group
+ * e = ceil(log2(maxabs / 6)) clamped to [-127, 128], with `search` the better of e - 1, e, e + 1 by squared error in f64
+ * (e wins ties), nearest E2M1 level by the midpoints, sign from the sign bit.  w [rows][cols] f32 ->
+ * packed [rows][cols/2], scales [rows][cols/32]: the reference's bytes.  An offline path (weights arrive quantized).
+ * w and packed 16-byte aligned. */
+int mk_dev_mxfp4_quantize(const float *w, size_t rows, size_t cols, int search, uint8_t *packed, uint8_t *scales, void *stream);
+
+/* dequant::quantize_fp8 (src/dequant.rs:50-74): e4m3fn codes with one e8m0 scale per 128x128 block,
+ * e = ceil(log2(maxabs / 448)) clamped to [-127, 8].  rows and cols multiples of 128; qw [rows][cols],
+ * scales [rows/128][cols/128]: the reference's bytes. */
+int mk_dev_quantize_fp8(const float *w, size_t rows, size_t cols, uint8_t *qw, uint8_t *scales, void *stream);
+
 /* ------------------------------------------- device level: MXFP4 matvecs */
 
 /* mxfp4::matvec_packed_q8 (src/mxfp4.rs:405-443): out[r] = sum_g idot_g * (2^(sb_g-128) * xs_g).
@@ -279,15 +291,19 @@ int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, si
  * _q8_attn  mla_attn_flash_q8_mqa (src/model.rs:1804-1908) for m queries q [m][nh][nope+rope]: query i attends the
  *           positions 0 ..= pos0 + i (m = 1: the decode step of mla_forward, src/model.rs:1980-1985; m > 1: the
  *           per-position loop of mla_prefill, src/model.rs:2080-2102).  out [m][nh][vd].
- *           workspace: mk_mla_heads_workspace_bytes(m, nh, nope, vd). */
+ *           workspace: mk_mla_heads_workspace_bytes(m, nh, nope, vd).
+ * hadamard  nonzero: the cache is kept in the rotated form of kv_hadamard (src/model.rs:1529-1554, MICROKIMI_KV_HADAMARD=1):
+ *           hadamard64 on every 64-chunk of a K-nope row, a V row and the query's nope part before quantization, the
+ *           factor 1/64 on the latent score, the output rotated back.  As in the reference it takes effect only when
+ *           nope and vd are multiples of 64.  All three calls of a cache must agree on it. */
 int mk_dev_mla_heads_append(const float *k_rows, const float *v_rows, size_t n_new, size_t nh, size_t nope, size_t rope, size_t vd,
-                            size_t pos0, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream);
+                            size_t pos0, int hadamard, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream);
 int mk_dev_mla_heads_to_f32(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t n, size_t nh,
-                            size_t nope, size_t rope, size_t vd, float *k, float *v, void *stream);
+                            size_t nope, size_t rope, size_t vd, int hadamard, float *k, float *v, void *stream);
 size_t mk_mla_heads_workspace_bytes(size_t m, size_t nh, size_t nope, size_t vd);
 int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t pos0,
-                             const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, void *workspace,
-                             float *out, void *stream);
+                             const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, int hadamard,
+                             void *workspace, float *out, void *stream);
 
 /* ---------------------------------- device level: prefill expert GEMM */
 
@@ -456,11 +472,15 @@ void mk_q8head_free(mk_q8head *h);
  *                           64 up to 512, R 32 or 64.  A position is given as (latent [L], rope [R]).
  *   mk_mla_cache_new_heads  the reference's own layout: per position and head a K-nope row and a V row (int8 + f32
  *                           scales) and one shared f32 rope row.  A position is given as the reference gives it to
- *                           MlaCache::push: (k_row [nh][nope+rope], v_row [nh][vd]).
+ *                           MlaCache::push: (k_row [nh][nope+rope], v_row [nh][vd]).  The Hadamard option is read
+ *                           from MICROKIMI_KV_HADAMARD when the cache is made, like kv_hadamard() (src/model.rs:1532-1535),
+ *                           or set with mk_mla_cache_set_hadamard while the cache is empty.
  * row0 / row1 below are those two rows; rows0 / rows1 are n of them, position-major. */
 typedef struct mk_mla_cache mk_mla_cache;
 int mk_mla_cache_new(size_t nh, size_t L, size_t R, size_t capacity, mk_mla_cache **out);
 int mk_mla_cache_new_heads(size_t nh, size_t nope, size_t rope, size_t vd, size_t capacity, mk_mla_cache **out);
+/* MlaCache.had (src/model.rs:1567) of a cache in the reference's layout; MK_ERR_INVALID once positions are held */
+int mk_mla_cache_set_hadamard(mk_mla_cache *c, int on);
 /* MlaCache::push (src/model.rs:1583-1618) */
 int mk_mla_cache_push(mk_mla_cache *c, const float *row0, const float *row1);
 /* MlaCache::assign_f32 (src/model.rs:1680-1692): the cache is emptied and refilled from n f32 positions (snapshot restore) */

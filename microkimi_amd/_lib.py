@@ -61,6 +61,8 @@ def _load():
         "mk_dev_fp8_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_dev_quantize_q8": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_quantize_mxfp8": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_mxfp4_quantize": (i32, [vp, sz, sz, i32, vp, vp, vp]),
+        "mk_dev_quantize_fp8": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_mxfp4_matvec_q8": (i32, [vp, vp, sz, sz, vp, vp, vp, vp]),
         "mk_dev_mxfp4_matvec_f32": (i32, [vp, vp, sz, sz, vp, vp, vp]),
         "mk_dev_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp, i32, vp, vp, vp]),
@@ -83,10 +85,10 @@ def _load():
         "mk_mla_decode_static_max_heads": (sz, []),
         "mk_dev_mla_q8_decode_static": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp]),
         "mk_dev_mla_cache_append": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, vp, vp]),
-        "mk_dev_mla_heads_append": (i32, [vp, vp, sz, sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
-        "mk_dev_mla_heads_to_f32": (i32, [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, vp, vp, vp]),
+        "mk_dev_mla_heads_append": (i32, [vp, vp, sz, sz, sz, sz, sz, sz, i32, vp, vp, vp, vp, vp, vp]),
+        "mk_dev_mla_heads_to_f32": (i32, [vp, vp, vp, vp, vp, sz, sz, sz, sz, sz, i32, vp, vp, vp]),
         "mk_mla_heads_workspace_bytes": (sz, [sz, sz, sz, sz]),
-        "mk_dev_mla_heads_q8_attn": (i32, [vp, vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, f32, vp, vp, vp]),
+        "mk_dev_mla_heads_q8_attn": (i32, [vp, vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, f32, i32, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
         "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),
         "mk_moe_prefill_workspace_layout": (i32, [sz, sz, sz, sz, sz, C.POINTER(PrefillLayout)]),
@@ -105,6 +107,7 @@ def _load():
         "mk_q8head_free": (None, [vp]),
         "mk_mla_cache_new": (i32, [sz, sz, sz, sz, C.POINTER(vp)]),
         "mk_mla_cache_new_heads": (i32, [sz, sz, sz, sz, sz, C.POINTER(vp)]),
+        "mk_mla_cache_set_hadamard": (i32, [vp, i32]),
         "mk_mla_cache_push": (i32, [vp, vp, vp]),
         "mk_mla_cache_assign_f32": (i32, [vp, vp, vp, sz]),
         "mk_mla_attn_prefill": (i32, [vp, vp, sz, f32, vp]),

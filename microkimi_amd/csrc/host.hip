@@ -561,6 +561,7 @@ extern "C" int mk_q8head_matvec(mk_q8head *h, const float *x, size_t batch, floa
 //     a K-nope row and a V row (int8 + f32 scales) and one shared f32 rope row.
 struct mk_mla_cache {
     int heads_layout = 0;
+    int had = 0;  // heads layout: rotated form (kv_hadamard, src/model.rs:1532-1535)
     size_t nh = 0, L = 0, R = 0, vd = 0, cap = 0, n = 0;  // heads layout: L = nope, R = rope
     int8_t *lat_q = nullptr, *rope_q = nullptr;            // heads layout: kq, vq
     void *lat_s = nullptr, *rope_s = nullptr;              // heads layout: ks (f32), vs (f32)
@@ -619,6 +620,10 @@ extern "C" int mk_mla_cache_new_heads(size_t nh, size_t nope, size_t rope, size_
     if ((s = bind_device()) != MK_OK) return s;
     mk_mla_cache *c = new mk_mla_cache();
     c->heads_layout = 1;
+    {
+        const char *e = getenv("MICROKIMI_KV_HADAMARD");
+        c->had = e && strcmp(e, "1") == 0;
+    }
     c->nh = nh;
     c->L = nope;
     c->R = rope;
@@ -642,6 +647,15 @@ extern "C" int mk_mla_cache_new_heads(size_t nh, size_t nope, size_t rope, size_
 
 extern "C" size_t mk_mla_cache_positions(const mk_mla_cache *c) { return c ? c->n : 0; }
 
+extern "C" int mk_mla_cache_set_hadamard(mk_mla_cache *c, int on) {
+    MK_REQUIRE(c, "null pointer");
+    MK_REQUIRE(c->heads_layout, "the Hadamard option belongs to the per-head layout (mk_mla_cache_new_heads)");
+    std::lock_guard<std::mutex> lk(g_mu);
+    MK_REQUIRE(c->n == 0, "the option can change only while the cache is empty");
+    c->had = on ? 1 : 0;
+    return MK_OK;
+}
+
 namespace {
 // widths of the two host rows a position is given as: (latent, rope) or (k_row = nh x (nope + rope), v_row = nh x vd)
 size_t row0_floats(const mk_mla_cache *c) { return c->heads_layout ? c->nh * (c->L + c->R) : c->L; }
@@ -661,7 +675,7 @@ int mla_append_host(mk_mla_cache *c, const float *r0, const float *r1, size_t n_
         MK_HIP_TRY(hipMemcpyAsync(d0, r0 + j0 * w0, nj * w0 * 4, hipMemcpyHostToDevice, g_ctx.stream));
         if (w1) MK_HIP_TRY(hipMemcpyAsync(d1, r1 + j0 * w1, nj * w1 * 4, hipMemcpyHostToDevice, g_ctx.stream));
         if (c->heads_layout)
-            s = mk_dev_mla_heads_append(d0, d1, nj, c->nh, c->L, c->R, c->vd, c->n, c->lat_q, (float *)c->lat_s, c->kr, c->rope_q, (float *)c->rope_s,
+            s = mk_dev_mla_heads_append(d0, d1, nj, c->nh, c->L, c->R, c->vd, c->n, c->had, c->lat_q, (float *)c->lat_s, c->kr, c->rope_q, (float *)c->rope_s,
                                         g_ctx.stream);
         else
             s = mk_dev_mla_cache_append(d0, d1, c->L, c->R, c->n, c->lat_q, c->lat_s, c->rope_q, c->rope_s, g_ctx.stream);
@@ -714,7 +728,7 @@ extern "C" int mk_mla_cache_to_f32(const mk_mla_cache *c, float *rows0, float *r
         void *dk = nullptr;
         if (mk_check_hip(hipMalloc(&dk, n * (w0 + w1) * 4), "hipMalloc(to_f32)") != MK_OK) return MK_ERR_NOMEM;
         float *k = (float *)dk, *v = k + n * w0;
-        s = mk_dev_mla_heads_to_f32(c->lat_q, (const float *)c->lat_s, c->kr, c->rope_q, (const float *)c->rope_s, n, c->nh, c->L, c->R, c->vd, k, v,
+        s = mk_dev_mla_heads_to_f32(c->lat_q, (const float *)c->lat_s, c->kr, c->rope_q, (const float *)c->rope_s, n, c->nh, c->L, c->R, c->vd, c->had, k, v,
                                     g_ctx.stream);
         std::vector<float> hk, hv;
         if (s == MK_OK) {
@@ -760,7 +774,7 @@ int mla_attn_host(mk_mla_cache *c, const float *q, size_t m, size_t pos0, float 
     MK_HIP_TRY(hipMemcpyAsync(c->q.p, q, qn * 4, hipMemcpyHostToDevice, g_ctx.stream));
     if (c->heads_layout) {
         s = mk_dev_mla_heads_q8_attn(c->lat_q, (const float *)c->lat_s, c->kr, c->rope_q, (const float *)c->rope_s, pos0, (const float *)c->q.p, m,
-                                     c->nh, c->L, c->R, c->vd, scale, c->ws.p, (float *)c->out.p, g_ctx.stream);
+                                     c->nh, c->L, c->R, c->vd, scale, c->had, c->ws.p, (float *)c->out.p, g_ctx.stream);
     } else {
         for (size_t i = 0; i < m && s == MK_OK; i++)
             s = mk_dev_mla_q8_decode(c->lat_q, c->lat_s, c->rope_q, c->rope_s, pos0 + i, (const float *)c->q.p + i * c->nh * (c->L + c->R), c->nh,

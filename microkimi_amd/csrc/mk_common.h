@@ -22,6 +22,7 @@ typedef int mk_i4 __attribute__((ext_vector_type(4)));
 typedef int mk_i8v __attribute__((ext_vector_type(8)));
 typedef float mk_f4 __attribute__((ext_vector_type(4)));
 typedef unsigned int mk_u2 __attribute__((ext_vector_type(2)));
+typedef unsigned int mk_v4u __attribute__((ext_vector_type(4)));
 typedef float mk_f16v __attribute__((ext_vector_type(16)));
 
 // Loads that tell the compiler the pointer is global memory.  A pointer that was

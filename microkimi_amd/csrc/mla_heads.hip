@@ -12,7 +12,11 @@
 //            Splits are merged by log-sum-exp.  With several queries (prefill, src/model.rs:2080-2102) query i
 //            attends positions 0 ..= pos0 + i.
 //
-// The Hadamard option (MICROKIMI_KV_HADAMARD, off by default) is not built: a cache in that mode stays on the CPU.
+// The Hadamard option (kv_hadamard / hadamard64, src/model.rs:1529-1554; MICROKIMI_KV_HADAMARD=1, off by default): every
+// 64-chunk of a K-nope row, a V row and a query's nope part goes through the unnormalized Walsh-Hadamard butterfly
+// before it is quantized; the latent score carries the factor 1/64 and the attention output is rotated back.  As in the
+// reference it applies only when nope and v are multiples of 64.  The butterfly is the reference's: the same six stages
+// of one addition or subtraction per element, so the rotated values (and the cache bytes) are identical.
 #include "mk_common.h"
 
 namespace {
@@ -23,6 +27,17 @@ constexpr int MAX_NB = 8;       // latent blocks per head the decode kernel hold
 constexpr int MAX_VD = 512;
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// hadamard64 (src/model.rs:1540-1554) on a 64-chunk held one element per lane by a whole wave: stage h pairs lane j
+// (bit h clear) with lane j + h: x[j] = a + b, x[j + h] = a - b.
+__device__ __forceinline__ float hadamard64_lane(float v, int lane) {
+#pragma unroll
+    for (int h = 1; h < 64; h <<= 1) {
+        const float o = __shfl_xor(v, h, MK_WAVE);
+        v = (lane & h) ? o - v : v + o;
+    }
+    return v;
+}
 
 // One 32-block per aligned group of 32 lanes: q8::quantize_q8_into (src/q8.rs:57-68).
 __device__ __forceinline__ void quantize_block32(float v, int8_t *q_out, float *s_out, int j) {
@@ -35,19 +50,23 @@ __device__ __forceinline__ void quantize_block32(float v, int8_t *q_out, float *
 // grid: (blocks of the position's rows, position).  Blocks 0 .. nh*nope/32-1: K-nope of head h; then nh*vd/32 V blocks;
 // the last workgroups copy the rope row of head 0.
 __global__ __launch_bounds__(256) void heads_append_kernel(const float *__restrict__ k_rows, const float *__restrict__ v_rows, int nh, int nope,
-                                                           int rope, int vd, size_t pos0, int8_t *__restrict__ kq, float *__restrict__ ks,
-                                                           float *__restrict__ kr, int8_t *__restrict__ vq, float *__restrict__ vs) {
+                                                           int rope, int vd, size_t pos0, int had, int8_t *__restrict__ kq,
+                                                           float *__restrict__ ks, float *__restrict__ kr, int8_t *__restrict__ vq,
+                                                           float *__restrict__ vs) {
+    // (with the Hadamard option nope and vd are multiples of 64: a wave then holds one 64-chunk, two blocks of one row)
     const int nbk = nh * nope / 32, nbv = nh * vd / 32;
     const size_t jn = blockIdx.y, pos = pos0 + jn;
     const int blk = (blockIdx.x * blockDim.x + threadIdx.x) >> 5, j = threadIdx.x & 31;
     const int qh = nope + rope;
     if (blk < nbk) {
         const int h = blk / (nope / 32), g = blk % (nope / 32);
-        const float v = k_rows[(jn * nh + h) * qh + g * 32 + j];
+        float v = k_rows[(jn * nh + h) * qh + g * 32 + j];
+        if (had) v = hadamard64_lane(v, threadIdx.x & 63);
         quantize_block32(v, kq + (pos * nh + h) * nope + g * 32, ks + pos * nbk + blk, j);
     } else if (blk < nbk + nbv) {
         const int b = blk - nbk, h = b / (vd / 32), g = b % (vd / 32);
-        const float v = v_rows[(jn * nh + h) * vd + g * 32 + j];
+        float v = v_rows[(jn * nh + h) * vd + g * 32 + j];
+        if (had) v = hadamard64_lane(v, threadIdx.x & 63);
         quantize_block32(v, vq + (pos * nh + h) * vd + g * 32, vs + pos * nbv + b, j);
     } else {
         const int d = (blk - nbk - nbv) * 32 + j;
@@ -71,14 +90,49 @@ __global__ __launch_bounds__(256) void heads_to_f32_kernel(const int8_t *__restr
     }
 }
 
+// The same with the Hadamard option: a wave per 64-chunk, dequantized, rotated back (butterfly, then / 64).
+__global__ __launch_bounds__(256) void heads_to_f32_had_kernel(const int8_t *__restrict__ kq, const float *__restrict__ ks,
+                                                               const float *__restrict__ kr, const int8_t *__restrict__ vq,
+                                                               const float *__restrict__ vs, int nh, int nope, int rope, int vd,
+                                                               float *__restrict__ k, float *__restrict__ v) {
+    const size_t j = blockIdx.y;
+    const int qh = nope + rope, lane = threadIdx.x & 63;
+    const int ck = nh * nope / 64, cv = nh * vd / 64;
+    for (int c = (blockIdx.x * blockDim.x + threadIdx.x) >> 6; c < ck + cv; c += (gridDim.x * blockDim.x) >> 6) {
+        if (c < ck) {
+            const int h = c / (nope / 64), d = (c % (nope / 64)) * 64 + lane;
+            const float x = (float)kq[(j * nh + h) * nope + d] * ks[(j * nh + h) * (nope / 32) + d / 32];
+            k[(j * nh + h) * qh + d] = hadamard64_lane(x, lane) / 64.0f;
+        } else {
+            const int cc = c - ck, h = cc / (vd / 64), d = (cc % (vd / 64)) * 64 + lane;
+            const float x = (float)vq[(j * nh + h) * vd + d] * vs[(j * nh + h) * (vd / 32) + d / 32];
+            v[(j * nh + h) * vd + d] = hadamard64_lane(x, lane) / 64.0f;
+        }
+    }
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < nh * rope; i += gridDim.x * blockDim.x) {
+        const int h = i / rope, d = i % rope;
+        k[(j * nh + h) * qh + nope + d] = kr[j * rope + d];
+    }
+}
+
+// The attention rows rotated back (src/model.rs:1896-1903): butterfly, then / 64, per 64-chunk.
+__global__ __launch_bounds__(256) void heads_out_had_kernel(float *__restrict__ out, size_t chunks) {
+    const size_t c = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (c >= chunks) return;
+    out[c * 64 + lane] = hadamard64_lane(out[c * 64 + lane], lane) / 64.0f;
+}
+
 // q8 of the latent part of every (query, head): (src/model.rs:1812-1821)
-__global__ __launch_bounds__(256) void heads_q_prep_kernel(const float *__restrict__ q, int rows, int nope, int rope, int8_t *__restrict__ qq,
-                                                           float *__restrict__ qs) {
+__global__ __launch_bounds__(256) void heads_q_prep_kernel(const float *__restrict__ q, int rows, int nope, int rope, int had,
+                                                           int8_t *__restrict__ qq, float *__restrict__ qs) {
     const int nb = nope / 32;
     const int blk = (blockIdx.x * blockDim.x + threadIdx.x) >> 5, j = threadIdx.x & 31;
-    if (blk >= rows * nb) return;
+    if (blk >= rows * nb) return;  // (with the Hadamard option nb is even: both halves of a wave stay or leave together)
     const int r = blk / nb, g = blk % nb;
-    quantize_block32(q[(size_t)r * (nope + rope) + g * 32 + j], qq + (size_t)r * nope + g * 32, qs + blk, j);
+    float v = q[(size_t)r * (nope + rope) + g * 32 + j];
+    if (had) v = hadamard64_lane(v, threadIdx.x & 63);
+    quantize_block32(v, qq + (size_t)r * nope + g * 32, qs + blk, j);
 }
 
 struct HeadsArgs {
@@ -92,6 +146,7 @@ struct HeadsArgs {
     const float *qs;   // [m][nh][nope/32]
     int nh, nope, rope, vd, n_pos0, split_len, n_splits;
     float scale;
+    float had_k;          // factor of the latent part of a score: 1/64 with the Hadamard option (src/model.rs:1823), else 1
     float *po, *pm, *pl;  // split partials (one query only)
     float *out;           // [m][nh][vd]
 };
@@ -123,7 +178,7 @@ __global__ __launch_bounds__(256) void heads_decode_kernel(HeadsArgs a) {
             const mk_i4 *src = reinterpret_cast<const mk_i4 *>(a.qq + qrow * nope + g * 32);
             qreg[k][0] = src[0];
             qreg[k][1] = src[1];
-            qsc[k] = a.qs[qrow * nb + g];
+            qsc[k] = a.qs[qrow * nb + g] * a.had_k;  // (a power of two: the product with 1/64 is exact)
         } else {
             qreg[k][0] = qreg[k][1] = mk_i4{0, 0, 0, 0};
             qsc[k] = 0.0f;
@@ -261,8 +316,11 @@ int check_shape(size_t nh, size_t nope, size_t rope, size_t vd) {
 
 }  // namespace
 
+// the option applies only when both widths are whole 64-chunks (src/model.rs:1590, 1631, 1811)
+static int had_applies(int hadamard, size_t nope, size_t vd) { return hadamard && nope % 64 == 0 && vd % 64 == 0; }
+
 extern "C" int mk_dev_mla_heads_append(const float *k_rows, const float *v_rows, size_t n_new, size_t nh, size_t nope, size_t rope, size_t vd,
-                                       size_t pos0, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream) {
+                                       size_t pos0, int hadamard, int8_t *kq, float *ks, float *kr, int8_t *vq, float *vs, void *stream) {
     MK_REQUIRE(k_rows && v_rows && kq && ks && vq && vs && (kr || rope == 0), "null pointer");
     int s = check_shape(nh, nope, rope, vd);
     if (s != MK_OK) return s;
@@ -270,12 +328,12 @@ extern "C" int mk_dev_mla_heads_append(const float *k_rows, const float *v_rows,
     MK_REQUIRE(n_new <= 65535, "at most 65535 positions per call");
     const size_t blocks32 = nh * nope / 32 + nh * vd / 32 + (rope + 31) / 32;
     hipLaunchKernelGGL(heads_append_kernel, dim3((unsigned)((blocks32 + 7) / 8), (unsigned)n_new), dim3(256), 0, (hipStream_t)stream, k_rows, v_rows,
-                       (int)nh, (int)nope, (int)rope, (int)vd, pos0, kq, ks, kr, vq, vs);
+                       (int)nh, (int)nope, (int)rope, (int)vd, pos0, had_applies(hadamard, nope, vd), kq, ks, kr, vq, vs);
     return mk_launch_status("heads_append");
 }
 
 extern "C" int mk_dev_mla_heads_to_f32(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t n,
-                                       size_t nh, size_t nope, size_t rope, size_t vd, float *k, float *v, void *stream) {
+                                       size_t nh, size_t nope, size_t rope, size_t vd, int hadamard, float *k, float *v, void *stream) {
     MK_REQUIRE(kq && ks && vq && vs && k && v && (kr || rope == 0), "null pointer");
     int s = check_shape(nh, nope, rope, vd);
     if (s != MK_OK) return s;
@@ -283,9 +341,14 @@ extern "C" int mk_dev_mla_heads_to_f32(const int8_t *kq, const float *ks, const 
     MK_REQUIRE(n <= 65535 * 64, "too many positions");
     for (size_t j0 = 0; j0 < n; j0 += 65535) {
         const size_t nj = n - j0 < 65535 ? n - j0 : 65535;
-        hipLaunchKernelGGL(heads_to_f32_kernel, dim3(8, (unsigned)nj), dim3(256), 0, (hipStream_t)stream, kq + j0 * nh * nope,
-                           ks + j0 * nh * (nope / 32), kr + j0 * rope, vq + j0 * nh * vd, vs + j0 * nh * (vd / 32), (int)nh, (int)nope, (int)rope,
-                           (int)vd, k + j0 * nh * (nope + rope), v + j0 * nh * vd);
+        if (had_applies(hadamard, nope, vd))
+            hipLaunchKernelGGL(heads_to_f32_had_kernel, dim3(8, (unsigned)nj), dim3(256), 0, (hipStream_t)stream, kq + j0 * nh * nope,
+                               ks + j0 * nh * (nope / 32), kr + j0 * rope, vq + j0 * nh * vd, vs + j0 * nh * (vd / 32), (int)nh, (int)nope,
+                               (int)rope, (int)vd, k + j0 * nh * (nope + rope), v + j0 * nh * vd);
+        else
+            hipLaunchKernelGGL(heads_to_f32_kernel, dim3(8, (unsigned)nj), dim3(256), 0, (hipStream_t)stream, kq + j0 * nh * nope,
+                               ks + j0 * nh * (nope / 32), kr + j0 * rope, vq + j0 * nh * vd, vs + j0 * nh * (vd / 32), (int)nh, (int)nope,
+                               (int)rope, (int)vd, k + j0 * nh * (nope + rope), v + j0 * nh * vd);
         if ((s = mk_launch_status("heads_to_f32")) != MK_OK) return s;
     }
     return MK_OK;
@@ -297,8 +360,8 @@ extern "C" size_t mk_mla_heads_workspace_bytes(size_t m, size_t nh, size_t nope,
 }
 
 extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const float *kr, const int8_t *vq, const float *vs, size_t pos0,
-                                        const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, void *workspace,
-                                        float *out, void *stream) {
+                                        const float *q, size_t m, size_t nh, size_t nope, size_t rope, size_t vd, float scale, int hadamard,
+                                        void *workspace, float *out, void *stream) {
     MK_REQUIRE(kq && ks && vq && vs && q && workspace && out && (kr || rope == 0), "null pointer");
     int s = check_shape(nh, nope, rope, vd);
     if (s != MK_OK) return s;
@@ -333,8 +396,11 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.n_pos0 = (int)pos0 + 1;
     a.scale = scale;
     a.out = out;
+    const int had = had_applies(hadamard, nope, vd);
+    a.had_k = had ? 1.0f / 64.0f : 1.0f;
     const int rows = (int)(m * nh);
-    hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, qq, qs);
+    hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, had, qq,
+                       qs);
     if ((s = mk_launch_status("heads_q_prep")) != MK_OK) return s;
     // one query: split the context so that about 1024 workgroups stream the cache; several queries (prefill): the
     // (query, head) grid is parallel enough, one split each
@@ -352,7 +418,14 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.n_splits = n_splits;
     hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);
     if ((s = mk_launch_status("heads_decode")) != MK_OK) return s;
-    if (n_splits == 1) return MK_OK;
-    hipLaunchKernelGGL(heads_merge_kernel, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
-    return mk_launch_status("heads_merge");
+    if (n_splits > 1) {
+        hipLaunchKernelGGL(heads_merge_kernel, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
+        if ((s = mk_launch_status("heads_merge")) != MK_OK) return s;
+    }
+    if (had) {
+        const size_t chunks = m * nh * vd / 64;
+        hipLaunchKernelGGL(heads_out_had_kernel, dim3((unsigned)((chunks + 3) / 4)), dim3(256), 0, st, out, chunks);
+        return mk_launch_status("heads_out_had");
+    }
+    return MK_OK;
 }

@@ -19,6 +19,21 @@ def dequant_fp8(w, scales, rows, cols):
     return out
 
 
+def quantize_fp8(w):
+    """dequant::quantize_fp8 (src/dequant.rs:50-74) of a device tensor [rows, cols] f32, both multiples of 128:
+    (e4m3fn codes [rows, cols], e8m0 scales [rows/128, cols/128])."""
+    import torch
+    _lib.require_device()
+    w = w.contiguous()
+    rows, cols = w.shape
+    if rows % 128 or cols % 128:
+        raise ValueError("fp8: rows and cols must be multiples of 128")
+    qw = torch.empty((rows, cols), dtype=torch.uint8, device=w.device)
+    scales = torch.empty((rows // 128, cols // 128), dtype=torch.uint8, device=w.device)
+    check(lib.mk_dev_quantize_fp8(ptr(w), rows, cols, ptr(qw), ptr(scales), cur_stream()))
+    return qw, scales
+
+
 def quantize_mxfp8(x):
     """deepseek::fp8_roundtrip with block 32 (src/deepseek.rs:312-322) in coded form: (e4m3 codes, e8m0 exponents)."""
     import torch

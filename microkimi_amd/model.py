@@ -136,9 +136,10 @@ class MlaHeadsCache:
     MlaCache::push, ::assign_f32, ::to_f32 and mla_attn_flash_q8_mqa; attn with several queries is the attention loop
     of mla_prefill (src/model.rs:2080-2102)."""
 
-    def __init__(self, nh, nope, rope, vd, capacity, device="cuda"):
+    def __init__(self, nh, nope, rope, vd, capacity, device="cuda", hadamard=False):
         import torch
         self.nh, self.nope, self.rope, self.vd, self.cap, self.n = nh, nope, rope, vd, capacity, 0
+        self.had = int(bool(hadamard))  # kv_hadamard (src/model.rs:1532-1535): takes effect when nope and vd are multiples of 64
         self.kq = torch.zeros((capacity, nh * nope), dtype=torch.int8, device=device)
         self.ks = torch.zeros((capacity, nh * nope // 32), dtype=torch.float32, device=device)
         self.kr = torch.zeros((capacity, rope), dtype=torch.float32, device=device)
@@ -157,7 +158,7 @@ class MlaHeadsCache:
         n_new = k_rows.shape[0]
         if self.n + n_new > self.cap:
             raise RuntimeError("MlaCache is full")
-        check(lib.mk_dev_mla_heads_append(ptr(k_rows), ptr(v_rows), n_new, self.nh, self.nope, self.rope, self.vd, self.n, ptr(self.kq),
+        check(lib.mk_dev_mla_heads_append(ptr(k_rows), ptr(v_rows), n_new, self.nh, self.nope, self.rope, self.vd, self.n, self.had, ptr(self.kq),
                                           ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), cur_stream()))
         self.n += n_new
 
@@ -173,7 +174,7 @@ class MlaHeadsCache:
         v = torch.empty((self.n, self.nh * self.vd), dtype=torch.float32, device=self.kq.device)
         if self.n:
             check(lib.mk_dev_mla_heads_to_f32(ptr(self.kq), ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), self.n, self.nh, self.nope,
-                                              self.rope, self.vd, ptr(k), ptr(v), cur_stream()))
+                                              self.rope, self.vd, self.had, ptr(k), ptr(v), cur_stream()))
         return k, v
 
     def attn(self, q, pos0, scale):
@@ -189,7 +190,7 @@ class MlaHeadsCache:
             self._ws = torch.empty(need, dtype=torch.uint8, device=q.device)
         out = torch.empty((m, self.nh * self.vd), dtype=torch.float32, device=q.device)
         check(lib.mk_dev_mla_heads_q8_attn(ptr(self.kq), ptr(self.ks), ptr(self.kr), ptr(self.vq), ptr(self.vs), pos0, ptr(q), m, self.nh,
-                                           self.nope, self.rope, self.vd, float(scale), ptr(self._ws), ptr(out), cur_stream()))
+                                           self.nope, self.rope, self.vd, float(scale), self.had, ptr(self._ws), ptr(out), cur_stream()))
         return out
 
 

@@ -31,6 +31,26 @@ def dequant(packed, scales, rows, cols):
     return out
 
 
+def quantize(w, search=True):
+    """mxfp4::quantize (search) / quantize_naive (src/mxfp4.rs:38-138) of a device tensor [rows, cols] f32: the
+    reference's (packed [rows, cols/2], scales [rows, cols/32]) bytes."""
+    import torch
+    _lib.require_device()
+    w = w.contiguous()
+    rows, cols = w.shape
+    if cols % 32:
+        raise ValueError("cols must be a multiple of 32")
+    packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+    scales = torch.empty((rows, cols // 32), dtype=torch.uint8, device=w.device)
+    check(lib.mk_dev_mxfp4_quantize(ptr(w), rows, cols, int(bool(search)), ptr(packed), ptr(scales), cur_stream()))
+    return packed, scales
+
+
+def quantize_naive(w):
+    """mxfp4::quantize_naive (src/mxfp4.rs:94-100)."""
+    return quantize(w, search=False)
+
+
 def matvec_packed_q8(packed, scales, rows, cols, xq, out):
     """mxfp4::matvec_packed_q8 (src/mxfp4.rs:405-443) on device tensors; xq is a q8.Q8Vec."""
     _check_shapes(packed, scales, rows, cols)

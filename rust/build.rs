@@ -9,7 +9,7 @@ use std::process::Command;
 
 const SOURCES: &[&str] = &[
     "host.hip", "codec.hip", "gemv_mxfp4.hip", "gemv_q8.hip", "moe.hip", "mla.hip", "mla_heads.hip", "gemm_mxfp4.hip",
-    "gemm_q8x.hip", "prefill.hip", "front.hip", "weights.hip", "vq1.hip",
+    "gemm_q8x.hip", "prefill.hip", "front.hip", "weights.hip", "vq1.hip", "quantize.hip",
 ];
 
 fn main() {

@@ -115,6 +115,8 @@ extern "C" {
     pub fn mk_dev_mxfp4_dequant(packed: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_fp8_dequant(w: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_q8(x: *const f32, nvec: usize, n: usize, q: *mut i8, scales: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4_quantize(w: *const f32, rows: usize, cols: usize, search: c_int, packed: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_quantize_fp8(w: *const f32, rows: usize, cols: usize, qw: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_mxfp8(x: *const f32, nvec: usize, n: usize, codes: *mut u8, exps: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_matvec_q8(packed: *const u8, scales: *const u8, rows: usize, cols: usize, xq: *const i8, xs: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_matvec_f32(packed: *const u8, scales: *const u8, rows: usize, cols: usize, x: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;
@@ -138,10 +140,10 @@ extern "C" {
     pub fn mk_mla_decode_static_max_heads() -> usize;
     pub fn mk_dev_mla_q8_decode_static(lat_q: *const i8, lat_s: *const c_void, rope_q: *const i8, rope_s: *const c_void, pos: usize, q: *const f32, nh: usize, L: usize, R: usize, scale: f32, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mla_cache_append(latent: *const f32, rope: *const f32, L: usize, R: usize, pos: usize, lat_q: *mut i8, lat_s: *mut c_void, rope_q: *mut i8, rope_s: *mut c_void, stream: *mut c_void) -> c_int;
-    pub fn mk_dev_mla_heads_append(k_rows: *const f32, v_rows: *const f32, n_new: usize, nh: usize, nope: usize, rope: usize, vd: usize, pos0: usize, kq: *mut i8, ks: *mut f32, kr: *mut f32, vq: *mut i8, vs: *mut f32, stream: *mut c_void) -> c_int;
-    pub fn mk_dev_mla_heads_to_f32(kq: *const i8, ks: *const f32, kr: *const f32, vq: *const i8, vs: *const f32, n: usize, nh: usize, nope: usize, rope: usize, vd: usize, k: *mut f32, v: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mla_heads_append(k_rows: *const f32, v_rows: *const f32, n_new: usize, nh: usize, nope: usize, rope: usize, vd: usize, pos0: usize, hadamard: c_int, kq: *mut i8, ks: *mut f32, kr: *mut f32, vq: *mut i8, vs: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mla_heads_to_f32(kq: *const i8, ks: *const f32, kr: *const f32, vq: *const i8, vs: *const f32, n: usize, nh: usize, nope: usize, rope: usize, vd: usize, hadamard: c_int, k: *mut f32, v: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_mla_heads_workspace_bytes(m: usize, nh: usize, nope: usize, vd: usize) -> usize;
-    pub fn mk_dev_mla_heads_q8_attn(kq: *const i8, ks: *const f32, kr: *const f32, vq: *const i8, vs: *const f32, pos0: usize, q: *const f32, m: usize, nh: usize, nope: usize, rope: usize, vd: usize, scale: f32, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mla_heads_q8_attn(kq: *const i8, ks: *const f32, kr: *const f32, vq: *const i8, vs: *const f32, pos0: usize, q: *const f32, m: usize, nh: usize, nope: usize, rope: usize, vd: usize, scale: f32, hadamard: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_grouped_gemm(packed_ptrs: *const *const u8, scales_ptrs: *const *const u8, n_groups: usize, rows: usize, cols: usize, codes: *const u8, exps: *const u8, offsets: *const i32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_moe_prefill_workspace_bytes(T: usize, topk: usize, n_experts: usize, d: usize, inter: usize) -> usize;
     pub fn mk_moe_prefill_workspace_layout(T: usize, topk: usize, n_experts: usize, d: usize, inter: usize, out: *mut MkPrefillLayout) -> c_int;
@@ -176,6 +178,7 @@ extern "C" {
     pub fn mk_q8head_free(h: *mut MkQ8Head);
     pub fn mk_mla_cache_new(nh: usize, L: usize, R: usize, capacity: usize, out: *mut *mut MkMlaCache) -> c_int;
     pub fn mk_mla_cache_new_heads(nh: usize, nope: usize, rope: usize, vd: usize, capacity: usize, out: *mut *mut MkMlaCache) -> c_int;
+    pub fn mk_mla_cache_set_hadamard(c: *mut MkMlaCache, on: c_int) -> c_int;
     pub fn mk_mla_cache_push(c: *mut MkMlaCache, row0: *const f32, row1: *const f32) -> c_int;
     pub fn mk_mla_cache_assign_f32(c: *mut MkMlaCache, rows0: *const f32, rows1: *const f32, n: usize) -> c_int;
     pub fn mk_mla_cache_positions(c: *const MkMlaCache) -> usize;

@@ -122,3 +122,61 @@ def test_quantize_mxfp8_bit_exact():
         _, c, e = oracle.fp8_roundtrip(x[r], 32)
         assert np.array_equal(exps[r], e), r
         assert np.array_equal(codes[r], c), r
+
+
+def _quantizer_inputs(rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    w *= np.exp2(rng.integers(-20, 20, size=(rows, cols // 32)).astype(np.float32)).repeat(32, axis=1)  # group scales all over
+    w[0, :32] = 0.0                                              # a zero group: scale byte 0, all nibbles 0
+    w[0, 32:64] = -0.0
+    w[1, :32] = 0.0
+    w[1, 0] = 6.0                                                # maxabs / 6 an exact power of two
+    w[1, 1:8] = [0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0]          # every midpoint: the upper level
+    w[1, 8:15] = [-0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0]
+    w[1, 15] = np.float32(0.24999999)
+    w[2, :32] = np.float32(6.0000005)                            # just above a power of two: the logarithm rounds down
+    w[2, 32:64] = np.float32(1e-41)                              # maxabs / 6 subnormal
+    w[3, :32] = np.float32(3e38)                                 # the largest exponents
+    w[3, 32:64] = np.float32(2.0 ** -126)
+    w[4, :32] = np.linspace(-7, 7, 32, dtype=np.float32)         # clamps at +-6
+    return w
+
+
+@pytest.mark.parametrize("search", [True, False])
+def test_mxfp4_quantize_gives_the_reference_bytes(search):
+    # mxfp4::quantize / quantize_naive (src/mxfp4.rs:38-138)
+    from microkimi_amd import mxfp4
+    rows, cols = 48, 256
+    w = _quantizer_inputs(rows, cols, 21)
+    wp, ws = oracle.mxfp4_quantize(w, rows, cols, search=search)
+    gp, gs = mxfp4.quantize(dev(w), search=search)
+    assert np.array_equal(gs.cpu().numpy(), ws)
+    assert np.array_equal(gp.cpu().numpy(), wp)
+    if search:  # the search moves some scales (else this case tests nothing beyond the naive one)
+        assert (ws != oracle.mxfp4_quantize(w, rows, cols, search=False)[1]).any()
+    # round trip through the device decoder (the rows of random values): inside the clamp the error is at most half the
+    # widest level step, 2^e
+    back = mxfp4.dequant(gp, gs, rows, cols).cpu().numpy()[5:]
+    step = np.exp2(gs.cpu().numpy()[5:].astype(np.float64) - 127.0).repeat(32, axis=1)
+    inside = np.abs(w[5:]) <= 6.0 * step
+    assert inside.mean() > 0.9 and np.all(np.abs(back.astype(np.float64) - w[5:])[inside] <= step[inside])
+
+
+def test_quantize_fp8_gives_the_reference_bytes():
+    # dequant::quantize_fp8 (src/dequant.rs:50-74)
+    from microkimi_amd import dequant
+    rows, cols = 256, 384
+    rng = np.random.default_rng(22)
+    w = rng.standard_normal((rows, cols)).astype(np.float32)
+    w[:128, :128] = 0.0                                          # a zero block: exponent byte 0
+    w[:128, 128:256] *= np.float32(1e6)                          # clamp of the exponent at 8: codes saturate at 448
+    w[128:, :128] *= np.float32(1e-30)
+    w[128, 128] = 448.0                                          # block maximum / 448 an exact power of two
+    w[128:, 128:256] = np.clip(w[128:, 128:256], -400, 400)
+    w[128, 128] = 448.0
+    wq, wsc = oracle.quantize_fp8(w, rows, cols)
+    gq, gsc = dequant.quantize_fp8(dev(w))
+    assert np.array_equal(gsc.cpu().numpy(), wsc)
+    assert np.array_equal(gq.cpu().numpy(), wq)
+    assert wsc[0, 0] == 0 and wsc[0, 1] == 135 and wsc[1, 1] == 127

@@ -134,3 +134,65 @@ def test_shapes_the_kernels_do_not_cover_are_refused():
     assert lib.mk_mla_cache_new_heads(4, 128, 64, 1024, 8, C.byref(h)) == -1   # V rows wider than the kernel holds
     assert lib.mk_mla_cache_new(4, 512, 0, 8, C.byref(h)) == -1                # the shared-latent cache needs a rope row
     assert lib.mk_mla_cache_new(4, 96, 64, 8, C.byref(h)) == -1                # latent width the decode kernel rejects
+
+
+@pytest.mark.parametrize("n,nh,nope,rope,vd,applies", [(37, 4, 128, 64, 128, True), (70, 3, 64, 32, 192, True), (300, 6, 128, 64, 128, True),
+                                                     (20, 3, 96, 32, 128, False)])
+def test_hadamard_option(n, nh, nope, rope, vd, applies):
+    # kv_hadamard (src/model.rs:1529-1554): rotated cache bytes, to_f32 and attention against the oracle in the same
+    # mode; widths that are not whole 64-chunks leave the option without effect, as in the reference
+    from microkimi_amd import model
+    k, v = rows(n, nh, nope, rope, vd, 300 + n)
+    k[0, :64] = 0.0
+    rng = np.random.default_rng(n)
+    q = rng.standard_normal(nh * (nope + rope)).astype(np.float32)
+    scale = float(np.float32(nope + rope) ** np.float32(-0.5))
+    want = oracle.MlaCache(nh, nope, rope, vd, had=True, capacity=n)
+    for j in range(n):
+        want.push(k[j], v[j])
+    c = model.MlaHeadsCache(nh, nope, rope, vd, n, hadamard=True)
+    c.push(dev(k), dev(v))
+    assert np.array_equal(c.kq[:n].cpu().numpy(), want.kq[:n]) and np.array_equal(c.vq[:n].cpu().numpy(), want.vq[:n])
+    assert np.array_equal(c.ks[:n].cpu().numpy().view(np.uint32), want.ks[:n].view(np.uint32))
+    assert np.array_equal(c.vs[:n].cpu().numpy().view(np.uint32), want.vs[:n].view(np.uint32))
+    plain = oracle_cache(k, v, nh, nope, rope, vd)
+    assert np.array_equal(want.kq[:n], plain.kq[:n]) != applies      # the rotation changes the bytes exactly when it applies
+    kf, vf = c.to_f32()
+    wk, wv = want.to_f32()
+    assert np.array_equal(kf.cpu().numpy().view(np.uint32), wk.view(np.uint32))
+    assert np.array_equal(vf.cpu().numpy().view(np.uint32), wv.view(np.uint32))
+    for pos in sorted({n - 1, n // 2}):
+        got = c.attn(dev(q), pos, scale).cpu().numpy()[0]
+        assert rel_l2(got, oracle.mla_attn_flash_q8_mqa(want, q, pos, scale)) <= TOL
+    m = min(5, n)
+    qs = rng.standard_normal((m, nh * (nope + rope))).astype(np.float32)
+    got = c.attn(dev(qs), n - m, scale).cpu().numpy()
+    for i in range(m):
+        assert rel_l2(got[i], oracle.mla_attn_flash_q8_mqa(want, qs[i], n - m + i, scale)) <= TOL
+
+
+def test_host_level_hadamard_switch():
+    torch_cuda()
+    from microkimi_amd._lib import check, hptr, lib
+    nh, nope, rope, vd, n = 4, 128, 64, 128, 12
+    k, v = rows(n, nh, nope, rope, vd, 11)
+    want = oracle.MlaCache(nh, nope, rope, vd, had=True, capacity=n)
+    for j in range(n):
+        want.push(k[j], v[j])
+    q = np.random.default_rng(12).standard_normal(nh * (nope + rope)).astype(np.float32)
+    scale = float(np.float32(nope + rope) ** np.float32(-0.5))
+    h = C.c_void_p()
+    check(lib.mk_mla_cache_new_heads(nh, nope, rope, vd, n, C.byref(h)))
+    try:
+        check(lib.mk_mla_cache_set_hadamard(h, 1))
+        check(lib.mk_mla_cache_assign_f32(h, hptr(k), hptr(v), n))
+        assert lib.mk_mla_cache_set_hadamard(h, 0) == -1              # not while positions are held
+        kf, vf = np.empty_like(k), np.empty_like(v)
+        check(lib.mk_mla_cache_to_f32(h, hptr(kf), hptr(vf)))
+        wk, wv = want.to_f32()
+        assert np.array_equal(kf.view(np.uint32), wk.view(np.uint32)) and np.array_equal(vf.view(np.uint32), wv.view(np.uint32))
+        out = np.empty(nh * vd, np.float32)
+        check(lib.mk_mla_attn(h, hptr(q), scale, hptr(out)))
+        assert rel_l2(out, oracle.mla_attn_flash_q8_mqa(want, q, n - 1, scale)) <= TOL
+    finally:
+        lib.mk_mla_cache_free(h)
