@@ -180,10 +180,16 @@ typedef struct {
     const uint8_t *const *w2p, *const *w2s;
     size_t d, inter;
     size_t n_experts;
+    /* A layer with VQ1 ("cold") experts (src/model.rs:729-730, 2243-2257): the file's global 256 x 16 f32 codebook on the
+     * device, or NULL when every expert is MXFP4.  A VQ1 expert has its index bytes ([rows][cols/16]) where the packed
+     * nibbles would be (w1p, w3p, w2p) and NULL scale pointers (w1s, w3s, w2s). */
+    const float *vq_codebook;
 } mk_expert_table;
 
 /* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
 size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
+/* Further bytes, directly behind those, when the table has a vq_codebook (the LUT GEMV's tables). */
+size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
 
 /* The expert section of moe_forward / ds_moe for B decode tokens in one grouped
  * pass (src/model.rs:2227-2264,2346-2351; src/deepseek.rs:1069-1106):
@@ -193,7 +199,9 @@ size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size
  *         + o(shared expert)    when shared >= 0, unweighted.
  * ids [B][topk] int32, weights [B][topk] f32, x [B][d], out [B][d]; all device.
  * mode MK_MODE_Q8 re-quantizes x and act per 32 exactly as matvec_packed does on
- * each call. */
+ * each call.  A selected expert that is VQ1 (table->vq_codebook set, NULL scale pointers) takes quant::matvec_vq
+ * (src/quant.rs:333-346) for its three products, on the f32 hidden and activation rows, whatever `mode` says
+ * (src/model.rs:2243-2257); the workspace then also holds mk_moe_decode_vq_workspace_bytes. */
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
 
@@ -415,9 +423,11 @@ typedef struct mk_expert_set mk_expert_set;
  * "<layer_prefix>block_sparse_moe.experts.<e>.w1|w2|w3" for e < n_experts (the names resolved in
  * src/model.rs:979-989), each MXFP4 blob copied as stored (256-byte aligned; scales = packed +
  * R*C/2), plus the device pointer arrays of an mk_expert_table.  w1 of expert 0 fixes
- * [inter, d]; every other tensor is checked against it.  Experts of another dtype (VQ1,
- * MXFP4SQ) give MK_ERR_UNSUPPORTED: such a layer stays on the caller's CPU path, as dtype 3/4
- * blobs do for the reference's GPU entry points.  This replaces the pointer-keyed upload cache
+ * [inter, d]; every other tensor is checked against it.  An expert stored as VQ1 (dtype 3, `slice --cold-vq`; its kind
+ * is taken from w1 as in src/model.rs:988-990, w2 and w3 must agree) keeps its index bytes and a NULL scale pointer, and
+ * the file's global "vq_codebook" (256 x 16 f32, src/model.rs:995-999) is uploaded with the set: table->vq_codebook.
+ * MXFP4SQ experts (dtype 4) give MK_ERR_UNSUPPORTED: a storage format the runtime matvec does not read
+ * (src/mxfp4.rs:150-151); such a layer stays on the caller's CPU path.  This replaces the pointer-keyed upload cache
  * of src/metal.rs:874-936 for callers that load whole layers. */
 int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix, size_t n_experts, mk_expert_set **out);
 const mk_expert_table *mk_expert_set_table(const mk_expert_set *s);

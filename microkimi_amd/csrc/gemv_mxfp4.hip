@@ -70,6 +70,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_q8_kernel(GemvArgs a) {
     // uniform pointers in scalar registers + 32-bit lane offsets: the loads take the scalar-base form
     const uint8_t *packed = mk_uniform_ptr(a.packed ? a.packed : a.packed_ptrs[mat]);
     const uint8_t *scales = mk_uniform_ptr(a.packed ? a.scales : a.scales_ptrs[mat]);
+    if (!scales) return;  // a matrix without scale bytes is not MXFP4 (a VQ1 expert of a mixed layer): not this kernel's
     float *out = a.packed ? a.out : a.out_ptrs[mat];
     const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
     const int8_t *xq = a.xq + (size_t)xi * NB * 32;
@@ -191,6 +192,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_f32_kernel(GemvArgs a) {
     const int mat = blockIdx.y;
     const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
     const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    if (!scales) return;  // (see the q8 kernel)
     float *out = a.packed ? a.out : a.out_ptrs[mat];
     const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
     const float *xf = a.xf + (size_t)xi * NB * 32;
@@ -260,6 +262,7 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_generic_kernel(GemvArgs a, int
     const int mat = blockIdx.y;
     const uint8_t *packed = a.packed ? a.packed : a.packed_ptrs[mat];
     const uint8_t *scales = a.packed ? a.scales : a.scales_ptrs[mat];
+    if (!scales) return;  // (see the q8 kernel)
     float *out = a.packed ? a.out : a.out_ptrs[mat];
     const int xi = (a.packed || !a.x_index) ? 0 : a.x_index[mat];
     const int lane = threadIdx.x & 63;

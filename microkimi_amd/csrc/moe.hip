@@ -23,6 +23,13 @@ int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const u
                              size_t cols, const int8_t *xq, const float *xs, const float *xf, const int32_t *x_index, float *const *out_ptrs,
                              hipStream_t st);
 
+// grouped VQ1 LUT GEMV of vq1.hip: tables for n_vec activation vectors, then the sweep over the matrices whose marker
+// pointer is null
+int mk_vq1_grouped_tables(const float *codebook, const float *x, size_t n_vec, size_t cols, const uint8_t *const *marker_ptrs, float *lut,
+                          hipStream_t st);
+int mk_vq1_grouped_sweep(const float *lut, const int32_t *vec_index, const uint8_t *const *idx_ptrs, const uint8_t *const *marker_ptrs,
+                         size_t n_mat, size_t rows, size_t cols, float *const *out_ptrs, hipStream_t st);
+
 int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t rows, size_t cols,
                    const int8_t *xq, const float *xs, const int32_t *arow, const int32_t *goff, const int32_t *gexp, const int32_t *ngroups,
                    const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream);
@@ -713,6 +720,12 @@ extern "C" size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_s
     return carve(nullptr, B, topk, has_shared, d, inter).bytes;
 }
 
+// behind it when the table holds VQ1 experts: the tables of the hidden rows, then those of the activation rows
+extern "C" size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter) {
+    const size_t P = B * (topk + (has_shared ? 1 : 0));
+    return align_up(B * (d / 16) * 256 * sizeof(float), 256) + align_up(P * (inter / 16) * 256 * sizeof(float), 256);
+}
+
 namespace {
 
 template <int NB>
@@ -808,8 +821,13 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
     const bool fast = mode == MK_MODE_Q8 && (nb == 32 || nb == 64 || nb == 128 || nb == 224) && (nbi == 32 || nbi == 64 || nbi == 128) &&
                       per <= MAX_PER && d % 2 == 0 && (size_t)per * nbi * 68 <= 150 * 1024;
     int s;
+    // A layer with VQ1 experts (src/model.rs:2243-2257) takes the composed kernels: which pairs are VQ1 is known on the
+    // device only, so both kinds of launch run over all pairs and each skips the other kind's.
+    const bool has_vq = table->vq_codebook != nullptr;
+    float *lut_x = reinterpret_cast<float *>((uint8_t *)workspace + w.bytes);
+    float *lut_a = reinterpret_cast<float *>((uint8_t *)lut_x + align_up(B * (d / 16) * 256 * sizeof(float), 256));
     // batched path: q8 mode, both projections in K tiles of 512, enough tokens for experts to repeat
-    const bool batched = mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
+    const bool batched = !has_vq && mode == MK_MODE_Q8 && d % 512 == 0 && inter % 512 == 0 && P <= (size_t)BATCHED_MAX_P &&
                          (int)B >= MK_TUNE("MK_MOE_BATCHED_MIN", 4) && inter * (d / 2) < 0xFFFFFFFFull && P * d < 0xFFFFFFFFull;
     if (batched) {
         {
@@ -845,7 +863,7 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         return mk_launch_status("moe_combine_grouped");
     }
     float *af = stage == STAGE_ALL ? w.af : act_io;  // [P][inter] activation rows in (token, slot) order
-    if (fast) {
+    if (fast && !has_vq) {
         FusedArgs fa;
         fa.tab = *table;
         fa.ids = ids;
@@ -887,6 +905,11 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         if (q8 && (s = mk_dev_quantize_q8(x, B, d, w.xq, w.xs, stream)) != MK_OK) return s;
         if ((s = mk_gemv_grouped_internal(q8, w.pt.w1p, w.pt.w1s, P, inter, d, w.xq, w.xs, x, w.pt.xidx, w.pt.gptr, st)) != MK_OK) return s;
         if ((s = mk_gemv_grouped_internal(q8, w.pt.w3p, w.pt.w3s, P, inter, d, w.xq, w.xs, x, w.pt.xidx, w.pt.uptr, st)) != MK_OK) return s;
+        if (has_vq) {  // quant::matvec_vq on the f32 hidden row (no q8 step for VQ1 experts)
+            if ((s = mk_vq1_grouped_tables(table->vq_codebook, x, B, d, nullptr, lut_x, st)) != MK_OK) return s;
+            if ((s = mk_vq1_grouped_sweep(lut_x, w.pt.xidx, w.pt.w1p, w.pt.w1s, P, inter, d, w.pt.gptr, st)) != MK_OK) return s;
+            if ((s = mk_vq1_grouped_sweep(lut_x, w.pt.xidx, w.pt.w3p, w.pt.w3s, P, inter, d, w.pt.uptr, st)) != MK_OK) return s;
+        }
         const int n = (int)(P * inter);
         hipLaunchKernelGGL(moe_act_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.pt.pw, (int)inter, n, act_kind, limit,
                            af);
@@ -894,6 +917,10 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
     }
     if (q8 && (s = mk_dev_quantize_q8(af, P, inter, w.aq, w.as, stream)) != MK_OK) return s;
     if ((s = mk_gemv_grouped_internal(q8, w.pt.w2p, w.pt.w2s, P, d, inter, w.aq, w.as, af, w.pt.aidx, w.pt.optr, st)) != MK_OK) return s;
+    if (has_vq) {
+        if ((s = mk_vq1_grouped_tables(table->vq_codebook, af, P, inter, w.pt.w2s, lut_a, st)) != MK_OK) return s;
+        if ((s = mk_vq1_grouped_sweep(lut_a, nullptr, w.pt.w2p, w.pt.w2s, P, d, inter, w.pt.optr, st)) != MK_OK) return s;
+    }
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((d + 255) / 256), (unsigned)B), dim3(256), 0, st, w.o, w.pt.pw, per, (int)topk, (int)d,
                        act_kind == MK_ACT_DS ? 1 : 0, out);
     return mk_launch_status("moe_combine");

@@ -232,6 +232,10 @@ extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts
                                   const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
     MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
     MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
+    if (table->vq_codebook) {  // quant::matvec_vq_nt experts (src/model.rs:2556-2566): mk_dev_vq1_matvec_nt per expert, not this call
+        mk_set_error("mk_dev_moe_prefill reads MXFP4 experts only; this layer holds VQ1 experts");
+        return MK_ERR_UNSUPPORTED;
+    }
     const size_t d = table->d, inter = table->inter;
     MK_REQUIRE(d % 128 == 0 && inter % 128 == 0 && d > 0 && inter > 0, "d and inter must be positive multiples of 128");
     MK_REQUIRE(n_experts >= 1 && n_experts <= 960 && T >= 1 && topk >= 1 && T <= 65535, "bad token / expert count");

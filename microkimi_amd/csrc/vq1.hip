@@ -77,6 +77,56 @@ __global__ __launch_bounds__(64) void vq1_sweep_exact_kernel(const float *__rest
     out[r] = a;
 }
 
+// Grouped forms for a MoE layer with VQ1 experts (src/model.rs:2243-2257): matrix p of a launch is the index bytes
+// idx_ptrs[p]; it belongs to this path when marker_ptrs[p] is null (an MXFP4 matrix has its scale bytes there).
+// tables: vector v of `x` (n_vec x cols) -> lut + v * (cols / 16) * 256; sweep: matrix p reads the table of vector
+// vec_index[p] (p itself when vec_index is null).
+__global__ __launch_bounds__(256) void vq1_table_grouped_kernel(const float *__restrict__ codebook, const float *__restrict__ x, int cols,
+                                                                const uint8_t *const *__restrict__ marker_ptrs, float *__restrict__ lut) {
+    __shared__ float xs[16];
+    const int g = blockIdx.x, v = blockIdx.y, k = threadIdx.x;
+    if (marker_ptrs && marker_ptrs[v]) return;
+    if (k < 16) xs[k] = x[(size_t)v * cols + g * 16 + k];
+    __syncthreads();
+    const mk_f4 *cb = reinterpret_cast<const mk_f4 *>(codebook + k * 16);
+    float s = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const mk_f4 c = cb[q];
+        s = mk_add(s, mk_mul(c.x, xs[q * 4 + 0]));
+        s = mk_add(s, mk_mul(c.y, xs[q * 4 + 1]));
+        s = mk_add(s, mk_mul(c.z, xs[q * 4 + 2]));
+        s = mk_add(s, mk_mul(c.w, xs[q * 4 + 3]));
+    }
+    lut[((size_t)v * (cols / 16) + g) * 256 + k] = s;
+}
+
+__global__ __launch_bounds__(256) void vq1_sweep_grouped_kernel(const float *__restrict__ lut, const int32_t *__restrict__ vec_index,
+                                                                const uint8_t *const *__restrict__ idx_ptrs,
+                                                                const uint8_t *const *__restrict__ marker_ptrs, int rows, int vpr,
+                                                                float *const *__restrict__ out_ptrs) {
+    const int p = blockIdx.y;
+    if (marker_ptrs[p]) return;
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;  // whole waves leave together
+    const float *tab = lut + (size_t)(vec_index ? vec_index[p] : p) * vpr * 256;
+    const uint8_t *ir = idx_ptrs[p] + (size_t)r * vpr;
+    float a = 0.0f;
+    for (int g0 = 0; g0 < vpr; g0 += 256) {  // four gathers in flight per lane
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int g = g0 + i * 64 + lane;
+            v[i] = g < vpr ? tab[g * 256 + ir[g]] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) a += v[i];
+    }
+    a = mk_wave_sum(a);
+    if (lane == 0) out_ptrs[p][r] = a;
+}
+
 // quant::matvec_vq_nt (src/quant.rs:353-376): m positions at once, every product added to its position's running sum in
 // (vector, j) order -- one sequential chain of cols multiply-adds per (row, position), not the per-vector partial sums of
 // matvec_vq.  A lane owns a row and 8 positions (the reference's block of 8): the codebook entry is gathered from LDS
@@ -147,6 +197,22 @@ extern "C" int mk_dev_vq1_matvec_nt(const float *codebook, const uint8_t *indice
     else
         hipLaunchKernelGGL(vq1_nt_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, codebook, indices, (int)rows, (int)(cols / 16), xt, (int)m, out);
     return mk_launch_status("vq1_nt");
+}
+
+int mk_vq1_grouped_tables(const float *codebook, const float *x, size_t n_vec, size_t cols, const uint8_t *const *marker_ptrs, float *lut,
+                          hipStream_t st) {
+    if (n_vec == 0) return MK_OK;
+    hipLaunchKernelGGL(vq1_table_grouped_kernel, dim3((unsigned)(cols / 16), (unsigned)n_vec), dim3(256), 0, st, codebook, x, (int)cols, marker_ptrs,
+                       lut);
+    return mk_launch_status("vq1_table_grouped");
+}
+
+int mk_vq1_grouped_sweep(const float *lut, const int32_t *vec_index, const uint8_t *const *idx_ptrs, const uint8_t *const *marker_ptrs,
+                         size_t n_mat, size_t rows, size_t cols, float *const *out_ptrs, hipStream_t st) {
+    if (n_mat == 0 || rows == 0) return MK_OK;
+    hipLaunchKernelGGL(vq1_sweep_grouped_kernel, dim3((unsigned)((rows + 3) / 4), (unsigned)n_mat), dim3(256), 0, st, lut, vec_index, idx_ptrs,
+                       marker_ptrs, (int)rows, (int)(cols / 16), out_ptrs);
+    return mk_launch_status("vq1_sweep_grouped");
 }
 
 extern "C" size_t mk_vq1_workspace_bytes(size_t cols) { return cols / 16 * 256 * sizeof(float); }

@@ -223,16 +223,25 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
         size_t size, half, dev_off;
     };
     std::vector<Blob> blobs(3 * n_experts);
+    std::vector<char> vq(n_experts, 0);
+    bool any_vq = false;
     size_t d = 0, inter = 0, off = 0;
     for (size_t e = 0; e < n_experts; e++) {
         for (int k = 0; k < 3; k++) {
             const std::string name = std::string(layer_prefix) + "block_sparse_moe.experts." + std::to_string(e) + "." + kind[k];
             mk_bin_entry en;
             if ((rc = mk_bin_find(f, name.c_str(), &en)) != MK_OK) return rc;
-            if (en.dtype != MK_DTYPE_MXFP4) {
-                // VQ1 and MXFP4SQ experts have no device kernel: the caller keeps such a layer on its CPU path
-                mk_set_error("%s has dtype %d; the device path reads mxfp4 (1) only", name.c_str(), (int)en.dtype);
+            if (en.dtype != MK_DTYPE_MXFP4 && en.dtype != MK_DTYPE_VQ1) {
+                // MXFP4SQ experts have no device kernel (storage format only, src/mxfp4.rs:150-151)
+                mk_set_error("%s has dtype %d; the device path reads mxfp4 (1) and vq1 (3)", name.c_str(), (int)en.dtype);
                 return MK_ERR_UNSUPPORTED;
+            }
+            if (k == 0) {
+                vq[e] = en.dtype == MK_DTYPE_VQ1;  // the reference takes the expert's kind from w1 (src/model.rs:988-990)
+                any_vq |= vq[e];
+            } else if ((en.dtype == MK_DTYPE_VQ1) != vq[e]) {
+                mk_set_error("%s: dtype %d differs from the expert's w1", name.c_str(), (int)en.dtype);
+                return MK_ERR_INVALID;
             }
             const size_t r = en.dims[0], c = en.dims[1];
             if (e == 0 && k == 0) {  // w1 of the first expert fixes the layer's shapes: w1, w3 [inter, d], w2 [d, inter]
@@ -248,9 +257,23 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
                 mk_set_error("%s: columns must be a multiple of 32", name.c_str());
                 return MK_ERR_INVALID;
             }
-            blobs[e * 3 + k] = {f->data + en.offset, (size_t)en.size, r * c / 2, off};
+            blobs[e * 3 + k] = {f->data + en.offset, (size_t)en.size, vq[e] ? 0 : r * c / 2, off};
             off = align_up(off + (size_t)en.size, 256);
         }
+    }
+    // one global codebook shared by every VQ1 tensor of the file (src/model.rs:995-999)
+    const uint8_t *cb_host = nullptr;
+    size_t cb_off = 0;
+    if (any_vq) {
+        mk_bin_entry en;
+        if ((rc = mk_bin_find(f, "vq_codebook", &en)) != MK_OK) return rc;
+        if (en.dtype != MK_DTYPE_F32 || en.size != 256 * 16 * sizeof(float)) {
+            mk_set_error("vq_codebook: bad dims (want 256 x 16 f32)");
+            return MK_ERR_INVALID;
+        }
+        cb_host = f->data + en.offset;
+        cb_off = off;
+        off = align_up(off + (size_t)en.size, 256);
     }
     const size_t tab_off = off, total = off + 6 * n_experts * sizeof(void *);
     mk_expert_set *s = new mk_expert_set;
@@ -274,9 +297,15 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
                 mk_set_error("upload of expert %zu failed", e);
                 return MK_ERR_HIP;
             }
-            ptrs[(size_t)(2 * k) * n_experts + e] = base + b.dev_off;               // packed
-            ptrs[(size_t)(2 * k + 1) * n_experts + e] = base + b.dev_off + b.half;  // scales
+            ptrs[(size_t)(2 * k) * n_experts + e] = base + b.dev_off;                                  // packed nibbles, or VQ1 index bytes
+            ptrs[(size_t)(2 * k + 1) * n_experts + e] = vq[e] ? nullptr : base + b.dev_off + b.half;  // scales (none: VQ1)
         }
+    }
+    if (cb_host && hipMemcpy(base + cb_off, cb_host, 256 * 16 * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        mk_expert_set_free(s);
+        mk_set_error("upload of the VQ codebook failed");
+        return MK_ERR_HIP;
     }
     if (hipMemcpy(base + tab_off, ptrs.data(), ptrs.size() * sizeof(void *), hipMemcpyHostToDevice) != hipSuccess) {
         (void)hipGetLastError();
@@ -294,6 +323,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->table.d = d;
     s->table.inter = inter;
     s->table.n_experts = n_experts;
+    s->table.vq_codebook = any_vq ? reinterpret_cast<const float *>(base + cb_off) : nullptr;
     *out = s;
     return MK_OK;
 }

@@ -196,16 +196,20 @@ class MlaHeadsCache:
 
 class PackedExperts:
     """Expert table of an MoE layer on the device: per expert w1, w3 [inter, d] and w2 [d, inter], each MXFP4
-    (packed, scales) in the reference layout.  Built from lists of device tensors."""
+    (packed, scales) in the reference layout, or -- a VQ1 expert (src/model.rs:729-730) -- (index bytes, None) with
+    the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors."""
 
-    def __init__(self, w1, w3, w2, d, inter):
+    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None):
         import torch
         self.d, self.inter, self.n = d, inter, len(w1)
-        self._keep = (w1, w3, w2)
+        self._keep = (w1, w3, w2, vq_codebook)
         dev = w1[0][0].device
-        arr = lambda lst, k: torch.tensor([t[k].data_ptr() for t in lst], dtype=torch.int64, device=dev)
+        arr = lambda lst, k: torch.tensor([t[k].data_ptr() if t[k] is not None else 0 for t in lst], dtype=torch.int64, device=dev)
         self._ptrs = [arr(w1, 0), arr(w1, 1), arr(w3, 0), arr(w3, 1), arr(w2, 0), arr(w2, 1)]
-        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n)
+        self.has_vq = vq_codebook is not None
+        if any(t[1] is None for lst in (w1, w3, w2) for t in lst) and not self.has_vq:
+            raise ValueError("a VQ1 expert needs the codebook")
+        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None)
         self._ws = None
 
 
@@ -216,7 +220,7 @@ def moe_decode(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_S
     import torch
     _lib.require_device()
     B, topk = ids.shape
-    need = lib.mk_moe_decode_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    need = _moe_ws_bytes(experts, B, topk, shared)
     if experts._ws is None or experts._ws.numel() < need:
         experts._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     if out is None:
@@ -226,9 +230,16 @@ def moe_decode(experts, ids, weights, x, shared=-1, mode=MODE_Q8, act_kind=ACT_S
     return out
 
 
+def _moe_ws_bytes(experts, B, topk, shared):
+    need = lib.mk_moe_decode_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    if getattr(experts, "has_vq", False):
+        need += lib.mk_moe_decode_vq_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    return need
+
+
 def _moe_ws(experts, B, topk, shared, device):
     import torch
-    need = lib.mk_moe_decode_workspace_bytes(B, topk, int(shared >= 0), experts.d, experts.inter)
+    need = _moe_ws_bytes(experts, B, topk, shared)
     if experts._ws is None or experts._ws.numel() < need:
         experts._ws = torch.empty(need, dtype=torch.uint8, device=device)
     return experts._ws

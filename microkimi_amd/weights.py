@@ -30,6 +30,7 @@ class DeviceExperts:
         t = lib.mk_expert_set_table(handle).contents
         self.table = t
         self.d, self.inter = int(t.d), int(t.inter)
+        self.has_vq = bool(t.vq_codebook)  # VQ1 experts among them (dtype 3): the file's codebook came along
         self.n = int(lib.mk_expert_set_count(handle))
         self.bytes = int(lib.mk_expert_set_bytes(handle))
         self._ws = None

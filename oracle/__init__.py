@@ -103,6 +103,7 @@ _lib.orc_router_softmax.argtypes = [_f32p, _sz, _sz, _u32p, _f32p]
 _lib.orc_expert_forward_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _sz, _sz, C.c_float, _f32p]
 _PP = C.POINTER(_u8p)
 _lib.orc_expert_packed.argtypes = [_u8p, _u8p, _u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+_lib.orc_expert_vq.argtypes = [_f32p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_float, C.c_float, _f32p]
 _lib.orc_expert_act.argtypes = [_u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
 _lib.orc_moe_decode.argtypes = [_PP, _PP, _PP, _PP, _PP, _PP, _sz, _sz, _sz, _sz, _u32p, _f32p, C.c_int, _f32p, C.c_int, C.c_int,
                                 C.c_float, _sz, _f32p]
@@ -517,6 +518,46 @@ def expert_act(w1, w3, d, inter, x, mode=1, act_kind=ACT_SWIGLU, limit=0.0, wgt=
     _lib.orc_expert_act(_p(w1p, _u8p), _p(w1s, _u8p), _p(w3p, _u8p), _p(w3s, _u8p), d, inter, _p(x, _f32p), mode, act_kind, limit, wgt,
                         _p(act, _f32p))
     return act
+
+
+def expert_vq(codebook, i1, i3, i2, d, inter, x, act_kind=ACT_SWIGLU, limit=0.0, wgt=1.0):
+    """A VQ1 expert (src/model.rs:2243-2259, vq branch): three quant::matvec_vq calls with the activation between."""
+    codebook, x = _c(codebook, np.float32), _c(x, np.float32)
+    i1, i3, i2 = _c(i1, np.uint8), _c(i3, np.uint8), _c(i2, np.uint8)
+    assert codebook.size == 256 * 16 and i1.size == inter * d // 16 == i3.size == i2.size and x.size == d
+    out = np.empty(d, np.float32)
+    _lib.orc_expert_vq(_p(codebook, _f32p), _p(i1, _u8p), _p(i3, _u8p), _p(i2, _u8p), d, inter, _p(x, _f32p), act_kind, limit, wgt,
+                       _p(out, _f32p))
+    return out
+
+
+def moe_decode_mixed(experts, codebook, d, inter, ids, weights, x, shared=-1, mode=1, act_kind=ACT_SWIGLU, limit=0.0):
+    """moe_forward's expert section for a layer that mixes MXFP4 and VQ1 experts (src/model.rs:2227-2264, 2346-2351):
+    experts[e] = ("mxfp4", w1, w3, w2) with (packed, scales) pairs or ("vq1", i1, i3, i2) index bytes.  Per token the
+    outputs are added in slot order, weight times output (ACT_DS: the weight sits inside the activation), then the
+    shared expert unweighted."""
+    ids, weights, x = _c(ids, np.uint32), _c(weights, np.float32), _c(x, np.float32)
+    B, topk = ids.shape
+    out = np.empty((B, d), np.float32)
+
+    def run(e, xt, wgt):
+        ex = experts[e]
+        if ex[0] == "vq1":
+            return expert_vq(codebook, ex[1], ex[2], ex[3], d, inter, xt, act_kind, limit, wgt)
+        return expert_packed(ex[1], ex[2], ex[3], d, inter, xt, mode, act_kind, limit, wgt)
+
+    for t in range(B):
+        y = np.zeros(d, np.float32)
+        for s in range(topk):
+            w = np.float32(weights[t, s])
+            if act_kind == ACT_DS:
+                y = y + run(int(ids[t, s]), x[t], float(w))
+            else:
+                y = y + w * run(int(ids[t, s]), x[t], 1.0)
+        if shared >= 0:
+            y = y + run(shared, x[t], 1.0)
+        out[t] = y
+    return out
 
 
 def moe_decode(table, ids, weights, x, shared=-1, mode=1, act_kind=ACT_SWIGLU, limit=0.0, threads=1):

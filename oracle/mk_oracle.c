@@ -1138,6 +1138,32 @@ ORC_API void orc_expert_act(const uint8_t *w1p, const uint8_t *w1s, const uint8_
     free(u);
 }
 
+/* A VQ1 ("cold") expert on one input (src/model.rs:2243-2259, vq branch): quant::matvec_vq for W1 and W3 on the f32
+ * row, the activation, quant::matvec_vq for W2 on the f32 activation.  i1, i3: index bytes [inter][d/16]; i2: [d][inter/16]. */
+ORC_API void orc_expert_vq(const float *codebook, const uint8_t *i1, const uint8_t *i3, const uint8_t *i2, size_t d, size_t inter,
+                           const float *x, int act_kind, float limit, float wgt, float *out) {
+    float *a = (float *)malloc(sizeof(float) * inter);
+    float *u = (float *)malloc(sizeof(float) * inter);
+    float *act = (float *)malloc(sizeof(float) * inter);
+    orc_vq1_matvec_lut(codebook, i1, inter, d, x, a);
+    orc_vq1_matvec_lut(codebook, i3, inter, d, x, u);
+    for (size_t j = 0; j < inter; j++) {
+        if (act_kind == ORC_ACT_SITU) {
+            act[j] = orc_situ(a[j], u[j]);
+        } else if (act_kind == ORC_ACT_DS) {
+            float g = fminf(a[j], limit);
+            float uu = clampf(u[j], -limit, limit);
+            act[j] = wgt * (g / (1.0f + expf(-g))) * uu;
+        } else {
+            act[j] = (a[j] / (1.0f + expf(-a[j]))) * u[j];
+        }
+    }
+    orc_vq1_matvec_lut(codebook, i2, d, inter, act, out);
+    free(a);
+    free(u);
+    free(act);
+}
+
 /* One packed expert on one input: the three matvec_packed calls of
  * src/model.rs:2246-2259 / src/deepseek.rs:1080-1089.  w1,w3: [inter][d],
  * w2: [d][inter]; each as (packed, scales).  mode as orc_matvec_packed. */

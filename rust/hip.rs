@@ -45,6 +45,8 @@ pub struct MkExpertTable {
     pub d: usize,
     pub inter: usize,
     pub n_experts: usize,
+    /// the file's 256 x 16 f32 VQ codebook on the device, or null when every expert is MXFP4
+    pub vq_codebook: *const f32,
 }
 
 /// mk_bin_entry: one directory entry of an MKIM file (weights::Entry, src/weights.rs:31-37).
@@ -127,6 +129,7 @@ extern "C" {
     pub fn mk_dev_q8_matvec(q: *const i8, scales: *const c_void, scales_f16: c_int, rows: usize, cols: usize, xq: *const i8, xs: *const f32, batch: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_argmax(logits: *const f32, batch: usize, n: usize, ws: *mut c_void, out_idx: *mut i32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_q8head_from_f32(w: *const f32, rows: usize, cols: usize, q: *mut i8, scales: *mut c_void, scales_f16: c_int, stream: *mut c_void) -> c_int;
+    pub fn mk_moe_decode_vq_workspace_bytes(B: usize, topk: usize, has_shared: c_int, d: usize, inter: usize) -> usize;
     pub fn mk_moe_decode_workspace_bytes(B: usize, topk: usize, has_shared: c_int, d: usize, inter: usize) -> usize;
     pub fn mk_dev_moe_decode(table: *const MkExpertTable, B: usize, topk: usize, ids: *const i32, weights: *const f32, shared: c_int, x: *const f32, mode: c_int, act_kind: c_int, limit: f32, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_decode_act(table: *const MkExpertTable, B: usize, topk: usize, ids: *const i32, weights: *const f32, shared: c_int, x: *const f32, mode: c_int, act_kind: c_int, limit: f32, workspace: *mut c_void, act: *mut f32, stream: *mut c_void) -> c_int;

@@ -287,3 +287,54 @@ def test_full_layer_257_experts_sampled_tokens():
         got1 = model.moe_decode(experts, ids[tok:tok + 1].contiguous(), wts[tok:tok + 1].contiguous(), x[tok:tok + 1].contiguous(), shared=ne, mode=1).cpu().numpy()
         flips += rows_match_up_to_q8_flips(got1, want, lambda t: [w2[e] for e in used], d, inter)
     assert flips <= 8
+
+
+@pytest.mark.parametrize("d,inter,B,topk,shared,act,mode", [
+    (1024, 512, 1, 3, 5, 1, 0),      # SiTU (the rule of the model that stores cold experts as VQ1), shared expert VQ1, f32 mode
+    (1024, 512, 5, 3, 4, 1, 0),      # shared expert MXFP4
+    (2048, 1024, 3, 2, -1, 0, 0),    # SwiGLU, no shared expert
+    (1024, 512, 4, 3, 5, 2, 0),      # DeepSeek rule (weight inside the activation)
+    (1024, 512, 6, 3, 5, 1, 1),      # q8 mode: the MXFP4 experts quantize their inputs, the VQ1 experts do not
+])
+def test_layer_with_vq1_experts(d, inter, B, topk, shared, act, mode):
+    # moe_forward over a layer that mixes MXFP4 and VQ1 ("cold") experts (src/model.rs:2227-2264): experts 1, 3, 5 are VQ1
+    torch_cuda()
+    from microkimi_amd import model, workloads
+    n_experts = 6
+    rng = np.random.default_rng(d + B)
+    codebook = (rng.standard_normal((256, 16)) * 0.05).astype(np.float32)
+    host, devs = [], ([], [], [])
+    for e in range(n_experts):
+        if e % 2:
+            idx = [rng.integers(0, 256, (inter, d // 16), dtype=np.uint8), rng.integers(0, 256, (inter, d // 16), dtype=np.uint8),
+                   rng.integers(0, 256, (d, inter // 16), dtype=np.uint8)]
+            host.append(("vq1", idx[0], idx[1], idx[2]))
+            for k in range(3):
+                devs[k].append((dev(idx[k]), None))
+        else:
+            m = [workloads.mxfp4_matrix(2, "w1", inter, d, e), workloads.mxfp4_matrix(2, "w3", inter, d, e),
+                 workloads.mxfp4_matrix(2, "w2", d, inter, e)]
+            host.append(("mxfp4", m[0], m[1], m[2]))
+            for k in range(3):
+                devs[k].append((dev(m[k][0]), dev(m[k][1])))
+    experts = model.PackedExperts(devs[0], devs[1], devs[2], d, inter, vq_codebook=dev(codebook))
+    n_routed = n_experts - (1 if shared >= 0 else 0)
+    ids = np.stack([rng.permutation(n_routed)[:topk] for _ in range(B)]).astype(np.int32)
+    wts = rng.random((B, topk)).astype(np.float32)
+    wts /= wts.sum(axis=1, keepdims=True)
+    x = (rng.standard_normal((B, d)) * 0.05).astype(np.float32)
+    limit = 10.0 if act == 2 else 0.0
+    got = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=mode, act_kind=act, limit=limit).cpu().numpy()
+    want = oracle.moe_decode_mixed(host, codebook, d, inter, ids.astype(np.uint32), wts, x, shared=shared, mode=mode, act_kind=act, limit=limit)
+    assert np.isfinite(got).all() and np.isfinite(want).all()
+    if mode == 0:
+        for t in range(B):
+            assert rel_l2(got[t], want[t]) <= TOL, (t, rel_l2(got[t], want[t]))
+    else:
+        w2_dev = devs[2]
+        used = lambda t: [w2_dev[int(e)] for e in list(ids[t]) + ([shared] if shared >= 0 else []) if int(e) % 2 == 0]
+        rows_match_up_to_q8_flips(got, want, used, d, inter)
+    # the two stages compose to the same rows
+    act_rows = model.moe_decode_act(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=mode, act_kind=act, limit=limit)
+    again = model.moe_decode_from_act(experts, dev(ids), dev(wts), act_rows, shared=shared, mode=mode, act_kind=act).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32))

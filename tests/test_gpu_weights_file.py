@@ -9,12 +9,21 @@ from gpu_util import dev, rel_l2, torch_cuda
 pytestmark = pytest.mark.gpu
 
 
-def make_file(path, n_experts, d, inter, bad_dtype_at=None, bad_shape_at=None):
+def make_file(path, n_experts, d, inter, bad_dtype_at=None, bad_shape_at=None, vq_experts=(), codebook=None):
     from microkimi_amd import workloads
     rng = np.random.default_rng(7)
     tensors = [("model.embed_tokens.weight", W.F32, (16, d), rng.standard_normal((16, d)).astype(np.float32))]
+    if codebook is not None:
+        tensors.append(("vq_codebook", W.F32, (256, 16), codebook))
     host = []
     for e in range(n_experts):
+        if e in vq_experts:   # a cold expert: one index byte per 16 weights (src/weights.rs:49-55)
+            idx = {"w1": rng.integers(0, 256, (inter, d // 16), dtype=np.uint8), "w3": rng.integers(0, 256, (inter, d // 16), dtype=np.uint8),
+                   "w2": rng.integers(0, 256, (d, inter // 16), dtype=np.uint8)}
+            host.append(("vq1", idx["w1"], idx["w3"], idx["w2"]))
+            for k, dims in (("w1", (inter, d)), ("w2", (d, inter)), ("w3", (inter, d))):
+                tensors.append((f"layers.2.block_sparse_moe.experts.{e}.{k}", W.VQ1, dims, idx[k].tobytes()))
+            continue
         w1 = workloads.mxfp4_matrix(2, "w1", inter, d, e)
         w3 = workloads.mxfp4_matrix(2, "w3", inter, d, e)
         w2 = workloads.mxfp4_matrix(2, "w2", d, inter, e)
@@ -65,14 +74,46 @@ def test_loaded_experts_match_tables_built_from_tensors(tmp_path):
     f.close()
 
 
+def test_layer_with_vq1_experts_from_a_file(tmp_path):
+    # experts 1 and 4 stored as VQ1 (dtype 3) with the file's global vq_codebook (src/model.rs:979-999): the loaded table
+    # drives the layer like one built from tensors, and the oracle's mixed layer agrees
+    torch_cuda()
+    from microkimi_amd import model, weights
+    n, d, inter, B, topk = 6, 1024, 512, 4, 3
+    codebook = (np.random.default_rng(11).standard_normal((256, 16)) * 0.05).astype(np.float32)
+    host = make_file(tmp_path / "cold.bin", n, d, inter, vq_experts=(1, 4), codebook=codebook)
+    f = weights.BinFile.open(tmp_path / "cold.bin")
+    ex = f.load_experts("layers.2.", n)
+    assert ex.has_vq and (ex.n, ex.d, ex.inter) == (n, d, inter)
+    oracle_experts = [h if h[0] == "vq1" else ("mxfp4", h[0], h[1], h[2]) for h in host]
+    rng = np.random.default_rng(5)
+    ids = np.stack([rng.permutation(n - 1)[:topk] for _ in range(B)]).astype(np.int32)
+    wts = rng.random((B, topk)).astype(np.float32)
+    x = (rng.standard_normal((B, d)) * 0.05).astype(np.float32)
+    got = model.moe_decode(ex, dev(ids), dev(wts), dev(x), shared=n - 1, mode=0, act_kind=1).cpu().numpy()
+    want = oracle.moe_decode_mixed(oracle_experts, codebook, d, inter, ids.astype(np.uint32), wts, x, shared=n - 1, mode=0, act_kind=1)
+    for t in range(B):
+        assert rel_l2(got[t], want[t]) <= 1e-5
+    from microkimi_amd._lib import MkError
+    with pytest.raises(MkError) as e:   # the prefill call reads MXFP4 experts only
+        model.moe_prefill(ex, dev(ids), dev(wts), dev(x))
+    assert e.value.status == -4
+    ex.close()
+    f.close()
+
+
 def test_unsupported_dtype_and_shape_mismatch(tmp_path):
     torch_cuda()
     from microkimi_amd import weights
     from microkimi_amd._lib import MkError
-    make_file(tmp_path / "vq.bin", 3, 256, 128, bad_dtype_at=(1, "w3"))
+    make_file(tmp_path / "vq.bin", 3, 256, 128, bad_dtype_at=(1, "w3"))   # one tensor of an MXFP4 expert stored as VQ1
     with pytest.raises(MkError) as e:
         weights.BinFile.open(tmp_path / "vq.bin").load_experts("layers.2.", 3)
-    assert e.value.status == -4 and "dtype 3" in str(e.value)
+    assert e.value.status == -1 and "differs from the expert's w1" in str(e.value)
+    make_file(tmp_path / "nocb.bin", 3, 256, 128, vq_experts=(1,))        # VQ1 expert, but the file has no codebook
+    with pytest.raises(MkError) as e:
+        weights.BinFile.open(tmp_path / "nocb.bin").load_experts("layers.2.", 3)
+    assert "missing tensor" in str(e.value) and "vq_codebook" in str(e.value)
     make_file(tmp_path / "shape.bin", 3, 256, 128, bad_shape_at=(2, "w2"))
     with pytest.raises(MkError) as e:
         weights.BinFile.open(tmp_path / "shape.bin").load_experts("layers.2.", 3)

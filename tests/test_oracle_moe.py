@@ -136,3 +136,30 @@ def test_situ_values():
     for g, u in [(0.3, -1.2), (5.0, 40.0), (-3.0, 0.1)]:
         want = 4 * np.tanh(g / 4) / (1 + np.exp(-g)) * 25 * np.tanh(u / 25)
         assert abs(oracle.situ(g, u) - want) <= 1e-6 * max(1.0, abs(want))
+
+
+def test_mixed_layer_composition_is_the_layer_and_the_vq_expert_is_three_matvec_vq():
+    # oracle.moe_decode_mixed restates the combine of orc_moe_decode in numpy: on a layer without VQ1 experts the two
+    # must give the same bits; oracle.expert_vq is matvec_vq, the activation, matvec_vq (src/model.rs:2243-2259)
+    rng = np.random.default_rng(0)
+    d, inter, ne = 64, 64, 5
+    mat = lambda r, c: (rng.integers(0, 256, (r, c // 2), dtype=np.uint8), rng.integers(120, 130, (r, c // 32), dtype=np.uint8))
+    w1, w3, w2 = [mat(inter, d) for _ in range(ne)], [mat(inter, d) for _ in range(ne)], [mat(d, inter) for _ in range(ne)]
+    tab = oracle.ExpertTable(w1, w3, w2, d, inter)
+    ids = np.array([[0, 2], [3, 1], [2, 0]], np.uint32)
+    wts = rng.random((3, 2)).astype(np.float32)
+    x = rng.standard_normal((3, d)).astype(np.float32)
+    ex = [("mxfp4", w1[e], w3[e], w2[e]) for e in range(ne)]
+    for act, limit in ((0, 0.0), (1, 0.0), (2, 7.0)):
+        a = oracle.moe_decode(tab, ids, wts, x, shared=4, act_kind=act, limit=limit)
+        b = oracle.moe_decode_mixed(ex, None, d, inter, ids, wts, x, shared=4, act_kind=act, limit=limit)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    cb = (rng.standard_normal((256, 16)) * 0.1).astype(np.float32)
+    i1, i3 = rng.integers(0, 256, (inter, d // 16), dtype=np.uint8), rng.integers(0, 256, (inter, d // 16), dtype=np.uint8)
+    i2 = rng.integers(0, 256, (d, inter // 16), dtype=np.uint8)
+    g = oracle.vq1_matvec(cb, i1, inter, d, x[0], lut=False)
+    u = oracle.vq1_matvec(cb, i3, inter, d, x[0], lut=False)
+    act = (g / (np.float32(1.0) + np.exp(-g.astype(np.float64)).astype(np.float32))) * u   # silu(g) * u
+    want = oracle.vq1_matvec(cb, i2, d, inter, act.astype(np.float32), lut=False)
+    got = oracle.expert_vq(cb, i1, i3, i2, d, inter, x[0])
+    assert np.linalg.norm(got - want) <= 1e-6 * np.linalg.norm(want)
