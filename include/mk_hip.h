@@ -101,6 +101,18 @@ int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes,
  * w and packed 16-byte aligned. */
 int mk_dev_mxfp4_quantize(const float *w, size_t rows, size_t cols, int search, uint8_t *packed, uint8_t *scales, void *stream);
 
+/* MXFP4SQ, the quadratic-scale storage variant (src/mxfp4.rs:140-229; dtype 4 of the weight file): e2m1 nibbles and
+ * groups of 32 as MXFP4, the scale byte q decodes to ((q + 1) / 256)^2 * smax with smax = max over the tensor's groups
+ * of maxabs / 6 (the trailing f32 of a dtype-4 blob).
+ *   _quantize  mxfp4::quantize_sq: q = ceil(256 sqrt(ideal / smax)) - 1 clamped to 0..255 (rounded up: nothing clips);
+ *              smax is written to a device float.  The reference's bytes.
+ *   _dequant   mxfp4::dequant_sq, bit-exact; smax from the device float smax_dev, or, when that is NULL, the value
+ *              `smax`.  With a dtype-4 blob (packed || scales || smax) this is mxfp4::dequant_any's second branch.
+ * The runtime matvecs read MXFP4 only, as in the reference (src/mxfp4.rs:150-151). */
+int mk_dev_mxfp4sq_quantize(const float *w, size_t rows, size_t cols, uint8_t *packed, uint8_t *scales, float *smax, void *stream);
+int mk_dev_mxfp4sq_dequant(const uint8_t *packed, const uint8_t *scales, const float *smax_dev, float smax, size_t rows, size_t cols,
+                           float *out, void *stream);
+
 /* dequant::quantize_fp8 (src/dequant.rs:50-74): e4m3fn codes with one e8m0 scale per 128x128 block,
  * e = ceil(log2(maxabs / 448)) clamped to [-127, 8].  rows and cols multiples of 128; qw [rows][cols],
  * scales [rows/128][cols/128]: the reference's bytes. */

@@ -63,6 +63,8 @@ def _load():
         "mk_dev_quantize_mxfp8": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_mxfp4_quantize": (i32, [vp, sz, sz, i32, vp, vp, vp]),
         "mk_dev_quantize_fp8": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_mxfp4sq_quantize": (i32, [vp, sz, sz, vp, vp, vp, vp]),
+        "mk_dev_mxfp4sq_dequant": (i32, [vp, vp, vp, f32, sz, sz, vp, vp]),
         "mk_dev_mxfp4_matvec_q8": (i32, [vp, vp, sz, sz, vp, vp, vp, vp]),
         "mk_dev_mxfp4_matvec_f32": (i32, [vp, vp, sz, sz, vp, vp, vp]),
         "mk_dev_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp, i32, vp, vp, vp]),

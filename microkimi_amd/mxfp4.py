@@ -46,6 +46,46 @@ def quantize(w, search=True):
     return packed, scales
 
 
+def quantize_sq(w):
+    """mxfp4::quantize_sq (src/mxfp4.rs:160-214) of a device tensor [rows, cols] f32: (packed, scale bytes, smax as a
+    one-element device tensor)."""
+    import torch
+    _lib.require_device()
+    w = w.contiguous()
+    rows, cols = w.shape
+    if cols % 32:
+        raise ValueError("cols must be a multiple of 32")
+    packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+    scales = torch.empty((rows, cols // 32), dtype=torch.uint8, device=w.device)
+    smax = torch.empty(1, dtype=torch.float32, device=w.device)
+    check(lib.mk_dev_mxfp4sq_quantize(ptr(w), rows, cols, ptr(packed), ptr(scales), ptr(smax), cur_stream()))
+    return packed, scales, smax
+
+
+def dequant_sq(packed, scales, smax, rows, cols):
+    """mxfp4::dequant_sq (src/mxfp4.rs:216-229) on device tensors; smax a float or a one-element device tensor."""
+    import torch
+    _lib.require_device()
+    _check_shapes(packed, scales, rows, cols)
+    out = torch.empty((rows, cols), dtype=torch.float32, device=packed.device)
+    on_dev = isinstance(smax, torch.Tensor)
+    check(lib.mk_dev_mxfp4sq_dequant(ptr(packed), ptr(scales), ptr(smax) if on_dev else None, 0.0 if on_dev else float(smax), rows, cols,
+                                     ptr(out), cur_stream()))
+    return out
+
+
+def dequant_any(dtype, blob, rows, cols):
+    """mxfp4::dequant_any (src/mxfp4.rs:231-240) on a raw blob of either flavour (a uint8 device tensor): packed || scales
+    for dtype 1, packed || scales || smax (f32) for dtype 4."""
+    n_p, n_s = rows * cols // 2, rows * cols // 32
+    if dtype == 1:
+        return dequant(blob[:n_p].contiguous(), blob[n_p:n_p + n_s].contiguous(), rows, cols)
+    if dtype == 4:
+        smax = float(blob[n_p + n_s:n_p + n_s + 4].cpu().numpy().view(np.float32)[0])
+        return dequant_sq(blob[:n_p].contiguous(), blob[n_p:n_p + n_s].contiguous(), smax, rows, cols)
+    raise ValueError(f"dequant_any: dtype {dtype} is not an mxfp4 flavor")
+
+
 def quantize_naive(w):
     """mxfp4::quantize_naive (src/mxfp4.rs:94-100)."""
     return quantize(w, search=False)

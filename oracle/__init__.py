@@ -103,6 +103,11 @@ _lib.orc_router_softmax.argtypes = [_f32p, _sz, _sz, _u32p, _f32p]
 _lib.orc_expert_forward_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _sz, _sz, C.c_float, _f32p]
 _PP = C.POINTER(_u8p)
 _lib.orc_expert_packed.argtypes = [_u8p, _u8p, _u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+_lib.orc_scale_sq.argtypes = [C.c_uint8, C.c_float]
+_lib.orc_scale_sq.restype = C.c_float
+_lib.orc_mxfp4sq_quantize.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
+_lib.orc_mxfp4sq_quantize.restype = C.c_float
+_lib.orc_mxfp4sq_dequant.argtypes = [_u8p, _u8p, C.c_float, _sz, _sz, _f32p]
 _lib.orc_expert_vq.argtypes = [_f32p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_float, C.c_float, _f32p]
 _lib.orc_expert_act.argtypes = [_u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
 _lib.orc_moe_decode.argtypes = [_PP, _PP, _PP, _PP, _PP, _PP, _sz, _sz, _sz, _sz, _u32p, _f32p, C.c_int, _f32p, C.c_int, C.c_int,
@@ -164,6 +169,30 @@ def mxfp4_quantize(w, rows, cols, search=True):
     scales = np.zeros((rows, cols // 32), np.uint8)
     _lib.orc_mxfp4_quantize(_p(w, _f32p), rows, cols, int(search), _p(packed, _u8p), _p(scales, _u8p))
     return packed, scales
+
+
+def scale_sq(q, smax):
+    """mxfp4::scale_sq (src/mxfp4.rs:154-158)."""
+    return float(_lib.orc_scale_sq(int(q), float(smax)))
+
+
+def mxfp4sq_quantize(w, rows, cols):
+    """mxfp4::quantize_sq (src/mxfp4.rs:160-214): (packed, scale bytes, smax)."""
+    w = _c(w, np.float32)
+    assert cols % 32 == 0 and w.size == rows * cols
+    packed = np.zeros((rows, cols // 2), np.uint8)
+    scales = np.zeros((rows, cols // 32), np.uint8)
+    smax = _lib.orc_mxfp4sq_quantize(_p(w, _f32p), rows, cols, _p(packed, _u8p), _p(scales, _u8p))
+    return packed, scales, np.float32(smax)
+
+
+def mxfp4sq_dequant(packed, scales, smax, rows, cols):
+    """mxfp4::dequant_sq (src/mxfp4.rs:216-229)."""
+    packed, scales = _c(packed, np.uint8), _c(scales, np.uint8)
+    assert packed.size == rows * cols // 2 and scales.size == rows * cols // 32
+    out = np.empty((rows, cols), np.float32)
+    _lib.orc_mxfp4sq_dequant(_p(packed, _u8p), _p(scales, _u8p), float(smax), rows, cols, _p(out, _f32p))
+    return out
 
 
 def search_mx_scale(group, e):

@@ -161,6 +161,63 @@ ORC_API void orc_mxfp4_quantize(const float *w, size_t rows, size_t cols, int se
     }
 }
 
+/* ---- MXFP4SQ: quadratic scale byte against a per-tensor smax (src/mxfp4.rs:140-240) */
+
+/* src/mxfp4.rs:154-158 */
+ORC_API float orc_scale_sq(uint8_t q, float smax) {
+    float t = ((float)q + 1.0f) * (1.0f / 256.0f);
+    return t * t * smax;
+}
+
+/* src/mxfp4.rs:160-214: returns smax; packed [rows][cols/2], scales [rows][cols/32] */
+ORC_API float orc_mxfp4sq_quantize(const float *w, size_t rows, size_t cols, uint8_t *packed, uint8_t *scales) {
+    size_t ng = rows * cols / 32;
+    float *ideal = (float *)malloc(sizeof(float) * (ng ? ng : 1));
+    float smax = 0.0f;
+    for (size_t gi = 0; gi < ng; gi++) {
+        float maxabs = 0.0f;
+        for (int i = 0; i < 32; i++) maxabs = fmaxf(maxabs, fabsf(w[gi * 32 + i]));
+        ideal[gi] = maxabs / 6.0f;
+        smax = fmaxf(smax, ideal[gi]);
+    }
+    memset(packed, 0, rows * cols / 2);
+    for (size_t gi = 0; gi < ng; gi++) {
+        int q = 0;
+        if (!(smax == 0.0f || ideal[gi] == 0.0f)) {
+            q = (int)ceilf(256.0f * sqrtf(ideal[gi] / smax)) - 1;
+            if (q < 0) q = 0;
+            if (q > 255) q = 255;
+        }
+        scales[gi] = (uint8_t)q;
+        float inv = 1.0f / orc_scale_sq((uint8_t)q, smax);
+        for (int j = 0; j < 32; j++) {
+            float qv = clampf(w[gi * 32 + j] * inv, -6.0f, 6.0f);
+            float mag = fabsf(qv);
+            int idx = 0;
+            while (idx < 7 && mag >= MX_BOUNDS[idx]) idx++;
+            if (signbit(qv)) idx += 8;
+            size_t c = gi * 32 + j; /* rows are whole groups: the element's index in the matrix */
+            uint8_t *byte = &packed[c / 2];
+            if (c % 2 == 0)
+                *byte |= (uint8_t)idx;
+            else
+                *byte |= (uint8_t)(idx << 4);
+        }
+    }
+    free(ideal);
+    return smax;
+}
+
+/* src/mxfp4.rs:216-229 */
+ORC_API void orc_mxfp4sq_dequant(const uint8_t *packed, const uint8_t *scales, float smax, size_t rows, size_t cols, float *out) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++) {
+            uint8_t byte = packed[r * cols / 2 + c / 2];
+            uint8_t nib = (c % 2 == 0) ? (byte & 0x0F) : (byte >> 4);
+            out[r * cols + c] = E2M1[nib] * orc_scale_sq(scales[r * cols / 32 + c / 32], smax);
+        }
+}
+
 /* src/dequant.rs:12-23 */
 ORC_API float orc_e4m3_to_f32(uint8_t b) {
     float sign = (b & 0x80) ? -1.0f : 1.0f;

@@ -118,6 +118,8 @@ extern "C" {
     pub fn mk_dev_fp8_dequant(w: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_q8(x: *const f32, nvec: usize, n: usize, q: *mut i8, scales: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_quantize(w: *const f32, rows: usize, cols: usize, search: c_int, packed: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4sq_quantize(w: *const f32, rows: usize, cols: usize, packed: *mut u8, scales: *mut u8, smax: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4sq_dequant(packed: *const u8, scales: *const u8, smax_dev: *const f32, smax: f32, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_fp8(w: *const f32, rows: usize, cols: usize, qw: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_mxfp8(x: *const f32, nvec: usize, n: usize, codes: *mut u8, exps: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_matvec_q8(packed: *const u8, scales: *const u8, rows: usize, cols: usize, xq: *const i8, xs: *const f32, out: *mut f32, stream: *mut c_void) -> c_int;

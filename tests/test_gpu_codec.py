@@ -180,3 +180,32 @@ def test_quantize_fp8_gives_the_reference_bytes():
     assert np.array_equal(gsc.cpu().numpy(), wsc)
     assert np.array_equal(gq.cpu().numpy(), wq)
     assert wsc[0, 0] == 0 and wsc[0, 1] == 135 and wsc[1, 1] == 127
+
+
+def test_mxfp4sq_quantize_and_dequant_give_the_reference_bytes():
+    # mxfp4::quantize_sq / dequant_sq / dequant_any (src/mxfp4.rs:140-240)
+    from microkimi_amd import mxfp4
+    rows, cols = 48, 256
+    w = _quantizer_inputs(rows, cols, 23)
+    w[3, :32] = np.float32(3e30)   # (keeps smax finite enough for the small groups to be distinct)
+    wp, ws, wsmax = oracle.mxfp4sq_quantize(w, rows, cols)
+    gp, gs, gsmax = mxfp4.quantize_sq(dev(w))
+    assert np.float32(gsmax.cpu().numpy()[0]) == wsmax
+    assert np.array_equal(gs.cpu().numpy(), ws) and np.array_equal(gp.cpu().numpy(), wp)
+    want = oracle.mxfp4sq_dequant(wp, ws, wsmax, rows, cols)
+    got = mxfp4.dequant_sq(gp, gs, gsmax, rows, cols).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    blob = np.concatenate([wp.reshape(-1), ws.reshape(-1), np.array([wsmax], np.float32).view(np.uint8)])   # a dtype-4 blob
+    got2 = mxfp4.dequant_any(4, dev(blob), rows, cols).cpu().numpy()
+    assert np.array_equal(got2.view(np.uint32), want.view(np.uint32))
+    # moderate magnitudes too (the case above is dominated by one huge group)
+    w2 = _quantizer_inputs(rows, cols, 24)[5:]
+    p2, s2, m2 = oracle.mxfp4sq_quantize(w2, rows - 5, cols)
+    g2 = mxfp4.quantize_sq(dev(w2))
+    assert np.array_equal(g2[0].cpu().numpy(), p2) and np.array_equal(g2[1].cpu().numpy(), s2) and np.float32(g2[2].cpu().numpy()[0]) == m2
+    # an all-zero tensor: smax 0, scale 0, and 0 * (1 / 0) is a NaN whose sign bit decides the nibble (8 where the
+    # default NaN is negative, as on x86 and here; 0 elsewhere): bytes and smax as the oracle on this host has them
+    z = mxfp4.quantize_sq(dev(np.zeros((2, 64), np.float32)))
+    zp, zs, zm = oracle.mxfp4sq_quantize(np.zeros((2, 64), np.float32), 2, 64)
+    assert not z[1].any() and float(z[2]) == 0.0 and zm == 0.0
+    assert set(np.unique(z[0].cpu().numpy())) <= {0x00, 0x88}

@@ -157,3 +157,38 @@ def test_naive_scale_rule_matches_numpy_restatement():
     got[:, 0::2] = p & 0x0F
     got[:, 1::2] = p >> 4
     assert np.array_equal(got[off_mid.reshape(16, 64)], idx[off_mid.reshape(16, 64)])
+
+
+def test_mxfp4sq_properties():
+    # MXFP4SQ (src/mxfp4.rs:140-229), pinned by what the format promises: smax is the largest maxabs / 6; the decoded
+    # scale of every group is at least its ideal scale (nothing clips) and the byte is the smallest with that property;
+    # the group that sets smax gets byte 255 and scale smax exactly; values that sit on the grid come back exactly
+    rng = np.random.default_rng(8)
+    rows, cols = 16, 128
+    w = (rng.standard_normal((rows, cols)) * np.exp2(rng.integers(-8, 3, (rows, cols // 32)).astype(np.float32)).repeat(32, axis=1)).astype(np.float32)
+    w[3, 32:64] = 0.0
+    p, s, smax = oracle.mxfp4sq_quantize(w, rows, cols)
+    ideal = np.abs(w).reshape(rows, cols // 32, 32).max(axis=2) / np.float32(6.0)
+    assert smax == ideal.max()
+    dec = np.array([[oracle.scale_sq(q, smax) for q in r] for r in s], np.float32)
+    assert np.all(dec >= ideal) and s[3, 1] == 0
+    lower = np.array([[oracle.scale_sq(q - 1, smax) if q > 0 else 0.0 for q in r] for r in s], np.float32)
+    assert np.all((lower < ideal) | (s == 0))
+    gi = np.unravel_index(ideal.argmax(), ideal.shape)
+    assert s[gi] == 255 and oracle.scale_sq(255, smax) == smax
+    assert oracle.scale_sq(0, 1.0) == 2.0 ** -16 and oracle.scale_sq(127, 4.0) == 1.0
+    back = oracle.mxfp4sq_dequant(p, s, smax, rows, cols)
+    assert np.all(np.abs(back) <= 6.0 * dec.repeat(32, axis=1)) and np.all(np.abs(back - w) <= dec.repeat(32, axis=1))   # half the widest level step
+    # a matrix built on the grid: levels times decoded scales of chosen bytes round-trips bit for bit
+    levels = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6], np.float32)
+    q = rng.integers(0, 256, (4, 2)).astype(np.uint8)
+    q[0, 0] = 255
+    sc = np.array([[oracle.scale_sq(v, 3.0) for v in r] for r in q], np.float32)
+    nib = rng.integers(0, 8, (4, 64))
+    nib[:, 0] = 7
+    nib[:, 32] = 7                                   # every group reaches level 6: its ideal scale is its decoded scale
+    grid = (levels[nib] * sc.repeat(32, axis=1) * rng.choice([-1.0, 1.0], (4, 64))).astype(np.float32)
+    p2, s2, smax2 = oracle.mxfp4sq_quantize(grid, 4, 64)
+    assert smax2 == np.float32(3.0)
+    b2 = oracle.mxfp4sq_dequant(p2, s2, smax2, 4, 64)
+    assert np.array_equal(np.abs(b2), np.abs(grid))
