@@ -103,6 +103,8 @@ _lib.orc_router_softmax.argtypes = [_f32p, _sz, _sz, _u32p, _f32p]
 _lib.orc_expert_forward_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _sz, _sz, C.c_float, _f32p]
 _PP = C.POINTER(_u8p)
 _lib.orc_expert_packed.argtypes = [_u8p, _u8p, _u8p, _u8p, _u8p, _u8p, _sz, _sz, _f32p, C.c_int, C.c_int, C.c_float, C.c_float, _f32p]
+_lib.orc_matvec_packed_q8_device_order.argtypes = [_u8p, _u8p, _sz, _sz, _i8p, _f32p, _f32p]
+_lib.orc_q8head_matvec_device_order.argtypes = [_i8p, _f32p, _sz, _sz, _i8p, _f32p, _f32p]
 _lib.orc_scale_sq.argtypes = [C.c_uint8, C.c_float]
 _lib.orc_scale_sq.restype = C.c_float
 _lib.orc_mxfp4sq_quantize.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
@@ -333,6 +335,25 @@ def matvec_packed_shader_emul(packed, scales, rows, cols, x, lanes=256):
     x = _c(x, np.float32)
     out = np.empty(rows, np.float32)
     _lib.orc_matvec_packed_shader_emul(_p(packed, _u8p), _p(scales, _u8p), rows, cols, _p(x, _f32p), _p(out, _f32p), lanes)
+    return out
+
+
+def matvec_packed_q8_device_order(packed, scales, rows, cols, xq, xs):
+    """matvec_packed_q8 with the row sums associated as the single-row MXFP4 GEMV kernel of the library associates them
+    (the counterpart of matvec_packed_shader_emul for this device)."""
+    packed, scales = _chk_packed(packed, scales, rows, cols)
+    xq, xs = _c(xq, np.int8), _c(xs, np.float32)
+    out = np.empty(rows, np.float32)
+    _lib.orc_matvec_packed_q8_device_order(_p(packed, _u8p), _p(scales, _u8p), rows, cols, _p(xq, _i8p), _p(xs, _f32p), _p(out, _f32p))
+    return out
+
+
+def q8head_matvec_device_order(q, ws, rows, cols, xq, xs):
+    """Q8Head::matvec with the row sums associated as the batch-1 q8 GEMV kernel associates them; cols % 1024 == 0."""
+    q, ws, xq, xs = _c(q, np.int8), _c(ws, np.float32), _c(xq, np.int8), _c(xs, np.float32)
+    assert cols % 1024 == 0 and q.size == rows * cols and ws.size == rows * cols // 32
+    out = np.empty(rows, np.float32)
+    _lib.orc_q8head_matvec_device_order(_p(q, _i8p), _p(ws, _f32p), rows, cols, _p(xq, _i8p), _p(xs, _f32p), _p(out, _f32p))
     return out
 
 

@@ -636,6 +636,78 @@ ORC_API void orc_matvec_packed_nt(const uint8_t *packed, const uint8_t *scales, 
 
 /* ------------------------------------------------------------- q8 head */
 
+/* ------------------------------------------- summation order of the device kernels
+ * What matvec_packed_shader_emul (src/mxfp4.rs:348-393) is for the reference's Metal kernel: the order in which the
+ * device kernels of this library add a row's terms, restated on the CPU.  The terms themselves are the reference's
+ * (exact integer block dots times the f32 scale product); only the association of the f32 sum differs.  With it the gap
+ * between the device's and the reference's order is bounded without a device, and on a device the kernels must give
+ * these values bit for bit. */
+
+/* The wave-wide sum of the kernels: four exchange steps inside each row of 16 lanes (lane ^ 1, lane ^ 2, mirror of the
+ * half row, mirror of the row), then (v[0] + v[16]) + (v[32] + v[48]). */
+static float wave_sum_order(const float *in) {
+    float v[64], n[64];
+    memcpy(v, in, sizeof(v));
+    for (int l = 0; l < 64; l++) n[l] = v[l] + v[l ^ 1];
+    memcpy(v, n, sizeof(v));
+    for (int l = 0; l < 64; l++) n[l] = v[l] + v[l ^ 2];
+    memcpy(v, n, sizeof(v));
+    for (int l = 0; l < 64; l++) n[l] = v[l] + v[(l & ~7) + 7 - (l & 7)];
+    memcpy(v, n, sizeof(v));
+    for (int l = 0; l < 64; l++) n[l] = v[l] + v[(l & ~15) + 15 - (l & 15)];
+    return (n[0] + n[16]) + (n[32] + n[48]);
+}
+
+static size_t gcd_sz(size_t a, size_t b) { return b == 0 ? a : gcd_sz(b, a % b); }
+
+/* matvec_packed_q8 in the order of the single-row MXFP4 GEMV kernel: a tile is lcm(nb, 64) blocks = RT whole rows; lane l
+ * takes the blocks l, l + 64, ... of the tile in turn and adds a block's term to the sum of the row the block belongs
+ * to (zero to the other row's); the lanes' sums of a row then meet in the wave-wide sum.  nb = cols / 32. */
+ORC_API void orc_matvec_packed_q8_device_order(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const int8_t *xq,
+                                               const float *xs, float *out) {
+    size_t nb = cols / 32, tile = nb / gcd_sz(nb, 64) * 64, T = tile / 64, RT = tile / nb;
+    for (size_t row = 0; row < rows; row++) {
+        size_t r = row % RT;
+        float lanes[64];
+        for (size_t l = 0; l < 64; l++) {
+            float acc = 0.0f;
+            for (size_t t = 0; t < T; t++) {
+                size_t b = t * 64 + l;
+                float term = 0.0f;
+                if (b / nb == r) {
+                    size_t g = b % nb;
+                    int32_t idot = orc_block_dot(packed + row * cols / 2 + g * 16, xq + g * 32);
+                    term = (float)idot * (orc_exp2_i((int)scales[row * nb + g] - 128) * xs[g]);
+                }
+                acc += term;
+            }
+            lanes[l] = acc;
+        }
+        out[row] = wave_sum_order(lanes);
+    }
+}
+
+/* Q8Head::matvec in the order of the batch-1 q8 GEMV kernel: lane l takes the half blocks (16 values) l, l + 64, ... of
+ * the row; a half block's term is (ws * xs) * (its integer dot); then the wave-wide sum.  cols a multiple of 1024. */
+ORC_API void orc_q8head_matvec_device_order(const int8_t *q, const float *ws, size_t rows, size_t cols, const int8_t *xq, const float *xs,
+                                            float *out) {
+    size_t nb = cols / 32, T = nb * 2 / 64;
+    for (size_t row = 0; row < rows; row++) {
+        float lanes[64];
+        for (size_t l = 0; l < 64; l++) {
+            float acc = 0.0f;
+            for (size_t t = 0; t < T; t++) {
+                size_t hb = t * 64 + l;
+                int32_t d = 0;
+                for (int i = 0; i < 16; i++) d += (int32_t)q[row * cols + hb * 16 + i] * (int32_t)xq[hb * 16 + i];
+                acc += (ws[row * nb + hb / 2] * xs[hb / 2]) * (float)d;
+            }
+            lanes[l] = acc;
+        }
+        out[row] = wave_sum_order(lanes);
+    }
+}
+
 /* src/model.rs:274-286: row-wise q8_0 copy of an f32 matrix */
 ORC_API void orc_q8head_from_f32(const float *w, size_t rows, size_t cols, int8_t *q, float *scales) {
     size_t nb = cols / 32;

@@ -273,3 +273,41 @@ def test_batched_q8_matvec_on_the_matrix_cores():
         for i in range(m):
             want = oracle.matvec_packed_q8(packed, scales, rows, cols, xq_h[i], xs_h[i])
             assert rel_l2(got[i], want) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,cols", [(77, 7168), (2048, 7168), (130, 2048), (333, 1024), (2048, 4096)])
+def test_mxfp4_gemv_equals_its_order_emulation_bit_for_bit(rows, cols):
+    # the kernel's terms are the reference's (exact block dots, the same scale product); the oracle restates the order in
+    # which the kernel adds them (matvec_packed_q8_device_order): the device must give exactly those floats
+    torch = torch_cuda()
+    from microkimi_amd import mxfp4, q8
+    rng = np.random.default_rng(rows + cols)
+    p = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)
+    s = rng.integers(118, 131, (rows, cols // 32), dtype=np.uint8)
+    x = rng.standard_normal(cols).astype(np.float32)
+    xq, xs = oracle.quantize_q8(x)
+    want = oracle.matvec_packed_q8_device_order(p, s, rows, cols, xq, xs)
+    out = torch.empty(rows, device="cuda")
+    mxfp4.matvec_packed_q8(dev(p), dev(s), rows, cols, q8.quantize_q8(dev(x)), out)
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), float(np.abs(got - want).max())
+
+
+@pytest.mark.parametrize("f16", [True, False])
+def test_lm_head_gemv_equals_its_order_emulation_bit_for_bit(f16):
+    # the batch-1 q8 head kernel at the benchmark's row length, against q8head_matvec_device_order
+    torch_cuda()
+    from microkimi_amd import model
+    rng = np.random.default_rng(44)
+    rows, cols = 3000, 7168
+    q = rng.integers(-127, 128, (rows, cols), dtype=np.int8)
+    s = (np.abs(rng.standard_normal((rows, cols // 32))) * 0.02 / 127).astype(np.float32)
+    if f16:
+        s16 = s.astype(np.float16)
+        s = s16.astype(np.float32)
+    head = model.Q8Head.from_q8(dev(q), dev(s16 if f16 else s), rows, cols)
+    x = rng.standard_normal((1, cols)).astype(np.float32)
+    xq, xs = oracle.quantize_q8(x[0])
+    want = oracle.q8head_matvec_device_order(q, s, rows, cols, xq, xs)
+    got = head.matvec(dev(x)).cpu().numpy()[0]
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), float(np.abs(got - want).max())

@@ -139,3 +139,41 @@ def test_q8head_matches_f32_reference_test():
 
 def test_argmax_ties_lowest_index():
     assert oracle.argmax(np.array([1, 3, 3, 2], np.float32)) == 1
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 128), (9, 1024), (5, 2048), (6, 4096), (7, 7168), (3, 96)])
+def test_device_order_emulation_bounds_the_gap_without_a_device(rows, cols):
+    # the association of a row's f32 sum as the library's MXFP4 GEMV kernel has it (the role matvec_packed_shader_emul,
+    # src/selftest.rs:534-595, plays for the Metal kernel): the same terms, another order -- a few ulp of the row's norm
+    p, s, x = make_case(rows, cols)
+    xq, xs = oracle.quantize_q8(x)
+    ref = oracle.matvec_packed_q8(p, s, rows, cols, xq, xs)
+    emu = oracle.matvec_packed_q8_device_order(p, s, rows, cols, xq, xs)
+    assert np.linalg.norm(ref.astype(np.float64) - emu) <= 2e-6 * np.linalg.norm(ref)
+    # one block per row: a single term, no association to differ in -> the same bits
+    if cols >= 64:
+        x1 = x.copy()
+        x1[32:] = 0.0
+        xq1, xs1 = oracle.quantize_q8(x1)
+        a = oracle.matvec_packed_q8(p, s, rows, cols, xq1, xs1)
+        b = oracle.matvec_packed_q8_device_order(p, s, rows, cols, xq1, xs1)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_q8head_device_order_emulation():
+    rng = np.random.default_rng(3)
+    rows, cols = 12, 7168
+    q = rng.integers(-127, 128, (rows, cols), dtype=np.int8)
+    ws = (np.abs(rng.standard_normal((rows, cols // 32))) * 0.02 / 127).astype(np.float32)
+    x = rng.standard_normal(cols).astype(np.float32)
+    xq, xs = oracle.quantize_q8(x)
+    ref = oracle.q8head_matvec(q, ws, rows, cols, x)
+    emu = oracle.q8head_matvec_device_order(q, ws, rows, cols, xq, xs)
+    assert np.linalg.norm(ref.astype(np.float64) - emu) <= 2e-6 * np.linalg.norm(ref)
+    # the first 16 values of the activation only: one half block per row, one term -> the same bits as the reference order
+    x1 = np.zeros(cols, np.float32)
+    x1[:16] = x[:16]
+    xq1, xs1 = oracle.quantize_q8(x1)
+    a = oracle.q8head_matvec(q, ws, rows, cols, x1)
+    b = oracle.q8head_matvec_device_order(q, ws, rows, cols, xq1, xs1)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
