@@ -138,3 +138,39 @@ def test_hadamard_involution():
     x = oracle.pattern(5, 64)
     y = oracle.hadamard64(oracle.hadamard64(x)) / 64.0
     assert np.abs(x - y).max() <= 1e-6
+
+
+def test_hadamard_is_the_sylvester_matrix():
+    # the butterfly of src/model.rs:1540-1554 is the natural-order Walsh-Hadamard transform: on integer vectors (exact
+    # arithmetic) it equals the product with scipy's Sylvester matrix, so a wrong stage, stride or sign shows
+    from scipy.linalg import hadamard
+    H = hadamard(64).astype(np.float64)
+    rng = np.random.default_rng(64)
+    for _ in range(4):
+        x = rng.integers(-50, 51, 64).astype(np.float32)
+        assert np.array_equal(oracle.hadamard64(x).astype(np.float64), H @ x.astype(np.float64))
+    e = np.zeros(64, np.float32)
+    e[37] = 1.0
+    assert np.array_equal(oracle.hadamard64(e).astype(np.float64), H[:, 37])
+
+
+def test_hadamard_cache_attends_like_the_plain_one():
+    # the rotation is orthogonal up to the factor the kernel takes out again: attention over a Hadamard-mode cache agrees
+    # with the plain q8 cache to the quantization noise of both (and both with the f32 attention)
+    rng = np.random.default_rng(9)
+    nh, nope, rope, vd, n = 3, 128, 64, 128, 40
+    k = rng.standard_normal((n, nh * (nope + rope))).astype(np.float32)
+    v = rng.standard_normal((n, nh * vd)).astype(np.float32)
+    q = rng.standard_normal(nh * (nope + rope)).astype(np.float32)
+    scale = float(np.float32(nope + rope) ** np.float32(-0.5))
+    plain, had = oracle.MlaCache(nh, nope, rope, vd, capacity=n), oracle.MlaCache(nh, nope, rope, vd, had=True, capacity=n)
+    for j in range(n):
+        plain.push(k[j], v[j])
+        had.push(k[j], v[j])
+    assert not np.array_equal(plain.kq[:n], had.kq[:n])
+    a = oracle.mla_attn_flash_q8_mqa(plain, q, n - 1, scale)
+    b = oracle.mla_attn_flash_q8_mqa(had, q, n - 1, scale)
+    assert np.linalg.norm(a - b) <= 2e-2 * np.linalg.norm(a)
+    kf, vf = had.to_f32()   # de-rotated rows: the q8 round trip (the rope part of a K row is head 0's for every head)
+    nope_cols = (np.arange(nh * (nope + rope)) % (nope + rope)) < nope
+    assert np.abs(kf - k)[:, nope_cols].max() <= 0.05 and np.abs(vf - v).max() <= 0.05
