@@ -494,9 +494,10 @@ def bench_gemm(torch):
     ms3 = time_region(torch, step3, 5, warmup=2)
     per_expert = 3 * (inter * d // 2 + inter * d // 32)
     fl3 = 3 * 2.0 * m * inter * d
-    # weights once per used expert; token rows in, MXFP8 gathered rows, f32 gate / up / down outputs and their re-reads
-    alg3 = used * per_expert + T * d * 4 + 2 * (m * d + m * d // 32) + 2 * 2 * m * inter * 4 + 2 * (m * inter + m * inter // 32) + 2 * m * d * 4 + T * d * 4
-    res["expert_section"] = {"workload": "512 tokens x top-8 over 256 experts: group, gather + MXFP8, gate, up, SwiGLU + MXFP8, down, combine",
+    # weights once per used expert; token rows in, MXFP8 gathered rows and MXFP8 activation rows written and read, f32 down
+    # rows written and read (gate and up go from the accumulators to the activation's MXFP8 form: no f32 round trip)
+    alg3 = used * per_expert + T * d * 4 + 2 * (m * d + m * d // 32) + 2 * (m * inter + m * inter // 32) + 2 * m * d * 4 + T * d * 4
+    res["expert_section"] = {"workload": "512 tokens x top-8 over 256 experts: group, gather + MXFP8, gate + up + SwiGLU + MXFP8 (one launch), down, combine",
                              "ms": ms3, "tok_s": T / (ms3 * 1e-3), "tflops": fl3 / (ms3 * 1e-3) / 1e12,
                              "mfma_frac_fp8_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
                              "mfma_frac_fp4_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP4_PEAK_TFLOPS, "weight_bytes": used * per_expert,

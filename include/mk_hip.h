@@ -346,7 +346,9 @@ size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, s
  *   order   [P] int32      grouped row -> pair index t * topk + s
  *   pos     [P] int32      pair index -> grouped row, -1 for an expert id out of range
  *   offsets [n_experts+1]  int32: expert e owns the grouped rows offsets[e] .. offsets[e+1]
- *   g, u    [P][inter] f32 the gate and up projections per grouped row (before the activation)
+ *   g, u    [P][inter] f32 the gate and up projections per grouped row (before the activation): written by
+ *                          mk_dev_moe_prefill_keep only (mk_dev_moe_prefill goes from the accumulators straight to the
+ *                          activation's MXFP8 form and leaves these rows untouched)
  *   o       [P][d] f32     the down projection per grouped row, before the weighted sum */
 typedef struct {
     size_t order, pos, offsets, g, u, o;
@@ -369,6 +371,10 @@ int mk_moe_prefill_workspace_layout(size_t T, size_t topk, size_t n_experts, siz
  * act_kind MK_ACT_SWIGLU or MK_ACT_SITU.  d, inter multiples of 128; T * topk <= 16384
  * per call (a longer prompt is split by the caller). */
 int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
+                       const float *x, int act_kind, void *workspace, float *out, void *stream);
+/* The same call, the same kernels and the same result bit for bit, with the f32 gate and up rows stored as well (for
+ * callers that inspect the intermediates, see mk_moe_prefill_workspace_layout). */
+int mk_dev_moe_prefill_keep(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                        const float *x, int act_kind, void *workspace, float *out, void *stream);
 
 /* ---------------------------------------- device level: VQ1 / LUT GEMV */

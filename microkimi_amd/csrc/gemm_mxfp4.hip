@@ -132,6 +132,11 @@ struct GemmArgs {
     const int32_t *offsets;
     float *out[2];
     int n_groups, n_mats, row_blocks;
+    // gate/up form (GU passes): a workgroup owns 128 rows of BOTH matrices of a group, and the epilogue applies the
+    // activation and writes its MXFP8 form (the input of the down projection); out[] is written only when `keep` is set
+    int act_kind, keep;
+    uint8_t *act_codes;  // [token rows][rows] e4m3
+    uint8_t *act_exps;   // [token rows][rows / 32] e8m0
 };
 
 // PIN: the weights are the instruction's M operand and the token rows its N operand, so a lane of the 16 x 16 result
@@ -205,13 +210,21 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // same form with a second copy of the units in registers ran at one wave per SIMD and 101-111 us).  All four row tiles
 // per read (step-major, in place) needs 43 registers more than two waves per SIMD allow.  The next thing to measure is a larger tile
 // per workgroup (256 x 128 tokens: half the bytes through the cache per FLOP) with a per-step timeline of one wave.
-template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false>
+// GU: the gate/up form.  The wave's row tiles 0, 1 are rows row0 .. row0 + 31 of the first matrix (gate) and its row tiles
+// 2, 3 the same rows of the second (up: packed3 / scales3), so a lane ends up with g and u of the same (row, token); the
+// epilogue forms ACT(g, u), quantizes each token's 32 values to MXFP8 (mk_mxfp8_quantize8's arithmetic with the whole
+// e8m0 range; the block's maximum crosses the four lanes of a token) and stores codes and exponent bytes: 1.03 bytes
+// per value instead of 8 written and 8 read back by a kernel of its own.
+template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
-                                          uint8_t *lds) {
+                                          uint8_t *lds, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr) {
+    static_assert(!GU || (FULL && PIN && !DEEP && MC <= 2), "the gate/up form exists for the small-group pass");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
-    const int row0 = rb * 256 + wave * 64;
+    const int row0 = GU ? rb * 128 + wave * 32 : rb * 256 + wave * 64;
+    // first row of the wave's row tile rt
+    auto tile_row = [&](int rt) { return GU ? row0 + (rt & 1) * 16 : row0 + rt * 16; };
     // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
     // FULL: weight loads take whole 128-byte lines: load j = 2i + h of a unit covers line i (of the K tile's two) of the
     // rows 8h .. 8h+7 of the row tile, lane (r3 = lane / 8, c = lane % 8) reading bytes 16c .. of row 8h + r3, and the
@@ -224,9 +237,9 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     for (int rt = 0; rt < 4; rt++) {
         if constexpr (FULL) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(row0 + rt * 16 + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
+            for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(tile_row(rt) + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
         } else {
-            woff[rt][0] = (uint32_t)min(row0 + rt * 16 + n, a.rows - 1) * (uint32_t)(cols / 2) + kb * 16;
+            woff[rt][0] = (uint32_t)min(tile_row(rt) + n, a.rows - 1) * (uint32_t)(cols / 2) + kb * 16;
         }
     }
     // after the lane rotation below, lane (kg, x, r3) holds what lane (r3, x, kg) loaded
@@ -234,9 +247,11 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     mk_i4 wa[KT_STEPS], wb[KT_STEPS];
     auto load_unit = [&](mk_i4 *w, int kt, int rt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
+        const uint8_t *pk = (GU && rt >= 2) ? packed3 : packed;
 #pragma unroll
         for (int j = 0; j < KT_STEPS; j++)
-            if constexpr (FULL && NT) w[j] = mk_ldg128_off_nt(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
+            if constexpr (GU) w[j] = mk_ldg128_off_nt(pk, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
+            else if constexpr (FULL && NT) w[j] = mk_ldg128_off_nt(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
             else if constexpr (FULL) w[j] = mk_ldg128_off(packed, woff[rt][j & 1] + ku * (KT_STEPS * 64) + (j >> 1) * 128);
             else w[j] = mk_ldg128_off(packed, woff[rt][0] + ku * (KT_STEPS * 64) + j * 64);
     };
@@ -246,7 +261,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // row the same 16 bytes) they were 4 of a wave's 29 loads per K tile and about half of its vector-cache
     // accesses: a 16-byte load whose lanes sit in 16 different lines is looked up once per lane and pass.
     mk_i4 st[2 * MC], ste, stw;
-    const uint32_t wsoff = (uint32_t)min(rb * 256 + tid, a.rows - 1) * (uint32_t)nb;
+    // (gate/up form: thread i is row slot (wave i / 64, row tile (i / 16) % 4, row i % 16) of the workgroup)
+    const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * 256 + tid;
+    const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? scales3 : scales;
+    const uint32_t wsoff = (uint32_t)min(ws_row, a.rows - 1) * (uint32_t)nb;
     uint32_t coff[2 * MC];  // the host checks that tokens x cols stays below 2^32
 #pragma unroll
     for (int k = 0; k < 2 * MC; k++) {
@@ -259,7 +277,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
         for (int k = 0; k < 2 * MC; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
         ste = mk_ldg128_off(a.exps, eoff + ku * 16);
-        stw = mk_ldg128_off(scales, wsoff + ku * 16);
+        stw = mk_ldg128_off(ws_base, wsoff + ku * 16);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
@@ -434,6 +452,49 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             __syncthreads();
         }
     }
+    if constexpr (GU) {
+        // lane (n, kb): token base + 16 c + n, rows row0 + 4 kb .. + 3 (tiles 0 / 2) and row0 + 16 + 4 kb .. (tiles 1 / 3)
+#pragma unroll
+        for (int c = 0; c < MC; c++) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[i] = mk_act(a.act_kind, acc[0][c][i], acc[2][c][i], 0.0f, 1.0f);
+                v[4 + i] = mk_act(a.act_kind, acc[1][c][i], acc[3][c][i], 0.0f, 1.0f);
+            }
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(v[i]));
+            amax = mk_rows_max(amax);  // the token's 32 rows: this lane's eight and those of the lanes n + 16, + 32, + 48
+            int e = mk_ceil_log2f(fmaxf(amax, 1e-4f) / 448.0f);
+            e = max(-127, min(127, e));
+            const uint32_t eb = (uint32_t)(e + 127);
+            const float inv = mk_scale_from_byte(254u - eb);
+            float q[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(v[i] * inv, -448.0f), 448.0f);
+            int w0 = 0, w1 = 0;
+            w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], w0, false);
+            w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
+            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], w1, false);
+            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
+            const int t = base + c * 16 + n;
+            if (t < tok1 && row0 + 31 < a.rows) {
+                uint8_t *dst = a.act_codes + (size_t)t * a.rows + row0 + kb * 4;
+                *reinterpret_cast<uint32_t *>(dst) = (uint32_t)w0;
+                *reinterpret_cast<uint32_t *>(dst + 16) = (uint32_t)w1;
+                if (kb == 0) a.act_exps[(size_t)t * (a.rows / 32) + row0 / 32] = (uint8_t)eb;
+            }
+        }
+        if (a.keep) {  // the f32 gate and up rows as well (tests read them)
+#pragma unroll
+            for (int c = 0; c < MC; c++) {
+                store_tile_pair<NT>(a.out[0], a.rows, base + c * 16, tok1, row0, n, kb, acc[0][c], acc[1][c]);
+                store_tile_pair<NT>(a.out[1], a.rows, base + c * 16, tok1, row0, n, kb, acc[2][c], acc[3][c]);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int rt = 0; rt < 4; rt += 2) {
         if constexpr (PIN) {
@@ -496,6 +557,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     }
 }
 
+// The gate/up form: workgroup -> (group, block of 128 rows), both matrices.  Groups of up to 16 tokens take one token
+// tile, larger ones passes of 32 tokens (a group beyond 32 passes over its weights again: the prefill shape has none).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_gu_kernel(GemmArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int per_group = a.row_blocks;  // blocks of 128 rows
+    int e, rb;
+    if (a.n_groups % 8 == 0) {  // a group's workgroups on one XCD (see the kernel above)
+        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        e = x + 8 * (j / per_group);
+        rb = j % per_group;
+    } else {
+        e = blockIdx.x / per_group;
+        rb = blockIdx.x % per_group;
+    }
+    const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
+    const int count = tok1 - tok0;
+    if (count <= 0) return;
+    const uint8_t *p1 = mk_uniform_ptr(a.packed_ptrs[0][e]), *s1 = mk_uniform_ptr(a.scales_ptrs[0][e]);
+    const uint8_t *p3 = mk_uniform_ptr(a.packed_ptrs[1][e]), *s3 = mk_uniform_ptr(a.scales_ptrs[1][e]);
+    if (count <= 16) {
+        gemm_pass<1, true, true, true, false, true>(a, p1, s1, nullptr, rb, tok0, tok1, lds, p3, s3);
+    } else {
+#pragma unroll 1
+        for (int base = tok0; base < tok1; base += 32) gemm_pass<2, true, true, true, false, true>(a, p1, s1, nullptr, rb, base, tok1, lds, p3, s3);
+    }
+}
+
 template <int MC>
 int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
     // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
@@ -550,6 +638,42 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         if (st != MK_OK) return st;
     }
     return MK_OK;
+}
+
+// Gate and up of the prefill section with the activation and its MXFP8 form in the epilogue (see mk_common.h).
+// MK_ERR_UNSUPPORTED for shapes the streaming kernel does not take: the caller then runs the separate steps.
+int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
+                                      size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
+                                      const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
+                                      float *keep_u, void *stream) {
+    MK_REQUIRE(w1p && w1s && w3p && w3s && codes && exps && offsets && act_codes && act_exps, "null pointer");
+    if (!(cols % 512 == 0 && rows % 128 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0 &&
+          ((uintptr_t)codes & 15) == 0 && ((uintptr_t)act_codes & 3) == 0 && n_groups * (rows / 128) < 0x7FFFFFFFull))
+        return MK_ERR_UNSUPPORTED;
+    if (m == 0) return MK_OK;
+    GemmArgs a{};
+    a.packed_ptrs[0] = w1p;
+    a.scales_ptrs[0] = w1s;
+    a.packed_ptrs[1] = w3p;
+    a.scales_ptrs[1] = w3s;
+    a.out[0] = keep_g;
+    a.out[1] = keep_u;
+    a.keep = keep_g && keep_u;
+    a.rows = (int)rows;
+    a.cols = (int)cols;
+    a.codes = codes;
+    a.exps = exps;
+    a.offsets = offsets;
+    a.n_groups = (int)n_groups;
+    a.n_mats = 2;
+    a.row_blocks = (int)(rows / 128);
+    a.act_kind = act_kind;
+    a.act_codes = act_codes;
+    a.act_exps = act_exps;
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_gu_kernel), 2 * a_buf_bytes(2));
+    if (s != MK_OK) return s;
+    hipLaunchKernelGGL(mxfp4_grouped_gemm_gu_kernel, dim3((unsigned)(n_groups * (rows / 128))), dim3(256), 2 * a_buf_bytes(2), (hipStream_t)stream, a);
+    return mk_launch_status("mxfp4_grouped_gemm_gu");
 }
 
 extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,

@@ -329,3 +329,10 @@ int mk_mla_static_init(void **out_ptr);
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                             size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
                             float *const *out, void *stream);
+// The gate and up matrices of every group against the same token rows, the activation ACT(gate, up) and its MXFP8 form
+// (e4m3 codes [m][rows], e8m0 bytes [m][rows / 32], whole exponent range) in one launch; the f32 gate / up rows are
+// written too when keep_g and keep_u are given.  MK_ERR_UNSUPPORTED (nothing launched) for shapes it does not take.
+int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
+                                      size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
+                                      const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
+                                      float *keep_u, void *stream);

@@ -228,8 +228,9 @@ extern "C" int mk_moe_prefill_workspace_layout(size_t T, size_t topk, size_t n_e
     return MK_OK;
 }
 
-extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
-                                  const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+namespace {
+int moe_prefill_impl(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
+                     const float *x, int act_kind, void *workspace, float *out, void *stream, bool keep) {
     MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
     MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
     if (table->vq_codebook) {  // quant::matvec_vq_nt experts (src/model.rs:2556-2566): mk_dev_vq1_matvec_nt per expert, not this call
@@ -254,17 +255,34 @@ extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts
     hipLaunchKernelGGL(prefill_gather_mxfp8_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
                        (int)n_experts, (int)topk, (int)d, w.codes, w.exps);
     if ((s = mk_launch_status("prefill_gather_mxfp8")) != MK_OK) return s;
-    {
+    // gate, up, activation and its MXFP8 form in one launch; shapes that launch does not take run the three steps
+    s = MK_TUNE("MK_PREFILL_SEPARATE", 0) ? MK_ERR_UNSUPPORTED
+                                         : mk_mxfp4_grouped_gemm_gate_up_act(table->w1p, table->w1s, table->w3p, table->w3s, n_experts, inter, d, w.codes,
+                                                                             w.exps, w.offsets, P, act_kind, w.codes2, w.exps2, keep ? w.g : nullptr,
+                                                                             keep ? w.u : nullptr, stream);
+    if (s == MK_ERR_UNSUPPORTED) {
         const uint8_t *const *pp[2] = {table->w1p, table->w3p};
         const uint8_t *const *sp[2] = {table->w1s, table->w3s};
         float *gu[2] = {w.g, w.u};
         if ((s = mk_mxfp4_grouped_gemm_n(2, pp, sp, n_experts, inter, d, w.codes, w.exps, w.offsets, P, gu, stream)) != MK_OK) return s;
+        hipLaunchKernelGGL(prefill_act_mxfp8_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
+                           (int)n_experts, (int)inter, act_kind, w.codes2, w.exps2);
+        s = mk_launch_status("prefill_act_mxfp8");
     }
-    hipLaunchKernelGGL(prefill_act_mxfp8_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
-                       (int)n_experts, (int)inter, act_kind, w.codes2, w.exps2);
-    if ((s = mk_launch_status("prefill_act_mxfp8")) != MK_OK) return s;
+    if (s != MK_OK) return s;
     if ((s = mk_dev_mxfp4_grouped_gemm(table->w2p, table->w2s, n_experts, d, inter, w.codes2, w.exps2, w.offsets, P, w.o, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");
+}
+}  // namespace
+
+extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                  const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    return moe_prefill_impl(table, n_experts, T, topk, ids, weights, x, act_kind, workspace, out, stream, false);
+}
+
+extern "C" int mk_dev_moe_prefill_keep(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                       const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    return moe_prefill_impl(table, n_experts, T, topk, ids, weights, x, act_kind, workspace, out, stream, true);
 }

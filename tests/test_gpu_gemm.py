@@ -80,7 +80,9 @@ def test_matches_oracle_prefill_expert_section():
     assert rel_l2(got, want) <= 2e-3
 
 
-@pytest.mark.parametrize("T,topk,n_experts,d,inter,act", [(24, 2, 4, 256, 128, "swiglu"), (40, 3, 7, 512, 256, "situ"), (5, 1, 3, 1024, 512, "swiglu")])
+@pytest.mark.parametrize("T,topk,n_experts,d,inter,act", [(24, 2, 4, 256, 128, "swiglu"), (40, 3, 7, 512, 256, "situ"), (5, 1, 3, 1024, 512, "swiglu"),
+                                                          # groups of about 50 and 75 tokens: several 32-token passes of the gate/up launch
+                                                          (100, 2, 4, 512, 256, "swiglu"), (150, 2, 4, 1024, 384, "situ")])
 def test_moe_prefill_on_device(T, topk, n_experts, d, inter, act):
     # grouping, gather, the three grouped GEMMs, activation and combine all on the device (mk_dev_moe_prefill) against
     # the oracle's moe_prefill with the MXFP8 rounding switched on; the looser bound is the device expf in front of an
@@ -135,8 +137,9 @@ def test_config4_full_size_expert_section():
     logits, x = W.config4_tokens()
     T = x.shape[0]
     ids, wts = model.router_softmax_topk(dev(logits), topk)
-    got = model.moe_prefill(experts, ids, wts, dev(x)).cpu().numpy()
-    assert np.isfinite(got).all()
+    plain = model.moe_prefill(experts, ids, wts, dev(x)).cpu().numpy()
+    got = model.moe_prefill(experts, ids, wts, dev(x), keep=True).cpu().numpy()   # the same kernels, gate / up rows stored as well
+    assert np.isfinite(got).all() and np.array_equal(plain.view(np.uint32), got.view(np.uint32))
     mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
     ids_h, wts_h = ids.cpu().numpy(), wts.cpu().numpy()
 
