@@ -262,8 +262,8 @@ def bench_mxfp4_gemv(torch, cpu=True):
         for i in range(nmat):
             check(lib.mk_dev_mxfp4_matvec_q8(ptr(mats[i][0]), ptr(mats[i][1]), rows, cols, ptr(xq.q), ptr(xq.scales), ptr(outs[i]), cur_stream()))
 
-    g_ms, _ = time_events(torch, grouped, 30, warmup=30)  # the GPU idles during the CPU baseline before this: let the clocks come back
-    r_ms = time_events_region(torch, grouped, 30, warmup=30, rounds=7)
+    g_ms, _ = time_events(torch, grouped, 30, warmup=300)  # the GPU idles during the CPU baseline before this: 25 ms of launches let the clocks come back
+    r_ms = time_events_region(torch, grouped, 30, warmup=100, rounds=9)
     s_ms = time_region(torch, singles, 10)
     xf = x.contiguous()
 
