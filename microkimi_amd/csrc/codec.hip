@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void mk_quantize_q8_kernel(const float *__rest
     mx = fmaxf(mx, mk_dpp<0xB1>(mx));
     mx = fmaxf(mx, mk_dpp<0x4E>(mx));
     mx = fmaxf(mx, mk_dpp<0x141>(mx));
-    const float dx = mx / 127.0f;
+    const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
     uint32_t packed = 0;
     if (dx != 0.0f) {
         float qf[4];

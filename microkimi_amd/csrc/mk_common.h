@@ -155,6 +155,7 @@ __device__ __forceinline__ float mk_half_wave_max(float v) {
 // away from zero, clamp to +-127.  dx > 0.
 __device__ __forceinline__ int mk_q8_round(float v, float dx) {
     float r = roundf(v / dx);
+    if (r != r) return 0;  // a NaN value, or inf / inf: the reference's `as i8` of NaN is 0 (fmaxf would drop the NaN and give -127)
     r = fminf(fmaxf(r, -127.0f), 127.0f);
     return (int)r;
 }

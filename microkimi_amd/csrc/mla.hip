@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void mla_q_prep_kernel(const float *__restrict
     const int h = blk / nb, g = blk % nb;
     float v = q[(size_t)h * (L + R) + g * 32 + j];
     float mx = mk_half_wave_max(fabsf(v));
-    float dx = mx / 127.0f;
+    float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
     int qi = dx != 0.0f ? mk_q8_round(v, dx) : 0;
     qq[(size_t)h * L + g * 32 + j] = (int8_t)qi;
     if (j == 0) qs[blk] = dx;
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
                     mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, MK_WAVE));
-                const float dx = mx / 127.0f;
+                const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
                 mk_i4 packed;
 #pragma unroll
                 for (int k = 0; k < 4; k++) {

@@ -42,7 +42,7 @@ __device__ __forceinline__ float hadamard64_lane(float v, int lane) {
 // One 32-block per aligned group of 32 lanes: q8::quantize_q8_into (src/q8.rs:57-68).
 __device__ __forceinline__ void quantize_block32(float v, int8_t *q_out, float *s_out, int j) {
     const float mx = mk_half_wave_max(fabsf(v));
-    const float dx = mx / 127.0f;
+    const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
     q_out[j] = (int8_t)(dx != 0.0f ? mk_q8_round(v, dx) : 0);
     if (j == 0) *s_out = dx;
 }

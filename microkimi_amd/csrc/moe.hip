@@ -240,7 +240,7 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
                 mx = fmaxf(mx, mk_dpp<0xB1>(mx));
                 mx = fmaxf(mx, mk_dpp<0x4E>(mx));
                 mx = fmaxf(mx, mk_dpp<0x141>(mx));
-                const float dx = mx / 127.0f;
+                const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
                 mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
                 if (dx != 0.0f) mk_q8_round4_f16(v[b], dx, lo, hi);
                 if (i < n_x) {
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a)
             mx = fmaxf(mx, mk_dpp<0xB1>(mx));
             mx = fmaxf(mx, mk_dpp<0x4E>(mx));
             mx = fmaxf(mx, mk_dpp<0x141>(mx));
-            const float dx = mx / 127.0f;
+            const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
             mk_h2 lo = {(_Float16)0.0f, (_Float16)0.0f}, hi = lo;
             if (dx != 0.0f) mk_q8_round4_f16(v[b], dx, lo, hi);
             if (i < n_a) {
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(1024) void moe_group_pairs_kernel(int B, int topk, 
         mx = fmaxf(mx, mk_dpp<0xB1>(mx));
         mx = fmaxf(mx, mk_dpp<0x4E>(mx));
         mx = fmaxf(mx, mk_dpp<0x141>(mx));
-        const float dx = mx / 127.0f;
+        const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
         uint32_t packed = 0;
         if (dx != 0.0f) {
             float qf[4];
@@ -686,7 +686,7 @@ __global__ __launch_bounds__(256) void moe_act_q8_grouped_kernel(const float *__
     mx = fmaxf(mx, mk_dpp<0xB1>(mx));
     mx = fmaxf(mx, mk_dpp<0x4E>(mx));
     mx = fmaxf(mx, mk_dpp<0x141>(mx));
-    const float dx = mx / 127.0f;
+    const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
     uint32_t packed = 0;
     if (dx != 0.0f) {
         float qf[4];

@@ -334,7 +334,7 @@ ORC_API void orc_quantize_q8(const float *x, size_t n, int8_t *q, float *scales)
         for (int j = 0; j < 32; j++) {
             float v = roundf(b[j] / dx); /* Rust f32::round: half away from zero */
             v = clampf(v, -127.0f, 127.0f);
-            q[g * 32 + j] = (int8_t)v;
+            q[g * 32 + j] = v != v ? 0 : (int8_t)v; /* Rust's `as i8` of NaN (a NaN value, or inf / inf) is 0 */
         }
     }
 }

@@ -87,6 +87,19 @@ def test_quantize_q8_bit_exact():
     qo, so = oracle.quantize_q8(y.reshape(-1))
     assert np.array_equal(vt.q.cpu().numpy().reshape(-1), qo)
     assert np.array_equal(bits(vt.scales.cpu().numpy().reshape(-1)), bits(so))
+    # NaN and inf: the maximum skips a NaN, a NaN quotient (a NaN value, inf / inf) gives 0 as the reference's cast does
+    z = rng.standard_normal((4, 64)).astype(np.float32)
+    z[0, 3] = np.nan
+    z[1, 7] = np.inf
+    z[1, 9] = -np.inf
+    z[2, :32] = np.nan
+    z[3, 33] = np.nan
+    z[3, 40] = np.inf
+    vz = q8.quantize_q8(dev(z))
+    for r in range(4):
+        qo, so = oracle.quantize_q8(z[r])
+        assert np.array_equal(vz.q.cpu().numpy()[r], qo), r
+        assert np.array_equal(bits(vz.scales.cpu().numpy()[r]), bits(so)), r
     # host-level entry point
     hv = q8.quantize_q8(x[0])
     assert np.array_equal(hv.q, q[0]) and np.array_equal(hv.scales, s[0])

@@ -192,3 +192,23 @@ def test_mxfp4sq_properties():
     assert smax2 == np.float32(3.0)
     b2 = oracle.mxfp4sq_dequant(p2, s2, smax2, 4, 64)
     assert np.array_equal(np.abs(b2), np.abs(grid))
+
+
+def test_quantize_q8_non_finite_values():
+    """src/q8.rs:49-69 on blocks with NaN or inf, fixed by the language rules the reference's expression runs under:
+    f32::max skips a NaN (the block maximum comes from the other values), f32::clamp keeps a NaN, and `NaN as i8` is 0;
+    a block with an inf has scale inf, finite / inf = 0 and inf / inf = NaN -> 0."""
+    x = np.zeros(96, dtype=np.float32)
+    x[:32] = np.linspace(-2.0, 2.0, 32, dtype=np.float32)
+    x[5] = np.nan
+    x[32:64] = 1.5
+    x[40] = np.inf
+    x[41] = -np.inf
+    x[64:96] = np.nan
+    q, s = oracle.quantize_q8(x)
+    clean = x[:32].copy()
+    clean[5] = 0.0
+    qc, sc = oracle.quantize_q8(clean)
+    assert s[0] == sc[0] and np.array_equal(q[:32], qc[:32]) and q[5] == 0
+    assert np.isinf(s[1]) and not q[32:64].any()
+    assert s[2] == 0.0 and not q[64:].any()   # every value skipped: maximum 0, the all-zero rule
