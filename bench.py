@@ -423,6 +423,51 @@ def bench_mla(torch, cpu=True):
     return res
 
 
+def bench_mla_heads(torch):
+    """The attention over the reference's own cache layout (per head a q8 K-nope row and a q8 V row, one f32 rope row per
+    position) on the case the reference publishes: 96 heads, nope 128 + rope 64, v 128 (KIMI.md:96, bench code
+    src/main.rs:389-479: 16k positions 79.7 ms with the all-heads q8 kernel on one CPU thread).  Every cache byte is
+    used once: HBM-bound.  Two caches alternate (each is larger than the Infinity Cache at 16k)."""
+    from microkimi_amd import model
+    nh, nope, rope, vd = 96, 128, 64, 128
+    g = torch.Generator(device="cuda").manual_seed(6)
+    res = {"workload": "96 heads, nope 128 + rope 64 (f32, shared), v 128, q8_0 with f32 scales: 27 904 B/position",
+           "published_cpu_ms_16k": 79.7}
+    q = torch.randn((1, nh * (nope + rope)), device="cuda", generator=g)
+    scale = float((nope + rope) ** -0.5)
+    for ctx in (1024, 4096, 16384):
+        caches = []
+        for _ in range(2):
+            c = model.MlaHeadsCache(nh, nope, rope, vd, ctx)
+            c.kq.copy_(torch.randint(-127, 128, c.kq.shape, dtype=torch.int8, device="cuda", generator=g))
+            c.vq.copy_(torch.randint(-127, 128, c.vq.shape, dtype=torch.int8, device="cuda", generator=g))
+            c.ks.copy_(torch.rand(c.ks.shape, device="cuda", generator=g) * 0.03 + 0.005)
+            c.vs.copy_(torch.rand(c.vs.shape, device="cuda", generator=g) * 0.03 + 0.005)
+            c.kr.copy_(torch.randn(c.kr.shape, device="cuda", generator=g))
+            c.n = ctx
+            caches.append(c)
+        caches[0].attn(q, ctx - 1, scale)  # workspaces allocated before the capture
+        caches[1].attn(q, ctx - 1, scale)
+        it = [0]
+
+        def step():
+            c = caches[it[0] % 2]
+            it[0] += 1
+            c.attn(q, ctx - 1, scale)
+
+        ms_eager = time_region(torch, step, 32, warmup=4)
+        it[0] = 0
+        ms_graph = time_graph(torch, [step] * 8)
+        ms = ms_graph if ms_graph is not None else ms_eager
+        alg = ctx * (nh * (nope + vd) * 9 // 8 + rope * 4) + nh * (nope + rope) * 4 + nh * vd * 4
+        res[f"ctx{ctx}"] = {"us": ms * 1e3, "us_python_loop": ms_eager * 1e3, "timing": "graph replay" if ms_graph is not None else "python loop",
+                            "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        if ctx == 16384:
+            res[f"ctx{ctx}"]["published_cpu_ms_over_this"] = 79.7 / ms
+        del caches
+    return res
+
+
 def bench_gemm(torch):
     """Configuration 4: 512 tokens routed top-8 over 256 experts (about 16 rows per expert), gate GEMM 2048 x 7168 per
     expert on the block-scaled MFMA; and a large-M variant (512 rows on each of 8 experts)."""
@@ -514,7 +559,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="",
-                    help="comma-separated names of extras (mxfp4_gemv, moe_decode, mla_decode, grouped_gemm, vq1_gemv): run only "
+                    help="comma-separated names of extras (mxfp4_gemv, moe_decode, mla_decode, mla_heads_decode, grouped_gemm, vq1_gemv): run only "
                          "those and print their figures as one JSON object (a development aid; the contract line needs a full run)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain 1 GiB device copies (a kernel of known traffic to scale rocprofv3 --pmc byte counters by)")
@@ -539,7 +584,8 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
     if args.only:
-        table = {"mxfp4_gemv": bench_mxfp4_gemv, "moe_decode": bench_moe, "mla_decode": bench_mla, "grouped_gemm": bench_gemm, "vq1_gemv": bench_vq1}
+        table = {"mxfp4_gemv": bench_mxfp4_gemv, "moe_decode": bench_moe, "mla_decode": bench_mla, "mla_heads_decode": bench_mla_heads,
+                 "grouped_gemm": bench_gemm, "vq1_gemv": bench_vq1}
         res = {}
         for name in args.only.split(","):
             log(name, "...")
@@ -558,7 +604,8 @@ def main():
     torch.cuda.empty_cache()
     extras = {"lm_head_batch8": head.pop("batch8")}
     if not args.no_extras:
-        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("grouped_gemm", bench_gemm), ("vq1_gemv", bench_vq1)):
+        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("mla_heads_decode", bench_mla_heads),
+                         ("grouped_gemm", bench_gemm), ("vq1_gemv", bench_vq1)):
             log(name, "...")
             try:
                 extras[name] = fn(torch, not args.no_cpu) if name in ("mxfp4_gemv", "moe_decode", "mla_decode") else fn(torch)

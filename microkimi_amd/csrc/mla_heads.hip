@@ -279,30 +279,221 @@ __global__ __launch_bounds__(256) void heads_decode_kernel(HeadsArgs a) {
     }
 }
 
+// The all-heads form for the reference's own head shape, nope 128 + rope 64 / v 128 (its mla_attn_flash_q8_mqa streams the
+// cache once, tile outer / head inner, src/model.rs:1804-1908): a workgroup takes 8 neighbouring heads over a split of the positions, a wave
+// every 4th position, 8 lanes a head.  One load instruction of a wave is then 1 KB of consecutive bytes (the K rows, or
+// the V rows, of the 8 heads at one position), the 8 heads' block scales are exactly one 128-byte line, the rope row is
+// read once for the 8 heads.  Every wave runs its own online softmax over its positions (no barrier and no LDS in the
+// loop); the four states of a head meet once at the end.  nh % 8 == 0.
+struct G8Pos {
+    mk_i4 k;
+    float ks;
+    mk_f4 r0, r1;
+    mk_i4 v;
+    float vs;
+};
+
+__global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
+        constexpr int NOPE = 128, ROPE = 64, VD = 128, U = 4;
+    __shared__ float o_l[4][8][VD + 4];
+    __shared__ float m_l[4][8], l_l[4][8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hgroups = a.nh >> 3;
+    // consecutive workgroup ids go round the 8 XCDs (each with its own L2): XCD x takes the splits x, x + 8, ... with all
+    // their head groups, so a position's rope row is fetched by one of them only
+    int split, hg;
+    if ((a.n_splits & 7) == 0) {
+        const int r = blockIdx.x >> 3;
+        split = (blockIdx.x & 7) + 8 * (r / hgroups);
+        hg = r % hgroups;
+    } else {
+        split = blockIdx.x / hgroups;
+        hg = blockIdx.x - split * hgroups;
+    }
+    const int qi = blockIdx.y;
+    const int hl = lane >> 3, c = lane & 7, h = hg * 8 + hl;
+    const uint32_t nh = (uint32_t)a.nh;
+    const int n_pos = a.n_pos0 + qi;
+    // Split s takes the steps (16 positions) s, s + n_splits, ...: at any time the launch reads one compact window of the
+    // cache (n_splits x 16 positions), not n_splits distant ranges.  (The softmax partials do not care which positions a
+    // split holds.)
+    const int p_end = n_pos;
+    const uint32_t last = (uint32_t)n_pos - 1u;
+    const size_t qrow = (size_t)qi * nh + h;
+    // lane c of a head: bytes 16 c .. of a K row (half of block c / 2), rope values 4 c .. and 32 + 4 c .., V dims 16 c ..
+    mk_i4 qk;
+    float qsc;
+    if (a.qq) {  // quantized by the launch before this one (the Hadamard option rotates the query first)
+        qk = mk_ldg128(a.qq + qrow * NOPE + c * 16);
+        qsc = a.qs[qrow * (NOPE / 32) + (c >> 1)] * a.had_k;
+    } else {  // quantize_q8 of the query's latent part here (src/model.rs:1812-1821): lanes c and c ^ 1 share a block
+        const mk_f4 *src = reinterpret_cast<const mk_f4 *>(a.q + qrow * (NOPE + ROPE) + c * 16);
+        mk_f4 v[4];
+        float mx = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[k] = src[k];
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(v[k].x), fabsf(v[k].y)), fmaxf(fabsf(v[k].z), fabsf(v[k].w))));
+        }
+        mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+        const float dx = mx / 127.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            uint32_t w = 0;
+            if (dx != 0.0f) {
+                float qf[4];
+                mk_q8_round4(v[k], dx, qf);
+                w = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                    ((uint32_t)(int)qf[3] << 24);
+            }
+            qk[k] = (int)w;
+        }
+        qsc = dx;
+    }
+    const mk_f4 qr0 = *reinterpret_cast<const mk_f4 *>(a.q + qrow * (NOPE + ROPE) + NOPE + c * 4);
+    const mk_f4 qr1 = *reinterpret_cast<const mk_f4 *>(a.q + qrow * (NOPE + ROPE) + NOPE + 32 + c * 4);
+    float o[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[e] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    // byte offsets are 32-bit (the host checks positions * heads * 128 < 2^32); a position past the end re-reads the last one
+    static_assert(U == 4, "a step is 16 positions");
+    for (int t0 = split * 16 + wave; t0 < p_end; t0 += 16 * a.n_splits) {
+        G8Pos t[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = min((uint32_t)(t0 + 4 * u), last);
+            const uint32_t row = j * nh + (uint32_t)h;
+            t[u].k = mk_ldg128_off_nt(a.kq, row * NOPE + c * 16);  // streamed once: non-temporal
+            t[u].ks = mk_ldg_f32_off(a.ks, (row * (NOPE / 32) + (c >> 1)) * 4);
+            t[u].r0 = __builtin_bit_cast(mk_f4, mk_ldg128_off(a.kr, (j * ROPE + c * 4) * 4));
+            t[u].r1 = __builtin_bit_cast(mk_f4, mk_ldg128_off(a.kr, (j * ROPE + 32 + c * 4) * 4));
+            t[u].v = mk_ldg128_off_nt(a.vq, row * VD + c * 16);
+            t[u].vs = mk_ldg_f32_off(a.vs, (row * (VD / 32) + (c >> 1)) * 4);
+        }
+        // ---- scores (src/model.rs:1833-1851): integer block dot, the block's scale product, the f32 rope part
+        float s[U];
+        float m_new = m;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int idot = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) idot = __builtin_amdgcn_sdot4(t[u].k[e], qk[e], idot, false);
+            idot += __builtin_amdgcn_update_dpp(0, idot, 0xB1, 0xF, 0xF, true);  // the other half of the block (lane ^ 1)
+            float x = (c & 1) ? 0.0f : (qsc * t[u].ks) * (float)idot;
+            x += qr0.x * t[u].r0.x + qr0.y * t[u].r0.y + qr0.z * t[u].r0.z + qr0.w * t[u].r0.w;
+            x += qr1.x * t[u].r1.x + qr1.y * t[u].r1.y + qr1.z * t[u].r1.z + qr1.w * t[u].r1.w;
+            x += mk_dpp<0xB1>(x);
+            x += mk_dpp<0x4E>(x);
+            x += mk_dpp<0x141>(x);
+            s[u] = (t0 + 4 * u < p_end) ? x * a.scale : -INFINITY;
+            m_new = fmaxf(m_new, s[u]);
+        }
+        // ---- online softmax of this wave's positions (the first position of the step is inside the split: m_new is finite)
+        const float corr = expf(m - m_new);
+        l *= corr;
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[e] *= corr;
+        m = m_new;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float p = expf(s[u] - m_new);  // a position past the end has score -inf: 0
+            l += p;
+            const float ps = p * t[u].vs;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const int w = t[u].v[d];
+                o[4 * d + 0] += ps * (float)(int8_t)w;
+                o[4 * d + 1] += ps * (float)(int8_t)(w >> 8);
+                o[4 * d + 2] += ps * (float)(int8_t)(w >> 16);
+                o[4 * d + 3] += ps * (float)(w >> 24);
+            }
+        }
+    }
+    // ---- the four waves' states of a head meet (a wave without a position has m = -inf, l = 0, o = 0: weight 0)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o_l[wave][hl][c * 16 + e] = o[e];
+    if (c == 0) {
+        m_l[wave][hl] = m;
+        l_l[wave][hl] = l;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < 8 * VD; idx += 256) {
+        const int hh = idx / VD, d = idx - hh * VD;
+        const float ms = fmaxf(fmaxf(m_l[0][hh], m_l[1][hh]), fmaxf(m_l[2][hh], m_l[3][hh]));
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float wt = expf(m_l[w][hh] - ms);
+            num += wt * o_l[w][hh][d];
+            den += wt * l_l[w][hh];
+        }
+        const size_t hrow = (size_t)hg * 8 + hh;
+        if (a.n_splits == 1) {
+            a.out[((size_t)qi * nh + hrow) * VD + d] = num / den;
+        } else {
+            a.po[((size_t)split * nh + hrow) * VD + d] = num;
+            if (d == 0) {
+                a.pm[split * nh + hrow] = ms;
+                a.pl[split * nh + hrow] = den;
+            }
+        }
+    }
+}
+
 // log-sum-exp merge of the splits of one query: a workgroup per head
 __global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
                                                           int nh, int vd, int n_splits, float *__restrict__ out) {
     __shared__ float w_l[MAX_SPLITS];
     __shared__ float den_l;
+    __shared__ float part_l[256];
     const int h = blockIdx.x, tid = threadIdx.x;
-    if (tid < 64) {
-        float mx = -INFINITY;
-        for (int s = tid; s < n_splits; s += 64) mx = fmaxf(mx, pm[s * nh + h]);
-        mx = mk_wave_max(mx);
-        float den = 0.0f;
-        for (int s = tid; s < n_splits; s += 64) {
-            const float w = expf(pm[s * nh + h] - mx);
-            w_l[s] = w;
-            den += pl[s * nh + h] * w;
+    // The partials come from other compute dies: every dependent round of loads costs a trip to memory.  Narrow rows
+    // (vd <= 128) take ONE round: the splits are shared out over 256 / vd groups of threads and a thread requests all
+    // its partial values before the weights exist (a split past the end re-reads the last one with weight 0).
+    const int groups = vd <= 128 ? 256 / vd : 1;
+    constexpr int PER = MAX_SPLITS / 2;
+    const int sg = tid / vd, d = tid - sg * vd;
+    float pv[PER];
+    if (groups > 1 && sg < groups) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int s = min(sg + groups * i, n_splits - 1);
+            pv[i] = po[((size_t)s * nh + h) * vd + d];
         }
-        den = mk_wave_sum(den);
+    }
+    if (tid < 64) {
+        static_assert(MAX_SPLITS <= 64, "one lane per split");
+        const float ms = tid < n_splits ? pm[tid * nh + h] : -INFINITY;
+        const float ls = tid < n_splits ? pl[tid * nh + h] : 0.0f;
+        const float mx = mk_wave_max(ms);
+        const float w = expf(ms - mx);  // (a lane past the last split: 0)
+        w_l[tid] = w;
+        const float den = mk_wave_sum(ls * w);
         if (tid == 0) den_l = den;
     }
     __syncthreads();
-    for (int d = tid; d < vd; d += 256) {
+    if (groups > 1) {
         float num = 0.0f;
-        for (int s = 0; s < n_splits; s++) num += po[((size_t)s * nh + h) * vd + d] * w_l[s];
-        out[(size_t)h * vd + d] = num / den_l;
+        if (sg < groups) {
+#pragma unroll
+            for (int i = 0; i < PER; i++) {
+                const int s = sg + groups * i;
+                num += pv[i] * (s < n_splits ? w_l[s] : 0.0f);
+            }
+            part_l[tid] = num;
+        }
+        __syncthreads();
+        if (tid < vd) {
+            for (int g = 1; g < groups; g++) num += part_l[g * vd + tid];
+            out[(size_t)h * vd + tid] = num / den_l;
+        }
+        return;
+    }
+    for (int dd = tid; dd < vd; dd += 256) {
+        float num = 0.0f;
+        for (int s = 0; s < n_splits; s++) num += po[((size_t)s * nh + h) * vd + dd] * w_l[s];
+        out[(size_t)h * vd + dd] = num / den_l;
     }
 }
 
@@ -398,10 +589,17 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.out = out;
     const int had = had_applies(hadamard, nope, vd);
     a.had_k = had ? 1.0f / 64.0f : 1.0f;
-    const int rows = (int)(m * nh);
-    hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, had, qq,
-                       qs);
-    if ((s = mk_launch_status("heads_q_prep")) != MK_OK) return s;
+    // the reference's own head shape in whole groups of 8 heads takes the all-heads kernel
+    const bool g8 = nope == 128 && rope == 64 && vd == 128 && nh % 8 == 0 && (pos0 + m) * nh * 128 < 0xFFFFFFFFull &&
+                      ((uintptr_t)vq & 15) == 0 && ((uintptr_t)kr & 15) == 0 && ((uintptr_t)q & 15) == 0 && !MK_TUNE("MK_MLA_HEADS_GENERIC", 0);
+    if (g8 && !had) {
+        a.qq = nullptr;  // the all-heads kernel quantizes the query itself
+    } else {
+        const int rows = (int)(m * nh);
+        hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, had, qq,
+                           qs);
+        if ((s = mk_launch_status("heads_q_prep")) != MK_OK) return s;
+    }
     // one query: split the context so that about 1024 workgroups stream the cache; several queries (prefill): the
     // (query, head) grid is parallel enough, one split each
     int n_splits = 1, split_len = (int)((pos0 + m + TJ - 1) / TJ) * TJ;
@@ -413,10 +611,20 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
         const int tps = (tiles + want - 1) / want;
         split_len = tps * TJ;
         n_splits = (tiles + tps - 1) / tps;
+        if (g8) {  // interleaved steps of 16 positions: any count up to the number of steps
+            const int steps = (int)((pos0 + 1 + 15) / 16);
+            n_splits = (int)((MK_TUNE("MK_MLA_HEADS_WGS", 768) + nh / 8 - 1) / (nh / 8));
+            if (n_splits > MAX_SPLITS) n_splits = MAX_SPLITS;
+            if (n_splits > steps) n_splits = steps;
+        }
     }
     a.split_len = split_len;
     a.n_splits = n_splits;
-    hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);
+    if (g8) {
+        hipLaunchKernelGGL(heads_decode_g8_kernel, dim3((unsigned)(n_splits * (nh / 8)), (unsigned)m), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);
+    }
     if ((s = mk_launch_status("heads_decode")) != MK_OK) return s;
     if (n_splits > 1) {
         hipLaunchKernelGGL(heads_merge_kernel, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);

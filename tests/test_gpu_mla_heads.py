@@ -56,7 +56,12 @@ def test_push_assign_and_to_f32_are_the_reference_bytes(n, nh, nope, rope, vd):
 
 @pytest.mark.parametrize("n,nh,nope,rope,vd,qscale", [(1, 4, 128, 64, 128, 1.0), (7, 4, 128, 64, 128, 1.0), (64, 6, 128, 64, 128, 1.0),
                                                      (65, 6, 128, 64, 128, 1.0), (512, 6, 128, 64, 128, 1.0), (300, 5, 64, 32, 96, 3.0),
-                                                     (4200, 24, 128, 64, 128, 1.0), (130, 2, 256, 64, 512, 0.0)])
+                                                     (4200, 24, 128, 64, 128, 1.0), (130, 2, 256, 64, 512, 0.0),
+                                                     # head counts in whole groups of 8 at the reference's head shape take the
+                                                     # streaming kernel: the same lengths, a context split over the chip, zero query
+                                                     (1, 8, 128, 64, 128, 1.0), (7, 8, 128, 64, 128, 1.0), (64, 16, 128, 64, 128, 1.0),
+                                                     (65, 8, 128, 64, 128, 3.0), (512, 8, 128, 64, 128, 1.0), (2100, 96, 128, 64, 128, 1.0),
+                                                     (200, 8, 128, 64, 128, 0.0)])
 def test_decode_matches_mla_attn_flash_q8_mqa(n, nh, nope, rope, vd, qscale):
     # the lengths of src/selftest.rs:871-876 (1, 7, 64, 65, 512), a long context (split over the chip), odd shapes,
     # an all-zero query (uniform weights)
@@ -75,10 +80,12 @@ def test_decode_matches_mla_attn_flash_q8_mqa(n, nh, nope, rope, vd, qscale):
         assert rel_l2(got, want) <= TOL, (pos, rel_l2(got, want))
 
 
-def test_prefill_loop_equals_one_decode_per_position():
-    # mla_prefill (src/model.rs:2080-2102): query i over the positions 0 ..= pos0 + i
+@pytest.mark.parametrize("nh", [6, 8])
+def test_prefill_loop_equals_one_decode_per_position(nh):
+    # mla_prefill (src/model.rs:2080-2102): query i over the positions 0 ..= pos0 + i (6 heads: the general kernel,
+    # 8: the streaming one)
     from microkimi_amd import model
-    nh, nope, rope, vd, n0, m = 6, 128, 64, 128, 40, 33
+    nope, rope, vd, n0, m = 128, 64, 128, 40, 33
     k, v = rows(n0 + m, nh, nope, rope, vd, 5)
     rng = np.random.default_rng(6)
     q = rng.standard_normal((m, nh * (nope + rope))).astype(np.float32)
@@ -137,7 +144,7 @@ def test_shapes_the_kernels_do_not_cover_are_refused():
 
 
 @pytest.mark.parametrize("n,nh,nope,rope,vd,applies", [(37, 4, 128, 64, 128, True), (70, 3, 64, 32, 192, True), (300, 6, 128, 64, 128, True),
-                                                     (20, 3, 96, 32, 128, False)])
+                                                     (20, 3, 96, 32, 128, False), (300, 8, 128, 64, 128, True)])
 def test_hadamard_option(n, nh, nope, rope, vd, applies):
     # kv_hadamard (src/model.rs:1529-1554): rotated cache bytes, to_f32 and attention against the oracle in the same
     # mode; widths that are not whole 64-chunks leave the option without effect, as in the reference
