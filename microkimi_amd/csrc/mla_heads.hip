@@ -293,8 +293,9 @@ struct G8Pos {
     float vs;
 };
 
+constexpr int G8_U = 2;  // positions a wave takes per step (4 measured the same with twice the registers)
 __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
-        constexpr int NOPE = 128, ROPE = 64, VD = 128, U = 4;
+        constexpr int NOPE = 128, ROPE = 64, VD = 128, U = G8_U;
     __shared__ float o_l[4][8][VD + 4];
     __shared__ float m_l[4][8], l_l[4][8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -314,8 +315,8 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
     const int hl = lane >> 3, c = lane & 7, h = hg * 8 + hl;
     const uint32_t nh = (uint32_t)a.nh;
     const int n_pos = a.n_pos0 + qi;
-    // Split s takes the steps (16 positions) s, s + n_splits, ...: at any time the launch reads one compact window of the
-    // cache (n_splits x 16 positions), not n_splits distant ranges.  (The softmax partials do not care which positions a
+    // Split s takes the steps (4 U positions) s, s + n_splits, ...: at any time the launch reads one compact window of the
+    // cache (n_splits x 4 U positions), not n_splits distant ranges.  (The softmax partials do not care which positions a
     // split holds.)
     const int p_end = n_pos;
     const uint32_t last = (uint32_t)n_pos - 1u;
@@ -357,9 +358,7 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
     for (int e = 0; e < 16; e++) o[e] = 0.0f;
     float m = -INFINITY, l = 0.0f;
     // byte offsets are 32-bit (the host checks positions * heads * 128 < 2^32); a position past the end re-reads the last one
-    static_assert(U == 4, "a step is 16 positions");
-    for (int t0 = split * 16 + wave; t0 < p_end; t0 += 16 * a.n_splits) {
-        G8Pos t[U];
+    auto load_step = [&](G8Pos *t, int t0) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const uint32_t j = min((uint32_t)(t0 + 4 * u), last);
@@ -371,6 +370,12 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
             t[u].v = mk_ldg128_off_nt(a.vq, row * VD + c * 16);
             t[u].vs = mk_ldg_f32_off(a.vs, (row * (VD / 32) + (c >> 1)) * 4);
         }
+    };
+    const int stride = 4 * U * a.n_splits;
+    G8Pos t[U], nx[U];
+    load_step(t, split * 4 * U + wave);
+    for (int t0 = split * 4 * U + wave; t0 < p_end; t0 += stride) {
+        load_step(nx, t0 + stride);  // the next step's values are requested before this step is worked on
         // ---- scores (src/model.rs:1833-1851): integer block dot, the block's scale product, the f32 rope part
         float s[U];
         float m_new = m;
@@ -409,6 +414,8 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
                 o[4 * d + 3] += ps * (float)(w >> 24);
             }
         }
+#pragma unroll
+        for (int u = 0; u < U; u++) t[u] = nx[u];
     }
     // ---- the four waves' states of a head meet (a wave without a position has m = -inf, l = 0, o = 0: weight 0)
 #pragma unroll
@@ -611,8 +618,8 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
         const int tps = (tiles + want - 1) / want;
         split_len = tps * TJ;
         n_splits = (tiles + tps - 1) / tps;
-        if (g8) {  // interleaved steps of 16 positions: any count up to the number of steps
-            const int steps = (int)((pos0 + 1 + 15) / 16);
+        if (g8) {  // interleaved steps of 4 U positions: any count up to the number of steps
+            const int steps = (int)((pos0 + 4 * G8_U) / (4 * G8_U));
             n_splits = (int)((MK_TUNE("MK_MLA_HEADS_WGS", 768) + nh / 8 - 1) / (nh / 8));
             if (n_splits > MAX_SPLITS) n_splits = MAX_SPLITS;
             if (n_splits > steps) n_splits = steps;
