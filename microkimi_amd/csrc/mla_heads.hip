@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void heads_decode_kernel(HeadsArgs a) {
 // every 4th position, 8 lanes a head.  One load instruction of a wave is then 1 KB of consecutive bytes (the K rows, or
 // the V rows, of the 8 heads at one position), the 8 heads' block scales are exactly one 128-byte line, the rope row is
 // read once for the 8 heads.  Every wave runs its own online softmax over its positions (no barrier and no LDS in the
-// loop); the four states of a head meet once at the end.  nh % 8 == 0.
+// loop); the four states of a head meet once at the end.
 struct G8Pos {
     mk_i4 k;
     float ks;
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
     __shared__ float o_l[4][8][VD + 4];
     __shared__ float m_l[4][8], l_l[4][8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hgroups = a.nh >> 3;
+    const int hgroups = (a.nh + 7) >> 3;  // a last group with fewer than 8 heads re-reads the last head in its idle lanes
     // consecutive workgroup ids go round the 8 XCDs (each with its own L2): XCD x takes the splits x, x + 8, ... with all
     // their head groups, so a position's rope row is fetched by one of them only
     int split, hg;
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
         hg = blockIdx.x - split * hgroups;
     }
     const int qi = blockIdx.y;
-    const int hl = lane >> 3, c = lane & 7, h = hg * 8 + hl;
+    const int hl = lane >> 3, c = lane & 7, h = min(hg * 8 + hl, a.nh - 1);
     const uint32_t nh = (uint32_t)a.nh;
     const int n_pos = a.n_pos0 + qi;
     // Split s takes the steps (4 U positions) s, s + n_splits, ...: at any time the launch reads one compact window of the
@@ -436,6 +436,7 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
             den += wt * l_l[w][hh];
         }
         const size_t hrow = (size_t)hg * 8 + hh;
+        if (hrow >= nh) continue;
         if (a.n_splits == 1) {
             a.out[((size_t)qi * nh + hrow) * VD + d] = num / den;
         } else {
@@ -596,8 +597,8 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.out = out;
     const int had = had_applies(hadamard, nope, vd);
     a.had_k = had ? 1.0f / 64.0f : 1.0f;
-    // the reference's own head shape in whole groups of 8 heads takes the all-heads kernel
-    const bool g8 = nope == 128 && rope == 64 && vd == 128 && nh % 8 == 0 && (pos0 + m) * nh * 128 < 0xFFFFFFFFull &&
+    // the reference's own head shape takes the all-heads kernel
+    const bool g8 = nope == 128 && rope == 64 && vd == 128 && (pos0 + m) * nh * 128 < 0xFFFFFFFFull &&
                       ((uintptr_t)vq & 15) == 0 && ((uintptr_t)kr & 15) == 0 && ((uintptr_t)q & 15) == 0 && !MK_TUNE("MK_MLA_HEADS_GENERIC", 0);
     if (g8 && !had) {
         a.qq = nullptr;  // the all-heads kernel quantizes the query itself
@@ -609,6 +610,7 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     }
     // one query: split the context so that about 1024 workgroups stream the cache; several queries (prefill): the
     // (query, head) grid is parallel enough, one split each
+    const int hgroups = (int)((nh + 7) / 8);
     int n_splits = 1, split_len = (int)((pos0 + m + TJ - 1) / TJ) * TJ;
     if (m == 1) {
         const int tiles = (int)((pos0 + 1 + TJ - 1) / TJ);
@@ -620,7 +622,7 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
         n_splits = (tiles + tps - 1) / tps;
         if (g8) {  // interleaved steps of 4 U positions: any count up to the number of steps
             const int steps = (int)((pos0 + 4 * G8_U) / (4 * G8_U));
-            n_splits = (int)((MK_TUNE("MK_MLA_HEADS_WGS", 768) + nh / 8 - 1) / (nh / 8));
+            n_splits = (int)((MK_TUNE("MK_MLA_HEADS_WGS", 768) + hgroups - 1) / hgroups);
             if (n_splits > MAX_SPLITS) n_splits = MAX_SPLITS;
             if (n_splits > steps) n_splits = steps;
         }
@@ -628,7 +630,7 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.split_len = split_len;
     a.n_splits = n_splits;
     if (g8) {
-        hipLaunchKernelGGL(heads_decode_g8_kernel, dim3((unsigned)(n_splits * (nh / 8)), (unsigned)m), dim3(256), 0, st, a);
+        hipLaunchKernelGGL(heads_decode_g8_kernel, dim3((unsigned)(n_splits * hgroups), (unsigned)m), dim3(256), 0, st, a);
     } else {
         hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);
     }

@@ -57,8 +57,9 @@ def test_push_assign_and_to_f32_are_the_reference_bytes(n, nh, nope, rope, vd):
 @pytest.mark.parametrize("n,nh,nope,rope,vd,qscale", [(1, 4, 128, 64, 128, 1.0), (7, 4, 128, 64, 128, 1.0), (64, 6, 128, 64, 128, 1.0),
                                                      (65, 6, 128, 64, 128, 1.0), (512, 6, 128, 64, 128, 1.0), (300, 5, 64, 32, 96, 3.0),
                                                      (4200, 24, 128, 64, 128, 1.0), (130, 2, 256, 64, 512, 0.0),
-                                                     # head counts in whole groups of 8 at the reference's head shape take the
-                                                     # streaming kernel: the same lengths, a context split over the chip, zero query
+                                                     # the reference's head shape (128 + 64 / 128) takes the all-heads kernel, 8 heads a
+                                                     # workgroup (the cases above with 4, 6 and 24 heads too; other shapes the
+                                                     # per-head one): whole groups, a context split over the chip, zero query
                                                      (1, 8, 128, 64, 128, 1.0), (7, 8, 128, 64, 128, 1.0), (64, 16, 128, 64, 128, 1.0),
                                                      (65, 8, 128, 64, 128, 3.0), (512, 8, 128, 64, 128, 1.0), (2100, 96, 128, 64, 128, 1.0),
                                                      (200, 8, 128, 64, 128, 0.0)])
@@ -82,8 +83,8 @@ def test_decode_matches_mla_attn_flash_q8_mqa(n, nh, nope, rope, vd, qscale):
 
 @pytest.mark.parametrize("nh", [6, 8])
 def test_prefill_loop_equals_one_decode_per_position(nh):
-    # mla_prefill (src/model.rs:2080-2102): query i over the positions 0 ..= pos0 + i (6 heads: the general kernel,
-    # 8: the streaming one)
+    # mla_prefill (src/model.rs:2080-2102): query i over the positions 0 ..= pos0 + i (6 heads: a partial group of the
+    # all-heads kernel, 8: a whole one)
     from microkimi_amd import model
     nope, rope, vd, n0, m = 128, 64, 128, 40, 33
     k, v = rows(n0 + m, nh, nope, rope, vd, 5)
