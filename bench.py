@@ -423,6 +423,37 @@ def bench_mla(torch, cpu=True):
     return res
 
 
+def bench_lm_head_published(torch):
+    """The q8 lm_head at the shape the reference publishes (KIMI.md:100: 65536 x 7168, int8 + f32 scale per 32 as
+    Q8Head::from_f32 builds it, 5.1 ms per call on 10 CPU threads).  Two heads alternate (528 MB each)."""
+    from microkimi_amd import model
+    rows, cols = 65536, 7168
+    g = torch.Generator(device="cuda").manual_seed(7)
+    heads = []
+    for _ in range(2):
+        q = torch.randint(-127, 128, (rows, cols), dtype=torch.int8, device="cuda", generator=g)
+        sc = torch.rand((rows, cols // 32), device="cuda", generator=g) * 0.01 + 0.001
+        heads.append(model.Q8Head.from_q8(q, sc, rows, cols))
+    x = torch.randn((1, cols), device="cuda", generator=g)
+    out = torch.empty((1, rows), device="cuda")
+    it = [0]
+
+    def step():
+        h = heads[it[0] % 2]
+        it[0] += 1
+        h.matvec(x, out)
+
+    ms_eager = time_region(torch, step, 40, warmup=6)
+    it[0] = 0
+    ms_graph = time_graph(torch, [step] * 8)
+    ms = ms_graph if ms_graph is not None else ms_eager
+    alg = rows * cols + rows * (cols // 32) * 4 + cols * 4 + rows * 4
+    return {"workload": "q8 lm_head 65536 x 7168, f32 scales, batch 1 (quantize + GEMV); the reference publishes 5.1 ms on 10 CPU threads",
+            "us": ms * 1e3, "us_python_loop": ms_eager * 1e3, "timing": "graph replay" if ms_graph is not None else "python loop",
+            "alg_bytes": alg, "gbs": alg / (ms * 1e-3) / 1e9, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "published_cpu_ms": 5.1, "published_cpu_ms_over_this": 5.1 / ms}
+
+
 def bench_mla_heads(torch):
     """The attention over the reference's own cache layout (per head a q8 K-nope row and a q8 V row, one f32 rope row per
     position) on the case the reference publishes: 96 heads, nope 128 + rope 64, v 128 (KIMI.md:96, bench code
@@ -559,7 +590,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="",
-                    help="comma-separated names of extras (mxfp4_gemv, moe_decode, mla_decode, mla_heads_decode, grouped_gemm, vq1_gemv): run only "
+                    help="comma-separated names of extras (mxfp4_gemv, moe_decode, mla_decode, mla_heads_decode, lm_head_published_shape, grouped_gemm, vq1_gemv): run only "
                          "those and print their figures as one JSON object (a development aid; the contract line needs a full run)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain 1 GiB device copies (a kernel of known traffic to scale rocprofv3 --pmc byte counters by)")
@@ -584,7 +615,7 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
     if args.only:
-        table = {"mxfp4_gemv": bench_mxfp4_gemv, "moe_decode": bench_moe, "mla_decode": bench_mla, "mla_heads_decode": bench_mla_heads,
+        table = {"mxfp4_gemv": bench_mxfp4_gemv, "moe_decode": bench_moe, "mla_decode": bench_mla, "mla_heads_decode": bench_mla_heads, "lm_head_published_shape": bench_lm_head_published,
                  "grouped_gemm": bench_gemm, "vq1_gemv": bench_vq1}
         res = {}
         for name in args.only.split(","):
@@ -604,7 +635,7 @@ def main():
     torch.cuda.empty_cache()
     extras = {"lm_head_batch8": head.pop("batch8")}
     if not args.no_extras:
-        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("mla_heads_decode", bench_mla_heads),
+        for name, fn in (("mxfp4_gemv", bench_mxfp4_gemv), ("moe_decode", bench_moe), ("mla_decode", bench_mla), ("mla_heads_decode", bench_mla_heads), ("lm_head_published_shape", bench_lm_head_published),
                          ("grouped_gemm", bench_gemm), ("vq1_gemv", bench_vq1)):
             log(name, "...")
             try:
