@@ -496,6 +496,24 @@ def bench_mla_heads(torch):
         if ctx == 16384:
             res[f"ctx{ctx}"]["published_cpu_ms_over_this"] = 79.7 / ms
         del caches
+    # the attention loop of mla_prefill over the same cache: a 512-token chunk at the start of a prompt and behind 3584
+    # cached positions (query i attends 0 ..= pos0 + i); 16 queries of a head share the K / V tiles on the matrix cores
+    m = 512
+    qs = torch.randn((m, nh * (nope + rope)), device="cuda", generator=g)
+    for pos0 in (0, 3584):
+        c = model.MlaHeadsCache(nh, nope, rope, vd, pos0 + m)
+        c.kq.copy_(torch.randint(-127, 128, c.kq.shape, dtype=torch.int8, device="cuda", generator=g))
+        c.vq.copy_(torch.randint(-127, 128, c.vq.shape, dtype=torch.int8, device="cuda", generator=g))
+        c.ks.copy_(torch.rand(c.ks.shape, device="cuda", generator=g) * 0.03 + 0.005)
+        c.vs.copy_(torch.rand(c.vs.shape, device="cuda", generator=g) * 0.03 + 0.005)
+        c.kr.copy_(torch.randn(c.kr.shape, device="cuda", generator=g))
+        c.n = pos0 + m
+        ms = time_region(torch, lambda: c.attn(qs, pos0, scale), 10, warmup=2)
+        pairs = sum(pos0 + i + 1 for i in range(m))
+        flops = 2.0 * pairs * nh * (nope + rope + vd)
+        res[f"prefill_{m}_at_{pos0}"] = {"ms": ms, "query_position_pairs": pairs, "tflops": flops / (ms * 1e-3) / 1e12,
+                                         "cache_bytes": (pos0 + m) * (nh * (nope + vd) * 9 // 8 + rope * 4)}
+        del c
     return res
 
 

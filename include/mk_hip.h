@@ -311,7 +311,10 @@ int mk_dev_mla_cache_append(const float *latent, const float *rope, size_t L, si
  * _q8_attn  mla_attn_flash_q8_mqa (src/model.rs:1804-1908) for m queries q [m][nh][nope+rope]: query i attends the
  *           positions 0 ..= pos0 + i (m = 1: the decode step of mla_forward, src/model.rs:1980-1985; m > 1: the
  *           per-position loop of mla_prefill, src/model.rs:2080-2102).  out [m][nh][vd].
- *           workspace: mk_mla_heads_workspace_bytes(m, nh, nope, vd).
+ *           workspace: mk_mla_heads_workspace_bytes(m, nh, nope, vd).  At the reference's own head shape (nope 128, rope 64,
+ *           vd 128) one query streams the cache once for all heads and 16 or more queries share every K / V tile on the
+ *           matrix cores; other shapes take a per-head kernel.  The results do not depend on which one runs beyond the
+ *           order of the sums.
  * hadamard  nonzero: the cache is kept in the rotated form of kv_hadamard (src/model.rs:1529-1554, MICROKIMI_KV_HADAMARD=1):
  *           hadamard64 on every 64-chunk of a K-nope row, a V row and the query's nope part before quantization, the
  *           factor 1/64 on the latent score, the output rotated back.  As in the reference it takes effect only when

@@ -449,6 +449,145 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
     }
 }
 
+// The attention loop of mla_prefill (src/model.rs:2080-2102) for the same head shape: 16 queries of one head share every
+// K / V tile on the matrix cores -- a wave per (head, 16 queries), tiles of 16 positions -- instead of one pass over the
+// cache per query.  The arithmetic keeps the reference's terms: integer block dots (v_mfma_i32_16x16x64_i8, issued once
+// with the second block's query bytes zeroed and once whole: the second block's dot is the difference), the per-block
+// scale product in f32, the f32 rope dot and P V on the f32 matrix instruction (v_mfma_f32_16x16x4_f32: f32 products,
+// f32 sums; V = scale * byte is formed exactly as the decode kernel forms it).  Only the order of the sums differs.
+// Operands (lane = j + 16 g): the scores are computed transposed, positions as rows and queries as columns, so that the
+// probabilities a lane holds -- query j, positions 4 g + r -- are already the B operand of P V (k = g at step r); the A
+// operand of P V is V transposed with output row i of tile t standing for dim 8 i + t, so a lane reads 8 consecutive V
+// bytes per position and ends with 8 consecutive output values per accumulator row.
+__global__ __launch_bounds__(64) void heads_prefill_mfma_kernel(HeadsArgs a, int m) {
+    constexpr int NOPE = 128, ROPE = 64, VD = 128;
+    const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
+    const int qg = (int)gridDim.x - 1 - (int)blockIdx.x;  // the groups with the longest contexts start first
+    const int h = blockIdx.y;
+    const uint32_t nh = (uint32_t)a.nh;
+    const int qi = min(qg * 16 + j, m - 1);            // this lane's query (a column of the score tile)
+    const size_t qrow = (size_t)qi * nh + h;
+    const int lim = a.n_pos0 - 1 + qi;                 // its last position
+    const int t_end = a.n_pos0 + min(qg * 16 + 15, m - 1);  // positions the group's last query sees
+    const uint32_t last = (uint32_t)(a.n_pos0 + m - 2);      // last cached position the call may read
+    // query side
+    mk_i4 bq[2], bq0[2];
+    float qsv[4], qr[16];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; s2++) {
+        bq[s2] = mk_ldg128(a.qq + qrow * NOPE + 64 * s2 + 16 * g);
+        bq0[s2] = g < 2 ? bq[s2] : mk_i4{0, 0, 0, 0};
+    }
+    {
+        const mk_f4 v = *reinterpret_cast<const mk_f4 *>(a.qs + qrow * (NOPE / 32));
+        qsv[0] = v.x * a.had_k, qsv[1] = v.y * a.had_k, qsv[2] = v.z * a.had_k, qsv[3] = v.w * a.had_k;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const mk_f4 v = *reinterpret_cast<const mk_f4 *>(a.q + qrow * (NOPE + ROPE) + NOPE + 16 * g + 4 * i);
+        qr[4 * i] = v.x, qr[4 * i + 1] = v.y, qr[4 * i + 2] = v.z, qr[4 * i + 3] = v.w;
+    }
+    mk_f4 o[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) o[t] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    float mrun = -INFINITY, lrun = 0.0f;
+    const mk_i4 zero4 = {0, 0, 0, 0};
+    // a tile's values as this lane needs them: as row j of the tile (position t0 + j) and as the rows 4 g + r of the results
+    struct Tile {
+        mk_i4 ak[2];
+        mk_f4 ar[4];
+        mk_f4 ksv[4];
+        mk_u2 vb[4];
+        float vsv[4];
+    };
+    auto load_tile = [&](Tile &T, int t0) {
+        const uint32_t pa = min((uint32_t)(t0 + j), last);
+        const uint32_t rowa = pa * nh + (uint32_t)h;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) T.ak[s2] = mk_ldg128_off(a.kq, rowa * NOPE + 64 * s2 + 16 * g);
+#pragma unroll
+        for (int i = 0; i < 4; i++) T.ar[i] = __builtin_bit_cast(mk_f4, mk_ldg128_off(a.kr, (pa * ROPE + 16 * g + 4 * i) * 4));
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t pr = min((uint32_t)(t0 + 4 * g + r), last);
+            const uint32_t rowr = pr * nh + (uint32_t)h;
+            T.ksv[r] = __builtin_bit_cast(mk_f4, mk_ldg128_off(a.ks, rowr * (NOPE / 32) * 4));
+            T.vb[r] = mk_ldg64(reinterpret_cast<const uint8_t *>(a.vq) + (size_t)rowr * VD + 8 * j);
+            T.vsv[r] = mk_ldg_f32_off(a.vs, (rowr * (VD / 32) + (j >> 2)) * 4);
+        }
+    };
+    // (requesting the next tile a tile ahead was measured: the same time with 50 more registers -- the kernel is bound by
+    // the issue of its matrix and vector instructions, 41 % and 48 % of the cycles, not by the loads)
+    for (int t0 = 0; t0 < t_end; t0 += 16) {
+        Tile cur;
+        load_tile(cur, t0);
+        const mk_i4 *ak = cur.ak;
+        const mk_f4 *ar = cur.ar, *ksv = cur.ksv;
+        const mk_u2 *vb = cur.vb;
+        const float *vsv = cur.vsv;
+        // ---- scores, transposed: rows = positions, columns = queries
+        mk_f4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) {
+            const mk_i4 c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(ak[s2], bq0[s2], zero4, 0, 0, 0);
+            const mk_i4 cf = __builtin_amdgcn_mfma_i32_16x16x64_i8(ak[s2], bq[s2], zero4, 0, 0, 0);
+            sc.x = fmaf(qsv[2 * s2 + 1] * ksv[0][2 * s2 + 1], (float)(cf[0] - c0[0]), fmaf(qsv[2 * s2] * ksv[0][2 * s2], (float)c0[0], sc.x));
+            sc.y = fmaf(qsv[2 * s2 + 1] * ksv[1][2 * s2 + 1], (float)(cf[1] - c0[1]), fmaf(qsv[2 * s2] * ksv[1][2 * s2], (float)c0[1], sc.y));
+            sc.z = fmaf(qsv[2 * s2 + 1] * ksv[2][2 * s2 + 1], (float)(cf[2] - c0[2]), fmaf(qsv[2 * s2] * ksv[2][2 * s2], (float)c0[2], sc.z));
+            sc.w = fmaf(qsv[2 * s2 + 1] * ksv[3][2 * s2 + 1], (float)(cf[3] - c0[3]), fmaf(qsv[2 * s2] * ksv[3][2 * s2], (float)c0[3], sc.w));
+        }
+        // (four chains of four dependent matrix instructions, not one of sixteen)
+        mk_f4 c4[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            c4[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ar[i].x, qr[4 * i], mk_f4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            c4[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ar[i].y, qr[4 * i + 1], c4[i], 0, 0, 0);
+            c4[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ar[i].z, qr[4 * i + 2], c4[i], 0, 0, 0);
+            c4[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ar[i].w, qr[4 * i + 3], c4[i], 0, 0, 0);
+        }
+        const mk_f4 cr = (c4[0] + c4[1]) + (c4[2] + c4[3]);
+        float sv[4];
+        sv[0] = (t0 + 4 * g + 0) <= lim ? (sc.x + cr.x) * a.scale : -INFINITY;
+        sv[1] = (t0 + 4 * g + 1) <= lim ? (sc.y + cr.y) * a.scale : -INFINITY;
+        sv[2] = (t0 + 4 * g + 2) <= lim ? (sc.z + cr.z) * a.scale : -INFINITY;
+        sv[3] = (t0 + 4 * g + 3) <= lim ? (sc.w + cr.w) * a.scale : -INFINITY;
+        // ---- online softmax of query j: its 16 scores of the tile sit in the lanes j, j + 16, j + 32, j + 48
+        // (position 0 is inside every query's range, so the running maximum is finite from the first tile on)
+        const float tm = mk_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+        const float m_new = fmaxf(mrun, tm);
+        const float corr = expf(mrun - m_new);
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) p[r] = expf(sv[r] - m_new);  // a position past the query's range: 0
+        lrun = lrun * corr + mk_rows_sum((p[0] + p[1]) + (p[2] + p[3]));
+        mrun = m_new;
+        if (__builtin_amdgcn_ballot_w64(corr != 1.0f)) {  // (after the first tiles a new maximum is rare)
+#pragma unroll
+            for (int t = 0; t < 8; t++) o[t] *= corr;
+        }
+        // ---- out^T += V^T P^T: step r takes the positions t0 + 4 g + r (k = g)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int byte = (int)(int8_t)((t < 4 ? vb[r][0] : vb[r][1]) >> (8 * (t & 3)));
+                o[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vsv[r] * (float)byte, p[r], o[t], 0, 0, 0);
+            }
+        }
+    }
+    // accumulator row i = 4 g + r of tile t is dim 8 i + t of query j
+    if (qg * 16 + j < m) {
+        const float inv = 1.0f / lrun;
+        float *dst = a.out + qrow * VD;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int d0 = 8 * (4 * g + r);
+            *reinterpret_cast<mk_f4 *>(dst + d0) = mk_f4{o[0][r] * inv, o[1][r] * inv, o[2][r] * inv, o[3][r] * inv};
+            *reinterpret_cast<mk_f4 *>(dst + d0 + 4) = mk_f4{o[4][r] * inv, o[5][r] * inv, o[6][r] * inv, o[7][r] * inv};
+        }
+    }
+}
+
 // log-sum-exp merge of the splits of one query: a workgroup per head
 __global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
                                                           int nh, int vd, int n_splits, float *__restrict__ out) {
@@ -600,7 +739,8 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     // the reference's own head shape takes the all-heads kernel
     const bool g8 = nope == 128 && rope == 64 && vd == 128 && (pos0 + m) * nh * 128 < 0xFFFFFFFFull &&
                       ((uintptr_t)vq & 15) == 0 && ((uintptr_t)kr & 15) == 0 && ((uintptr_t)q & 15) == 0 && !MK_TUNE("MK_MLA_HEADS_GENERIC", 0);
-    if (g8 && !had) {
+    const bool many = g8 && m >= (size_t)MK_TUNE("MK_MLA_HEADS_PREFILL_MIN", 16);
+    if (g8 && !had && !many) {
         a.qq = nullptr;  // the all-heads kernel quantizes the query itself
     } else {
         const int rows = (int)(m * nh);
@@ -629,7 +769,11 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     }
     a.split_len = split_len;
     a.n_splits = n_splits;
-    if (g8) {
+    if (g8 && m >= (size_t)MK_TUNE("MK_MLA_HEADS_PREFILL_MIN", 16) && ((uintptr_t)out & 15) == 0 && ((uintptr_t)ks & 15) == 0 &&
+        ((uintptr_t)vq & 7) == 0) {
+        // several queries: 16 of them share every K / V tile on the matrix cores
+        hipLaunchKernelGGL(heads_prefill_mfma_kernel, dim3((unsigned)((m + 15) / 16), (unsigned)nh), dim3(64), 0, st, a, (int)m);
+    } else if (g8) {
         hipLaunchKernelGGL(heads_decode_g8_kernel, dim3((unsigned)(n_splits * hgroups), (unsigned)m), dim3(256), 0, st, a);
     } else {
         hipLaunchKernelGGL(heads_decode_kernel, dim3((unsigned)n_splits, (unsigned)nh, (unsigned)m), dim3(256), 0, st, a);

@@ -81,6 +81,28 @@ def test_decode_matches_mla_attn_flash_q8_mqa(n, nh, nope, rope, vd, qscale):
         assert rel_l2(got, want) <= TOL, (pos, rel_l2(got, want))
 
 
+@pytest.mark.parametrize("nh,n0,m,had", [(8, 300, 70, False), (3, 0, 40, False), (16, 1000, 16, True), (4, 17, 130, False)])
+def test_prefill_on_the_matrix_cores(nh, n0, m, had):
+    # 16 and more queries at the reference's head shape share the K / V tiles on the matrix cores: every query against
+    # its own decode in the oracle (a prompt from position 0, a chunk behind a long context, a last group of queries
+    # that is not full, the Hadamard option)
+    from microkimi_amd import model
+    nope, rope, vd = 128, 64, 128
+    k, v = rows(n0 + m, nh, nope, rope, vd, 50 + m)
+    rng = np.random.default_rng(m)
+    q = rng.standard_normal((m, nh * (nope + rope))).astype(np.float32)
+    scale = float(np.float32(nope + rope) ** np.float32(-0.5))
+    want_c = oracle.MlaCache(nh, nope, rope, vd, had=had, capacity=n0 + m)
+    for i in range(n0 + m):
+        want_c.push(k[i], v[i])
+    c = model.MlaHeadsCache(nh, nope, rope, vd, n0 + m, hadamard=had)
+    c.push(dev(k), dev(v))
+    got = c.attn(dev(q), n0, scale).cpu().numpy()
+    assert np.isfinite(got).all()
+    worst = max(rel_l2(got[i], oracle.mla_attn_flash_q8_mqa(want_c, q[i], n0 + i, scale)) for i in range(m))
+    assert worst <= TOL, worst
+
+
 @pytest.mark.parametrize("nh", [6, 8])
 def test_prefill_loop_equals_one_decode_per_position(nh):
     # mla_prefill (src/model.rs:2080-2102): query i over the positions 0 ..= pos0 + i (6 heads: a partial group of the
