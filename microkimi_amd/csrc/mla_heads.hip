@@ -135,6 +135,31 @@ __global__ __launch_bounds__(256) void heads_q_prep_kernel(const float *__restri
     quantize_block32(v, qq + (size_t)r * nope + g * 32, qs + blk, j);
 }
 
+// The same without the rotation, 8 lanes a block and four values a lane (quantize_q8_into, src/q8.rs:57-68).
+__global__ __launch_bounds__(256) void heads_q_prep4_kernel(const float *__restrict__ q, size_t n_blocks, int nope, int rope,
+                                                            int8_t *__restrict__ qq, float *__restrict__ qs) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_blocks * 8) return;  // whole groups of 8 lanes leave together
+    const int nb = nope / 32;
+    const size_t blk = i >> 3, r = blk / nb;
+    const int g = (int)(blk - r * nb), c = (int)(i & 7);
+    const mk_f4 v = *reinterpret_cast<const mk_f4 *>(q + r * (nope + rope) + g * 32 + c * 4);
+    float mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    mx = fmaxf(mx, mk_dpp<0xB1>(mx));
+    mx = fmaxf(mx, mk_dpp<0x4E>(mx));
+    mx = fmaxf(mx, mk_dpp<0x141>(mx));
+    const float dx = fmaxf(mx, 0.0f) / 127.0f;  // (a block of NaN only: the reference's maximum, folded from 0, is 0)
+    uint32_t packed = 0;
+    if (dx != 0.0f) {
+        float qf[4];
+        mk_q8_round4(v, dx, qf);
+        packed = ((uint32_t)(int)qf[0] & 255u) | (((uint32_t)(int)qf[1] & 255u) << 8) | (((uint32_t)(int)qf[2] & 255u) << 16) |
+                 ((uint32_t)(int)qf[3] << 24);
+    }
+    reinterpret_cast<uint32_t *>(qq)[i] = packed;  // qq is [rows][nope]: block blk starts at byte 32 blk
+    if (c == 0) qs[blk] = dx;
+}
+
 struct HeadsArgs {
     const int8_t *kq;
     const float *ks;
@@ -744,8 +769,14 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
         a.qq = nullptr;  // the all-heads kernel quantizes the query itself
     } else {
         const int rows = (int)(m * nh);
-        hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, had, qq,
-                           qs);
+        if (!had && ((uintptr_t)q & 15) == 0 && (nope + rope) % 4 == 0) {
+            const size_t n_blocks = (size_t)rows * (nope / 32);
+            hipLaunchKernelGGL(heads_q_prep4_kernel, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, st, q, n_blocks, (int)nope, (int)rope,
+                               qq, qs);
+        } else {
+            hipLaunchKernelGGL(heads_q_prep_kernel, dim3((unsigned)((rows * (nope / 32) + 7) / 8)), dim3(256), 0, st, q, rows, (int)nope, (int)rope, had,
+                               qq, qs);
+        }
         if ((s = mk_launch_status("heads_q_prep")) != MK_OK) return s;
     }
     // one query: split the context so that about 1024 workgroups stream the cache; several queries (prefill): the
