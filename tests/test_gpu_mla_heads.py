@@ -151,6 +151,11 @@ def test_host_level_handle_in_the_reference_layout():
         check(lib.mk_mla_attn_prefill(h, hptr(q), 4, scale, hptr(outs)))  # the last 4 positions as a prompt
         for i in range(4):
             assert rel_l2(outs[i], oracle.mla_attn_flash_q8_mqa(want_c, q[i], n - 4 + i, scale)) <= TOL
+        q20 = rng.standard_normal((20, nh * (nope + rope))).astype(np.float32)
+        outs = np.empty((20, nh * vd), np.float32)
+        check(lib.mk_mla_attn_prefill(h, hptr(q20), 20, scale, hptr(outs)))  # 16 and more queries: the matrix-core kernel
+        for i in range(20):
+            assert rel_l2(outs[i], oracle.mla_attn_flash_q8_mqa(want_c, q20[i], n - 20 + i, scale)) <= TOL
         assert lib.mk_mla_cache_push(h, hptr(k[0]), hptr(v[0])) == -5   # full: MK_ERR_NOMEM
     finally:
         lib.mk_mla_cache_free(h)
