@@ -484,7 +484,7 @@ __global__ __launch_bounds__(256) void heads_decode_g8_kernel(HeadsArgs a) {
 // probabilities a lane holds -- query j, positions 4 g + r -- are already the B operand of P V (k = g at step r); the A
 // operand of P V is V transposed with output row i of tile t standing for dim 8 i + t, so a lane reads 8 consecutive V
 // bytes per position and ends with 8 consecutive output values per accumulator row.
-__global__ __launch_bounds__(64) void heads_prefill_mfma_kernel(HeadsArgs a, int m) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) void heads_prefill_mfma_kernel(HeadsArgs a, int m) {
     constexpr int NOPE = 128, ROPE = 64, VD = 128;
     const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
     const int qg = (int)gridDim.x - 1 - (int)blockIdx.x;  // the groups with the longest contexts start first
