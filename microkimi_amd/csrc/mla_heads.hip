@@ -614,6 +614,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3))) void he
 }
 
 // log-sum-exp merge of the splits of one query: a workgroup per head
+// GROUPS: thread groups that share out the splits of a dim; a workgroup takes 256 / GROUPS consecutive dims of a row
+// (blockIdx.y-th such chunk).  GROUPS = 0: the group count follows vd (256 / vd for vd <= 128, else a plain loop).
+template <int GROUPS>
 __global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restrict__ po, const float *__restrict__ pm, const float *__restrict__ pl,
                                                           int nh, int vd, int n_splits, float *__restrict__ out) {
     __shared__ float w_l[MAX_SPLITS];
@@ -623,9 +626,10 @@ __global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restric
     // The partials come from other compute dies: every dependent round of loads costs a trip to memory.  Narrow rows
     // (vd <= 128) take ONE round: the splits are shared out over 256 / vd groups of threads and a thread requests all
     // its partial values before the weights exist (a split past the end re-reads the last one with weight 0).
-    const int groups = vd <= 128 ? 256 / vd : 1;
-    constexpr int PER = MAX_SPLITS / 2;
-    const int sg = tid / vd, d = tid - sg * vd;
+    const int groups = GROUPS ? GROUPS : (vd <= 128 ? 256 / vd : 1);
+    constexpr int PER = MAX_SPLITS / (GROUPS ? GROUPS : 2);
+    const int vdc = GROUPS ? 256 / GROUPS : vd, d0 = GROUPS ? (int)blockIdx.y * vdc : 0;  // this workgroup's dims d0 .. d0 + vdc - 1
+    const int sg = tid / vdc, d = d0 + tid - sg * vdc;
     float pv[PER];
     if (groups > 1 && sg < groups) {
 #pragma unroll
@@ -656,9 +660,9 @@ __global__ __launch_bounds__(256) void heads_merge_kernel(const float *__restric
             part_l[tid] = num;
         }
         __syncthreads();
-        if (tid < vd) {
-            for (int g = 1; g < groups; g++) num += part_l[g * vd + tid];
-            out[(size_t)h * vd + tid] = num / den_l;
+        if (tid < vdc) {
+            for (int g = 1; g < groups; g++) num += part_l[g * vdc + tid];
+            out[(size_t)h * vd + d0 + tid] = num / den_l;
         }
         return;
     }
@@ -811,7 +815,10 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     }
     if ((s = mk_launch_status("heads_decode")) != MK_OK) return s;
     if (n_splits > 1) {
-        hipLaunchKernelGGL(heads_merge_kernel, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
+        if (vd % 64 == 0 && vd <= 512 && n_splits > 16 && MK_TUNE("MK_MLA_HEADS_MERGE4", 1))  // 64 dims a workgroup, four split groups
+            hipLaunchKernelGGL(heads_merge_kernel<4>, dim3((unsigned)nh, (unsigned)(vd / 64)), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
+        else
+            hipLaunchKernelGGL(heads_merge_kernel<0>, dim3((unsigned)nh), dim3(256), 0, st, a.po, a.pm, a.pl, (int)nh, (int)vd, n_splits, out);
         if ((s = mk_launch_status("heads_merge")) != MK_OK) return s;
     }
     if (had) {
