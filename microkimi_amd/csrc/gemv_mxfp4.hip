@@ -359,6 +359,128 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__res
 }
 
 
+// matvec_packed_nt for four and more positions on the f32 matrix instruction (v_mfma_f32_16x16x4_f32: f32 products, f32
+// sums), cols % 128 == 0.  A workgroup takes 16 weight rows, its four waves a quarter of the 128-column steps each; a
+// lane (i = lane % 16, g = lane / 16) holds the 32 weights of block 4 T + g of row i for step T, dequantized exactly
+// (e2m1 value times 2^(sb - 127): the scale rides on every weight because one instruction sums over four blocks), and
+// the 32 matching activations of position j = lane % 16.  Up to 64 positions a pass (four accumulator tiles) against the
+// same weight registers.  The terms are the reference's (src/model.rs:2412-2447); the order of the sums is not.
+template <int WAVES, int NTT>
+__global__ __launch_bounds__(64 * WAVES) void mxfp4_gemm_nt_mfma_kernel(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scales,
+                                                                        int rows, int nb, const float *__restrict__ x, int m,
+                                                                        float *__restrict__ out) {
+    __shared__ mk_f4 red_l[WAVES - 1][NTT][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
+    const int row = min((int)blockIdx.x * 16 + i, rows - 1);
+    const int tok0 = blockIdx.y * 16 * NTT;  // NTT tiles of 16 positions a pass (positions past the end: the last one, not stored)
+    const size_t cols = (size_t)nb * 32;
+    const int steps = nb / 4;
+    mk_f4 acc[NTT];
+#pragma unroll
+    for (int tt = 0; tt < NTT; tt++) acc[tt] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    // Everything is requested one item ahead: the next step's weights and scale byte before this step is worked on, the
+    // next tile's activations (from L2) before this tile's matrix instructions.  Past the end: the last one again.
+    auto load_w = [&](int T, mk_i4 &wq, uint32_t &sb) {
+        const size_t blk = (size_t)row * nb + 4 * min(T, steps - 1) + g;
+        wq = mk_ldg128_nt(packed + blk * 16);
+        sb = mk_ldg_u8(scales + blk);
+    };
+    auto load_x = [&](mk_f4 *xr, int T, int tt) {
+        const int tok = min(tok0 + 16 * tt + i, m - 1);
+        const mk_f4 *xv = reinterpret_cast<const mk_f4 *>(x + (size_t)tok * cols + (size_t)(4 * min(T, steps - 1) + g) * 32);
+#pragma unroll
+        for (int k = 0; k < 8; k++) xr[k] = xv[k];
+    };
+    mk_i4 wq, wq_n;
+    uint32_t sb, sb_n;
+    mk_f4 xa[8], xb[8];
+    load_w(wave, wq, sb);
+    load_x(xa, wave, 0);
+    for (int T = wave; T < steps; T += WAVES) {
+        load_w(T + WAVES, wq_n, sb_n);
+        __builtin_amdgcn_sched_barrier(0);
+        const float sc = mk_scale_from_byte(sb);
+        float wf[32];
+        // (the hardware conversion gives the e2m1 values; the power of two is applied in f32: exact)
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t wd = (uint32_t)wq[d];
+            const mk_f2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 0), p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 1);
+            const mk_f2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 2), p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 3);
+            wf[8 * d + 0] = p0.x * sc, wf[8 * d + 1] = p0.y * sc, wf[8 * d + 2] = p1.x * sc, wf[8 * d + 3] = p1.y * sc;
+            wf[8 * d + 4] = p2.x * sc, wf[8 * d + 5] = p2.y * sc, wf[8 * d + 6] = p3.x * sc, wf[8 * d + 7] = p3.y * sc;
+        }
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            if (tt + 1 < NTT) load_x(xb, T, tt + 1);
+            else load_x(xb, T + WAVES, 0);
+            __builtin_amdgcn_sched_barrier(0);  // (the requests stay in front of the matrix instructions that cover them)
+            // two chains of dependent matrix instructions, added at the end
+            mk_f4 c1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) {
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k], xa[k].x, acc[tt], 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 4], xa[k + 1].x, c1, 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 1], xa[k].y, acc[tt], 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 5], xa[k + 1].y, c1, 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 2], xa[k].z, acc[tt], 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 6], xa[k + 1].z, c1, 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 3], xa[k].w, acc[tt], 0, 0, 0);
+                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 7], xa[k + 1].w, c1, 0, 0, 0);
+            }
+            acc[tt] += c1;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) xa[k] = xb[k];
+        }
+        wq = wq_n;
+        sb = sb_n;
+    }
+    // the waves' partial sums meet; result tile: column = position j = lane % 16, rows 4 g + r
+    if (wave > 0) {
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) red_l[wave - 1][tt][lane] = acc[tt];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            mk_f4 v = acc[tt];
+#pragma unroll
+            for (int w = 0; w < WAVES - 1; w++) v += red_l[w][tt][lane];
+            const int tok = tok0 + 16 * tt + i;
+            const int r0 = (int)blockIdx.x * 16 + 4 * g;
+            if (tok < m) {
+                float *dst = out + (size_t)tok * rows + r0;
+                if (r0 + 0 < rows) dst[0] = v.x;
+                if (r0 + 1 < rows) dst[1] = v.y;
+                if (r0 + 2 < rows) dst[2] = v.z;
+                if (r0 + 3 < rows) dst[3] = v.w;
+            }
+        }
+    }
+}
+
+template <int WAVES, int NTT>
+int launch_nt_mfma(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m, float *out, hipStream_t st) {
+    const dim3 grid((unsigned)((rows + 15) / 16), (unsigned)((m + 16 * NTT - 1) / (16 * NTT)));
+    hipLaunchKernelGGL((mxfp4_gemm_nt_mfma_kernel<WAVES, NTT>), grid, dim3(64 * WAVES), 0, st, packed, scales, (int)rows, (int)(cols / 32), x, (int)m, out);
+    return mk_launch_status("mxfp4_gemm_nt_mfma");
+}
+template <int WAVES>
+int launch_nt_mfma_w(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m, float *out, hipStream_t st) {
+    // tiles of 16 positions a workgroup takes against its weight registers: as many as leaves the chip 512 workgroups
+    const size_t row_tiles = (rows + 15) / 16, tiles = (m + 15) / 16;
+    size_t ntt = std::min<size_t>(4, tiles);
+    while (ntt > 1 && row_tiles * ((tiles + ntt - 1) / ntt) < 512) ntt--;
+    switch (ntt) {
+        case 1: return launch_nt_mfma<WAVES, 1>(packed, scales, rows, cols, x, m, out, st);
+        case 2: return launch_nt_mfma<WAVES, 2>(packed, scales, rows, cols, x, m, out, st);
+        case 3: return launch_nt_mfma<WAVES, 3>(packed, scales, rows, cols, x, m, out, st);
+        default: return launch_nt_mfma<WAVES, 4>(packed, scales, rows, cols, x, m, out, st);
+    }
+}
+
 template <int NB>
 int launch_fast(const GemvArgs &a0, bool q8, size_t nmat, hipStream_t st) {
     constexpr int RT = lcm_c(NB, 64) / NB;
@@ -483,6 +605,12 @@ extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scal
     MK_REQUIRE(shape_ok(rows, cols), "cols must be a positive multiple of 32");
     MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)x & 15) == 0, "packed and x must be 16-byte aligned");
     if (rows == 0 || m == 0) return MK_OK;
+    if (m >= (size_t)MK_TUNE("MK_MXFP4_NT_MFMA_MIN", 4) && cols % 128 == 0 && m <= 65535 * 64) {
+        // waves of a workgroup = shares of the 128-column steps: eight for long rows while the grid is small
+        if (cols / 128 >= 16 && (rows + 15) / 16 * ((m + 63) / 64) < 2048)
+            return launch_nt_mfma_w<8>(packed, scales, rows, cols, x, m, out, (hipStream_t)stream);
+        return launch_nt_mfma_w<4>(packed, scales, rows, cols, x, m, out, (hipStream_t)stream);
+    }
     hipLaunchKernelGGL(mxfp4_gemv_nt_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, packed, scales, (int)rows,
                        (int)(cols / 32), x, (int)m, out);
     return mk_launch_status("mxfp4_gemv_nt");

@@ -110,7 +110,10 @@ def test_grouped_launch_matches_per_matrix():
         del keep
 
 
-@pytest.mark.parametrize("rows,cols,m", [(64, 128, 8), (33, 64, 5), (128, 512, 24), (40, 7168, 3)])
+@pytest.mark.parametrize("rows,cols,m", [(64, 128, 8), (33, 64, 5), (128, 512, 24), (40, 7168, 3),
+                                         # four and more positions at cols % 128 == 0 run on the f32 matrix instruction: ragged rows,
+                                         # position counts around the tiles of 16 and the passes of 64, the model shapes
+                                         (37, 7168, 4), (2048, 7168, 17), (100, 2048, 70), (7168, 2048, 16), (16, 128, 130)])
 def test_matvec_packed_nt(rows, cols, m):
     from microkimi_amd import model
     p, s, _ = quantized_case(rows, cols)
