@@ -597,6 +597,16 @@ def bench_gemm(torch):
                              "mfma_frac_fp4_peak": fl3 / (ms3 * 1e-3) / 1e12 / FP4_PEAK_TFLOPS, "weight_bytes": used * per_expert,
                              "alg_bytes": alg3, "gbs": alg3 / (ms3 * 1e-3) / 1e9, "hbm_frac": alg3 / (ms3 * 1e-3) / 1e9 / HBM_PEAK_GBS,
                              "finite": bool(torch.isfinite(out).all().item())}
+    # the same section in the reference's own arithmetic (f32 rows against the dequantized weights, f32 matrix instruction)
+
+    def step4():
+        model.moe_prefill(experts, ids_d, wts_d, x_d, out=out, exact=True)
+
+    ms4 = time_region(torch, step4, 3, warmup=1)
+    res["expert_section_f32"] = {"workload": "the same section, mk_dev_moe_prefill_f32: group, gate + up (one launch), activation, down, combine in f32",
+                                 "ms": ms4, "tok_s": T / (ms4 * 1e-3), "tflops": fl3 / (ms4 * 1e-3) / 1e12,
+                                 "mfma_frac_fp32_peak": fl3 / (ms4 * 1e-3) / 1e12 / 157.3,
+                                 "finite": bool(torch.isfinite(out).all().item())}
     return res
 
 

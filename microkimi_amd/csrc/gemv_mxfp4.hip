@@ -360,11 +360,132 @@ __global__ __launch_bounds__(256) void mxfp4_gemv_nt_kernel(const uint8_t *__res
 
 
 // matvec_packed_nt for four and more positions on the f32 matrix instruction (v_mfma_f32_16x16x4_f32: f32 products, f32
-// sums), cols % 128 == 0.  A workgroup takes 16 weight rows, its four waves a quarter of the 128-column steps each; a
-// lane (i = lane % 16, g = lane / 16) holds the 32 weights of block 4 T + g of row i for step T, dequantized exactly
-// (e2m1 value times 2^(sb - 127): the scale rides on every weight because one instruction sums over four blocks), and
-// the 32 matching activations of position j = lane % 16.  Up to 64 positions a pass (four accumulator tiles) against the
-// same weight registers.  The terms are the reference's (src/model.rs:2412-2447); the order of the sums is not.
+// sums), cols % 128 == 0.  A wave works on 16 weight rows and a step of 128 columns at a time.  Lane (i = lane % 16,
+// g = lane / 16) loads the 16 packed bytes of block 4 T + g of row i; a 4 x 4 exchange between the lanes i, i + 16,
+// i + 32, i + 48 then leaves it dword g of each of the four blocks, i.e. the columns 32 b + 8 g .. + 7 (b = 0..3) of the
+// step, dequantized exactly (e2m1 value times 2^(sb - 127): the scale rides on every weight because one instruction
+// sums over columns of four blocks).  The activations of position j = lane % 16 for the same columns are 32 contiguous
+// bytes per block, and the four lanes of a position read whole 128-byte lines between them (a lane that read its own
+// block instead would touch 64 lines with every load instruction, and the address unit of the CU becomes the limit).
+// Up to 16 NTT positions a pass (NTT accumulator tiles) against the same weight registers.  The terms are the
+// reference's (src/model.rs:2412-2447); the order of the sums is not.
+//
+// The 4 x 4 exchange and the dequantization of one step: wq = the lane's 16 packed bytes of block g, sb = the scale
+// bytes of the step's four blocks; wf[8 b + c] = weight of column 32 b + 8 g + c.  All 64 lanes must be active.
+__device__ __forceinline__ void nt_dequant(mk_i4 wq, uint32_t sb, float (&wf)[32]) {
+    // dword d of lane row g <-> dword g of lane row d (rows of 16 lanes): two swaps between the halves of the wave,
+    // two between neighbouring rows
+    const mk_u2 a = __builtin_amdgcn_permlane32_swap((unsigned)wq[0], (unsigned)wq[2], false, false);
+    const mk_u2 b = __builtin_amdgcn_permlane32_swap((unsigned)wq[1], (unsigned)wq[3], false, false);
+    const mk_u2 c = __builtin_amdgcn_permlane16_swap((unsigned)a[0], (unsigned)b[0], false, false);
+    const mk_u2 e = __builtin_amdgcn_permlane16_swap((unsigned)a[1], (unsigned)b[1], false, false);
+    const uint32_t w[4] = {c[0], c[1], e[0], e[1]};
+    // (the hardware conversion gives the e2m1 values; the power of two is applied in f32: exact)
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        const uint32_t wd = w[d];
+        const float sc = mk_scale_from_byte((sb >> (8 * d)) & 255u);
+        const mk_f2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 0), p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 1);
+        const mk_f2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 2), p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 3);
+        wf[8 * d + 0] = p0.x * sc, wf[8 * d + 1] = p0.y * sc, wf[8 * d + 2] = p1.x * sc, wf[8 * d + 3] = p1.y * sc;
+        wf[8 * d + 4] = p2.x * sc, wf[8 * d + 5] = p2.y * sc, wf[8 * d + 6] = p3.x * sc, wf[8 * d + 7] = p3.y * sc;
+    }
+}
+// 16 weight rows x 16 positions x the step's 128 columns: xa[2 b + h] = the position's columns 32 b + 8 g + 4 h .. + 3.
+// Two chains of dependent matrix instructions, added at the end.
+__device__ __forceinline__ void nt_mfma_tile(const float (&wf)[32], const mk_f4 (&xa)[8], mk_f4 &acc) {
+    mk_f4 c1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < 8; k += 2) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k], xa[k].x, acc, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 4], xa[k + 1].x, c1, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 1], xa[k].y, acc, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 5], xa[k + 1].y, c1, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 2], xa[k].z, acc, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 6], xa[k + 1].z, c1, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 3], xa[k].w, acc, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 7], xa[k + 1].w, c1, 0, 0, 0);
+    }
+    acc += c1;
+}
+
+// nt_mfma_pass: this wave's share (steps wave, wave + WAVES, ..) of one pass.  xp[tt] is the lane's activation row of
+// tile tt, already moved to column 8 g; ntl (uniform, 1 .. NTT) tiles are in use.  All 64 lanes must be active.
+template <int WAVES, int NTT>
+__device__ __forceinline__ void nt_mfma_pass(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scales, int row, int nb, int wave,
+                                             int g, const float *const (&xp)[NTT], int ntl, mk_f4 (&acc)[NTT]) {
+    const int steps = nb / 4;
+    // Everything is requested one item ahead: the next step's weights and scale byte before this step is worked on, the
+    // next tile's activations (from L2) before this tile's matrix instructions.  Past the end: the last one again.
+    const bool sc_al4 = ((uintptr_t)scales & 3) == 0;  // (nb % 4 == 0: every row's scale bytes then start on a dword)
+    auto load_w = [&](int T, mk_i4 &wq, uint32_t &sb) {
+        const size_t blk = (size_t)row * nb + 4 * min(T, steps - 1);
+        wq = mk_ldg128_nt(packed + (blk + g) * 16);
+        if (sc_al4) sb = mk_ldg_u32(scales + blk);  // the scale bytes of the step's four blocks
+        else sb = mk_ldg_u8(scales + blk) | (mk_ldg_u8(scales + blk + 1) << 8) | (mk_ldg_u8(scales + blk + 2) << 16) | (mk_ldg_u8(scales + blk + 3) << 24);
+    };
+    auto load_x = [&](mk_f4 *xr, const float *xrow, int T) {
+        const mk_f4 *xv = reinterpret_cast<const mk_f4 *>(xrow + (size_t)min(T, steps - 1) * 128);
+#pragma unroll
+        for (int k = 0; k < 8; k++) xr[k] = xv[8 * (k >> 1) + (k & 1)];  // columns 32 b + 8 g + 4 h of the step, k = 2 b + h
+    };
+    mk_i4 wq, wq_n;
+    uint32_t sb, sb_n;
+    mk_f4 xa[8], xb[8];
+    load_w(wave, wq, sb);
+    load_x(xa, xp[0], wave);
+    for (int T = wave; T < steps; T += WAVES) {
+        load_w(T + WAVES, wq_n, sb_n);
+        __builtin_amdgcn_sched_barrier(0);
+        float wf[32];
+        nt_dequant(wq, sb, wf);
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            if (tt >= ntl) continue;
+            if (tt + 1 < NTT && tt + 1 < ntl) load_x(xb, xp[tt + 1 < NTT ? tt + 1 : 0], T);
+            else load_x(xb, xp[0], T + WAVES);
+            __builtin_amdgcn_sched_barrier(0);  // (the requests stay in front of the matrix instructions that cover them)
+            nt_mfma_tile(wf, xa, acc[tt]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) xa[k] = xb[k];
+        }
+        wq = wq_n;
+        sb = sb_n;
+    }
+}
+
+// The waves' partial sums of one pass meet in wave 0, which stores tile tt's rows 4 g + r of position tok0 + 16 tt + i
+// (result tile: column = position = lane % 16) for positions below tok_end.  Every wave of the workgroup calls it.
+template <int WAVES, int NTT>
+__device__ __forceinline__ void nt_mfma_store(mk_f4 (*red_l)[NTT][64], int wave, int lane, const mk_f4 (&acc)[NTT], int ntl, int row0, int rows,
+                                              int tok0, int tok_end, float *__restrict__ out) {
+    const int i = lane & 15, g = lane >> 4;
+    if (wave > 0) {
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) red_l[wave - 1][tt][lane] = acc[tt];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            if (tt >= ntl) continue;
+            mk_f4 v = acc[tt];
+#pragma unroll
+            for (int w = 0; w < WAVES - 1; w++) v += red_l[w][tt][lane];
+            const int tok = tok0 + 16 * tt + i;
+            const int r0 = row0 + 4 * g;
+            if (tok < tok_end) {
+                float *dst = out + (size_t)tok * rows + r0;
+                if (r0 + 0 < rows) dst[0] = v.x;
+                if (r0 + 1 < rows) dst[1] = v.y;
+                if (r0 + 2 < rows) dst[2] = v.z;
+                if (r0 + 3 < rows) dst[3] = v.w;
+            }
+        }
+    }
+}
+
 template <int WAVES, int NTT>
 __global__ __launch_bounds__(64 * WAVES) void mxfp4_gemm_nt_mfma_kernel(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ scales,
                                                                         int rows, int nb, const float *__restrict__ x, int m,
@@ -374,88 +495,117 @@ __global__ __launch_bounds__(64 * WAVES) void mxfp4_gemm_nt_mfma_kernel(const ui
     const int row = min((int)blockIdx.x * 16 + i, rows - 1);
     const int tok0 = blockIdx.y * 16 * NTT;  // NTT tiles of 16 positions a pass (positions past the end: the last one, not stored)
     const size_t cols = (size_t)nb * 32;
-    const int steps = nb / 4;
     mk_f4 acc[NTT];
+    const float *xp[NTT];
 #pragma unroll
-    for (int tt = 0; tt < NTT; tt++) acc[tt] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
-    // Everything is requested one item ahead: the next step's weights and scale byte before this step is worked on, the
-    // next tile's activations (from L2) before this tile's matrix instructions.  Past the end: the last one again.
+    for (int tt = 0; tt < NTT; tt++) {
+        acc[tt] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        xp[tt] = x + (size_t)min(tok0 + 16 * tt + i, m - 1) * cols + (size_t)g * 8;
+    }
+    nt_mfma_pass<WAVES, NTT>(packed, scales, row, nb, wave, g, xp, NTT, acc);
+    nt_mfma_store<WAVES, NTT>(red_l, wave, lane, acc, NTT, (int)blockIdx.x * 16, rows, tok0, m, out);
+}
+
+// The same product for groups of positions that each meet their own matrices (the experts of a prompt section): group e
+// owns the grouped rows offsets[e] .. offsets[e+1] of out ([.][rows]); grouped row p reads activation row xrow[p] / xdiv
+// of x (xrow null: row p).  Grid (tiles of 16 RW weight rows, groups, matrices per group).  The waves of a workgroup take
+// 16 weight rows each and all the column steps of them, against the same activations: the workgroup stages each step's
+// 16 NTT x 128 activations in LDS once (two buffers, one barrier a step; loaded a step ahead), so that the L1 sees them
+// once per 16 RW weight rows instead of once per 16.  A workgroup walks its group in passes of 16 NTT rows.
+struct NtGroupedArgs {
+    const uint8_t *const *packed[2];
+    const uint8_t *const *scales[2];
+    float *out[2];
+    const float *x;
+    const int32_t *xrow;
+    const int32_t *offsets;
+    int rows, nb, xdiv;
+};
+template <int RW, int NTT>
+__global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupedArgs a) {
+    constexpr int XS = 132;                            // floats a staged row takes (128 + 4: neighbouring rows start 4 banks apart)
+    constexpr int PER = NTT * 16 * 32 / (64 * RW);     // 16-byte pieces of a step's activations per thread
+    static_assert(PER >= 1 && PER * 64 * RW == NTT * 16 * 32, "threads must divide the staged activations");
+    __shared__ float xs_l[2][NTT * 16][XS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
+    const int grp = blockIdx.y, mat = blockIdx.z;
+    const int p_begin = a.offsets[grp], p_end = a.offsets[grp + 1];
+    if (p_end <= p_begin) return;  // (the whole workgroup)
+    const uint8_t *__restrict__ packed = a.packed[mat][grp];
+    const uint8_t *__restrict__ scales = a.scales[mat][grp];
+    float *__restrict__ out = a.out[mat];
+    const int nb = a.nb, steps = nb / 4;
+    const int row0 = ((int)blockIdx.x * RW + wave) * 16;   // (a wave past the last row works on the last row and stores nothing)
+    const int row = min(row0 + i, a.rows - 1);
+    const size_t cols = (size_t)nb * 32;
+    const bool sc_al4 = ((uintptr_t)scales & 3) == 0;
     auto load_w = [&](int T, mk_i4 &wq, uint32_t &sb) {
-        const size_t blk = (size_t)row * nb + 4 * min(T, steps - 1) + g;
-        wq = mk_ldg128_nt(packed + blk * 16);
-        sb = mk_ldg_u8(scales + blk);
+        const size_t blk = (size_t)row * nb + 4 * min(T, steps - 1);
+        wq = mk_ldg128_nt(packed + (blk + g) * 16);
+        if (sc_al4) sb = mk_ldg_u32(scales + blk);
+        else sb = mk_ldg_u8(scales + blk) | (mk_ldg_u8(scales + blk + 1) << 8) | (mk_ldg_u8(scales + blk + 2) << 16) | (mk_ldg_u8(scales + blk + 3) << 24);
     };
-    auto load_x = [&](mk_f4 *xr, int T, int tt) {
-        const int tok = min(tok0 + 16 * tt + i, m - 1);
-        const mk_f4 *xv = reinterpret_cast<const mk_f4 *>(x + (size_t)tok * cols + (size_t)(4 * min(T, steps - 1) + g) * 32);
+    for (int p0 = p_begin; p0 < p_end; p0 += 16 * NTT) {
+        const int ntl = min(NTT, (p_end - p0 + 15) >> 4);
+        // staging: piece q of this thread is 4 columns (sc) of staged row sr; rows of unused tiles are not touched
+        const float *sp[PER];
+        int so[PER];
 #pragma unroll
-        for (int k = 0; k < 8; k++) xr[k] = xv[k];
-    };
-    mk_i4 wq, wq_n;
-    uint32_t sb, sb_n;
-    mk_f4 xa[8], xb[8];
-    load_w(wave, wq, sb);
-    load_x(xa, wave, 0);
-    for (int T = wave; T < steps; T += WAVES) {
-        load_w(T + WAVES, wq_n, sb_n);
-        __builtin_amdgcn_sched_barrier(0);
-        const float sc = mk_scale_from_byte(sb);
-        float wf[32];
-        // (the hardware conversion gives the e2m1 values; the power of two is applied in f32: exact)
-#pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const uint32_t wd = (uint32_t)wq[d];
-            const mk_f2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 0), p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 1);
-            const mk_f2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 2), p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(wd, 1.0f, 3);
-            wf[8 * d + 0] = p0.x * sc, wf[8 * d + 1] = p0.y * sc, wf[8 * d + 2] = p1.x * sc, wf[8 * d + 3] = p1.y * sc;
-            wf[8 * d + 4] = p2.x * sc, wf[8 * d + 5] = p2.y * sc, wf[8 * d + 6] = p3.x * sc, wf[8 * d + 7] = p3.y * sc;
+        for (int q = 0; q < PER; q++) {
+            const int idx = (int)threadIdx.x + q * 64 * RW, sr = idx >> 5, sc = (idx & 31) * 4;
+            const int p = min(p0 + sr, p_end - 1);
+            const int xr = a.xrow ? a.xrow[p] / a.xdiv : p;
+            sp[q] = sr < 16 * ntl ? a.x + (size_t)xr * cols + sc : nullptr;
+            so[q] = sr * XS + sc;
         }
+        mk_f4 st[PER];
 #pragma unroll
-        for (int tt = 0; tt < NTT; tt++) {
-            if (tt + 1 < NTT) load_x(xb, T, tt + 1);
-            else load_x(xb, T + WAVES, 0);
-            __builtin_amdgcn_sched_barrier(0);  // (the requests stay in front of the matrix instructions that cover them)
-            // two chains of dependent matrix instructions, added at the end
-            mk_f4 c1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int q = 0; q < PER; q++)
+            if (sp[q]) *reinterpret_cast<mk_f4 *>(&xs_l[0][0][0] + so[q]) = *reinterpret_cast<const mk_f4 *>(sp[q]);
+        mk_f4 acc[NTT];
 #pragma unroll
-            for (int k = 0; k < 8; k += 2) {
-                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k], xa[k].x, acc[tt], 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 4], xa[k + 1].x, c1, 0, 0, 0);
-                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 1], xa[k].y, acc[tt], 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 5], xa[k + 1].y, c1, 0, 0, 0);
-                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 2], xa[k].z, acc[tt], 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 6], xa[k + 1].z, c1, 0, 0, 0);
-                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 3], xa[k].w, acc[tt], 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[4 * k + 7], xa[k + 1].w, c1, 0, 0, 0);
+        for (int tt = 0; tt < NTT; tt++) acc[tt] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        mk_i4 wq, wq_n;
+        uint32_t sb, sb_n;
+        load_w(0, wq, sb);
+        __syncthreads();
+        for (int T = 0; T < steps; T++) {
+            const bool more = T + 1 < steps;
+#pragma unroll
+            for (int q = 0; q < PER; q++)
+                if (more && sp[q]) st[q] = *reinterpret_cast<const mk_f4 *>(sp[q] + (size_t)(T + 1) * 128);
+            load_w(T + 1, wq_n, sb_n);
+            float wf[32];
+            nt_dequant(wq, sb, wf);
+            const float *xb = &xs_l[T & 1][0][0] + i * XS + 8 * g;
+#pragma unroll
+            for (int tt = 0; tt < NTT; tt++) {
+                if (tt >= ntl) continue;
+                mk_f4 xa[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) xa[k] = *reinterpret_cast<const mk_f4 *>(xb + tt * 16 * XS + 32 * (k >> 1) + 4 * (k & 1));
+                nt_mfma_tile(wf, xa, acc[tt]);
             }
-            acc[tt] += c1;
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int k = 0; k < 8; k++) xa[k] = xb[k];
+            for (int q = 0; q < PER; q++)
+                if (more && sp[q]) *reinterpret_cast<mk_f4 *>(&xs_l[(T + 1) & 1][0][0] + so[q]) = st[q];
+            wq = wq_n;
+            sb = sb_n;
+            __syncthreads();  // (the next step reads what was just written; the step after it overwrites what was just read)
         }
-        wq = wq_n;
-        sb = sb_n;
-    }
-    // the waves' partial sums meet; result tile: column = position j = lane % 16, rows 4 g + r
-    if (wave > 0) {
-#pragma unroll
-        for (int tt = 0; tt < NTT; tt++) red_l[wave - 1][tt][lane] = acc[tt];
-    }
-    __syncthreads();
-    if (wave == 0) {
+        // result tile: column = grouped row p0 + 16 tt + i, rows row0 + 4 g + r
 #pragma unroll
         for (int tt = 0; tt < NTT; tt++) {
-            mk_f4 v = acc[tt];
-#pragma unroll
-            for (int w = 0; w < WAVES - 1; w++) v += red_l[w][tt][lane];
-            const int tok = tok0 + 16 * tt + i;
-            const int r0 = (int)blockIdx.x * 16 + 4 * g;
-            if (tok < m) {
-                float *dst = out + (size_t)tok * rows + r0;
-                if (r0 + 0 < rows) dst[0] = v.x;
-                if (r0 + 1 < rows) dst[1] = v.y;
-                if (r0 + 2 < rows) dst[2] = v.z;
-                if (r0 + 3 < rows) dst[3] = v.w;
+            if (tt >= ntl) continue;
+            const int p = p0 + 16 * tt + i, r0 = row0 + 4 * g;
+            if (p < p_end && r0 < a.rows) {
+                float *dst = out + (size_t)p * a.rows + r0;
+                if (r0 + 3 < a.rows) *reinterpret_cast<mk_f4 *>(dst) = acc[tt];
+                else {
+                    dst[0] = acc[tt].x;
+                    if (r0 + 1 < a.rows) dst[1] = acc[tt].y;
+                    if (r0 + 2 < a.rows) dst[2] = acc[tt].z;
+                }
             }
         }
     }
@@ -479,6 +629,13 @@ int launch_nt_mfma_w(const uint8_t *packed, const uint8_t *scales, size_t rows, 
         case 3: return launch_nt_mfma<WAVES, 3>(packed, scales, rows, cols, x, m, out, st);
         default: return launch_nt_mfma<WAVES, 4>(packed, scales, rows, cols, x, m, out, st);
     }
+}
+
+template <int RW>
+int launch_nt_grouped(const NtGroupedArgs &a, size_t n_groups, int n_mats, hipStream_t st) {
+    const dim3 grid((unsigned)((a.rows + 16 * RW - 1) / (16 * RW)), (unsigned)n_groups, (unsigned)n_mats);
+    hipLaunchKernelGGL((mxfp4_gemm_nt_grouped_kernel<RW, 2>), grid, dim3(64 * RW), 0, st, a);
+    return mk_launch_status("mxfp4_gemm_nt_grouped");
 }
 
 template <int NB>
@@ -597,6 +754,23 @@ int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const u
     a.xf = xf;
     a.rows = (int)rows;
     return launch_gemv(a, q8, nmat, cols, st);
+}
+
+int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
+                             size_t rows, size_t cols, const float *x, const int32_t *xrow, int xdiv, const int32_t *offsets, float *const *out,
+                             void *stream) {
+    MK_REQUIRE((n_mats == 1 || n_mats == 2) && packed_ptrs && scales_ptrs && x && offsets && out, "bad argument");
+    MK_REQUIRE(rows > 0 && cols > 0 && cols % 128 == 0 && n_groups >= 1 && n_groups <= 65535, "cols must be a multiple of 128, at most 65535 groups");
+    MK_REQUIRE(rows <= (size_t)INT32_MAX && ((uintptr_t)x & 15) == 0 && (!xrow || xdiv >= 1), "bad shape or alignment");
+    NtGroupedArgs a{};
+    for (int k = 0; k < n_mats; k++) {
+        MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k], "null pointer");
+        a.packed[k] = packed_ptrs[k], a.scales[k] = scales_ptrs[k], a.out[k] = out[k];
+    }
+    a.x = x, a.xrow = xrow, a.offsets = offsets, a.rows = (int)rows, a.nb = (int)(cols / 32), a.xdiv = xdiv;
+    MK_REQUIRE(rows % 4 == 0 && ((uintptr_t)out[0] & 15) == 0 && (n_mats == 1 || ((uintptr_t)out[1] & 15) == 0), "rows % 4 and 16-byte aligned results");
+    if (MK_TUNE("MK_MXFP4_NT_GROUPED_WAVES", 8) == 8) return launch_nt_grouped<8>(a, n_groups, n_mats, (hipStream_t)stream);
+    return launch_nt_grouped<4>(a, n_groups, n_mats, (hipStream_t)stream);
 }
 
 extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m,

@@ -187,6 +187,17 @@ __global__ __launch_bounds__(256) void prefill_act_mxfp8_kernel(const float *__r
     if ((i & 3) == 0) exps[i >> 2] = (uint8_t)eb;
 }
 
+// ACT(gate, up) in f32, written over the gate rows (src/model.rs:2589-2595)
+__global__ __launch_bounds__(256) void prefill_act_f32_kernel(float *__restrict__ g, const float *__restrict__ u, const int32_t *__restrict__ offsets,
+                                                              int n_experts, int inter, int act_kind) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 4 values
+    const size_t n = (size_t)offsets[n_experts] * (inter / 4);
+    if (i >= n) return;
+    const mk_f4 gv = reinterpret_cast<const mk_f4 *>(g)[i], uv = reinterpret_cast<const mk_f4 *>(u)[i];
+    reinterpret_cast<mk_f4 *>(g)[i] = mk_f4{mk_act(act_kind, gv.x, uv.x, 0.0f, 1.0f), mk_act(act_kind, gv.y, uv.y, 0.0f, 1.0f),
+                                           mk_act(act_kind, gv.z, uv.z, 0.0f, 1.0f), mk_act(act_kind, gv.w, uv.w, 0.0f, 1.0f)};
+}
+
 // out_t = sum_s w[t][s] * o[pos(t, s)] in slot order, multiply then add (src/model.rs:2690-2700)
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ o, const int32_t *__restrict__ pos,
                                                               const float *__restrict__ weights, int topk, int d, float *__restrict__ out) {
@@ -276,6 +287,47 @@ int moe_prefill_impl(const mk_expert_table *table, size_t n_experts, size_t T, s
     return mk_launch_status("prefill_combine");
 }
 }  // namespace
+
+// The section in the reference's own arithmetic: f32 hidden rows and f32 activation against the dequantized weights.
+extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                      const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
+    MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
+    if (table->vq_codebook) {
+        mk_set_error("mk_dev_moe_prefill_f32 reads MXFP4 experts only; this layer holds VQ1 experts");
+        return MK_ERR_UNSUPPORTED;
+    }
+    const size_t d = table->d, inter = table->inter;
+    MK_REQUIRE(d % 128 == 0 && inter % 128 == 0 && d > 0 && inter > 0, "d and inter must be positive multiples of 128");
+    MK_REQUIRE(n_experts >= 1 && n_experts <= 960 && T >= 1 && topk >= 1 && T <= 65535, "bad token / expert count");
+    MK_REQUIRE(T * topk <= (size_t)GROUP_MAX_P, "at most 16384 (token, slot) pairs per call: split the prompt");
+    MK_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)x & 15) == 0,
+               "workspace must be 256-byte, x and out 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const size_t P = T * topk;
+    PrefillWs w = carve(workspace, P, n_experts, d, inter);
+    const size_t group_lds = ((size_t)GROUP_WAVES * n_experts + n_experts + 1) * sizeof(int);
+    MK_REQUIRE(group_lds <= 64 * 1024, "too many experts for the grouping kernel (17 counters per expert in 64 KiB of LDS)");
+    hipLaunchKernelGGL(prefill_group_kernel, dim3(1), dim3(GROUP_WAVES * 64), group_lds, st, ids, (int)P, (int)n_experts, w.order, w.pos,
+                       w.offsets);
+    int s = mk_launch_status("prefill_group");
+    if (s != MK_OK) return s;
+    // gate and up read the hidden row of their pair through the grouping (pair index / topk), no gathered copy
+    const uint8_t *const *pp[2] = {table->w1p, table->w3p};
+    const uint8_t *const *sp[2] = {table->w1s, table->w3s};
+    float *gu[2] = {w.g, w.u};
+    if ((s = mk_mxfp4_grouped_gemm_nt(2, pp, sp, n_experts, inter, d, x, w.order, (int)topk, w.offsets, gu, stream)) != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_act_f32_kernel, dim3((unsigned)((P * (inter / 4) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
+                       (int)n_experts, (int)inter, act_kind);
+    if ((s = mk_launch_status("prefill_act_f32")) != MK_OK) return s;
+    const uint8_t *const *pd[1] = {table->w2p};
+    const uint8_t *const *sd[1] = {table->w2s};
+    float *od[1] = {w.o};
+    if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, od, stream)) != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
+                       (int)d, out);
+    return mk_launch_status("prefill_combine");
+}
 
 extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
                                   const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {

@@ -107,6 +107,46 @@ def test_moe_prefill_on_device(T, topk, n_experts, d, inter, act):
     assert rel_l2(got, want) <= 2e-3
 
 
+@pytest.mark.parametrize("T,topk,n_experts,d,inter,act", [(24, 2, 4, 256, 128, "swiglu"), (40, 3, 7, 512, 256, "situ"), (5, 1, 3, 1024, 512, "swiglu"),
+                                                          # groups of about 50 and 75 tokens: several 32-row passes per workgroup
+                                                          (100, 2, 4, 512, 256, "swiglu"), (150, 2, 4, 1024, 384, "situ"),
+                                                          # one group of exactly 16, 17, 32 and 33 rows (tile and pass boundaries)
+                                                          (16, 1, 1, 256, 128, "swiglu"), (17, 1, 1, 256, 128, "swiglu"),
+                                                          (32, 1, 1, 128, 256, "situ"), (33, 1, 1, 128, 256, "situ")])
+def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
+    # the section in the reference's own arithmetic (mk_dev_moe_prefill_f32: f32 rows against the dequantized weights on
+    # the f32 matrix instruction) against oracle.moe_prefill without any rounding; the order of the sums is the only
+    # difference, hence 1e-5.  The stored intermediates are checked stage by stage as well.
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(T * 11 + n_experts)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.uint32)
+    if n_experts > 4:
+        ids[ids == 2] = 5  # an expert nobody selects
+    wts = rng.random((T, topk)).astype(np.float32)
+    kind = oracle.ACT_SITU if act == "situ" else oracle.ACT_SWIGLU
+    want = oracle.moe_prefill(table, ids, wts, x, act_kind=kind, round_mxfp8=False)
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x), act_kind=model.ACT_SITU if act == "situ" else model.ACT_SWIGLU,
+                            exact=True).cpu().numpy()
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, want) <= 1e-5
+    # stages: up rows and down rows per grouped row, in f64 from the dequantized weights
+    mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
+    order = np.argsort(ids.reshape(-1), kind="stable")
+    assert np.array_equal(mid["order"], order.astype(np.int32))
+    for r in range(0, T * topk, max(1, T * topk // 7)):
+        e, t = int(ids.reshape(-1)[order[r]]), int(order[r]) // topk
+        W3 = oracle.mxfp4_dequant(host[e][1][0], host[e][1][1], inter, d).astype(np.float64)
+        W2 = oracle.mxfp4_dequant(host[e][2][0], host[e][2][1], d, inter).astype(np.float64)
+        assert rel_l2(mid["u"][r], W3 @ x[t].astype(np.float64)) <= 1e-5
+        assert rel_l2(mid["o"][r], W2 @ mid["g"][r].astype(np.float64)) <= 1e-5  # "g" holds ACT(gate, up) after this call
+
+
 def test_config4_full_size_expert_section():
     """Configuration 4 at its full size: 512 prompt tokens routed top-8 (seeded logits, uneven groups) over 256
     experts of 2048 x 7168 / 7168 x 2048 (6 GB of MXFP4 drawn on the device), mk_dev_moe_prefill end to end.
@@ -119,6 +159,8 @@ def test_config4_full_size_expert_section():
       tokens     the output rows of ten sampled tokens against oracle.moe_prefill(round_mxfp8=2: MXFP8 inputs, full scale range), which gets the
                  eight experts of that token; the distance to the reference's own arithmetic (pure f32
                  matvec_packed_nt) is reported beside it
+      f32 mode   mk_dev_moe_prefill_f32 on the same weights: the up and down rows of two experts and the same ten
+                 token rows against the oracle without rounding (the reference's arithmetic): relative L2 <= 1e-5
     The looser bound on the last two is one e4m3 rounding step of the activation (2^-4 relative) where the device's
     expf and the CPU's differ in the last bit in front of a rounding boundary: see test_moe_prefill_on_device."""
     torch = torch_cuda()
@@ -175,8 +217,25 @@ def test_config4_full_size_expert_section():
         err = rel_l2(mid["o"][r0:r1], want_o)
         assert err <= 2e-3, f"expert {e}: down rows {err:.2e}"
 
+    # ---- the same section in the reference's own arithmetic (mk_dev_moe_prefill_f32), against the oracle without rounding
+    got_f32 = model.moe_prefill(experts, ids, wts, dev(x), exact=True).cpu().numpy()
+    assert np.isfinite(got_f32).all()
+    mid32 = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
+    assert np.array_equal(mid32["order"], order) and np.array_equal(mid32["offsets"], offsets)
+    for e in (nonempty[-1], nonempty[0]):
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        toks = order[r0:r1] // topk
+        table = oracle.ExpertTable([host(w1[e])], [host(w3[e])], [host(w2[e])], d, inter)
+        m = r1 - r0
+        want_o = oracle.moe_prefill(table, np.zeros((m, 1), np.uint32), np.ones((m, 1), np.float32), x[toks], round_mxfp8=False)
+        err = rel_l2(mid32["o"][r0:r1], want_o)
+        assert err <= 1e-5, f"expert {e}: f32 down rows {err:.2e}"
+        Wd = oracle.mxfp4_dequant(*host(w3[e]), inter, d).astype(np.float64)
+        err = rel_l2(mid32["u"][r0:r1], x[toks].astype(np.float64) @ Wd.T)
+        assert err <= 1e-5, f"expert {e}: f32 up rows {err:.2e}"
+
     # ---- ten tokens end to end
-    worst, worst_f32 = 0.0, 0.0
+    worst, worst_f32, worst_exact = 0.0, 0.0, 0.0
     for tok in (0, 1, 63, 64, 127, 200, 255, 256, 400, 511):
         used = [int(e) for e in ids_h[tok]]
         table = oracle.ExpertTable([host(w1[e]) for e in used], [host(w3[e]) for e in used], [host(w2[e]) for e in used], d, inter)
@@ -185,6 +244,9 @@ def test_config4_full_size_expert_section():
         plain = oracle.moe_prefill(table, lid, wts_h[tok:tok + 1], x[tok:tok + 1], round_mxfp8=False)
         worst = max(worst, rel_l2(got[tok], want[0]))
         worst_f32 = max(worst_f32, rel_l2(got[tok], plain[0]))
+        worst_exact = max(worst_exact, rel_l2(got_f32[tok], plain[0]))
     print(f"config 4 full size: worst token row vs MXFP8 oracle {worst:.2e}, vs the pure-f32 reference path {worst_f32:.2e}")
+    print(f"config 4 full size, f32 mode: worst token row vs the pure-f32 reference path {worst_exact:.2e}")
     assert worst <= 2e-3
+    assert worst_exact <= 1e-5
     assert worst_f32 < 0.06  # the e4m3 rounding of the activations: reported, not a parity claim
