@@ -520,6 +520,9 @@ struct NtGroupedArgs {
     const int32_t *xrow;
     const int32_t *offsets;
     int rows, nb, xdiv;
+    // offsets null: one matrix (packed1, scales1) for all m1 rows of x; blockIdx.y then counts passes of 16 NTT rows
+    const uint8_t *packed1, *scales1;
+    int m1;
 };
 template <int RW, int NTT>
 __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupedArgs a) {
@@ -529,10 +532,11 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
     __shared__ float xs_l[2][NTT * 16][XS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
     const int grp = blockIdx.y, mat = blockIdx.z;
-    const int p_begin = a.offsets[grp], p_end = a.offsets[grp + 1];
+    const bool one = a.offsets == nullptr;
+    const int p_begin = one ? grp * 16 * NTT : a.offsets[grp], p_end = one ? min(a.m1, p_begin + 16 * NTT) : a.offsets[grp + 1];
     if (p_end <= p_begin) return;  // (the whole workgroup)
-    const uint8_t *__restrict__ packed = a.packed[mat][grp];
-    const uint8_t *__restrict__ scales = a.scales[mat][grp];
+    const uint8_t *__restrict__ packed = one ? a.packed1 : a.packed[mat][grp];
+    const uint8_t *__restrict__ scales = one ? a.scales1 : a.scales[mat][grp];
     float *__restrict__ out = a.out[mat];
     const int nb = a.nb, steps = nb / 4;
     const int row0 = ((int)blockIdx.x * RW + wave) * 16;   // (a wave past the last row works on the last row and stores nothing)
@@ -631,10 +635,10 @@ int launch_nt_mfma_w(const uint8_t *packed, const uint8_t *scales, size_t rows, 
     }
 }
 
-template <int RW>
+template <int RW, int NTT = 2>
 int launch_nt_grouped(const NtGroupedArgs &a, size_t n_groups, int n_mats, hipStream_t st) {
     const dim3 grid((unsigned)((a.rows + 16 * RW - 1) / (16 * RW)), (unsigned)n_groups, (unsigned)n_mats);
-    hipLaunchKernelGGL((mxfp4_gemm_nt_grouped_kernel<RW, 2>), grid, dim3(64 * RW), 0, st, a);
+    hipLaunchKernelGGL((mxfp4_gemm_nt_grouped_kernel<RW, NTT>), grid, dim3(64 * RW), 0, st, a);
     return mk_launch_status("mxfp4_gemm_nt_grouped");
 }
 
@@ -757,8 +761,8 @@ int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const u
 }
 
 int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
-                             size_t rows, size_t cols, const float *x, const int32_t *xrow, int xdiv, const int32_t *offsets, float *const *out,
-                             void *stream) {
+                             size_t rows, size_t cols, const float *x, const int32_t *xrow, int xdiv, const int32_t *offsets, size_t m,
+                             float *const *out, void *stream) {
     MK_REQUIRE((n_mats == 1 || n_mats == 2) && packed_ptrs && scales_ptrs && x && offsets && out, "bad argument");
     MK_REQUIRE(rows > 0 && cols > 0 && cols % 128 == 0 && n_groups >= 1 && n_groups <= 65535, "cols must be a multiple of 128, at most 65535 groups");
     MK_REQUIRE(rows <= (size_t)INT32_MAX && ((uintptr_t)x & 15) == 0 && (!xrow || xdiv >= 1), "bad shape or alignment");
@@ -769,6 +773,9 @@ int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptr
     }
     a.x = x, a.xrow = xrow, a.offsets = offsets, a.rows = (int)rows, a.nb = (int)(cols / 32), a.xdiv = xdiv;
     MK_REQUIRE(rows % 4 == 0 && ((uintptr_t)out[0] & 15) == 0 && (n_mats == 1 || ((uintptr_t)out[1] & 15) == 0), "rows % 4 and 16-byte aligned results");
+    // passes of 64 grouped rows (twice the LDS, half the workgroups a CU holds) pay from about 48 rows a group
+    const int tiles = MK_TUNE("MK_MXFP4_NT_GROUPED_TILES", 0);
+    if (tiles == 4 || (tiles == 0 && m >= 48 * n_groups)) return launch_nt_grouped<8, 4>(a, n_groups, n_mats, (hipStream_t)stream);
     if (MK_TUNE("MK_MXFP4_NT_GROUPED_WAVES", 8) == 8) return launch_nt_grouped<8>(a, n_groups, n_mats, (hipStream_t)stream);
     return launch_nt_grouped<4>(a, n_groups, n_mats, (hipStream_t)stream);
 }
@@ -780,6 +787,14 @@ extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scal
     MK_REQUIRE(((uintptr_t)packed & 15) == 0 && ((uintptr_t)x & 15) == 0, "packed and x must be 16-byte aligned");
     if (rows == 0 || m == 0) return MK_OK;
     if (m >= (size_t)MK_TUNE("MK_MXFP4_NT_MFMA_MIN", 4) && cols % 128 == 0 && m <= 65535 * 64) {
+        // many positions: 64 weight rows a workgroup, each step's activations staged in LDS once for all of them
+        if (m >= (size_t)MK_TUNE("MK_MXFP4_NT_STAGED_MIN", 512) && m <= 65535 * 32 && rows % 4 == 0 && ((uintptr_t)out & 15) == 0 && rows <= (size_t)INT32_MAX) {
+            NtGroupedArgs a{};
+            a.out[0] = out, a.x = x, a.rows = (int)rows, a.nb = (int)(cols / 32), a.xdiv = 1;
+            a.packed1 = packed, a.scales1 = scales, a.m1 = (int)m;
+            if (MK_TUNE("MK_MXFP4_NT_STAGED_TILES", 4) == 4) return launch_nt_grouped<4, 4>(a, (m + 63) / 64, 1, (hipStream_t)stream);
+            return launch_nt_grouped<4, 2>(a, (m + 31) / 32, 1, (hipStream_t)stream);
+        }
         // waves of a workgroup = shares of the 128-column steps: eight for long rows while the grid is small
         if (cols / 128 >= 16 && (rows + 15) / 16 * ((m + 63) / 64) < 2048)
             return launch_nt_mfma_w<8>(packed, scales, rows, cols, x, m, out, (hipStream_t)stream);

@@ -316,14 +316,14 @@ extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_exp
     const uint8_t *const *pp[2] = {table->w1p, table->w3p};
     const uint8_t *const *sp[2] = {table->w1s, table->w3s};
     float *gu[2] = {w.g, w.u};
-    if ((s = mk_mxfp4_grouped_gemm_nt(2, pp, sp, n_experts, inter, d, x, w.order, (int)topk, w.offsets, gu, stream)) != MK_OK) return s;
+    if ((s = mk_mxfp4_grouped_gemm_nt(2, pp, sp, n_experts, inter, d, x, w.order, (int)topk, w.offsets, P, gu, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_act_f32_kernel, dim3((unsigned)((P * (inter / 4) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
                        (int)n_experts, (int)inter, act_kind);
     if ((s = mk_launch_status("prefill_act_f32")) != MK_OK) return s;
     const uint8_t *const *pd[1] = {table->w2p};
     const uint8_t *const *sd[1] = {table->w2s};
     float *od[1] = {w.o};
-    if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, od, stream)) != MK_OK) return s;
+    if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, P, od, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");

@@ -112,7 +112,9 @@ def test_moe_prefill_on_device(T, topk, n_experts, d, inter, act):
                                                           (100, 2, 4, 512, 256, "swiglu"), (150, 2, 4, 1024, 384, "situ"),
                                                           # one group of exactly 16, 17, 32 and 33 rows (tile and pass boundaries)
                                                           (16, 1, 1, 256, 128, "swiglu"), (17, 1, 1, 256, 128, "swiglu"),
-                                                          (32, 1, 1, 128, 256, "situ"), (33, 1, 1, 128, 256, "situ")])
+                                                          (32, 1, 1, 128, 256, "situ"), (33, 1, 1, 128, 256, "situ"),
+                                                          # 48 and more rows a group: passes of 64 rows
+                                                          (64, 1, 1, 256, 128, "swiglu"), (65, 1, 1, 256, 128, "swiglu"), (49, 1, 1, 128, 128, "situ")])
 def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
     # the section in the reference's own arithmetic (mk_dev_moe_prefill_f32: f32 rows against the dequantized weights on
     # the f32 matrix instruction) against oracle.moe_prefill without any rounding; the order of the sums is the only

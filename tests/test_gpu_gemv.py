@@ -113,7 +113,11 @@ def test_grouped_launch_matches_per_matrix():
 @pytest.mark.parametrize("rows,cols,m", [(64, 128, 8), (33, 64, 5), (128, 512, 24), (40, 7168, 3),
                                          # four and more positions at cols % 128 == 0 run on the f32 matrix instruction: ragged rows,
                                          # position counts around the tiles of 16 and the passes of 64, the model shapes
-                                         (37, 7168, 4), (2048, 7168, 17), (100, 2048, 70), (7168, 2048, 16), (16, 128, 130)])
+                                         (37, 7168, 4), (2048, 7168, 17), (100, 2048, 70), (7168, 2048, 16), (16, 128, 130),
+                                         (100, 2048, 129), (2048, 7168, 160),
+                                         # from 512 positions the activations of a step are staged in LDS for 64 weight rows: ragged
+                                         # rows and positions, and a row count the staged stores do not take
+                                         (100, 2048, 515), (260, 128, 513), (38, 256, 520), (512, 7168, 512)])
 def test_matvec_packed_nt(rows, cols, m):
     from microkimi_amd import model
     p, s, _ = quantized_case(rows, cols)
