@@ -149,6 +149,34 @@ def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
         assert rel_l2(mid["o"][r], W2 @ mid["g"][r].astype(np.float64)) <= 1e-5  # "g" holds ACT(gate, up) after this call
 
 
+@pytest.mark.parametrize("exact", [False, True])
+def test_moe_prefill_skips_ids_out_of_range(exact):
+    # a pair whose expert id lies outside the table adds nothing to its token (include/mk_hip.h): the result equals the
+    # oracle's with that pair pointed at a valid expert with routing weight 0; a token whose pairs are all out of range
+    # comes out as zeros
+    from microkimi_amd import model, workloads
+    T, topk, n_experts, d, inter = 37, 3, 5, 256, 128
+    rng = np.random.default_rng(5)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.int32)
+    wts = (rng.random((T, topk)) + 0.1).astype(np.float32)
+    bad = rng.random((T, topk)) < 0.25
+    bad[7, :] = True
+    dev_ids = ids.copy()
+    dev_ids[bad] = np.where(rng.random(int(bad.sum())) < 0.5, -1, n_experts + 2)
+    ref_ids, ref_wts = ids.copy(), wts.copy()
+    ref_wts[bad] = 0.0
+    want = oracle.moe_prefill(table, ref_ids.astype(np.uint32), ref_wts, x, round_mxfp8=False if exact else 2)
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    got = model.moe_prefill(experts, dev(dev_ids), dev(wts), dev(x), exact=exact).cpu().numpy()
+    assert np.all(np.isfinite(got)) and not got[7].any()
+    assert rel_l2(got, want) <= (1e-5 if exact else 2e-3)
+
+
 def test_config4_full_size_expert_section():
     """Configuration 4 at its full size: 512 prompt tokens routed top-8 (seeded logits, uneven groups) over 256
     experts of 2048 x 7168 / 7168 x 2048 (6 GB of MXFP4 drawn on the device), mk_dev_moe_prefill end to end.
