@@ -372,7 +372,8 @@ int mk_moe_prefill_workspace_layout(size_t T, size_t topk, size_t n_experts, siz
  * table entries 0..n_experts-1 are used; ids [T][topk] int32 (a pair whose id is
  * out of range contributes nothing), weights [T][topk], x [T][d], out [T][d].
  * act_kind MK_ACT_SWIGLU or MK_ACT_SITU.  d, inter multiples of 128; T * topk <= 16384
- * per call (a longer prompt is split by the caller). */
+ * per call (a longer prompt is split by the caller).  MK_ERR_UNSUPPORTED for a table with VQ1 experts
+ * (mk_dev_moe_prefill_f32 takes those). */
 int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                        const float *x, int act_kind, void *workspace, float *out, void *stream);
 /* The same call, the same kernels and the same result bit for bit, with the f32 gate and up rows stored as well (for
@@ -384,8 +385,10 @@ int mk_dev_moe_prefill_keep(const mk_expert_table *table, size_t n_experts, size
  * it at src/model.rs:2580-2599): f32 hidden rows and f32 activation against the exactly dequantized weights on the f32
  * matrix instruction, f32 products and sums.  Only the order of the sums inside a dot product differs from the
  * reference (relative L2 below 1e-5).  Same arguments, same workspace and same layout of the intermediates as
- * mk_dev_moe_prefill; afterwards g holds ACT(gate, up), u the up rows, o the down rows.  About three times the time of
- * the MXFP8 path at 512 tokens over 256 experts. */
+ * mk_dev_moe_prefill; afterwards g holds ACT(gate, up), u the up rows, o the down rows.  About four times the time of
+ * the MXFP8 path at 512 tokens over 256 experts.  A table with a vq_codebook is taken too: the three products of a VQ1
+ * expert (NULL scale pointers) are quant::matvec_vq_nt's (src/quant.rs:353-376, src/model.rs:2576-2593) with the
+ * codebook entries as the weights, again with the order of the sums as the only difference. */
 int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                            const float *x, int act_kind, void *workspace, float *out, void *stream);
 

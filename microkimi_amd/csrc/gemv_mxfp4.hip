@@ -523,13 +523,19 @@ struct NtGroupedArgs {
     // offsets null: one matrix (packed1, scales1) for all m1 rows of x; blockIdx.y then counts passes of 16 NTT rows
     const uint8_t *packed1, *scales1;
     int m1;
+    // VQ instantiation: the file's 256 x 16 f32 codebook; a group's "packed" pointer then holds index bytes [rows][cols / 16]
+    const float *codebook;
 };
-template <int RW, int NTT>
+// VQ = false takes the groups whose matrix has scale bytes (MXFP4) and leaves the others alone; VQ = true takes the groups
+// with a null scale pointer, whose matrix is VQ1 (W[r][16 v .. 16 v + 16] = codebook[index[r][v]], src/quant.rs:353-376):
+// the codebook sits in LDS and a lane fetches the halves of the four vectors that hold its columns.
+template <int RW, int NTT, bool VQ = false>
 __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupedArgs a) {
     constexpr int XS = 132;                            // floats a staged row takes (128 + 4: neighbouring rows start 4 banks apart)
     constexpr int PER = NTT * 16 * 32 / (64 * RW);     // 16-byte pieces of a step's activations per thread
     static_assert(PER >= 1 && PER * 64 * RW == NTT * 16 * 32, "threads must divide the staged activations");
     __shared__ float xs_l[2][NTT * 16][XS];
+    __shared__ __attribute__((aligned(16))) float cb_l[VQ ? 256 * 16 : 4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
     const int grp = blockIdx.y, mat = blockIdx.z;
     const bool one = a.offsets == nullptr;
@@ -537,13 +543,26 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
     if (p_end <= p_begin) return;  // (the whole workgroup)
     const uint8_t *__restrict__ packed = one ? a.packed1 : a.packed[mat][grp];
     const uint8_t *__restrict__ scales = one ? a.scales1 : a.scales[mat][grp];
+    if ((scales == nullptr) != VQ) return;  // (the other instantiation's group)
     float *__restrict__ out = a.out[mat];
     const int nb = a.nb, steps = nb / 4;
+    if (VQ) {
+        for (int k = threadIdx.x; k < 256 * 4; k += 64 * RW) reinterpret_cast<mk_f4 *>(cb_l)[k] = reinterpret_cast<const mk_f4 *>(a.codebook)[k];
+        // (the barrier in front of the first step also covers the codebook)
+    }
     const int row0 = ((int)blockIdx.x * RW + wave) * 16;   // (a wave past the last row works on the last row and stores nothing)
     const int row = min(row0 + i, a.rows - 1);
     const size_t cols = (size_t)nb * 32;
     const bool sc_al4 = ((uintptr_t)scales & 3) == 0;
     auto load_w = [&](int T, mk_i4 &wq, uint32_t &sb) {
+        if (VQ) {
+            // the index bytes of the vectors 2 b + g / 2 (b = 0..3) of the step's eight
+            const uint8_t *ip = packed + (size_t)row * (nb * 2) + 8 * min(T, steps - 1) + (g >> 1);
+#pragma unroll
+            for (int b = 0; b < 4; b++) wq[b] = (int)mk_ldg_u8(ip + 2 * b);
+            sb = 0;
+            return;
+        }
         const size_t blk = (size_t)row * nb + 4 * min(T, steps - 1);
         wq = mk_ldg128_nt(packed + (blk + g) * 16);
         if (sc_al4) sb = mk_ldg_u32(scales + blk);
@@ -580,7 +599,17 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
                 if (more && sp[q]) st[q] = *reinterpret_cast<const mk_f4 *>(sp[q] + (size_t)(T + 1) * 128);
             load_w(T + 1, wq_n, sb_n);
             float wf[32];
-            nt_dequant(wq, sb, wf);
+            if (VQ) {
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const mk_f4 *e = reinterpret_cast<const mk_f4 *>(cb_l + wq[b] * 16 + 8 * (g & 1));
+                    const mk_f4 lo = e[0], hi = e[1];
+                    wf[8 * b + 0] = lo.x, wf[8 * b + 1] = lo.y, wf[8 * b + 2] = lo.z, wf[8 * b + 3] = lo.w;
+                    wf[8 * b + 4] = hi.x, wf[8 * b + 5] = hi.y, wf[8 * b + 6] = hi.z, wf[8 * b + 7] = hi.w;
+                }
+            } else {
+                nt_dequant(wq, sb, wf);
+            }
             const float *xb = &xs_l[T & 1][0][0] + i * XS + 8 * g;
 #pragma unroll
             for (int tt = 0; tt < NTT; tt++) {
@@ -639,7 +668,11 @@ template <int RW, int NTT = 2>
 int launch_nt_grouped(const NtGroupedArgs &a, size_t n_groups, int n_mats, hipStream_t st) {
     const dim3 grid((unsigned)((a.rows + 16 * RW - 1) / (16 * RW)), (unsigned)n_groups, (unsigned)n_mats);
     hipLaunchKernelGGL((mxfp4_gemm_nt_grouped_kernel<RW, NTT>), grid, dim3(64 * RW), 0, st, a);
-    return mk_launch_status("mxfp4_gemm_nt_grouped");
+    int s = mk_launch_status("mxfp4_gemm_nt_grouped");
+    if (s != MK_OK || !a.codebook) return s;
+    // a layer with VQ1 experts: their groups in a second launch (which groups they are is known on the device only)
+    hipLaunchKernelGGL((mxfp4_gemm_nt_grouped_kernel<RW, 2, true>), grid, dim3(64 * RW), 0, st, a);
+    return mk_launch_status("vq1_gemm_nt_grouped");
 }
 
 template <int NB>
@@ -762,7 +795,7 @@ int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const u
 
 int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                              size_t rows, size_t cols, const float *x, const int32_t *xrow, int xdiv, const int32_t *offsets, size_t m,
-                             float *const *out, void *stream) {
+                             const float *vq_codebook, float *const *out, void *stream) {
     MK_REQUIRE((n_mats == 1 || n_mats == 2) && packed_ptrs && scales_ptrs && x && offsets && out, "bad argument");
     MK_REQUIRE(rows > 0 && cols > 0 && cols % 128 == 0 && n_groups >= 1 && n_groups <= 65535, "cols must be a multiple of 128, at most 65535 groups");
     MK_REQUIRE(rows <= (size_t)INT32_MAX && ((uintptr_t)x & 15) == 0 && (!xrow || xdiv >= 1), "bad shape or alignment");
@@ -772,6 +805,8 @@ int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptr
         a.packed[k] = packed_ptrs[k], a.scales[k] = scales_ptrs[k], a.out[k] = out[k];
     }
     a.x = x, a.xrow = xrow, a.offsets = offsets, a.rows = (int)rows, a.nb = (int)(cols / 32), a.xdiv = xdiv;
+    MK_REQUIRE(!vq_codebook || ((uintptr_t)vq_codebook & 15) == 0, "the codebook must be 16-byte aligned");
+    a.codebook = vq_codebook;
     MK_REQUIRE(rows % 4 == 0 && ((uintptr_t)out[0] & 15) == 0 && (n_mats == 1 || ((uintptr_t)out[1] & 15) == 0), "rows % 4 and 16-byte aligned results");
     // passes of 64 grouped rows (twice the LDS, half the workgroups a CU holds) pay from about 48 rows a group
     const int tiles = MK_TUNE("MK_MXFP4_NT_GROUPED_TILES", 0);

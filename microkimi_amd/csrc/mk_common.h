@@ -333,10 +333,12 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
 // matvec_packed_nt (f32 products and sums, gemv_mxfp4.hip) for groups of rows that each meet their own n_mats (1 or 2)
 // matrices: group e owns the grouped rows offsets[e] .. offsets[e+1]; grouped row p multiplies activation row
 // xrow[p] / xdiv of x (xrow null: row p itself); matrix k's [. x rows] result goes to out[k] at the grouped row.  m: the
-// number of grouped rows in all (only the choice of the pass size looks at it).
+// number of grouped rows in all (only the choice of the pass size looks at it).  vq_codebook (may be null): with it, a
+// group whose scale pointer is null has a VQ1 matrix (index bytes where the packed nibbles would be) and is multiplied
+// with the codebook's entries (quant::matvec_vq_nt's terms).
 int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                              size_t rows, size_t cols, const float *x, const int32_t *xrow, int xdiv, const int32_t *offsets, size_t m,
-                             float *const *out, void *stream);
+                             const float *vq_codebook, float *const *out, void *stream);
 // The gate and up matrices of every group against the same token rows, the activation ACT(gate, up) and its MXFP8 form
 // (e4m3 codes [m][rows], e8m0 bytes [m][rows / 32], whole exponent range) in one launch; the f32 gate / up rows are
 // written too when keep_g and keep_u are given.  MK_ERR_UNSUPPORTED (nothing launched) for shapes it does not take.

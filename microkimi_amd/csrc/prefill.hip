@@ -293,10 +293,6 @@ extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_exp
                                       const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
     MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
     MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
-    if (table->vq_codebook) {
-        mk_set_error("mk_dev_moe_prefill_f32 reads MXFP4 experts only; this layer holds VQ1 experts");
-        return MK_ERR_UNSUPPORTED;
-    }
     const size_t d = table->d, inter = table->inter;
     MK_REQUIRE(d % 128 == 0 && inter % 128 == 0 && d > 0 && inter > 0, "d and inter must be positive multiples of 128");
     MK_REQUIRE(n_experts >= 1 && n_experts <= 960 && T >= 1 && topk >= 1 && T <= 65535, "bad token / expert count");
@@ -316,14 +312,14 @@ extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_exp
     const uint8_t *const *pp[2] = {table->w1p, table->w3p};
     const uint8_t *const *sp[2] = {table->w1s, table->w3s};
     float *gu[2] = {w.g, w.u};
-    if ((s = mk_mxfp4_grouped_gemm_nt(2, pp, sp, n_experts, inter, d, x, w.order, (int)topk, w.offsets, P, gu, stream)) != MK_OK) return s;
+    if ((s = mk_mxfp4_grouped_gemm_nt(2, pp, sp, n_experts, inter, d, x, w.order, (int)topk, w.offsets, P, table->vq_codebook, gu, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_act_f32_kernel, dim3((unsigned)((P * (inter / 4) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
                        (int)n_experts, (int)inter, act_kind);
     if ((s = mk_launch_status("prefill_act_f32")) != MK_OK) return s;
     const uint8_t *const *pd[1] = {table->w2p};
     const uint8_t *const *sd[1] = {table->w2s};
     float *od[1] = {w.o};
-    if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, P, od, stream)) != MK_OK) return s;
+    if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, P, table->vq_codebook, od, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");

@@ -177,6 +177,53 @@ def test_moe_prefill_skips_ids_out_of_range(exact):
     assert rel_l2(got, want) <= (1e-5 if exact else 2e-3)
 
 
+@pytest.mark.parametrize("T,topk,d,inter,act", [(40, 3, 256, 128, 0), (90, 2, 512, 256, 1), (7, 1, 128, 384, 0)])
+def test_moe_prefill_f32_with_vq1_experts(T, topk, d, inter, act):
+    # moe_prefill over a layer that mixes MXFP4 and VQ1 ("cold") experts (src/model.rs:2556-2599: matvec_vq_nt for the
+    # three products of a VQ1 expert, matvec_packed_nt for the others): experts 1, 3, 5 are VQ1.  The oracle is the
+    # per-token form of the same layer in f32 (both nt functions keep their per-position terms; the order of the sums
+    # is what differs on the device).  mk_dev_moe_prefill (MXFP8) still refuses such a layer.
+    from microkimi_amd import model, workloads
+    n_experts = 6
+    rng = np.random.default_rng(T + d)
+    codebook = (rng.standard_normal((256, 16)) * 0.05).astype(np.float32)
+    host, devs = [], ([], [], [])
+    for e in range(n_experts):
+        if e % 2:
+            idx = [rng.integers(0, 256, (inter, d // 16), dtype=np.uint8), rng.integers(0, 256, (inter, d // 16), dtype=np.uint8),
+                   rng.integers(0, 256, (d, inter // 16), dtype=np.uint8)]
+            host.append(("vq1", idx[0], idx[1], idx[2]))
+            for k in range(3):
+                devs[k].append((dev(idx[k]), None))
+        else:
+            m = [workloads.mxfp4_matrix(2, "w1", inter, d, e), workloads.mxfp4_matrix(2, "w3", inter, d, e),
+                 workloads.mxfp4_matrix(2, "w2", d, inter, e)]
+            host.append(("mxfp4", m[0], m[1], m[2]))
+            for k in range(3):
+                devs[k].append((dev(m[k][0]), dev(m[k][1])))
+    experts = model.PackedExperts(devs[0], devs[1], devs[2], d, inter, vq_codebook=dev(codebook))
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.int32)
+    wts = rng.random((T, topk)).astype(np.float32)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    want = oracle.moe_decode_mixed(host, codebook, d, inter, ids.astype(np.uint32), wts, x, shared=-1, mode=0, act_kind=act, limit=0.0)
+    got = model.moe_prefill(experts, dev(ids), dev(wts), dev(x), act_kind=act, exact=True).cpu().numpy()
+    assert np.isfinite(got).all() and np.isfinite(want).all()
+    for t in range(T):
+        assert rel_l2(got[t], want[t]) <= 1e-5, (t, rel_l2(got[t], want[t]))
+    # the batched VQ1 product of the oracle on one expert's group: the up rows
+    mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
+    e = 3
+    r0, r1 = int(mid["offsets"][e]), int(mid["offsets"][e + 1])
+    toks = mid["order"][r0:r1] // topk
+    m8 = (len(toks) + 7) // 8 * 8
+    xt = np.zeros((d, m8), np.float32)
+    xt[:, :len(toks)] = x[toks].T
+    want_u = oracle.vq1_matvec_nt(codebook, host[e][2], inter, d, xt, m8)[:len(toks)]
+    assert len(toks) > 0 and rel_l2(mid["u"][r0:r1], want_u) <= 1e-5
+    with pytest.raises(Exception):
+        model.moe_prefill(experts, dev(ids), dev(wts), dev(x), act_kind=act)
+
+
 def test_config4_full_size_expert_section():
     """Configuration 4 at its full size: 512 prompt tokens routed top-8 (seeded logits, uneven groups) over 256
     experts of 2048 x 7168 / 7168 x 2048 (6 GB of MXFP4 drawn on the device), mk_dev_moe_prefill end to end.
