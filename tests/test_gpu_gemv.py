@@ -130,6 +130,27 @@ def test_matvec_packed_nt(rows, cols, m):
     assert rel_l2(got, want) <= TOL
 
 
+@pytest.mark.parametrize("sb,m", [(0, 16), (1, 16), (2, 16), (1, 3), (250, 16), (1, 600)])
+def test_matvec_packed_nt_extreme_scale_bytes(sb, m):
+    # scale bytes 0..2 make every weight a subnormal or the smallest normals (byte 0 is 2^-127, src/mxfp4.rs:340-346),
+    # byte 250 the largest that keeps the sums finite: the matrix-instruction paths (m >= 4, m >= 512) and the vector
+    # path (m = 3) keep subnormal weights and products as the reference's f32 loop does
+    from microkimi_amd import model
+    rows, cols = 64, 256
+    rng = np.random.default_rng(sb + m)
+    packed = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)
+    scales = np.full((rows, cols // 32), sb, np.uint8)
+    x = (rng.standard_normal((m, cols)) * (1.0 if sb < 100 else 1e-30)).astype(np.float32)
+    got = model.matvec_packed_nt(dev(packed), dev(scales), rows, cols, dev(x), m).cpu().numpy()
+    m8 = (m + 7) // 8 * 8
+    xt = np.zeros((cols, m8), np.float32)
+    xt[:, :m] = x.T
+    want = oracle.matvec_packed_nt(packed, scales, rows, cols, xt, m8)[:m]
+    assert np.isfinite(want).all() and np.abs(want).max() > 0
+    err = np.linalg.norm(got.astype(np.float64) - want) / np.linalg.norm(want.astype(np.float64))
+    assert err <= TOL
+
+
 @pytest.mark.parametrize("rows,cols,batch,f16", [(512, 1024, 1, True), (512, 1024, 8, True), (512, 1024, 3, False), (100, 7168, 1, True),
                                                   (100, 7168, 8, True), (37, 96, 2, True), (37, 96, 1, False), (64, 2048, 5, True),
                                                   (1000, 4096, 1, False),
