@@ -149,6 +149,31 @@ def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
         assert rel_l2(mid["o"][r], W2 @ mid["g"][r].astype(np.float64)) <= 1e-5  # "g" holds ACT(gate, up) after this call
 
 
+def test_moe_prefill_f32_random_shapes():
+    # a dozen seeded random shapes (token counts, top-k, expert counts, d and inter in multiples of 128, both
+    # activations; routing with repeats allowed across tokens only) against the oracle without rounding
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(2024)
+    for case in range(12):
+        n_experts = int(rng.integers(1, 9))
+        topk = int(rng.integers(1, min(n_experts, 4) + 1))
+        T = int(rng.integers(1, 130))
+        d, inter = 128 * int(rng.integers(1, 5)), 128 * int(rng.integers(1, 4))
+        act = int(rng.integers(0, 2))
+        host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+                 workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+        table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+        x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+        ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.uint32)
+        wts = rng.random((T, topk)).astype(np.float32)
+        want = oracle.moe_prefill(table, ids, wts, x, act_kind=act, round_mxfp8=False)
+        pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+        experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+        got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x), act_kind=act, exact=True).cpu().numpy()
+        err = rel_l2(got, want)
+        assert np.isfinite(got).all() and err <= 1e-5, (case, T, topk, n_experts, d, inter, act, err)
+
+
 @pytest.mark.parametrize("exact", [False, True])
 def test_moe_prefill_skips_ids_out_of_range(exact):
     # a pair whose expert id lies outside the table adds nothing to its token (include/mk_hip.h): the result equals the
