@@ -607,6 +607,16 @@ def bench_gemm(torch):
                                  "ms": ms4, "tok_s": T / (ms4 * 1e-3), "tflops": fl3 / (ms4 * 1e-3) / 1e12,
                                  "mfma_frac_fp32_peak": fl3 / (ms4 * 1e-3) / 1e12 / 157.3,
                                  "finite": bool(torch.isfinite(out).all().item())}
+    # and with bfloat16 activations (exact weights, bf16 matrix instruction)
+
+    def step5():
+        model.moe_prefill(experts, ids_d, wts_d, x_d, out=out, bf16=True)
+
+    ms5 = time_region(torch, step5, 5, warmup=2)
+    res["expert_section_bf16"] = {"workload": "the same section, mk_dev_moe_prefill_bf16: group, gather + bf16, gate + up (one launch), activation + bf16, down, combine",
+                                  "ms": ms5, "tok_s": T / (ms5 * 1e-3), "tflops": fl3 / (ms5 * 1e-3) / 1e12,
+                                  "mfma_frac_bf16_peak": fl3 / (ms5 * 1e-3) / 1e12 / 2500.0, "weight_bytes": used * per_expert,
+                                  "weight_gbs": used * per_expert / (ms5 * 1e-3) / 1e9, "finite": bool(torch.isfinite(out).all().item())}
     return res
 
 

@@ -392,6 +392,17 @@ int mk_dev_moe_prefill_keep(const mk_expert_table *table, size_t n_experts, size
 int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                            const float *x, int act_kind, void *workspace, float *out, void *stream);
 
+/* The same section with bfloat16 activations: the hidden rows and the activation rows are rounded to bfloat16 (nearest
+ * even) once, the MXFP4 weights are exact in bfloat16, and v_mfma_f32_16x16x32_bf16 gives f32 products and f32 sums: the
+ * results are those of moe_prefill (src/model.rs:2528-2602) on bfloat16-rounded inputs, with the order of the sums as
+ * the only further difference (about 2e-3 of a row's norm from the reference's f32 arithmetic, where the MXFP8 call
+ * differs by 2-5 %).  Same arguments, workspace and intermediates as mk_dev_moe_prefill_f32 (g holds the gate rows
+ * here: the activation is kept as bfloat16 elsewhere in the workspace).  MK_ERR_UNSUPPORTED unless d and inter are
+ * multiples of 512, and for a table with VQ1 experts.  Weights whose value lies below 2^-126 may be flushed to zero by
+ * the hardware conversion. */
+int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
+                            const float *x, int act_kind, void *workspace, float *out, void *stream);
+
 /* ---------------------------------------- device level: VQ1 / LUT GEMV */
 
 /* Bytes of device scratch for the lookup tables of one activation: cols/16 tables of 256 f32. */

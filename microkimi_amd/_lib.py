@@ -98,6 +98,7 @@ def _load():
         "mk_dev_moe_prefill": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_dev_moe_prefill_keep": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_dev_moe_prefill_f32": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
+        "mk_dev_moe_prefill_bf16": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),
         "mk_mxfp4_matvec": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp]),
         "mk_matvec_f32": (i32, [vp, sz, sz, vp, vp]),

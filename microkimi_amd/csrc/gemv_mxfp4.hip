@@ -531,7 +531,7 @@ struct NtGroupedArgs {
 // the codebook sits in LDS and a lane fetches the halves of the four vectors that hold its columns.
 template <int RW, int NTT, bool VQ = false>
 __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupedArgs a) {
-    constexpr int XS = 132;                            // floats a staged row takes (128 + 4: neighbouring rows start 4 banks apart)
+    constexpr int XS = 136;                            // floats a staged row takes (128 + 8: neighbouring rows start 8 banks apart)
     constexpr int PER = NTT * 16 * 32 / (64 * RW);     // 16-byte pieces of a step's activations per thread
     static_assert(PER >= 1 && PER * 64 * RW == NTT * 16 * 32, "threads must divide the staged activations");
     __shared__ float xs_l[2][NTT * 16][XS];
@@ -638,6 +638,159 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
                     dst[0] = acc[tt].x;
                     if (r0 + 1 < a.rows) dst[1] = acc[tt].y;
                     if (r0 + 2 < a.rows) dst[2] = acc[tt].z;
+                }
+            }
+        }
+    }
+}
+
+// The grouped product with bfloat16 activations on v_mfma_f32_16x16x32_bf16: the weights are exact in bf16 (an e2m1
+// value times a power of two), the products exact in f32 and summed in f32, so the one rounding is that of the
+// activations (done by the caller, once per row).  cols % 512 == 0.  Same split of the work as the f32 kernel above: a
+// wave owns 16 weight rows and all their columns, the workgroup stages the group's activation rows in LDS, here a K
+// tile of 512 columns at a time (two buffers, one barrier a K tile).
+//
+// Weight side: the 256 bytes a row has in a K tile are fetched as whole 128-byte lines (a load takes 8 rows x 128 bytes:
+// lane (r3 = lane / 8, c = lane % 8) reads bytes 16 c .. of row 8 h + r3; loads 2 i and 2 i + 1 cover line i of rows 0-7
+// and 8-15), non-temporally, a K tile ahead; a rotation of the lane index by three bits (ds_bpermute) and an exchange
+// of the 8-lane halves of every 16-lane row between two registers (DPP row_ror:8 under a bank mask) then give lane
+// (i = lane % 16, g = lane / 16) the 16 bytes of block 4 u + g of row i for the four steps u of the K tile.  Dword s2 of
+// such a block and the block's scale become the eight bf16 values lane group g feeds to matrix instruction (u, s2)
+// through v_cvt_scalef32_pk_bf16_fp4.  The activations of those columns, 128 u + 32 g + 8 s2 .. + 7, are one 16-byte
+// LDS read; the staging stores piece 4 g + s2 of a step at place 4 s2 + g, so that the four lanes of a position read
+// 64 contiguous bytes (with the pieces in column order the same reads ran into bank conflicts: 2.1-2.2 ms for the
+// 512-token section against 1.7), and rows are 32 bytes of padding apart (16: 2.7 times the conflict cycles).
+// Measured on the way: loads of 16 rows x 64 bytes in the operand's own form streamed at 4.1 TB/s with everything
+// else compiled out, the whole-line loads at 5.0; held to 128 registers (two workgroups a CU) 1.68 ms, at 138
+// registers (one workgroup) 1.96-2.1 ms; ordinary instead of non-temporal loads 1.77 ms.
+typedef __bf16 mk_bf8 __attribute__((ext_vector_type(8)));
+typedef __bf16 mk_bf2 __attribute__((ext_vector_type(2)));
+struct Bf16GroupedArgs {
+    const uint8_t *const *packed[2];
+    const uint8_t *const *scales[2];
+    float *out[2];
+    const uint16_t *x;       // [grouped rows][cols] bf16
+    const int32_t *offsets;  // [groups + 1]
+    int rows, nb;
+};
+template <int RW, int NTT>
+__global__ __launch_bounds__(64 * RW) __attribute__((amdgpu_waves_per_eu(4))) void mxfp4_gemm_bf16_grouped_kernel(Bf16GroupedArgs a) {
+    constexpr int XSB = 512 * 2 + 32;                   // bytes a staged row takes (32 of padding: neighbouring rows 8 banks apart)
+    constexpr int PER = NTT * 16 * 64 / (64 * RW);      // 16-byte pieces of a K tile per thread
+    static_assert(PER >= 1 && PER * 64 * RW == NTT * 16 * 64, "threads must divide the staged activations");
+    __shared__ __attribute__((aligned(16))) uint8_t xs_l[2][NTT * 16 * XSB];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
+    const int grp = blockIdx.y, mat = blockIdx.z;
+    const int p_begin = a.offsets[grp], p_end = a.offsets[grp + 1];
+    if (p_end <= p_begin) return;  // (the whole workgroup)
+    const uint8_t *__restrict__ packed = a.packed[mat][grp];
+    const uint8_t *__restrict__ scales = a.scales[mat][grp];
+    float *__restrict__ out = a.out[mat];
+    const int nb = a.nb, ktiles = nb / 16;
+    const int row0 = ((int)blockIdx.x * RW + wave) * 16;  // (a wave past the last row works on the last row and stores nothing)
+    const size_t cols = (size_t)nb * 32;
+    const uint8_t *wline[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) wline[h] = packed + (size_t)min(row0 + 8 * h + (lane >> 3), a.rows - 1) * (cols / 2) + (lane & 7) * 16;
+    const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
+    const uint8_t *srow = scales + (size_t)min(row0 + i, a.rows - 1) * nb;
+    const int sc_al = ((uintptr_t)scales & 15) == 0 ? 16 : ((uintptr_t)scales & 3) == 0 ? 4 : 1;  // (nb % 16 == 0)
+    auto load_w = [&](int kt, mk_i4 (&wl)[4], mk_i4 &sc) {
+        const size_t ku = (size_t)min(kt, ktiles - 1);
+#pragma unroll
+        for (int j = 0; j < 4; j++) wl[j] = mk_ldg128_nt(wline[j & 1] + ku * 256 + (j >> 1) * 128);
+        const uint8_t *sp = srow + ku * 16;  // the scale bytes of the row's 16 blocks in the K tile
+        if (sc_al == 16) sc = *reinterpret_cast<const mk_i4 *>(sp);
+        else if (sc_al == 4) sc = mk_i4{(int)mk_ldg_u32(sp), (int)mk_ldg_u32(sp + 4), (int)mk_ldg_u32(sp + 8), (int)mk_ldg_u32(sp + 12)};
+        else {
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                sc[k] = (int)(mk_ldg_u8(sp + 4 * k) | (mk_ldg_u8(sp + 4 * k + 1) << 8) | (mk_ldg_u8(sp + 4 * k + 2) << 16) | (mk_ldg_u8(sp + 4 * k + 3) << 24));
+        }
+    };
+    for (int p0 = p_begin; p0 < p_end; p0 += 16 * NTT) {
+        const int ntl = min(NTT, (p_end - p0 + 15) >> 4);
+        // staging: piece q of this thread is 8 columns (16 bytes) of staged row sr; rows of unused tiles are not touched
+        const uint8_t *sp[PER];
+        int so[PER];
+#pragma unroll
+        for (int q = 0; q < PER; q++) {
+            const int idx = (int)threadIdx.x + q * 64 * RW, sr = idx >> 6, pc = idx & 63;
+            const int p = min(p0 + sr, p_end - 1);
+            sp[q] = sr < 16 * ntl ? reinterpret_cast<const uint8_t *>(a.x) + ((size_t)p * cols) * 2 + pc * 16 : nullptr;
+            // inside a step's 16 pieces, piece 4 g + s2 (block g, dword s2) goes to place 4 s2 + g: the four lanes of a
+            // position then read 64 contiguous bytes for a matrix instruction
+            so[q] = sr * XSB + ((pc & 48) | ((pc & 3) << 2) | ((pc >> 2) & 3)) * 16;
+        }
+        mk_i4 st[PER];
+#pragma unroll
+        for (int q = 0; q < PER; q++)
+            if (sp[q]) *reinterpret_cast<mk_i4 *>(&xs_l[0][so[q]]) = *reinterpret_cast<const mk_i4 *>(sp[q]);
+        mk_f4 acc[NTT][2];
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) acc[tt][0] = acc[tt][1] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        mk_i4 wl[4], wl_n[4], sc, sc_n;
+        load_w(0, wl, sc);
+        __syncthreads();
+        for (int kt = 0; kt < ktiles; kt++) {
+            const bool more = kt + 1 < ktiles;
+#pragma unroll
+            for (int q = 0; q < PER; q++)
+                if (more && sp[q]) st[q] = *reinterpret_cast<const mk_i4 *>(sp[q] + (size_t)(kt + 1) * 1024);
+            load_w(kt + 1, wl_n, sc_n);
+            // operand form of the K tile's two lines: lane (i, g) gets the 16 bytes of block 4 u + g of row i
+            mk_i4 w[4];
+#pragma unroll
+            for (int l2 = 0; l2 < 2; l2++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int ra = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * l2][k]), rb = __builtin_amdgcn_ds_bpermute(rot_idx, wl[2 * l2 + 1][k]);
+                    w[2 * l2][k] = __builtin_amdgcn_update_dpp(ra, rb, 0x128 /* row_ror:8 */, 0xF, 0xC, false);
+                    w[2 * l2 + 1][k] = __builtin_amdgcn_update_dpp(rb, ra, 0x128 /* row_ror:8 */, 0xF, 0x3, false);
+                }
+            const uint8_t *xb = &xs_l[kt & 1][0] + i * XSB + 16 * g;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                mk_bf8 wa[4];
+                const float scf = mk_scale_from_byte(((uint32_t)sc[u] >> (8 * g)) & 255u);  // block 4 u + g
+#pragma unroll
+                for (int s2 = 0; s2 < 4; s2++) {
+                    const uint32_t wd = (uint32_t)w[u][s2];
+                    const mk_bf2 c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, scf, 0), c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, scf, 1);
+                    const mk_bf2 c2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, scf, 2), c3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(wd, scf, 3);
+                    wa[s2] = mk_bf8{c0[0], c0[1], c1[0], c1[1], c2[0], c2[1], c3[0], c3[1]};
+                }
+#pragma unroll
+                for (int tt = 0; tt < NTT; tt++) {
+                    if (tt >= ntl) continue;
+#pragma unroll
+                    for (int s2 = 0; s2 < 4; s2++) {
+                        const mk_bf8 xv = *reinterpret_cast<const mk_bf8 *>(xb + tt * 16 * XSB + u * 256 + 64 * s2);
+                        acc[tt][s2 & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s2], xv, acc[tt][s2 & 1], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < PER; q++)
+                if (more && sp[q]) *reinterpret_cast<mk_i4 *>(&xs_l[(kt + 1) & 1][so[q]]) = st[q];
+#pragma unroll
+            for (int u = 0; u < 4; u++) wl[u] = wl_n[u];
+            sc = sc_n;
+            __syncthreads();  // (the next K tile reads what was just written; the one after it overwrites what was just read)
+        }
+        // result tile: column = grouped row p0 + 16 tt + i, rows row0 + 4 g + r
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) {
+            if (tt >= ntl) continue;
+            const mk_f4 v = acc[tt][0] + acc[tt][1];
+            const int p = p0 + 16 * tt + i, r0 = row0 + 4 * g;
+            if (p < p_end && r0 < a.rows) {
+                float *dst = out + (size_t)p * a.rows + r0;
+                if (r0 + 3 < a.rows) *reinterpret_cast<mk_f4 *>(dst) = v;
+                else {
+                    dst[0] = v.x;
+                    if (r0 + 1 < a.rows) dst[1] = v.y;
+                    if (r0 + 2 < a.rows) dst[2] = v.z;
                 }
             }
         }
@@ -813,6 +966,26 @@ int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptr
     if (tiles == 4 || (tiles == 0 && m >= 48 * n_groups)) return launch_nt_grouped<8, 4>(a, n_groups, n_mats, (hipStream_t)stream);
     if (MK_TUNE("MK_MXFP4_NT_GROUPED_WAVES", 8) == 8) return launch_nt_grouped<8>(a, n_groups, n_mats, (hipStream_t)stream);
     return launch_nt_grouped<4>(a, n_groups, n_mats, (hipStream_t)stream);
+}
+
+int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
+                               size_t rows, size_t cols, const uint16_t *x, const int32_t *offsets, float *const *out, void *stream) {
+    MK_REQUIRE((n_mats == 1 || n_mats == 2) && packed_ptrs && scales_ptrs && x && offsets && out, "bad argument");
+    if (cols == 0 || cols % 512 != 0 || rows % 4 != 0) {
+        mk_set_error("the bf16 grouped product takes cols % 512 == 0 and rows % 4 == 0");
+        return MK_ERR_UNSUPPORTED;
+    }
+    MK_REQUIRE(rows > 0 && n_groups >= 1 && n_groups <= 65535 && rows <= (size_t)INT32_MAX && ((uintptr_t)x & 15) == 0, "bad shape or alignment");
+    Bf16GroupedArgs a{};
+    for (int k = 0; k < n_mats; k++) {
+        MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k] && ((uintptr_t)out[k] & 15) == 0, "null or unaligned pointer");
+        a.packed[k] = packed_ptrs[k], a.scales[k] = scales_ptrs[k], a.out[k] = out[k];
+    }
+    a.x = x, a.offsets = offsets, a.rows = (int)rows, a.nb = (int)(cols / 32);
+    constexpr int RW = 8;
+    const dim3 grid((unsigned)((rows + 16 * RW - 1) / (16 * RW)), (unsigned)n_groups, (unsigned)n_mats);
+    hipLaunchKernelGGL((mxfp4_gemm_bf16_grouped_kernel<RW, 2>), grid, dim3(64 * RW), 0, (hipStream_t)stream, a);
+    return mk_launch_status("mxfp4_gemm_bf16_grouped");
 }
 
 extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m,

@@ -33,6 +33,7 @@ struct PrefillWs {
     float *g, *u;             // [P][inter]
     uint8_t *codes2, *exps2;  // [P][inter], [P][inter/32]
     float *o;                 // [P][d]
+    uint16_t *xb;             // [P][max(d, inter)] bf16: the hidden rows, then the activation rows, of the bf16 section
     size_t bytes;
 };
 
@@ -55,6 +56,7 @@ PrefillWs carve(void *base, size_t P, size_t n_experts, size_t d, size_t inter) 
     w.codes2 = take(P * inter);
     w.exps2 = take(P * (inter / 32));
     w.o = (float *)take(P * d * 4);
+    w.xb = (uint16_t *)take(P * (d > inter ? d : inter) * 2);
     w.bytes = off;
     return w;
 }
@@ -198,6 +200,40 @@ __global__ __launch_bounds__(256) void prefill_act_f32_kernel(float *__restrict_
                                            mk_act(act_kind, gv.z, uv.z, 0.0f, 1.0f), mk_act(act_kind, gv.w, uv.w, 0.0f, 1.0f)};
 }
 
+// bfloat16 (round to nearest even) of the hidden row of each grouped pair: a lane takes 8 consecutive values
+__global__ __launch_bounds__(256) void prefill_gather_bf16_kernel(const float *__restrict__ x, const int32_t *__restrict__ order,
+                                                                  const int32_t *__restrict__ offsets, int n_experts, int topk, int d,
+                                                                  uint16_t *__restrict__ xb) {
+    const int per_row = d / 8;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t rows = (size_t)offsets[n_experts];
+    if (i >= rows * per_row) return;
+    const size_t r = i / per_row, c = i % per_row;
+    const int t = order[r] / topk;
+    const mk_f4 *src = reinterpret_cast<const mk_f4 *>(x + (size_t)t * d) + 2 * c;
+    const mk_f4 a = src[0], b = src[1];
+    typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+    const bf8 v = {(__bf16)a.x, (__bf16)a.y, (__bf16)a.z, (__bf16)a.w, (__bf16)b.x, (__bf16)b.y, (__bf16)b.z, (__bf16)b.w};
+    reinterpret_cast<bf8 *>(xb)[i] = v;
+}
+
+// act = ACT(gate, up) in f32, stored as bfloat16 (round to nearest even)
+__global__ __launch_bounds__(256) void prefill_act_bf16_kernel(const float *__restrict__ g, const float *__restrict__ u,
+                                                               const int32_t *__restrict__ offsets, int n_experts, int inter, int act_kind,
+                                                               uint16_t *__restrict__ ab) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 8 values
+    const size_t n = (size_t)offsets[n_experts] * (inter / 8);
+    if (i >= n) return;
+    const mk_f4 g0 = reinterpret_cast<const mk_f4 *>(g)[2 * i], g1 = reinterpret_cast<const mk_f4 *>(g)[2 * i + 1];
+    const mk_f4 u0 = reinterpret_cast<const mk_f4 *>(u)[2 * i], u1 = reinterpret_cast<const mk_f4 *>(u)[2 * i + 1];
+    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w}, uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+    typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+    bf8 v;
+#pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = (__bf16)mk_act(act_kind, gv[k], uv[k], 0.0f, 1.0f);
+    reinterpret_cast<bf8 *>(ab)[i] = v;
+}
+
 // out_t = sum_s w[t][s] * o[pos(t, s)] in slot order, multiply then add (src/model.rs:2690-2700)
 __global__ __launch_bounds__(256) void prefill_combine_kernel(const float *__restrict__ o, const int32_t *__restrict__ pos,
                                                               const float *__restrict__ weights, int topk, int d, float *__restrict__ out) {
@@ -320,6 +356,53 @@ extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_exp
     const uint8_t *const *sd[1] = {table->w2s};
     float *od[1] = {w.o};
     if ((s = mk_mxfp4_grouped_gemm_nt(1, pd, sd, n_experts, d, inter, w.g, nullptr, 1, w.offsets, P, table->vq_codebook, od, stream)) != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
+                       (int)d, out);
+    return mk_launch_status("prefill_combine");
+}
+
+// The section with bfloat16 hidden rows and activation rows against the exact weights (bf16 matrix instruction).
+extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                       const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
+    MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
+    if (table->vq_codebook) {
+        mk_set_error("mk_dev_moe_prefill_bf16 reads MXFP4 experts only; this layer holds VQ1 experts (mk_dev_moe_prefill_f32 takes them)");
+        return MK_ERR_UNSUPPORTED;
+    }
+    const size_t d = table->d, inter = table->inter;
+    if (d == 0 || inter == 0 || d % 512 != 0 || inter % 512 != 0) {
+        mk_set_error("mk_dev_moe_prefill_bf16 takes d and inter in multiples of 512");
+        return MK_ERR_UNSUPPORTED;
+    }
+    MK_REQUIRE(n_experts >= 1 && n_experts <= 960 && T >= 1 && topk >= 1 && T <= 65535, "bad token / expert count");
+    MK_REQUIRE(T * topk <= (size_t)GROUP_MAX_P, "at most 16384 (token, slot) pairs per call: split the prompt");
+    MK_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)x & 15) == 0,
+               "workspace must be 256-byte, x and out 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const size_t P = T * topk;
+    PrefillWs w = carve(workspace, P, n_experts, d, inter);
+    const size_t group_lds = ((size_t)GROUP_WAVES * n_experts + n_experts + 1) * sizeof(int);
+    MK_REQUIRE(group_lds <= 64 * 1024, "too many experts for the grouping kernel (17 counters per expert in 64 KiB of LDS)");
+    hipLaunchKernelGGL(prefill_group_kernel, dim3(1), dim3(GROUP_WAVES * 64), group_lds, st, ids, (int)P, (int)n_experts, w.order, w.pos,
+                       w.offsets);
+    int s = mk_launch_status("prefill_group");
+    if (s != MK_OK) return s;
+    hipLaunchKernelGGL(prefill_gather_bf16_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
+                       (int)n_experts, (int)topk, (int)d, w.xb);
+    if ((s = mk_launch_status("prefill_gather_bf16")) != MK_OK) return s;
+    const uint8_t *const *pp[2] = {table->w1p, table->w3p};
+    const uint8_t *const *sp[2] = {table->w1s, table->w3s};
+    float *gu[2] = {w.g, w.u};
+    if ((s = mk_mxfp4_grouped_gemm_bf16(2, pp, sp, n_experts, inter, d, w.xb, w.offsets, gu, stream)) != MK_OK) return s;
+    // (the hidden rows are used up: the activation rows take their place)
+    hipLaunchKernelGGL(prefill_act_bf16_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
+                       (int)n_experts, (int)inter, act_kind, w.xb);
+    if ((s = mk_launch_status("prefill_act_bf16")) != MK_OK) return s;
+    const uint8_t *const *pd[1] = {table->w2p};
+    const uint8_t *const *sd[1] = {table->w2s};
+    float *od[1] = {w.o};
+    if ((s = mk_mxfp4_grouped_gemm_bf16(1, pd, sd, n_experts, d, inter, w.xb, w.offsets, od, stream)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");

@@ -287,14 +287,16 @@ def moe_prefill_intermediates(experts, T, topk):
             "g": f32(lay.g, P, experts.inter), "u": f32(lay.u, P, experts.inter), "o": f32(lay.o, P, experts.d)}
 
 
-def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None, keep=False, exact=False):
+def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None, keep=False, exact=False, bf16=False):
     """The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) for T prompt positions: pairs grouped by
     expert, gate / up / activation / down per used expert on the block-scaled matrix cores (MXFP8 activations),
     per-token weighted sum in slot order.  ids [T, topk] int32, weights [T, topk] f32, x [T, d] f32; returns [T, d].
     keep: also store the f32 gate and up rows (moe_prefill_intermediates reads them); the result is the same.
     exact: the reference's own arithmetic instead (f32 rows and activation against the dequantized weights, f32 products
     and sums on the f32 matrix instruction: matvec_packed_nt per expert, src/model.rs:2580-2599); the intermediates then
-    hold ACT(gate, up) in "g", the up rows in "u" and the down rows in "o"."""
+    hold ACT(gate, up) in "g", the up rows in "u" and the down rows in "o".
+    bf16: hidden rows and activation rows rounded to bfloat16, exact weights, f32 products and sums on the bf16 matrix
+    instruction (mk_dev_moe_prefill_bf16); "g" and "u" then hold the gate and up rows."""
     import torch
     _lib.require_device()
     T, topk = ids.shape
@@ -303,7 +305,7 @@ def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None, keep=Fa
         experts._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((T, experts.d), dtype=torch.float32, device=x.device)
-    fn = lib.mk_dev_moe_prefill_f32 if exact else lib.mk_dev_moe_prefill_keep if keep else lib.mk_dev_moe_prefill
+    fn = lib.mk_dev_moe_prefill_bf16 if bf16 else lib.mk_dev_moe_prefill_f32 if exact else lib.mk_dev_moe_prefill_keep if keep else lib.mk_dev_moe_prefill
     check(fn(C.byref(experts.table), experts.n, T, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), ptr(x.contiguous()), act_kind,
              ptr(experts._ws), ptr(out), cur_stream()))
     return out

@@ -623,7 +623,8 @@ def moe_decode(table, ids, weights, x, shared=-1, mode=1, act_kind=ACT_SWIGLU, l
 
 def moe_prefill(table, ids, weights, x, act_kind=ACT_SWIGLU, round_mxfp8=False):
     """round_mxfp8: False/0 the reference's f32 arithmetic; True/1 inputs and activation through the reference's
-    fp8_roundtrip per 32; 2 the same with the full e8m0 scale range (no saturation)."""
+    fp8_roundtrip per 32; 2 the same with the full e8m0 scale range (no saturation); 3 inputs and activation rounded
+    to bfloat16 (nearest even)."""
     ids, weights, x = _c(ids, np.uint32), _c(weights, np.float32), _c(x, np.float32)
     n, topk = ids.shape
     out = np.empty((n, table.d), np.float32)

@@ -1391,7 +1391,23 @@ ORC_API void orc_moe_decode(const uint8_t *const *w1p, const uint8_t *const *w1s
  * input precision of the block-scaled MFMA GEMM, and the oracle it is compared
  * against tightly.  1: the reference's orc_fp8_roundtrip (scale exponent
  * clamped at 8); 2: the full e8m0 range (orc_fp8_roundtrip_emax with 127), the
- * encoding of the device's prefill section. */
+ * encoding of the device's prefill section; 3: hidden rows and activation
+ * rounded to bfloat16 (round to nearest even), the inputs of the device's
+ * bf16 prefill section. */
+static void orc_round_bf16(float *x, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        uint32_t b;
+        memcpy(&b, &x[i], 4);
+        if ((b & 0x7F800000u) == 0x7F800000u) continue; /* inf / NaN stay */
+        b += 0x7FFFu + ((b >> 16) & 1u);
+        b &= 0xFFFF0000u;
+        memcpy(&x[i], &b, 4);
+    }
+}
+static void orc_round_inputs(float *x, size_t n, int mode) {
+    if (mode == 3) orc_round_bf16(x, n);
+    else if (mode) orc_fp8_roundtrip_emax(x, n, 32, mode == 2 ? 127 : 8, NULL, NULL);
+}
 ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                              const uint8_t *const *w2p, const uint8_t *const *w2s, size_t n_experts, size_t d, size_t inter, size_t n,
                              size_t topk, const uint32_t *ids, const float *weights, const float *x, int act_kind, int round_mxfp8,
@@ -1413,7 +1429,7 @@ ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1
         for (size_t i = 0; i < m; i++) {
             size_t t = pairs[i] / topk;
             memcpy(tmp, x + t * d, sizeof(float) * d);
-            if (round_mxfp8) orc_fp8_roundtrip_emax(tmp, d, 32, round_mxfp8 == 2 ? 127 : 8, NULL, NULL);
+            orc_round_inputs(tmp, d, round_mxfp8);
             for (size_t c = 0; c < d; c++) ht[c * m8 + i] = tmp[c];
         }
         float *a = (float *)malloc(sizeof(float) * m8 * inter);
@@ -1426,7 +1442,7 @@ ORC_API void orc_moe_prefill(const uint8_t *const *w1p, const uint8_t *const *w1
                 float g = a[i * inter + j], uu = u[i * inter + j];
                 tmp[j] = (act_kind == ORC_ACT_SITU) ? orc_situ(g, uu) : (g / (1.0f + expf(-g))) * uu;
             }
-            if (round_mxfp8) orc_fp8_roundtrip_emax(tmp, inter, 32, round_mxfp8 == 2 ? 127 : 8, NULL, NULL);
+            orc_round_inputs(tmp, inter, round_mxfp8);
             for (size_t j = 0; j < inter; j++) act_t[j * m8 + i] = tmp[j];
         }
         float *o = (float *)malloc(sizeof(float) * m8 * d);

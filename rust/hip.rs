@@ -155,6 +155,7 @@ extern "C" {
     pub fn mk_dev_moe_prefill(table: *const MkExpertTable, n_experts: usize, T: usize, topk: usize, ids: *const i32, weights: *const f32, x: *const f32, act_kind: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_prefill_keep(table: *const MkExpertTable, n_experts: usize, T: usize, topk: usize, ids: *const i32, weights: *const f32, x: *const f32, act_kind: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_prefill_f32(table: *const MkExpertTable, n_experts: usize, T: usize, topk: usize, ids: *const i32, weights: *const f32, x: *const f32, act_kind: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_moe_prefill_bf16(table: *const MkExpertTable, n_experts: usize, T: usize, topk: usize, ids: *const i32, weights: *const f32, x: *const f32, act_kind: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_vq1_workspace_bytes(cols: usize) -> usize;
     pub fn mk_dev_vq1_matvec(codebook: *const f32, indices: *const u8, rows: usize, cols: usize, x: *const f32, exact: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_vq1_matvec_nt(codebook: *const f32, indices: *const u8, rows: usize, cols: usize, xt: *const f32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;

@@ -149,6 +149,66 @@ def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
         assert rel_l2(mid["o"][r], W2 @ mid["g"][r].astype(np.float64)) <= 1e-5  # "g" holds ACT(gate, up) after this call
 
 
+def bf16_round(a):
+    """bfloat16, round to nearest even, of an f32 array (as f32 values)."""
+    b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    b = ((b + 0x7FFF + ((b >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    return b.view(np.float32).reshape(np.shape(a))
+
+
+@pytest.mark.parametrize("T,topk,n_experts,d,inter,act", [(24, 2, 4, 512, 512, "swiglu"), (100, 2, 4, 1024, 512, "situ"), (5, 1, 3, 512, 1024, "swiglu"),
+                                                          # one group of 16, 17, 32, 33 rows: tile and pass boundaries
+                                                          (16, 1, 1, 512, 512, "swiglu"), (17, 1, 1, 512, 512, "situ"),
+                                                          (32, 1, 1, 1024, 512, "swiglu"), (33, 1, 1, 512, 512, "swiglu")])
+def test_moe_prefill_bf16_on_device(T, topk, n_experts, d, inter, act):
+    # mk_dev_moe_prefill_bf16: hidden rows and activation rows rounded to bfloat16 once, exact weights, f32 products and
+    # sums on the bf16 matrix instruction.
+    #   gate / up rows  against the f64 product of the dequantized weights and the bf16-rounded hidden rows: 1e-5
+    #   token rows      against oracle.moe_prefill(round_mxfp8=3) (the reference's loops on bf16-rounded inputs): 3e-4 --
+    #                   the device's expf and the CPU's can differ in the last bit in front of a bfloat16 rounding
+    #                   boundary of an activation value; one such step is 2^-8 of that value, about 1e-4 of a row of
+    #                   2048 activations (config 4 measures 6e-5 on its worst token row)
+    #   and the distance to the reference's own f32 arithmetic, which is the bfloat16 rounding of the two inputs
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(T * 13 + n_experts)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.uint32)
+    wts = rng.random((T, topk)).astype(np.float32)
+    kind = oracle.ACT_SITU if act == "situ" else oracle.ACT_SWIGLU
+    want = oracle.moe_prefill(table, ids, wts, x, act_kind=kind, round_mxfp8=3)
+    plain = oracle.moe_prefill(table, ids, wts, x, act_kind=kind, round_mxfp8=False)
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x), act_kind=model.ACT_SITU if act == "situ" else model.ACT_SWIGLU,
+                            bf16=True).cpu().numpy()
+    assert np.all(np.isfinite(got))
+    assert rel_l2(got, want) <= 3e-4
+    assert rel_l2(got, plain) <= 6e-3
+    mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
+    order = np.argsort(ids.reshape(-1), kind="stable")
+    for r in range(0, T * topk, max(1, T * topk // 7)):
+        e, t = int(ids.reshape(-1)[order[r]]), int(order[r]) // topk
+        xb = bf16_round(x[t]).astype(np.float64)
+        for name, k in (("g", 0), ("u", 1)):
+            Wd = oracle.mxfp4_dequant(host[e][k][0], host[e][k][1], inter, d).astype(np.float64)
+            assert rel_l2(mid[name][r], Wd @ xb) <= 1e-5, (name, r)
+
+
+def test_moe_prefill_bf16_refuses_other_shapes():
+    # d or inter not in multiples of 512, or a layer with VQ1 experts: MK_ERR_UNSUPPORTED, nothing computed
+    from microkimi_amd import model, workloads
+    d, inter = 256, 512
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, 0), workloads.mxfp4_matrix(4, "w3", inter, d, 0), workloads.mxfp4_matrix(4, "w2", d, inter, 0))]
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    x = np.zeros((4, d), np.float32)
+    with pytest.raises(Exception, match="512"):
+        model.moe_prefill(experts, dev(np.zeros((4, 1), np.int32)), dev(np.ones((4, 1), np.float32)), dev(x), bf16=True)
+
+
 def test_moe_prefill_f32_random_shapes():
     # a dozen seeded random shapes (token counts, top-k, expert counts, d and inter in multiples of 128, both
     # activations; routing with repeats allowed across tokens only) against the oracle without rounding
@@ -174,13 +234,14 @@ def test_moe_prefill_f32_random_shapes():
         assert np.isfinite(got).all() and err <= 1e-5, (case, T, topk, n_experts, d, inter, act, err)
 
 
-@pytest.mark.parametrize("exact", [False, True])
-def test_moe_prefill_skips_ids_out_of_range(exact):
+@pytest.mark.parametrize("arith", ["mxfp8", "f32", "bf16"])
+def test_moe_prefill_skips_ids_out_of_range(arith):
     # a pair whose expert id lies outside the table adds nothing to its token (include/mk_hip.h): the result equals the
     # oracle's with that pair pointed at a valid expert with routing weight 0; a token whose pairs are all out of range
     # comes out as zeros
     from microkimi_amd import model, workloads
-    T, topk, n_experts, d, inter = 37, 3, 5, 256, 128
+    T, topk, n_experts, d, inter = 37, 3, 5, 512, 512
+    exact = arith == "f32"
     rng = np.random.default_rng(5)
     host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
              workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
@@ -194,12 +255,12 @@ def test_moe_prefill_skips_ids_out_of_range(exact):
     dev_ids[bad] = np.where(rng.random(int(bad.sum())) < 0.5, -1, n_experts + 2)
     ref_ids, ref_wts = ids.copy(), wts.copy()
     ref_wts[bad] = 0.0
-    want = oracle.moe_prefill(table, ref_ids.astype(np.uint32), ref_wts, x, round_mxfp8=False if exact else 2)
+    want = oracle.moe_prefill(table, ref_ids.astype(np.uint32), ref_wts, x, round_mxfp8={"f32": False, "mxfp8": 2, "bf16": 3}[arith])
     pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
     experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
-    got = model.moe_prefill(experts, dev(dev_ids), dev(wts), dev(x), exact=exact).cpu().numpy()
+    got = model.moe_prefill(experts, dev(dev_ids), dev(wts), dev(x), exact=exact, bf16=arith == "bf16").cpu().numpy()
     assert np.all(np.isfinite(got)) and not got[7].any()
-    assert rel_l2(got, want) <= (1e-5 if exact else 2e-3)
+    assert rel_l2(got, want) <= {"f32": 1e-5, "mxfp8": 2e-3, "bf16": 3e-4}[arith]
 
 
 @pytest.mark.parametrize("T,topk,d,inter,act", [(40, 3, 256, 128, 0), (90, 2, 512, 256, 1), (7, 1, 128, 384, 0)])
@@ -261,6 +322,8 @@ def test_config4_full_size_expert_section():
       tokens     the output rows of ten sampled tokens against oracle.moe_prefill(round_mxfp8=2: MXFP8 inputs, full scale range), which gets the
                  eight experts of that token; the distance to the reference's own arithmetic (pure f32
                  matvec_packed_nt) is reported beside it
+      bf16 mode  mk_dev_moe_prefill_bf16 on the same weights: gate rows of two experts against the f64 product with the
+                 bf16-rounded hidden rows (1e-5), the ten token rows against the oracle on bf16-rounded inputs (3e-4)
       f32 mode   mk_dev_moe_prefill_f32 on the same weights: the up and down rows of two experts and the same ten
                  token rows against the oracle without rounding (the reference's arithmetic): relative L2 <= 1e-5
     The looser bound on the last two is one e4m3 rounding step of the activation (2^-4 relative) where the device's
@@ -336,8 +399,19 @@ def test_config4_full_size_expert_section():
         err = rel_l2(mid32["u"][r0:r1], x[toks].astype(np.float64) @ Wd.T)
         assert err <= 1e-5, f"expert {e}: f32 up rows {err:.2e}"
 
+    # ---- the bf16 section (mk_dev_moe_prefill_bf16) on the same weights
+    got_bf16 = model.moe_prefill(experts, ids, wts, dev(x), bf16=True).cpu().numpy()
+    assert np.isfinite(got_bf16).all()
+    mid16 = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
+    for e in (nonempty[-1], nonempty[0]):
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        toks = order[r0:r1] // topk
+        Wd = oracle.mxfp4_dequant(*host(w1[e]), inter, d).astype(np.float64)
+        err = rel_l2(mid16["g"][r0:r1], bf16_round(x[toks]).astype(np.float64) @ Wd.T)
+        assert err <= 1e-5, f"expert {e}: bf16 gate rows {err:.2e}"
+
     # ---- ten tokens end to end
-    worst, worst_f32, worst_exact = 0.0, 0.0, 0.0
+    worst, worst_f32, worst_exact, worst_bf16, worst_bf16_f32 = 0.0, 0.0, 0.0, 0.0, 0.0
     for tok in (0, 1, 63, 64, 127, 200, 255, 256, 400, 511):
         used = [int(e) for e in ids_h[tok]]
         table = oracle.ExpertTable([host(w1[e]) for e in used], [host(w3[e]) for e in used], [host(w2[e]) for e in used], d, inter)
@@ -347,8 +421,13 @@ def test_config4_full_size_expert_section():
         worst = max(worst, rel_l2(got[tok], want[0]))
         worst_f32 = max(worst_f32, rel_l2(got[tok], plain[0]))
         worst_exact = max(worst_exact, rel_l2(got_f32[tok], plain[0]))
+        want16 = oracle.moe_prefill(table, lid, wts_h[tok:tok + 1], x[tok:tok + 1], round_mxfp8=3)
+        worst_bf16 = max(worst_bf16, rel_l2(got_bf16[tok], want16[0]))
+        worst_bf16_f32 = max(worst_bf16_f32, rel_l2(got_bf16[tok], plain[0]))
     print(f"config 4 full size: worst token row vs MXFP8 oracle {worst:.2e}, vs the pure-f32 reference path {worst_f32:.2e}")
     print(f"config 4 full size, f32 mode: worst token row vs the pure-f32 reference path {worst_exact:.2e}")
+    print(f"config 4 full size, bf16 mode: worst token row vs the bf16-input oracle {worst_bf16:.2e}, vs the pure-f32 reference path {worst_bf16_f32:.2e}")
     assert worst <= 2e-3
+    assert worst_bf16 <= 3e-4 and worst_bf16_f32 <= 6e-3
     assert worst_exact <= 1e-5
     assert worst_f32 < 0.06  # the e4m3 rounding of the activations: reported, not a parity claim
