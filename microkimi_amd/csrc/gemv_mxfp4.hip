@@ -537,8 +537,18 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
     __shared__ float xs_l[2][NTT * 16][XS];
     __shared__ __attribute__((aligned(16))) float cb_l[VQ ? 256 * 16 : 4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
-    const int grp = blockIdx.y, mat = blockIdx.z;
     const bool one = a.offsets == nullptr;
+    // (groups in a multiple of 8: a group's workgroups on one XCD, see the bf16 kernel below)
+    int grp = blockIdx.y, mat = blockIdx.z, rblk = blockIdx.x;
+    if (!one && (gridDim.y & 7) == 0) {
+        const int per = gridDim.x * gridDim.z;
+        const int lin = (int)blockIdx.x + (int)gridDim.x * ((int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z);
+        const int xcd = lin & 7, slot = lin >> 3;
+        grp = (slot / per) * 8 + xcd;
+        const int inner = slot % per;
+        mat = inner / (int)gridDim.x;
+        rblk = inner % (int)gridDim.x;
+    }
     const int p_begin = one ? grp * 16 * NTT : a.offsets[grp], p_end = one ? min(a.m1, p_begin + 16 * NTT) : a.offsets[grp + 1];
     if (p_end <= p_begin) return;  // (the whole workgroup)
     const uint8_t *__restrict__ packed = one ? a.packed1 : a.packed[mat][grp];
@@ -550,7 +560,7 @@ __global__ __launch_bounds__(64 * RW) void mxfp4_gemm_nt_grouped_kernel(NtGroupe
         for (int k = threadIdx.x; k < 256 * 4; k += 64 * RW) reinterpret_cast<mk_f4 *>(cb_l)[k] = reinterpret_cast<const mk_f4 *>(a.codebook)[k];
         // (the barrier in front of the first step also covers the codebook)
     }
-    const int row0 = ((int)blockIdx.x * RW + wave) * 16;   // (a wave past the last row works on the last row and stores nothing)
+    const int row0 = (rblk * RW + wave) * 16;   // (a wave past the last row works on the last row and stores nothing)
     const int row = min(row0 + i, a.rows - 1);
     const size_t cols = (size_t)nb * 32;
     const bool sc_al4 = ((uintptr_t)scales & 3) == 0;
@@ -680,14 +690,26 @@ __global__ __launch_bounds__(64 * RW) __attribute__((amdgpu_waves_per_eu(4))) vo
     static_assert(PER >= 1 && PER * 64 * RW == NTT * 16 * 64, "threads must divide the staged activations");
     __shared__ __attribute__((aligned(16))) uint8_t xs_l[2][NTT * 16 * XSB];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = lane & 15, g = lane >> 4;
-    const int grp = blockIdx.y, mat = blockIdx.z;
+    // Workgroup ids go round the eight XCDs in turn, each with its own L2: with a multiple of 8 groups, id -> (XCD,
+    // slot) and a group's workgroups (row blocks x matrices) take consecutive slots of one XCD, so that the group's
+    // activation rows are fetched into one L2 instead of eight.
+    int grp = blockIdx.y, mat = blockIdx.z, rblk = blockIdx.x;
+    if ((gridDim.y & 7) == 0) {
+        const int per = gridDim.x * gridDim.z;
+        const int lin = (int)blockIdx.x + (int)gridDim.x * ((int)blockIdx.y + (int)gridDim.y * (int)blockIdx.z);
+        const int xcd = lin & 7, slot = lin >> 3;
+        grp = (slot / per) * 8 + xcd;
+        const int inner = slot % per;
+        mat = inner / (int)gridDim.x;
+        rblk = inner % (int)gridDim.x;
+    }
     const int p_begin = a.offsets[grp], p_end = a.offsets[grp + 1];
     if (p_end <= p_begin) return;  // (the whole workgroup)
     const uint8_t *__restrict__ packed = a.packed[mat][grp];
     const uint8_t *__restrict__ scales = a.scales[mat][grp];
     float *__restrict__ out = a.out[mat];
     const int nb = a.nb, ktiles = nb / 16;
-    const int row0 = ((int)blockIdx.x * RW + wave) * 16;  // (a wave past the last row works on the last row and stores nothing)
+    const int row0 = (rblk * RW + wave) * 16;  // (a wave past the last row works on the last row and stores nothing)
     const size_t cols = (size_t)nb * 32;
     const uint8_t *wline[2];
 #pragma unroll
