@@ -340,6 +340,18 @@ int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, const uint8_t *
                               size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
                               void *stream);
 
+/* The same grouped product in the reference's own arithmetic, matvec_packed_nt per group (src/model.rs:2412-2447,
+ * called per expert at src/model.rs:2580-2599): x [m][cols] f32, exactly dequantized weights, f32 products and sums on
+ * the f32 matrix instruction (order of the sums apart: relative L2 below 1e-5).  cols % 128 == 0, rows % 4 == 0,
+ * x and out 16-byte aligned; same offsets and out as above. */
+int mk_dev_mxfp4_grouped_gemm_f32(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                  size_t cols, const float *x, const int32_t *offsets, size_t m, float *out, void *stream);
+/* And with bfloat16 activations x [m][cols] (the caller rounds them once): the weights are exact in bfloat16, the
+ * products exact in f32 and summed in f32 on v_mfma_f32_16x16x32_bf16.  MK_ERR_UNSUPPORTED unless cols % 512 == 0 and
+ * rows % 4 == 0. */
+int mk_dev_mxfp4_grouped_gemm_bf16(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                   size_t cols, const uint16_t *x, const int32_t *offsets, size_t m, float *out, void *stream);
+
 /* Bytes of device scratch mk_dev_moe_prefill needs. */
 size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter);
 

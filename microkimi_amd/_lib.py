@@ -93,6 +93,8 @@ def _load():
         "mk_mla_heads_workspace_bytes": (sz, [sz, sz, sz, sz]),
         "mk_dev_mla_heads_q8_attn": (i32, [vp, vp, vp, vp, vp, sz, vp, sz, sz, sz, sz, sz, f32, i32, vp, vp, vp]),
         "mk_dev_mxfp4_grouped_gemm": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
+        "mk_dev_mxfp4_grouped_gemm_f32": (i32, [vp, vp, sz, sz, sz, vp, vp, sz, vp, vp]),
+        "mk_dev_mxfp4_grouped_gemm_bf16": (i32, [vp, vp, sz, sz, sz, vp, vp, sz, vp, vp]),
         "mk_moe_prefill_workspace_bytes": (sz, [sz, sz, sz, sz, sz]),
         "mk_moe_prefill_workspace_layout": (i32, [sz, sz, sz, sz, sz, C.POINTER(PrefillLayout)]),
         "mk_dev_moe_prefill": (i32, [C.POINTER(ExpertTable), sz, sz, sz, vp, vp, vp, i32, vp, vp, vp]),

@@ -1010,6 +1010,19 @@ int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_p
     return mk_launch_status("mxfp4_gemm_bf16_grouped");
 }
 
+extern "C" int mk_dev_mxfp4_grouped_gemm_f32(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                             size_t cols, const float *x, const int32_t *offsets, size_t m, float *out, void *stream) {
+    MK_REQUIRE(packed_ptrs && scales_ptrs && x && offsets && out, "null pointer");
+    return mk_mxfp4_grouped_gemm_nt(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, x, nullptr, 1, offsets, m, nullptr, &out, stream);
+}
+
+extern "C" int mk_dev_mxfp4_grouped_gemm_bf16(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                              size_t cols, const uint16_t *x, const int32_t *offsets, size_t m, float *out, void *stream) {
+    MK_REQUIRE(packed_ptrs && scales_ptrs && x && offsets && out, "null pointer");
+    (void)m;
+    return mk_mxfp4_grouped_gemm_bf16(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, x, offsets, &out, stream);
+}
+
 extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m,
                                       float *out, void *stream) {
     MK_REQUIRE(packed && scales && x && out, "null pointer");

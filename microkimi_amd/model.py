@@ -369,6 +369,24 @@ def router_softmax_topk(logits, k):
     return ids, w
 
 
+def grouped_gemm_f32(packed_list, scales_list, rows, cols, x, offsets, bf16=False):
+    """matvec_packed_nt per group (src/model.rs:2412-2447 as called at src/model.rs:2580-2599): rows
+    offsets[e]..offsets[e+1] of x [m, cols] against expert e -> [m, rows] f32.  x f32: the reference's f32 arithmetic on
+    the f32 matrix instruction; bf16=True: x is a torch.bfloat16 tensor, exact weights, f32 products and sums on the
+    bf16 matrix instruction."""
+    import torch
+    _lib.require_device()
+    dev = x.device
+    pp = torch.tensor([t.data_ptr() for t in packed_list], dtype=torch.int64, device=dev)
+    sp = torch.tensor([t.data_ptr() for t in scales_list], dtype=torch.int64, device=dev)
+    m = x.shape[0]
+    assert x.is_contiguous() and x.dtype == (torch.bfloat16 if bf16 else torch.float32)
+    out = torch.empty((m, rows), dtype=torch.float32, device=dev)
+    fn = lib.mk_dev_mxfp4_grouped_gemm_bf16 if bf16 else lib.mk_dev_mxfp4_grouped_gemm_f32
+    check(fn(ptr(pp), ptr(sp), len(packed_list), rows, cols, ptr(x), ptr(offsets), m, ptr(out), cur_stream()))
+    return out
+
+
 def grouped_gemm_mxfp8(packed_list, scales_list, rows, cols, codes, exps, offsets):
     """Per-expert batched evaluation of moe_prefill (src/model.rs:2539-2602) on the block-scaled matrix cores:
     rows offsets[e]..offsets[e+1] of the MXFP8 activations (codes, exps) against expert e -> [m, rows] f32."""

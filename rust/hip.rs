@@ -150,6 +150,8 @@ extern "C" {
     pub fn mk_mla_heads_workspace_bytes(m: usize, nh: usize, nope: usize, vd: usize) -> usize;
     pub fn mk_dev_mla_heads_q8_attn(kq: *const i8, ks: *const f32, kr: *const f32, vq: *const i8, vs: *const f32, pos0: usize, q: *const f32, m: usize, nh: usize, nope: usize, rope: usize, vd: usize, scale: f32, hadamard: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_grouped_gemm(packed_ptrs: *const *const u8, scales_ptrs: *const *const u8, n_groups: usize, rows: usize, cols: usize, codes: *const u8, exps: *const u8, offsets: *const i32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4_grouped_gemm_f32(packed_ptrs: *const *const u8, scales_ptrs: *const *const u8, n_groups: usize, rows: usize, cols: usize, x: *const f32, offsets: *const i32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4_grouped_gemm_bf16(packed_ptrs: *const *const u8, scales_ptrs: *const *const u8, n_groups: usize, rows: usize, cols: usize, x: *const u16, offsets: *const i32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_moe_prefill_workspace_bytes(T: usize, topk: usize, n_experts: usize, d: usize, inter: usize) -> usize;
     pub fn mk_moe_prefill_workspace_layout(T: usize, topk: usize, n_experts: usize, d: usize, inter: usize, out: *mut MkPrefillLayout) -> c_int;
     pub fn mk_dev_moe_prefill(table: *const MkExpertTable, n_experts: usize, T: usize, topk: usize, ids: *const i32, weights: *const f32, x: *const f32, act_kind: c_int, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;

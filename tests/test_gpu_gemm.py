@@ -149,6 +149,28 @@ def test_moe_prefill_f32_on_device(T, topk, n_experts, d, inter, act):
         assert rel_l2(mid["o"][r], W2 @ mid["g"][r].astype(np.float64)) <= 1e-5  # "g" holds ACT(gate, up) after this call
 
 
+@pytest.mark.parametrize("rows,cols,counts,bf16", [(128, 512, [5, 0, 20, 33], False), (100, 256, [16, 17], False), (64, 1024, [3, 70], True),
+                                                  (256, 512, [0, 0, 16, 1, 32, 0, 7, 9], True)])
+def test_grouped_gemm_f32_and_bf16(rows, cols, counts, bf16):
+    # the grouped products on their own (a caller that keeps its own grouping): every group's rows against the f64
+    # product of its dequantized matrix and the rows (bf16: the rows as the kernel gets them), empty groups included
+    torch = torch_cuda()
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(rows + cols)
+    mats = [workloads.mxfp4_matrix(4, "w1", rows, cols, e) for e in range(len(counts))]
+    m = int(sum(counts))
+    x = (rng.standard_normal((m, cols)) * 0.1).astype(np.float32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    xd = dev(x).to(torch.bfloat16).contiguous() if bf16 else dev(x)
+    got = model.grouped_gemm_f32([dev(p) for p, _ in mats], [dev(s) for _, s in mats], rows, cols, xd, dev(offsets), bf16=bf16).cpu().numpy()
+    xin = xd.to(torch.float32).cpu().numpy().astype(np.float64) if bf16 else x.astype(np.float64)
+    for e, (p, s) in enumerate(mats):
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        if r1 > r0:
+            Wd = oracle.mxfp4_dequant(p, s, rows, cols).astype(np.float64)
+            assert rel_l2(got[r0:r1], xin[r0:r1] @ Wd.T) <= 1e-5, e
+
+
 def bf16_round(a):
     """bfloat16, round to nearest even, of an f32 array (as f32 values)."""
     b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
