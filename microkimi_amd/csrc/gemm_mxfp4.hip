@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 // through readfirstlane, which hides the loop counter from the induction
 // variable widening that would otherwise rebuild 64-bit pointers per lane.
 constexpr int KT_STEPS = 4;
-constexpr int A_STRIDE = 512 + 16;  // LDS row stride of the activation tile: 16 rows fall in distinct banks
+constexpr int A_STRIDE = 512 + 32;  // LDS row stride of the activation tile: rows 8 banks apart (with 4 or 16 banks the 16-byte operand reads counted 2.5 times the bank-conflict cycles)
 constexpr int a_codes_bytes(int mc) { return 16 * mc * A_STRIDE; }
 constexpr int a_wsc_off(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }      // codes, then 16 scale bytes per token,
 constexpr int a_buf_bytes(int mc) { return a_wsc_off(mc) + 256 * 16; }            // then the K tile's 16 scale bytes of the 256 weight rows
