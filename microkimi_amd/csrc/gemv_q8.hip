@@ -205,7 +205,12 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
     mk_i4 *xl = reinterpret_cast<mk_i4 *>(lds);                      // [cols/16][8]
     float *xsl = reinterpret_cast<float *>(lds + (size_t)cols * 8);  // [nb][8]
     const int group_bytes = 16 * nb * SB;
-    uint8_t *sl = lds + (size_t)cols * 8 + (size_t)nb * 32 + (size_t)(threadIdx.x >> 6) * group_bytes;  // this wave's scale tile
+    // A row of the wave's scale tile takes row_bytes + 4 in LDS when the row is a whole number of 16-byte chunks: the
+    // 16 rows a step's 2-byte reads touch then start in different banks (at 448 bytes a row they fell on four).
+    const int row_bytes = nb * SB, cpr = row_bytes / 16;
+    const bool padded = (row_bytes & 15) == 0;
+    const int row_stride = padded ? row_bytes + 4 : row_bytes;
+    uint8_t *sl = lds + (size_t)cols * 8 + (size_t)nb * 32 + (size_t)(threadIdx.x >> 6) * (group_bytes + 64);  // this wave's scale tile
     for (int i = threadIdx.x; i < (cols / 16) * 8; i += WAVES * 64) {
         const int c = i >> 3, b = i & 7;
         mk_i4 v = {0, 0, 0, 0};
@@ -242,13 +247,23 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
                            : mk_i4{0, 0, 0, 0};
         }
     };
+    int soff[NIT];  // where chunk it * 64 + lane of a group's scales goes in the tile
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int c = it * 64 + lane;
+        soff[it] = padded ? (c / cpr) * row_stride + (c % cpr) * 16 : c * 16;
+    }
     if (wave < n_groups) prefetch_scales(wave);
     // 16-row groups are dealt round-robin to the resident waves
     for (int grp = wave; grp < n_groups; grp += n_waves) {
 #pragma unroll
         for (int it = 0; it < NIT; it++) {
             const int off = (it * 64 + lane) * 16;
-            if (off < group_bytes) *reinterpret_cast<mk_i4 *>(sl + off) = spre[it];
+            if (off < group_bytes) {
+                // (a padded row starts 4 bytes later than the one before: the chunk is stored as four words)
+                uint32_t *dst = reinterpret_cast<uint32_t *>(sl + soff[it]);
+                dst[0] = (uint32_t)spre[it][0], dst[1] = (uint32_t)spre[it][1], dst[2] = (uint32_t)spre[it][2], dst[3] = (uint32_t)spre[it][3];
+            }
         }
         if (grp + n_waves < n_groups) prefetch_scales(grp + n_waves);
         const int row = grp * 16 + n;
@@ -263,7 +278,7 @@ __global__ __launch_bounds__(WAVES * 64) void q8_gemv_mfma_kernel(const int8_t *
 #pragma unroll
         for (int h = 0; h < 2; h++) wline[h] = q + (size_t)min(grp * 16 + 8 * h + (lane >> 3), rows - 1) * cols + (lane & 7) * 16;
         const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
-        const uint8_t *srow = sl + (size_t)(n * nb + par) * SB;
+        const uint8_t *srow = sl + (size_t)n * row_stride + (size_t)par * SB;
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         mk_i4 wa[S], wb[S];
         auto load_block = [&](mk_i4 *wv, int s0) {
@@ -465,7 +480,7 @@ int launch_q8(const int8_t *q, const void *scales, size_t rows, size_t cols, con
         const int n_groups = (int)((rows + 15) / 16);
         int blocks = MK_TUNE("MK_Q8_MFMA_BLOCKS", 256);  // one per CU
         if (blocks * WAVES > n_groups) blocks = (n_groups + WAVES - 1) / WAVES;
-        const size_t lds = cols * 8 + (size_t)nb * 32 + (size_t)WAVES * 16 * nb * (F16 ? 2 : 4);
+        const size_t lds = cols * 8 + (size_t)nb * 32 + (size_t)WAVES * (16 * nb * (F16 ? 2 : 4) + 64);
         if (nb % 4 == 0 && !MK_TUNE("MK_Q8_MFMA_HALF_LINES", 0))  // rows are whole 128-byte lines
             hipLaunchKernelGGL((q8_gemv_mfma_kernel<F16, WAVES, true>), dim3(blocks), dim3(WAVES * 64), lds, st, q, scales, (int)rows, nb, xq,
                                xs, (int)batch, out);
