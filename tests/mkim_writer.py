@@ -2,8 +2,8 @@
 
 Blob offsets in write order: routed-expert tensors (name contains ".block_sparse_moe.experts." and ends in .w1/.w2/.w3,
 src/weights.rs:417-419) start on an `expert_align` boundary (4096 by default), everything else on 64; padding is zeros.
-No file of this format ships with the reference, so the loader is checked against files made here and against a header
-assembled byte by byte in the test itself.
+The loader is checked against three things: tests/golden/mkim_ref.bin, a file written by the reference's own exporter
+(nano/export.py), files made here by these rules, and a header assembled byte by byte in the test itself.
 """
 import json
 import struct
