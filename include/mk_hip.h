@@ -196,7 +196,21 @@ typedef struct {
      * device, or NULL when every expert is MXFP4.  A VQ1 expert has its index bytes ([rows][cols/16]) where the packed
      * nibbles would be (w1p, w3p, w2p) and NULL scale pointers (w1s, w3s, w2s). */
     const float *vq_codebook;
+    /* Optional (NULL: not there): per expert, W2 once more in slab-major tiles (mk_dev_mxfp4_to_slab).  With it, up to 4
+     * decode tokens in q8 mode take the one-launch form of the layer (see mk_dev_moe_decode). */
+    const uint8_t *const *w2t;
 } mk_expert_table;
+
+/* A second layout of an MXFP4 matrix [rows][cols] for the kernel that multiplies ONE q8 block of the activation into
+ * the matching 32 columns of every row (the down projection of the one-launch MoE decode): tile (b, i), at byte
+ * (b * rows / 256 + i) * 4352, holds block b (columns 32 b .. 32 b + 31) of the rows 256 i .. 256 i + 255 as
+ * 4 x 64 x 16 nibble bytes (row 256 i + 64 j + l at j * 1024 + l * 16, the 16 bytes as in the reference layout,
+ * src/mxfp4.rs:1-3) and 64 x 4 scale bytes (row 256 i + 64 j + l at 4096 + 4 l + j).  The same bytes in another order:
+ * mk_dev_mxfp4_slab_dequant gives mxfp4::dequant (src/mxfp4.rs:19-31) bit for bit.  rows % 256 == 0, cols % 32 == 0;
+ * mk_mxfp4_slab_bytes = rows * cols / 32 * 17, the size of packed + scales.  packed and slab 16-byte aligned. */
+size_t mk_mxfp4_slab_bytes(size_t rows, size_t cols);
+int mk_dev_mxfp4_to_slab(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, uint8_t *slab, void *stream);
+int mk_dev_mxfp4_slab_dequant(const uint8_t *slab, size_t rows, size_t cols, float *out, void *stream);
 
 /* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
 size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
@@ -213,7 +227,12 @@ size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, s
  * mode MK_MODE_Q8 re-quantizes x and act per 32 exactly as matvec_packed does on
  * each call.  A selected expert that is VQ1 (table->vq_codebook set, NULL scale pointers) takes quant::matvec_vq
  * (src/quant.rs:333-346) for its three products, on the f32 hidden and activation rows, whatever `mode` says
- * (src/model.rs:2243-2257); the workspace then also holds mk_moe_decode_vq_workspace_bytes. */
+ * (src/model.rs:2243-2257); the workspace then also holds mk_moe_decode_vq_workspace_bytes.
+ * Kernels by batch (q8 mode, MXFP4 experts, model-like shapes): 1-3 tokens with table->w2t: one streaming launch in
+ * which a workgroup takes 64 rows of W1 and W3 of a pair, forms the two q8 blocks of the activation they give and
+ * multiplies them into the matching slabs of W2, then a small kernel that adds the partial rows in a fixed order;
+ * without w2t: a gate/up launch and a down launch; from 4 tokens: the pairs grouped by expert on the matrix cores.
+ * Every form adds the reference's block terms (src/mxfp4.rs:405-443); only the order of the sum over blocks differs. */
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
 

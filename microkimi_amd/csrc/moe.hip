@@ -16,7 +16,7 @@
 // intermediates (act: 2 KiB + 256 B per pair, o: 28 KiB per pair) are noise.
 #include <stdlib.h>
 
-#include "mk_common.h"
+#include "mk_moe.h"
 
 // grouped MXFP4 GEMV of gemv_mxfp4.hip: q8 (xq, xs) or f32 (xf) activations, one launch over nmat matrices
 int mk_gemv_grouped_internal(bool q8, const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t nmat, size_t rows,
@@ -65,10 +65,13 @@ struct Workspace {
     int32_t *goff;     // [P + 1] first grouped row of every group
     int32_t *gexp;     // [P] expert of every group
     int32_t *ngroups;  // [2]: number of groups, index of the largest group
+    float *part;       // one-launch path (up to SLAB_MAX_B tokens): [P][inter / 32][d] partial rows
     size_t bytes;
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+constexpr int SLAB_MAX_B = 4;  // tokens the one-launch path (moe_slab.hip) takes: its partial rows are 1.8 MB a pair at the model shape
 
 Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, size_t inter) {
     const size_t P = B * (topk + (has_shared ? 1 : 0));
@@ -106,15 +109,9 @@ Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, siz
     w.goff = (int32_t *)take((P + 1) * 4);
     w.gexp = (int32_t *)take(P * 4);
     w.ngroups = (int32_t *)take(8);
+    w.part = (float *)take(B <= (size_t)SLAB_MAX_B && mk_moe_slab_takes(d, inter, (int)(P / B)) ? mk_moe_slab_part_bytes(P, d, inter) : 0);
     w.bytes = off;
     return w;
-}
-
-// Expert id of a routed pair.  When the table states its size, an id outside it selects entry 0 with routing weight 0:
-// the pair then adds nothing to the token's row (the pointer arrays are never read out of bounds).
-__device__ __forceinline__ int mk_checked_expert(int e, size_t n_experts, bool &ok) {
-    ok = n_experts == 0 || (unsigned)e < (unsigned)n_experts;
-    return ok ? e : 0;
 }
 
 __global__ void moe_setup_kernel(mk_expert_table tab, int B, int topk, int shared, const int32_t *__restrict__ ids,
@@ -139,19 +136,6 @@ __global__ void moe_setup_kernel(mk_expert_table tab, int B, int topk, int share
     pt.pw[p] = s < topk ? (ok ? weights[t * topk + s] : 0.0f) : 1.0f;
 }
 
-__device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
-    float h = 0.0f;
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        uint32_t wd = (uint32_t)w[d];
-        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 0), xr[d * 4 + 0], h, false);
-        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 1), xr[d * 4 + 1], h, false);
-        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 2), xr[d * 4 + 2], h, false);
-        h = __builtin_amdgcn_fdot2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(wd, 1.0f, 3), xr[d * 4 + 3], h, false);
-    }
-    return h;
-}
-
 // ------------------------------------------------------------ fused fast path
 // Two launches per layer, no setup / quantize / combine kernels:
 //
@@ -169,17 +153,6 @@ __device__ __forceinline__ float dot32_fp4_f16(const mk_i4 w, const mk_h2 *xr) {
 //            pair in slot order and accumulates y += w * (W2_e act) in registers,
 //            so the weighted sum of src/model.rs:2346-2351 needs no intermediate
 //            buffer.
-struct FusedArgs {
-    mk_expert_table tab;
-    const int32_t *ids;
-    const float *weights;
-    const float *x;
-    int topk, shared, per, d, inter, act_kind, ds_rule;
-    float limit;
-    float *af;   // [P][inter]  activation values in f32 (the down kernel forms their q8 blocks)
-    float *out;  // [B][d]
-};
-
 // Row-owner gate/up: wave w owns the rows w, w + W, ... of W1 and W3 in every pair
 // (three units = 3 x 2 rows in flight per wave).  Tokens are taken in groups
 // that fit LDS (q8 of the hidden rows as f16 pairs); a lane keeps the activation
@@ -328,7 +301,7 @@ __global__ __launch_bounds__(512) void moe_gate_up_rows_kernel(FusedArgs a, int 
                 float s1 = 0.0f, s3 = 0.0f;
 #pragma unroll
                 for (int t = 0; t < T; t++) {
-                    const float h1 = dot32_fp4_f16(U.w1[t], xr[t]), h3 = dot32_fp4_f16(U.w3[t], xr[t]);
+                    const float h1 = mk_dot32_fp4_f16(U.w1[t], xr[t]), h3 = mk_dot32_fp4_f16(U.w3[t], xr[t]);
                     s1 += (h1 + h1) * (mk_half_scale_from_byte(U.s1[t]) * cf[t]);
                     s3 += (h3 + h3) * (mk_half_scale_from_byte(U.s3[t]) * cf[t]);
                 }
@@ -479,7 +452,7 @@ __global__ __launch_bounds__(WAVES * 64) void moe_down_fused_kernel(FusedArgs a)
             for (int r = 0; r < RT; r++) acc[r] = 0.0f;
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                float h = dot32_fp4_f16(w[u][t], xr[t]);
+                float h = mk_dot32_fp4_f16(w[u][t], xr[t]);
                 float term = (h + h) * (mk_half_scale_from_byte(sc[u][t]) * cf[t]);
                 const int rit = (t * 64 + lane) / NB;
 #pragma unroll
@@ -795,7 +768,7 @@ int launch_down_fused(const FusedArgs &a, size_t B, hipStream_t st) {
 }  // namespace
 
 namespace {
-enum { STAGE_ALL = 0, STAGE_ACT = 1, STAGE_FROM_ACT = 2 };
+enum { STAGE_ALL = MK_MOE_STAGE_ALL, STAGE_ACT = MK_MOE_STAGE_ACT, STAGE_FROM_ACT = MK_MOE_STAGE_FROM_ACT };
 
 // The layer, or one of its two stages: STAGE_ACT stops after the activation rows (act_io [B * per][inter], out),
 // STAGE_FROM_ACT starts from given activation rows (act_io, in).  Both run the kernels the whole layer runs.
@@ -863,7 +836,10 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         return mk_launch_status("moe_combine_grouped");
     }
     float *af = stage == STAGE_ALL ? w.af : act_io;  // [P][inter] activation rows in (token, slot) order
-    if (fast && !has_vq) {
+    // one streaming launch + a small reduction when the table carries W2 in slab-major tiles
+    const bool slab = !has_vq && mode == MK_MODE_Q8 && table->w2t != nullptr && B <= (size_t)SLAB_MAX_B &&
+                      mk_moe_slab_takes(d, inter, per) && ((uintptr_t)x & 15) == 0 && !MK_TUNE("MK_MOE_NO_SLAB", 0);
+    if ((fast || slab) && !has_vq) {
         FusedArgs fa;
         fa.tab = *table;
         fa.ids = ids;
@@ -879,6 +855,7 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         fa.limit = limit;
         fa.af = af;
         fa.out = out;
+        if (slab) return mk_moe_slab_launch(fa, B, stage, w.part, st);
         if (stage != STAGE_FROM_ACT) {
             switch (nb) {
                 case 32: s = launch_gate_up_rows<32>(fa, B, st); break;

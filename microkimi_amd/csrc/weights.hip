@@ -275,7 +275,12 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
         cb_off = off;
         off = align_up(off + (size_t)en.size, 256);
     }
-    const size_t tab_off = off, total = off + 6 * n_experts * sizeof(void *);
+    // W2 of every expert once more in slab-major tiles (mk_dev_mxfp4_to_slab) for the one-launch decode layer, when the
+    // layer's shapes allow it and MK_W2_SLAB is not 0: as many bytes again as W2 itself
+    const bool with_slab = !any_vq && d % 1024 == 0 && inter % 32 == 0 && mk_env_int("MK_W2_SLAB", 1) != 0;
+    const size_t slab_each = with_slab ? align_up(mk_mxfp4_slab_bytes(d, inter), 256) : 0, slab_off = off;
+    off += slab_each * n_experts;
+    const size_t tab_off = off, total = off + 7 * n_experts * sizeof(void *);
     mk_expert_set *s = new mk_expert_set;
     if (hipMalloc(&s->dev, total) != hipSuccess) {
         (void)hipGetLastError();
@@ -287,7 +292,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->n = n_experts;
     uint8_t *base = (uint8_t *)s->dev;
     // pass 2: one copy per blob straight out of the mapping, then the pointer arrays
-    std::vector<const uint8_t *> ptrs(6 * n_experts);
+    std::vector<const uint8_t *> ptrs(7 * n_experts);
     for (size_t e = 0; e < n_experts; e++) {
         for (int k = 0; k < 3; k++) {
             const Blob &b = blobs[e * 3 + k];
@@ -300,6 +305,22 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
             ptrs[(size_t)(2 * k) * n_experts + e] = base + b.dev_off;                                  // packed nibbles, or VQ1 index bytes
             ptrs[(size_t)(2 * k + 1) * n_experts + e] = vq[e] ? nullptr : base + b.dev_off + b.half;  // scales (none: VQ1)
         }
+    }
+    for (size_t e = 0; e < n_experts; e++) {
+        ptrs[6 * n_experts + e] = nullptr;
+        if (!with_slab) continue;
+        uint8_t *slab = base + slab_off + e * slab_each;
+        if (mk_dev_mxfp4_to_slab(ptrs[4 * n_experts + e], ptrs[5 * n_experts + e], d, inter, slab, nullptr) != MK_OK) {
+            mk_expert_set_free(s);
+            return MK_ERR_HIP;
+        }
+        ptrs[6 * n_experts + e] = slab;
+    }
+    if (with_slab && hipDeviceSynchronize() != hipSuccess) {
+        (void)hipGetLastError();
+        mk_expert_set_free(s);
+        mk_set_error("the slab-major copy of W2 failed");
+        return MK_ERR_HIP;
     }
     if (cb_host && hipMemcpy(base + cb_off, cb_host, 256 * 16 * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
         (void)hipGetLastError();
@@ -324,6 +345,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->table.inter = inter;
     s->table.n_experts = n_experts;
     s->table.vq_codebook = any_vq ? reinterpret_cast<const float *>(base + cb_off) : nullptr;
+    s->table.w2t = with_slab ? tab + 6 * n_experts : nullptr;
     *out = s;
     return MK_OK;
 }

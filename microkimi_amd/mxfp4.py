@@ -31,6 +31,26 @@ def dequant(packed, scales, rows, cols):
     return out
 
 
+def to_slab(packed, scales, rows, cols):
+    """The slab-major copy of an MXFP4 matrix on the device (mk_dev_mxfp4_to_slab): block b of the rows 256 i .. 256 i + 255
+    as one 4352-byte tile, tiles of a block contiguous.  The layout the one-launch MoE decode reads W2 in."""
+    import torch
+    _lib.require_device()
+    _check_shapes(packed, scales, rows, cols)
+    slab = torch.empty(lib.mk_mxfp4_slab_bytes(rows, cols), dtype=torch.uint8, device=packed.device)
+    check(lib.mk_dev_mxfp4_to_slab(ptr(packed), ptr(scales), rows, cols, ptr(slab), cur_stream()))
+    return slab
+
+
+def dequant_slab(slab, rows, cols):
+    """mxfp4::dequant (src/mxfp4.rs:19-31) read from the slab-major copy: f32 [rows, cols], bit-exact."""
+    import torch
+    _lib.require_device()
+    out = torch.empty((rows, cols), dtype=torch.float32, device=slab.device)
+    check(lib.mk_dev_mxfp4_slab_dequant(ptr(slab), rows, cols, ptr(out), cur_stream()))
+    return out
+
+
 def quantize(w, search=True):
     """mxfp4::quantize (search) / quantize_naive (src/mxfp4.rs:38-138) of a device tensor [rows, cols] f32: the
     reference's (packed [rows, cols/2], scales [rows, cols/32]) bytes."""

@@ -40,7 +40,7 @@ def rows_match_up_to_q8_flips(got, want, w2_of_token, d, inter, max_flips=2):
     return flips
 
 
-def build(n_experts, d, inter, cfg=2):
+def build(n_experts, d, inter, cfg=2, slab=None):
     from microkimi_amd import model, workloads
     host = [(workloads.mxfp4_matrix(cfg, "w1", inter, d, e), workloads.mxfp4_matrix(cfg, "w3", inter, d, e),
              workloads.mxfp4_matrix(cfg, "w2", d, inter, e)) for e in range(n_experts)]
@@ -49,7 +49,7 @@ def build(n_experts, d, inter, cfg=2):
     w2 = [h[2] for h in host]
     table = oracle.ExpertTable(w1, w3, w2, d, inter)
     todev = lambda lst: [(dev(p), dev(s)) for p, s in lst]
-    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter)
+    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter, slab=slab)
     return table, experts
 
 
@@ -62,7 +62,7 @@ def table_host(table, k):
 @pytest.mark.parametrize("d,inter,n_experts,B,topk,shared,act", [
     (7168, 2048, 12, 1, 8, 11, 0),    # benchmark layer shapes, batch 1, shared expert
     (7168, 2048, 12, 4, 8, 11, 0),    # batch 4 (the smallest batch on the batched path)
-    (7168, 2048, 12, 3, 8, 11, 0),    # batch 3 (two-kernel path)
+    (7168, 2048, 12, 3, 8, 11, 0),    # batch 3 (one-launch path)
     (2048, 1024, 6, 3, 2, -1, 1),     # SiTU (K3 rule), no shared expert
     (4096, 2048, 5, 2, 3, 4, 2),      # DeepSeek rule: clamp, weight before W2, plain sum
     (1024, 512, 4, 16, 2, 3, 0),      # batch 16
@@ -73,7 +73,7 @@ def table_host(table, k):
     (4096, 2048, 5, 11, 3, 4, 2),     # batched path, DeepSeek rule, groups of more than four tokens (several passes)
     (7168, 2048, 12, 16, 8, 11, 0),   # batched path at the benchmark layer's shapes, batch 16
     (1024, 512, 4, 5, 3, -1, 0),      # batched path, an odd number of pairs
-    (7168, 2048, 12, 2, 8, 11, 100),  # hidden ~ N(0, 1) as the benchmark configuration states (saturated silu), two-kernel path
+    (7168, 2048, 12, 2, 8, 11, 100),  # hidden ~ N(0, 1) as the benchmark configuration states (saturated silu), one-launch path
     (7168, 2048, 12, 8, 8, 11, 100),  # the same on the batched path
 ])
 def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
@@ -103,7 +103,7 @@ def test_moe_decode_q8(d, inter, n_experts, B, topk, shared, act):
 
 STAGE_CASES = [
     # d, inter, n_experts, B, topk, shared, act, hidden scale
-    (7168, 2048, 12, 1, 8, 11, 0, 1.0),    # benchmark layer shapes, batch 1 (two-kernel path), hidden ~ N(0, 1)
+    (7168, 2048, 12, 1, 8, 11, 0, 1.0),    # benchmark layer shapes, batch 1 (one-launch path), hidden ~ N(0, 1)
     (7168, 2048, 12, 3, 8, 11, 0, 1.0),    # batch 3
     (7168, 2048, 12, 4, 8, 11, 0, 1.0),    # batch 4: batched path (pairs grouped by expert, matrix cores)
     (7168, 2048, 12, 16, 8, 11, 0, 1.0),   # batch 16
@@ -182,6 +182,71 @@ def test_stages_compose_to_the_layer():
         assert np.array_equal(one.view(np.uint32), two.view(np.uint32)), (d, inter, B)
 
 
+def slab_layout_np(p, s, rows, cols):
+    """The slab-major layout as include/mk_hip.h states it: tile (b, i) = block b of the rows 256 i .. 256 i + 255, 4 x 64 x 16
+    nibble bytes (row 256 i + 64 j + l at j * 1024 + l * 16) then 64 x 4 scale bytes (at 4096 + 4 l + j)."""
+    nb, nt = cols // 32, rows // 256
+    nib = p.reshape(nt, 4, 64, nb, 16).transpose(3, 0, 1, 2, 4).reshape(nb, nt, 4096)
+    sc = s.reshape(nt, 4, 64, nb).transpose(3, 0, 2, 1).reshape(nb, nt, 256)
+    return np.concatenate([nib, sc], axis=2).reshape(-1)
+
+
+@pytest.mark.parametrize("rows,cols", [(256, 32), (1024, 512), (7168, 2048)])
+def test_slab_copy_is_the_same_matrix_bit_for_bit(rows, cols):
+    # W2 in slab-major tiles: the bytes sit where the header says, and dequant(slab) is mxfp4::dequant bit for bit
+    torch_cuda()
+    from microkimi_amd import mxfp4
+    rng = np.random.default_rng(rows + cols)
+    p = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)   # every nibble, -0.0 (nibble 8) included
+    s = rng.integers(0, 256, (rows, cols // 32), dtype=np.uint8)  # every scale byte, the subnormal byte 0 included
+    s[0, 0], s[rows - 1, cols // 32 - 1] = 0, 255
+    slab = mxfp4.to_slab(dev(p), dev(s), rows, cols)
+    assert np.array_equal(slab.cpu().numpy(), slab_layout_np(p, s, rows, cols))
+    got = mxfp4.dequant_slab(slab, rows, cols).cpu().numpy()
+    want = oracle.mxfp4_dequant(p, s, rows, cols)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+TWO_LAUNCH_CASES = [
+    (7168, 2048, 12, 1, 8, 11, 0, 1.0),   # benchmark layer shapes, batch 1
+    (7168, 2048, 12, 3, 8, 11, 0, 1.0),   # batch 3
+    (2048, 1024, 6, 3, 2, -1, 1, 0.05),   # SiTU, no shared expert
+    (4096, 2048, 5, 2, 3, 4, 2, 1.0),     # DeepSeek rule, clamp active
+    (1024, 4096, 4, 3, 2, 3, 0, 0.02),    # two rows of W1/W3 per wave
+]
+
+
+@pytest.mark.parametrize("d,inter,n_experts,B,topk,shared,act,hs", TWO_LAUNCH_CASES)
+def test_two_launch_path_without_the_slab_copy(d, inter, n_experts, B, topk, shared, act, hs):
+    """A table without the slab-major copy of W2 takes the gate/up launch and the down launch (up to 3 tokens): both
+    stages against the oracle to TOL with nothing removed, the stages compose to the layer bit for bit, and the
+    activation rows equal the one-launch path's bit for bit (the same sums in the same order)."""
+    from microkimi_amd import model
+    table, experts = build(n_experts, d, inter, slab=False)
+    _, with_slab = build(n_experts, d, inter, slab=True)
+    assert experts.table.w2t is None and with_slab.table.w2t is not None
+    host = (table_host(table, 0), table_host(table, 1))
+    ids, wts, x = stage_inputs(d, inter, n_experts, B, topk, shared, hs)
+    limit = 10.0 if act == 2 else 0.0
+    a = model.moe_decode_act(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit)
+    want_a = oracle_act_rows(host, ids, wts, x, shared, d, inter, 1, act, limit)
+    got_a = a.cpu().numpy()
+    worst = max(rel_l2(got_a[t, s], want_a[t, s]) for t in range(B) for s in range(got_a.shape[1]))
+    assert worst <= TOL, f"worst activation row rel-L2 {worst:.2e}"
+    a_slab = model.moe_decode_act(with_slab, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
+    assert np.array_equal(a_slab.view(np.uint32), got_a.view(np.uint32))
+    want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=shared, mode=1, act_kind=act, limit=limit, threads=8)
+    got = model.moe_decode_from_act(experts, dev(ids), dev(wts), dev(want_a), shared=shared, mode=1, act_kind=act).cpu().numpy()
+    worst = max(rel_l2(got[t], want[t]) for t in range(B))
+    assert worst <= TOL, f"worst row rel-L2 {worst:.2e}"
+    two = model.moe_decode_from_act(experts, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
+    one = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
+    assert np.array_equal(one.view(np.uint32), two.view(np.uint32))
+    # the one-launch path on the same activation rows: the same block terms, added in another order
+    slab_rows = model.moe_decode_from_act(with_slab, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
+    assert max(rel_l2(slab_rows[t], two[t]) for t in range(B)) <= 2e-6
+
+
 def test_out_of_range_expert_id_adds_nothing():
     # a table that states its size: a routed id outside it contributes nothing (and no pointer is read out of bounds)
     from microkimi_amd import model
@@ -247,7 +312,7 @@ def test_router_softmax_topk():
 def test_full_layer_257_experts_sampled_tokens():
     """Configuration 2 at its full size (256 routed + 1 shared expert at 2048 x 7168, 6 GB of MXFP4 drawn on the
     device, batch 16 routed by the seeded logits): the rows of sampled tokens against the oracle, which gets only the
-    nine experts of that token copied to the host, at batch 16 (batched path) and at batch 1 (two-kernel path).
+    nine experts of that token copied to the host, at batch 16 (batched path) and at batch 1 (one-launch path).
 
     The layer re-quantizes the f32 activation to q8 before W2 (matvec_packed's own step, src/mxfp4.rs:476-479), which
     is a step function of its input: the gate/up sums here differ from the CPU's in their last bits (the order of
@@ -283,7 +348,7 @@ def test_full_layer_257_experts_sampled_tokens():
         local_ids = np.arange(topk, dtype=np.uint32)[None, :]
         want = oracle.moe_decode(table, local_ids, wts_h[tok:tok + 1], hidden[tok:tok + 1], shared=topk, mode=1, threads=8)
         flips += rows_match_up_to_q8_flips(got16[tok:tok + 1], want, lambda t: [w2[e] for e in used], d, inter)
-        # batch 1 takes the two-kernel path, batch 16 the batched one: the same arithmetic per block, another order of the sum
+        # batch 1 takes the one-launch path, batch 16 the batched one: the same arithmetic per block, another order of the sum
         got1 = model.moe_decode(experts, ids[tok:tok + 1].contiguous(), wts[tok:tok + 1].contiguous(), x[tok:tok + 1].contiguous(), shared=ne, mode=1).cpu().numpy()
         flips += rows_match_up_to_q8_flips(got1, want, lambda t: [w2[e] for e in used], d, inter)
     assert flips <= 8
