@@ -196,21 +196,28 @@ typedef struct {
      * device, or NULL when every expert is MXFP4.  A VQ1 expert has its index bytes ([rows][cols/16]) where the packed
      * nibbles would be (w1p, w3p, w2p) and NULL scale pointers (w1s, w3s, w2s). */
     const float *vq_codebook;
-    /* Optional (NULL: not there): per expert, W2 once more in slab-major tiles (mk_dev_mxfp4_to_slab).  With it, up to 4
-     * decode tokens in q8 mode take the one-launch form of the layer (see mk_dev_moe_decode). */
-    const uint8_t *const *w2t;
+    /* Optional (NULL: not there; all three or none): per expert, the three matrices once more in the matrix instruction's
+     * operand order (mk_dev_mxfp4_to_tiles: w1t and w3t with col_major = 0, w2t with col_major = 1).  With them, up to 3 decode tokens in
+     * q8 mode take the one-launch form of the layer (see mk_dev_moe_decode). */
+    const uint8_t *const *w1t, *const *w3t, *const *w2t;
 } mk_expert_table;
 
-/* A second layout of an MXFP4 matrix [rows][cols] for the kernel that multiplies ONE q8 block of the activation into
- * the matching 32 columns of every row (the down projection of the one-launch MoE decode): tile (b, i), at byte
- * (b * rows / 256 + i) * 4352, holds block b (columns 32 b .. 32 b + 31) of the rows 256 i .. 256 i + 255 as
- * 4 x 64 x 16 nibble bytes (row 256 i + 64 j + l at j * 1024 + l * 16, the 16 bytes as in the reference layout,
- * src/mxfp4.rs:1-3) and 64 x 4 scale bytes (row 256 i + 64 j + l at 4096 + 4 l + j).  The same bytes in another order:
- * mk_dev_mxfp4_slab_dequant gives mxfp4::dequant (src/mxfp4.rs:19-31) bit for bit.  rows % 256 == 0, cols % 32 == 0;
- * mk_mxfp4_slab_bytes = rows * cols / 32 * 17, the size of packed + scales.  packed and slab 16-byte aligned. */
-size_t mk_mxfp4_slab_bytes(size_t rows, size_t cols);
-int mk_dev_mxfp4_to_slab(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, uint8_t *slab, void *stream);
-int mk_dev_mxfp4_slab_dequant(const uint8_t *slab, size_t rows, size_t cols, float *out, void *stream);
+/* A second layout of an MXFP4 matrix [rows][cols], in the operand order of v_mfma_scale_f32_16x16x128_f8f6f4: a CHUNK is
+ * what one instruction takes, 64 lanes x 16 bytes, lane l = n + 16 kb holding one 32-block of row n (the 16 bytes as in the
+ * reference layout, src/mxfp4.rs:1-3) and one scale byte a lane.  Two consecutive chunks share a 2176-byte container (17
+ * whole lines): chunk ci at (ci >> 1) * 2176 + (ci & 1) * 1024, lane l at + 16 l, its scale byte at (ci >> 1) * 2176 + 2048 +
+ * 2 l + (ci & 1).
+ *   col_major == 0 (W1, W3 of the one-launch MoE decode): chunk ci = (r / 16) * (cols / 128) + c / 128 holds rows
+ *     16 (r / 16) .. + 15, columns 128 (c / 128) .. + 127; lane = r % 16 + 16 * ((c / 32) % 4).  The chunks of 16 rows are
+ *     contiguous along the columns.  rows % 16 == 0, cols % 256 == 0.
+ *   col_major != 0 (W2): chunk ci = (c / 64) * (rows / 32) + r / 32 holds rows 32 (r / 32) .. + 31, columns 64 (c / 64) .. +
+ *     63; lane = r % 16 + 16 * (2 * ((r / 16) % 2) + (c / 32) % 2).  The chunks of 64 columns are contiguous along the
+ *     rows.  rows % 64 == 0, cols % 64 == 0.
+ * The same bytes in another order: mk_dev_mxfp4_tiles_dequant gives mxfp4::dequant (src/mxfp4.rs:19-31) bit for bit.
+ * mk_mxfp4_tiles_bytes = rows * cols / 32 * 17, the size of packed + scales.  packed and tiles 16-byte aligned. */
+size_t mk_mxfp4_tiles_bytes(size_t rows, size_t cols);
+int mk_dev_mxfp4_to_tiles(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, int col_major, uint8_t *tiles, void *stream);
+int mk_dev_mxfp4_tiles_dequant(const uint8_t *tiles, size_t rows, size_t cols, int col_major, float *out, void *stream);
 
 /* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
 size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
@@ -228,10 +235,11 @@ size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, s
  * each call.  A selected expert that is VQ1 (table->vq_codebook set, NULL scale pointers) takes quant::matvec_vq
  * (src/quant.rs:333-346) for its three products, on the f32 hidden and activation rows, whatever `mode` says
  * (src/model.rs:2243-2257); the workspace then also holds mk_moe_decode_vq_workspace_bytes.
- * Kernels by batch (q8 mode, MXFP4 experts, model-like shapes): 1-3 tokens with table->w2t: one streaming launch in
- * which a workgroup takes 64 rows of W1 and W3 of a pair, forms the two q8 blocks of the activation they give and
- * multiplies them into the matching slabs of W2, then a small kernel that adds the partial rows in a fixed order;
- * without w2t: a gate/up launch and a down launch; from 4 tokens: the pairs grouped by expert on the matrix cores.
+ * Kernels by batch (q8 mode, MXFP4 experts, model-like shapes): 1-3 tokens with the table's tiled copies: one streaming
+ * launch in which a workgroup takes 64 rows of W1 and W3 of a pair, forms the two q8 blocks of the activation they
+ * give and multiplies them into the matching 64 columns of W2, then a small kernel that adds the partial rows in a
+ * fixed order; without the copies: a gate/up launch and a down launch; from 4 tokens: the pairs grouped by expert on
+ * the matrix cores.
  * Every form adds the reference's block terms (src/mxfp4.rs:405-443); only the order of the sum over blocks differs. */
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);

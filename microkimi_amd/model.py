@@ -197,11 +197,11 @@ class MlaHeadsCache:
 class PackedExperts:
     """Expert table of an MoE layer on the device: per expert w1, w3 [inter, d] and w2 [d, inter], each MXFP4
     (packed, scales) in the reference layout, or -- a VQ1 expert (src/model.rs:729-730) -- (index bytes, None) with
-    the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors.  slab: also keep W2 of every expert in
-    slab-major tiles (mk_dev_mxfp4_to_slab; as many bytes again as W2), which lets up to 3 decode tokens take the
-    one-launch form of the layer; None = when the shapes allow it and no expert is VQ1."""
+    the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors.  tiles: also keep every expert's matrices
+    in the matrix instruction's operand order (mk_dev_mxfp4_to_tiles; as many bytes again), which lets up to 3 decode
+    tokens take the one-launch form of the layer; None = when the shapes allow it and no expert is VQ1."""
 
-    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, slab=None):
+    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, tiles=None):
         import torch
         self.d, self.inter, self.n = d, inter, len(w1)
         self._keep = (w1, w3, w2, vq_codebook)
@@ -209,22 +209,25 @@ class PackedExperts:
         arr = lambda lst, k: torch.tensor([t[k].data_ptr() if t[k] is not None else 0 for t in lst], dtype=torch.int64, device=dev)
         self._ptrs = [arr(w1, 0), arr(w1, 1), arr(w3, 0), arr(w3, 1), arr(w2, 0), arr(w2, 1)]
         self.has_vq = vq_codebook is not None
-        if any(t[1] is None for lst in (w1, w3, w2) for t in lst) and not self.has_vq:
-            raise ValueError("a VQ1 expert needs the codebook")
         any_vq = any(t[1] is None for lst in (w1, w3, w2) for t in lst)
-        if slab is None:
-            slab = not any_vq and d % 1024 == 0 and inter % 32 == 0
-        self._slabs, w2t = None, None
-        if slab:
-            if any_vq or d % 256 or inter % 32:
-                raise ValueError("the slab-major copy needs MXFP4 experts, d % 256 == 0 and inter % 32 == 0")
-            each = (lib.mk_mxfp4_slab_bytes(d, inter) + 255) // 256 * 256
-            self._slabs = torch.empty(self.n * each, dtype=torch.uint8, device=dev)
-            for i, t in enumerate(w2):
-                check(lib.mk_dev_mxfp4_to_slab(ptr(t[0]), ptr(t[1]), d, inter, self._slabs.data_ptr() + i * each, cur_stream()))
-            self._w2t = torch.tensor([self._slabs.data_ptr() + i * each for i in range(self.n)], dtype=torch.int64, device=dev)
-            w2t = self._w2t.data_ptr()
-        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None, w2t)
+        if any_vq and not self.has_vq:
+            raise ValueError("a VQ1 expert needs the codebook")
+        if tiles is None:
+            tiles = not any_vq and d % 256 == 0 and inter % 64 == 0
+        self._tiles, tptrs = None, [None, None, None]
+        if tiles:
+            if any_vq or d % 256 or inter % 64:
+                raise ValueError("the tiled copies need MXFP4 experts, d % 256 == 0 and inter % 64 == 0")
+            each = (lib.mk_mxfp4_tiles_bytes(d, inter) + 255) // 256 * 256
+            self._tiles = torch.empty(3 * self.n * each, dtype=torch.uint8, device=dev)
+            base = self._tiles.data_ptr()
+            self._tptrs = []
+            for k, (lst, r, c) in enumerate(((w1, inter, d), (w3, inter, d), (w2, d, inter))):
+                for i, t in enumerate(lst):
+                    check(lib.mk_dev_mxfp4_to_tiles(ptr(t[0]), ptr(t[1]), r, c, int(k == 2), base + (k * self.n + i) * each, cur_stream()))
+                self._tptrs.append(torch.tensor([base + (k * self.n + i) * each for i in range(self.n)], dtype=torch.int64, device=dev))
+            tptrs = [p.data_ptr() for p in self._tptrs]
+        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None, *tptrs)
         self._ws = None
 
 

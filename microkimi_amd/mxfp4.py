@@ -31,23 +31,24 @@ def dequant(packed, scales, rows, cols):
     return out
 
 
-def to_slab(packed, scales, rows, cols):
-    """The slab-major copy of an MXFP4 matrix on the device (mk_dev_mxfp4_to_slab): block b of the rows 256 i .. 256 i + 255
-    as one 4352-byte tile, tiles of a block contiguous.  The layout the one-launch MoE decode reads W2 in."""
+def to_tiles(packed, scales, rows, cols, col_major=False):
+    """The tiled copy of an MXFP4 matrix on the device (mk_dev_mxfp4_to_tiles): the blocks in the operand order of the
+    block-scaled matrix instruction, chunks of 16 rows contiguous along the columns (col_major False) or chunks of 64
+    columns contiguous along the rows (True).  The layouts the one-launch MoE decode reads W1 / W3 and W2 in."""
     import torch
     _lib.require_device()
     _check_shapes(packed, scales, rows, cols)
-    slab = torch.empty(lib.mk_mxfp4_slab_bytes(rows, cols), dtype=torch.uint8, device=packed.device)
-    check(lib.mk_dev_mxfp4_to_slab(ptr(packed), ptr(scales), rows, cols, ptr(slab), cur_stream()))
-    return slab
+    tiles = torch.empty(lib.mk_mxfp4_tiles_bytes(rows, cols), dtype=torch.uint8, device=packed.device)
+    check(lib.mk_dev_mxfp4_to_tiles(ptr(packed), ptr(scales), rows, cols, int(bool(col_major)), ptr(tiles), cur_stream()))
+    return tiles
 
 
-def dequant_slab(slab, rows, cols):
-    """mxfp4::dequant (src/mxfp4.rs:19-31) read from the slab-major copy: f32 [rows, cols], bit-exact."""
+def dequant_tiles(tiles, rows, cols, col_major=False):
+    """mxfp4::dequant (src/mxfp4.rs:19-31) read from the tiled copy: f32 [rows, cols], bit-exact."""
     import torch
     _lib.require_device()
-    out = torch.empty((rows, cols), dtype=torch.float32, device=slab.device)
-    check(lib.mk_dev_mxfp4_slab_dequant(ptr(slab), rows, cols, ptr(out), cur_stream()))
+    out = torch.empty((rows, cols), dtype=torch.float32, device=tiles.device)
+    check(lib.mk_dev_mxfp4_tiles_dequant(ptr(tiles), rows, cols, int(bool(col_major)), ptr(out), cur_stream()))
     return out
 
 

@@ -40,7 +40,7 @@ def rows_match_up_to_q8_flips(got, want, w2_of_token, d, inter, max_flips=2):
     return flips
 
 
-def build(n_experts, d, inter, cfg=2, slab=None):
+def build(n_experts, d, inter, cfg=2, tiles=None):
     from microkimi_amd import model, workloads
     host = [(workloads.mxfp4_matrix(cfg, "w1", inter, d, e), workloads.mxfp4_matrix(cfg, "w3", inter, d, e),
              workloads.mxfp4_matrix(cfg, "w2", d, inter, e)) for e in range(n_experts)]
@@ -49,7 +49,7 @@ def build(n_experts, d, inter, cfg=2, slab=None):
     w2 = [h[2] for h in host]
     table = oracle.ExpertTable(w1, w3, w2, d, inter)
     todev = lambda lst: [(dev(p), dev(s)) for p, s in lst]
-    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter, slab=slab)
+    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter, tiles=tiles)
     return table, experts
 
 
@@ -182,27 +182,39 @@ def test_stages_compose_to_the_layer():
         assert np.array_equal(one.view(np.uint32), two.view(np.uint32)), (d, inter, B)
 
 
-def slab_layout_np(p, s, rows, cols):
-    """The slab-major layout as include/mk_hip.h states it: tile (b, i) = block b of the rows 256 i .. 256 i + 255, 4 x 64 x 16
-    nibble bytes (row 256 i + 64 j + l at j * 1024 + l * 16) then 64 x 4 scale bytes (at 4096 + 4 l + j)."""
-    nb, nt = cols // 32, rows // 256
-    nib = p.reshape(nt, 4, 64, nb, 16).transpose(3, 0, 1, 2, 4).reshape(nb, nt, 4096)
-    sc = s.reshape(nt, 4, 64, nb).transpose(3, 0, 2, 1).reshape(nb, nt, 256)
-    return np.concatenate([nib, sc], axis=2).reshape(-1)
+def tiles_layout_np(p, s, rows, cols, col_major):
+    """The tiled layout as include/mk_hip.h states it, element by element: the 32-block (r, b) of the matrix sits in chunk
+    ci at lane l; the 16 nibble bytes at (ci >> 1) * 2176 + (ci & 1) * 1024 + 16 l, the scale byte at (ci >> 1) * 2176 + 2048 +
+    2 l + (ci & 1)."""
+    nb = cols // 32
+    r, b = np.meshgrid(np.arange(rows), np.arange(nb), indexing="ij")
+    if col_major:
+        ci = (b >> 1) * (rows // 32) + (r >> 5)
+        lane = (r & 15) + 16 * (2 * ((r >> 4) & 1) + (b & 1))
+    else:
+        ci = (r >> 4) * (nb // 4) + (b >> 2)
+        lane = (r & 15) + 16 * (b & 3)
+    base = (ci >> 1) * 2176
+    out = np.zeros(rows * nb * 17, np.uint8)
+    nib_at = (base + (ci & 1) * 1024 + 16 * lane)[..., None] + np.arange(16)
+    out[nib_at.reshape(-1)] = p.reshape(rows, nb, 16).reshape(-1)
+    out[(base + 2048 + 2 * lane + (ci & 1)).reshape(-1)] = s.reshape(-1)
+    return out
 
 
-@pytest.mark.parametrize("rows,cols", [(256, 32), (1024, 512), (7168, 2048)])
-def test_slab_copy_is_the_same_matrix_bit_for_bit(rows, cols):
-    # W2 in slab-major tiles: the bytes sit where the header says, and dequant(slab) is mxfp4::dequant bit for bit
+@pytest.mark.parametrize("rows,cols,col_major", [(16, 256, 0), (64, 64, 1), (1024, 512, 1), (7168, 2048, 1), (2048, 7168, 0), (512, 1024, 0)])
+def test_tiled_copy_is_the_same_matrix_bit_for_bit(rows, cols, col_major):
+    # the experts in the matrix instruction's operand order: the bytes sit where the header says, and dequant(tiles) is
+    # mxfp4::dequant bit for bit
     torch_cuda()
     from microkimi_amd import mxfp4
     rng = np.random.default_rng(rows + cols)
     p = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)   # every nibble, -0.0 (nibble 8) included
     s = rng.integers(0, 256, (rows, cols // 32), dtype=np.uint8)  # every scale byte, the subnormal byte 0 included
     s[0, 0], s[rows - 1, cols // 32 - 1] = 0, 255
-    slab = mxfp4.to_slab(dev(p), dev(s), rows, cols)
-    assert np.array_equal(slab.cpu().numpy(), slab_layout_np(p, s, rows, cols))
-    got = mxfp4.dequant_slab(slab, rows, cols).cpu().numpy()
+    tiles = mxfp4.to_tiles(dev(p), dev(s), rows, cols, col_major)
+    assert np.array_equal(tiles.cpu().numpy(), tiles_layout_np(p, s, rows, cols, col_major))
+    got = mxfp4.dequant_tiles(tiles, rows, cols, col_major).cpu().numpy()
     want = oracle.mxfp4_dequant(p, s, rows, cols)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
@@ -217,14 +229,14 @@ TWO_LAUNCH_CASES = [
 
 
 @pytest.mark.parametrize("d,inter,n_experts,B,topk,shared,act,hs", TWO_LAUNCH_CASES)
-def test_two_launch_path_without_the_slab_copy(d, inter, n_experts, B, topk, shared, act, hs):
-    """A table without the slab-major copy of W2 takes the gate/up launch and the down launch (up to 3 tokens): both
-    stages against the oracle to TOL with nothing removed, the stages compose to the layer bit for bit, and the
-    activation rows equal the one-launch path's bit for bit (the same sums in the same order)."""
+def test_two_launch_path_without_the_tiled_copies(d, inter, n_experts, B, topk, shared, act, hs):
+    """A table without the tiled copies takes the gate/up launch and the down launch (up to 3 tokens): both stages
+    against the oracle to TOL with nothing removed, the stages compose to the layer bit for bit, and the one-launch
+    path fed the same activation rows adds the same block terms in another order."""
     from microkimi_amd import model
-    table, experts = build(n_experts, d, inter, slab=False)
-    _, with_slab = build(n_experts, d, inter, slab=True)
-    assert experts.table.w2t is None and with_slab.table.w2t is not None
+    table, experts = build(n_experts, d, inter, tiles=False)
+    _, with_tiles = build(n_experts, d, inter, tiles=True)
+    assert experts.table.w2t is None and with_tiles.table.w2t is not None
     host = (table_host(table, 0), table_host(table, 1))
     ids, wts, x = stage_inputs(d, inter, n_experts, B, topk, shared, hs)
     limit = 10.0 if act == 2 else 0.0
@@ -233,8 +245,8 @@ def test_two_launch_path_without_the_slab_copy(d, inter, n_experts, B, topk, sha
     got_a = a.cpu().numpy()
     worst = max(rel_l2(got_a[t, s], want_a[t, s]) for t in range(B) for s in range(got_a.shape[1]))
     assert worst <= TOL, f"worst activation row rel-L2 {worst:.2e}"
-    a_slab = model.moe_decode_act(with_slab, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
-    assert np.array_equal(a_slab.view(np.uint32), got_a.view(np.uint32))
+    a_tiles = model.moe_decode_act(with_tiles, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
+    assert max(rel_l2(a_tiles[t, s], got_a[t, s]) for t in range(B) for s in range(got_a.shape[1])) <= 2e-6
     want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=shared, mode=1, act_kind=act, limit=limit, threads=8)
     got = model.moe_decode_from_act(experts, dev(ids), dev(wts), dev(want_a), shared=shared, mode=1, act_kind=act).cpu().numpy()
     worst = max(rel_l2(got[t], want[t]) for t in range(B))
@@ -243,8 +255,8 @@ def test_two_launch_path_without_the_slab_copy(d, inter, n_experts, B, topk, sha
     one = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
     assert np.array_equal(one.view(np.uint32), two.view(np.uint32))
     # the one-launch path on the same activation rows: the same block terms, added in another order
-    slab_rows = model.moe_decode_from_act(with_slab, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
-    assert max(rel_l2(slab_rows[t], two[t]) for t in range(B)) <= 2e-6
+    tile_rows = model.moe_decode_from_act(with_tiles, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
+    assert max(rel_l2(tile_rows[t], two[t]) for t in range(B)) <= 2e-6
 
 
 def test_out_of_range_expert_id_adds_nothing():
