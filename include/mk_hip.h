@@ -196,28 +196,34 @@ typedef struct {
      * device, or NULL when every expert is MXFP4.  A VQ1 expert has its index bytes ([rows][cols/16]) where the packed
      * nibbles would be (w1p, w3p, w2p) and NULL scale pointers (w1s, w3s, w2s). */
     const float *vq_codebook;
-    /* Optional (NULL: not there; all three or none): per expert, the three matrices once more in the matrix instruction's
-     * operand order (mk_dev_mxfp4_to_tiles: w1t and w3t with col_major = 0, w2t with col_major = 1).  With them, up to 3 decode tokens in
-     * q8 mode take the one-launch form of the layer (see mk_dev_moe_decode). */
-    const uint8_t *const *w1t, *const *w3t, *const *w2t;
+    /* Optional (NULL: not there; both or none): per expert, the matrices once more in the order the one-launch decode
+     * kernel streams them (mk_dev_moe_pack_gate_up -> w13t, mk_dev_moe_pack_down -> w2t).  With them, up to 3 decode tokens in
+     * q8 mode at d = 7168 or 5120, inter = 2048 on a 256-CU device take the one-launch form of the layer (see
+     * mk_dev_moe_decode); such calls must not overlap on one device. */
+    const uint8_t *const *w13t, *const *w2t;
 } mk_expert_table;
 
-/* A second layout of an MXFP4 matrix [rows][cols], in the operand order of v_mfma_scale_f32_16x16x128_f8f6f4: a CHUNK is
- * what one instruction takes, 64 lanes x 16 bytes, lane l = n + 16 kb holding one 32-block of row n (the 16 bytes as in the
- * reference layout, src/mxfp4.rs:1-3) and one scale byte a lane.  Two consecutive chunks share a 2176-byte container (17
- * whole lines): chunk ci at (ci >> 1) * 2176 + (ci & 1) * 1024, lane l at + 16 l, its scale byte at (ci >> 1) * 2176 + 2048 +
- * 2 l + (ci & 1).
- *   col_major == 0 (W1, W3 of the one-launch MoE decode): chunk ci = (r / 16) * (cols / 128) + c / 128 holds rows
- *     16 (r / 16) .. + 15, columns 128 (c / 128) .. + 127; lane = r % 16 + 16 * ((c / 32) % 4).  The chunks of 16 rows are
- *     contiguous along the columns.  rows % 16 == 0, cols % 256 == 0.
- *   col_major != 0 (W2): chunk ci = (c / 64) * (rows / 32) + r / 32 holds rows 32 (r / 32) .. + 31, columns 64 (c / 64) .. +
- *     63; lane = r % 16 + 16 * (2 * ((r / 16) % 2) + (c / 32) % 2).  The chunks of 64 columns are contiguous along the
- *     rows.  rows % 64 == 0, cols % 64 == 0.
- * The same bytes in another order: mk_dev_mxfp4_tiles_dequant gives mxfp4::dequant (src/mxfp4.rs:19-31) bit for bit.
- * mk_mxfp4_tiles_bytes = rows * cols / 32 * 17, the size of packed + scales.  packed and tiles 16-byte aligned. */
-size_t mk_mxfp4_tiles_bytes(size_t rows, size_t cols);
-int mk_dev_mxfp4_to_tiles(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, int col_major, uint8_t *tiles, void *stream);
-int mk_dev_mxfp4_tiles_dequant(const uint8_t *tiles, size_t rows, size_t cols, int col_major, float *out, void *stream);
+/* The experts of a layer in the operand order of v_mfma_scale_f32_16x16x128_f8f6f4, for the one-launch decode kernel: the
+ * same bytes as (packed, scales) in another order -- mk_dev_moe_unpack_* restores the reference layout byte for byte
+ * (src/mxfp4.rs:1-3), so mxfp4::dequant of the restored matrices is the reference's bit for bit.
+ *   gate/up pack (W1 and W3 [inter][d] together): chunk (t, s) = rows 8 t .. 8 t + 7 of W1 and of W3, columns 128 s .. + 127, 64 lanes
+ *     x 16 bytes: the 32-block b of row r of matrix m (0: W1, 1: W3) sits at lane (r % 8 + 8 m) + 16 (b % 4) of chunk
+ *     ci = (r / 8) * (d / 128) + b / 4.  Two chunks share a 2176-byte container: chunk ci at (ci >> 1) * 2176 + (ci & 1) * 1024,
+ *     lane l at + 16 l, its scale byte at (ci >> 1) * 2176 + 2048 + 2 l + (ci & 1).  d % 256 == 0, inter % 8 == 0;
+ *     2 * inter * d / 32 * 17 bytes.
+ *   down pack (W2 [d][inter]): the rows in 256 groups of rw = d / 256 (17 .. 32); one K step of a group (128 columns) is
+ *     STEP = (1024 + 64 rb + 64 + 4 rb) rounded up to 128 bytes, rb = rw - 16, at (group * (inter / 128) + b / 4) * STEP: row
+ *     i < 16 of the group has its block at 16 (i + 16 (b % 4)) and its scale byte at 1024 + 64 rb + i + 16 (b % 4); row
+ *     i >= 16 at 1024 + 16 ((b % 4) rb + i - 16) and 1024 + 64 rb + 64 + (b % 4) rb + i - 16; the padding is zero.
+ *     256 * (inter / 128) * STEP bytes.
+ * mk_moe_pack_bytes(d, inter, down): the size of the gate/up pack (down == 0) or of the down pack (0: d not covered). */
+size_t mk_moe_pack_bytes(size_t d, size_t inter, int down);
+int mk_dev_moe_pack_gate_up(const uint8_t *w1p, const uint8_t *w1s, const uint8_t *w3p, const uint8_t *w3s, size_t d, size_t inter,
+                            uint8_t *pack, void *stream);
+int mk_dev_moe_unpack_gate_up(const uint8_t *pack, size_t d, size_t inter, uint8_t *w1p, uint8_t *w1s, uint8_t *w3p, uint8_t *w3s,
+                              void *stream);
+int mk_dev_moe_pack_down(const uint8_t *w2p, const uint8_t *w2s, size_t d, size_t inter, uint8_t *pack, void *stream);
+int mk_dev_moe_unpack_down(const uint8_t *pack, size_t d, size_t inter, uint8_t *w2p, uint8_t *w2s, void *stream);
 
 /* Bytes of device scratch mk_dev_moe_decode needs for B tokens of topk(+shared) experts. */
 size_t mk_moe_decode_workspace_bytes(size_t B, size_t topk, int has_shared, size_t d, size_t inter);
@@ -235,14 +241,18 @@ size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, s
  * each call.  A selected expert that is VQ1 (table->vq_codebook set, NULL scale pointers) takes quant::matvec_vq
  * (src/quant.rs:333-346) for its three products, on the f32 hidden and activation rows, whatever `mode` says
  * (src/model.rs:2243-2257); the workspace then also holds mk_moe_decode_vq_workspace_bytes.
- * Kernels by batch (q8 mode, MXFP4 experts, model-like shapes): 1-3 tokens with the table's tiled copies: one streaming
- * launch in which a workgroup takes 64 rows of W1 and W3 of a pair, forms the two q8 blocks of the activation they
- * give and multiplies them into the matching 64 columns of W2, then a small kernel that adds the partial rows in a
- * fixed order; without the copies: a gate/up launch and a down launch; from 4 tokens: the pairs grouped by expert on
- * the matrix cores.
+ * Kernels by batch (q8 mode, MXFP4 experts, model-like shapes): 1-3 tokens with the table's packed copies (w13t, w2t):
+ * ONE launch of one resident workgroup per CU -- every workgroup takes 8 rows of W1 and W3 of every pair, publishes their
+ * activation values through the workspace (8-byte units that carry the launch's tag), then takes d / 256 rows of W2 of
+ * every pair; every wait is bounded, a workgroup that gives up writes NaN to its rows and raises the flag that
+ * mk_dev_moe_decode_gave_up reads.  Without the copies: a gate/up launch and a down launch.  From 4 tokens: the pairs
+ * grouped by expert on the matrix cores.
  * Every form adds the reference's block terms (src/mxfp4.rs:405-443); only the order of the sum over blocks differs. */
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
+/* *flag = 1 if a workgroup of the one-launch form ever gave up waiting on this device (its rows are NaN), else 0.
+ * Synchronous (a device-to-host copy).  Has no counterpart in the reference. */
+int mk_dev_moe_decode_gave_up(int *flag);
 
 /* The two halves of mk_dev_moe_decode on their own, for callers that keep the reference's call structure (two
  * matvec_packed calls, the activation, then the third matvec_packed: src/model.rs:2246-2259, src/deepseek.rs:1080-1089)

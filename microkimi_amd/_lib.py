@@ -27,7 +27,7 @@ class BinEntry(C.Structure):
 class ExpertTable(C.Structure):
     _fields_ = [("w1p", C.c_void_p), ("w1s", C.c_void_p), ("w3p", C.c_void_p), ("w3s", C.c_void_p), ("w2p", C.c_void_p),
                 ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t), ("n_experts", C.c_size_t), ("vq_codebook", C.c_void_p),
-                ("w1t", C.c_void_p), ("w3t", C.c_void_p), ("w2t", C.c_void_p)]
+                ("w13t", C.c_void_p), ("w2t", C.c_void_p)]
 
 
 class Prof(C.Structure):
@@ -75,9 +75,12 @@ def _load():
         "mk_dev_q8_matvec": (i32, [vp, vp, i32, sz, sz, vp, vp, sz, vp, vp]),
         "mk_dev_argmax": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_q8head_from_f32": (i32, [vp, sz, sz, vp, vp, i32, vp]),
-        "mk_mxfp4_tiles_bytes": (sz, [sz, sz]),
-        "mk_dev_mxfp4_to_tiles": (i32, [vp, vp, sz, sz, i32, vp, vp]),
-        "mk_dev_mxfp4_tiles_dequant": (i32, [vp, sz, sz, i32, vp, vp]),
+        "mk_moe_pack_bytes": (sz, [sz, sz, i32]),
+        "mk_dev_moe_pack_gate_up": (i32, [vp, vp, vp, vp, sz, sz, vp, vp]),
+        "mk_dev_moe_unpack_gate_up": (i32, [vp, sz, sz, vp, vp, vp, vp, vp]),
+        "mk_dev_moe_pack_down": (i32, [vp, vp, sz, sz, vp, vp]),
+        "mk_dev_moe_unpack_down": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_moe_decode_gave_up": (i32, [C.POINTER(C.c_int)]),
         "mk_moe_decode_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_moe_decode_vq_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_dev_moe_decode": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),

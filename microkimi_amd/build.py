@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmk_hip.so")
-SOURCES = ["host.hip", "codec.hip", "gemv_mxfp4.hip", "gemv_q8.hip", "moe.hip", "moe_tiles.hip", "mla.hip", "mla_heads.hip", "gemm_mxfp4.hip", "gemm_q8x.hip", "prefill.hip", "front.hip", "weights.hip", "vq1.hip", "quantize.hip"]
+SOURCES = ["host.hip", "codec.hip", "gemv_mxfp4.hip", "gemv_q8.hip", "moe.hip", "moe_persist.hip", "mla.hip", "mla_heads.hip", "gemm_mxfp4.hip", "gemm_q8x.hip", "prefill.hip", "front.hip", "weights.hip", "vq1.hip", "quantize.hip"]
 
 
 def hipcc():

@@ -38,12 +38,12 @@ struct FusedArgs {
 
 enum { MK_MOE_STAGE_ALL = 0, MK_MOE_STAGE_ACT = 1, MK_MOE_STAGE_FROM_ACT = 2 };
 
-// moe_tiles.hip: the one-launch expert section over a table that carries the tiled copies (tab.w1t, w3t, w2t).
-//   stage ALL       x -> out                      (a.af unused)
+// moe_persist.hip: the one-launch expert section (one resident workgroup per CU) over a table that carries the packed
+// copies (tab.w13t, tab.w2t).
+//   stage ALL       x -> out                      (a.af unused; the activation values go through `lines`)
 //   stage ACT       x -> a.af, nothing else
 //   stage FROM_ACT  a.af -> out
-// part: [P][inter / 64][d] f32 partial rows.  Returns MK_ERR_UNSUPPORTED (nothing launched) for a shape the kernel does
-// not take.
-bool mk_moe_tiles_takes(size_t d, size_t inter, int per);
-size_t mk_moe_tiles_part_bytes(size_t P, size_t d, size_t inter);
-int mk_moe_tiles_launch(const FusedArgs &a, size_t B, int stage, float *part, hipStream_t st);
+// lines: [P][inter] 8-byte units of the caller's workspace.
+bool mk_moe_persist_takes(size_t B, size_t d, size_t inter, int per);
+size_t mk_moe_persist_lines_bytes(size_t P, size_t inter);
+int mk_moe_persist_launch(const FusedArgs &a, size_t B, int stage, void *lines, hipStream_t st);

@@ -65,13 +65,12 @@ struct Workspace {
     int32_t *goff;     // [P + 1] first grouped row of every group
     int32_t *gexp;     // [P] expert of every group
     int32_t *ngroups;  // [2]: number of groups, index of the largest group
-    float *part;       // one-launch path (up to TILES_MAX_B tokens): [P][inter / 64][d] partial rows
+    void *lines;       // one-launch path: [P][inter] 8-byte units (activation value, launch tag)
     size_t bytes;
 };
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-constexpr int TILES_MAX_B = 4;  // tokens the one-launch path (moe_tiles.hip) takes: its partial rows are 0.9 MB a pair at the model shape
 
 Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, size_t inter) {
     const size_t P = B * (topk + (has_shared ? 1 : 0));
@@ -109,7 +108,7 @@ Workspace carve(void *base, size_t B, size_t topk, int has_shared, size_t d, siz
     w.goff = (int32_t *)take((P + 1) * 4);
     w.gexp = (int32_t *)take(P * 4);
     w.ngroups = (int32_t *)take(8);
-    w.part = (float *)take(B <= (size_t)TILES_MAX_B && mk_moe_tiles_takes(d, inter, (int)(P / B)) ? mk_moe_tiles_part_bytes(P, d, inter) : 0);
+    w.lines = (void *)take(B <= 3 ? mk_moe_persist_lines_bytes(P, inter) : 0);
     w.bytes = off;
     return w;
 }
@@ -836,10 +835,10 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         return mk_launch_status("moe_combine_grouped");
     }
     float *af = stage == STAGE_ALL ? w.af : act_io;  // [P][inter] activation rows in (token, slot) order
-    // one streaming launch + a small reduction when the table carries the tiled copies of its matrices
-    const bool tiled = !has_vq && mode == MK_MODE_Q8 && table->w1t && table->w3t && table->w2t && B <= (size_t)TILES_MAX_B &&
-                      mk_moe_tiles_takes(d, inter, per) && ((uintptr_t)x & 15) == 0 && !MK_TUNE("MK_MOE_NO_TILES", 0);
-    if ((fast || tiled) && !has_vq) {
+    // one launch of one resident workgroup per CU when the table carries the packed copies of its matrices
+    const bool persist = !has_vq && mode == MK_MODE_Q8 && table->w13t && table->w2t && mk_moe_persist_takes(B, d, inter, per) &&
+                         ((uintptr_t)x & 15) == 0 && !MK_TUNE("MK_MOE_NO_PERSIST", 0);
+    if ((fast || persist) && !has_vq) {
         FusedArgs fa;
         fa.tab = *table;
         fa.ids = ids;
@@ -855,7 +854,7 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
         fa.limit = limit;
         fa.af = af;
         fa.out = out;
-        if (tiled) return mk_moe_tiles_launch(fa, B, stage, w.part, st);
+        if (persist) return mk_moe_persist_launch(fa, B, stage, w.lines, st);
         if (stage != STAGE_FROM_ACT) {
             switch (nb) {
                 case 32: s = launch_gate_up_rows<32>(fa, B, st); break;

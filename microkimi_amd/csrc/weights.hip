@@ -275,12 +275,13 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
         cb_off = off;
         off = align_up(off + (size_t)en.size, 256);
     }
-    // every expert's matrices once more in the matrix instruction's operand order (mk_dev_mxfp4_to_tiles) for the one-launch decode layer, when the
-    // layer's shapes allow it and MK_EXPERT_TILES is not 0: as many bytes again as the experts themselves
-    const bool with_tiles = !any_vq && d % 256 == 0 && inter % 64 == 0 && mk_env_int("MK_EXPERT_TILES", 1) != 0;
-    const size_t tiles_each = with_tiles ? align_up(mk_mxfp4_tiles_bytes(d, inter), 256) : 0, tiles_off = off;
-    off += 3 * tiles_each * n_experts;
-    const size_t tab_off = off, total = off + 9 * n_experts * sizeof(void *);
+    // every expert's matrices once more in the one-launch decode kernel's order (mk_dev_moe_pack_gate_up / _down), when the
+    // layer's shapes are the ones that kernel takes and MK_EXPERT_PACK is not 0: as many bytes again as the experts themselves
+    const size_t pk13 = align_up(mk_moe_pack_bytes(d, inter, 0), 256), pk2 = align_up(mk_moe_pack_bytes(d, inter, 1), 256);
+    const bool with_pack = !any_vq && (d == 7168 || d == 5120) && inter == 2048 && pk2 > 0 && mk_env_int("MK_EXPERT_PACK", 1) != 0;
+    const size_t pack_off = off;
+    if (with_pack) off += (pk13 + pk2) * n_experts;
+    const size_t tab_off = off, total = off + 8 * n_experts * sizeof(void *);
     mk_expert_set *s = new mk_expert_set;
     if (hipMalloc(&s->dev, total) != hipSuccess) {
         (void)hipGetLastError();
@@ -292,7 +293,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->n = n_experts;
     uint8_t *base = (uint8_t *)s->dev;
     // pass 2: one copy per blob straight out of the mapping, then the pointer arrays
-    std::vector<const uint8_t *> ptrs(9 * n_experts, nullptr);
+    std::vector<const uint8_t *> ptrs(8 * n_experts, nullptr);
     for (size_t e = 0; e < n_experts; e++) {
         for (int k = 0; k < 3; k++) {
             const Blob &b = blobs[e * 3 + k];
@@ -306,22 +307,20 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
             ptrs[(size_t)(2 * k + 1) * n_experts + e] = vq[e] ? nullptr : base + b.dev_off + b.half;  // scales (none: VQ1)
         }
     }
-    for (size_t e = 0; with_tiles && e < n_experts; e++) {
-        for (int k = 0; k < 3; k++) {  // w1, w3 (chunks of 16 rows contiguous), w2 (chunks of 64 columns contiguous)
-            uint8_t *t = base + tiles_off + (e * 3 + k) * tiles_each;
-            const size_t r = k == 2 ? d : inter, c = k == 2 ? inter : d;
-            if (mk_dev_mxfp4_to_tiles(ptrs[(size_t)(2 * k) * n_experts + e], ptrs[(size_t)(2 * k + 1) * n_experts + e], r, c, k == 2 ? 1 : 0, t,
-                                      nullptr) != MK_OK) {
-                mk_expert_set_free(s);
-                return MK_ERR_HIP;
-            }
-            ptrs[(size_t)(6 + k) * n_experts + e] = t;
+    for (size_t e = 0; with_pack && e < n_experts; e++) {
+        uint8_t *t13 = base + pack_off + e * (pk13 + pk2), *t2 = t13 + pk13;
+        if (mk_dev_moe_pack_gate_up(ptrs[e], ptrs[n_experts + e], ptrs[2 * n_experts + e], ptrs[3 * n_experts + e], d, inter, t13, nullptr) != MK_OK ||
+            mk_dev_moe_pack_down(ptrs[4 * n_experts + e], ptrs[5 * n_experts + e], d, inter, t2, nullptr) != MK_OK) {
+            mk_expert_set_free(s);
+            return MK_ERR_HIP;
         }
+        ptrs[6 * n_experts + e] = t13;
+        ptrs[7 * n_experts + e] = t2;
     }
-    if (with_tiles && hipDeviceSynchronize() != hipSuccess) {
+    if (with_pack && hipDeviceSynchronize() != hipSuccess) {
         (void)hipGetLastError();
         mk_expert_set_free(s);
-        mk_set_error("the tiled copies of the experts failed");
+        mk_set_error("the packed copies of the experts failed");
         return MK_ERR_HIP;
     }
     if (cb_host && hipMemcpy(base + cb_off, cb_host, 256 * 16 * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
@@ -347,9 +346,8 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->table.inter = inter;
     s->table.n_experts = n_experts;
     s->table.vq_codebook = any_vq ? reinterpret_cast<const float *>(base + cb_off) : nullptr;
-    s->table.w1t = with_tiles ? tab + 6 * n_experts : nullptr;
-    s->table.w3t = with_tiles ? tab + 7 * n_experts : nullptr;
-    s->table.w2t = with_tiles ? tab + 8 * n_experts : nullptr;
+    s->table.w13t = with_pack ? tab + 6 * n_experts : nullptr;
+    s->table.w2t = with_pack ? tab + 7 * n_experts : nullptr;
     *out = s;
     return MK_OK;
 }

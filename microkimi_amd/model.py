@@ -197,11 +197,12 @@ class MlaHeadsCache:
 class PackedExperts:
     """Expert table of an MoE layer on the device: per expert w1, w3 [inter, d] and w2 [d, inter], each MXFP4
     (packed, scales) in the reference layout, or -- a VQ1 expert (src/model.rs:729-730) -- (index bytes, None) with
-    the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors.  tiles: also keep every expert's matrices
-    in the matrix instruction's operand order (mk_dev_mxfp4_to_tiles; as many bytes again), which lets up to 3 decode
-    tokens take the one-launch form of the layer; None = when the shapes allow it and no expert is VQ1."""
+    the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors.  pack: also keep every expert's matrices
+    in the order the one-launch decode kernel streams them (mk_dev_moe_pack_gate_up / _down; as many bytes again), which
+    lets up to 3 decode tokens take that kernel (calls on it must not overlap on one device); None = when the shapes are
+    the ones it takes (d 7168 or 5120, inter 2048) and no expert is VQ1."""
 
-    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, tiles=None):
+    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, pack=None):
         import torch
         self.d, self.inter, self.n = d, inter, len(w1)
         self._keep = (w1, w3, w2, vq_codebook)
@@ -212,20 +213,22 @@ class PackedExperts:
         any_vq = any(t[1] is None for lst in (w1, w3, w2) for t in lst)
         if any_vq and not self.has_vq:
             raise ValueError("a VQ1 expert needs the codebook")
-        if tiles is None:
-            tiles = not any_vq and d % 256 == 0 and inter % 64 == 0
-        self._tiles, tptrs = None, [None, None, None]
-        if tiles:
-            if any_vq or d % 256 or inter % 64:
-                raise ValueError("the tiled copies need MXFP4 experts, d % 256 == 0 and inter % 64 == 0")
-            each = (lib.mk_mxfp4_tiles_bytes(d, inter) + 255) // 256 * 256
-            self._tiles = torch.empty(3 * self.n * each, dtype=torch.uint8, device=dev)
-            base = self._tiles.data_ptr()
-            self._tptrs = []
-            for k, (lst, r, c) in enumerate(((w1, inter, d), (w3, inter, d), (w2, d, inter))):
-                for i, t in enumerate(lst):
-                    check(lib.mk_dev_mxfp4_to_tiles(ptr(t[0]), ptr(t[1]), r, c, int(k == 2), base + (k * self.n + i) * each, cur_stream()))
-                self._tptrs.append(torch.tensor([base + (k * self.n + i) * each for i in range(self.n)], dtype=torch.int64, device=dev))
+        fits = not any_vq and d in (7168, 5120) and inter == 2048
+        if pack is None:
+            pack = fits
+        self._pack, tptrs = None, [None, None]
+        if pack:
+            if not fits:
+                raise ValueError("the packed copies need MXFP4 experts at d = 7168 or 5120 and inter = 2048")
+            b13 = (lib.mk_moe_pack_bytes(d, inter, 0) + 255) // 256 * 256
+            b2 = (lib.mk_moe_pack_bytes(d, inter, 1) + 255) // 256 * 256
+            self._pack = torch.empty(self.n * (b13 + b2), dtype=torch.uint8, device=dev)
+            base = self._pack.data_ptr()
+            for i in range(self.n):
+                at = base + i * (b13 + b2)
+                check(lib.mk_dev_moe_pack_gate_up(ptr(w1[i][0]), ptr(w1[i][1]), ptr(w3[i][0]), ptr(w3[i][1]), d, inter, at, cur_stream()))
+                check(lib.mk_dev_moe_pack_down(ptr(w2[i][0]), ptr(w2[i][1]), d, inter, at + b13, cur_stream()))
+            self._tptrs = [torch.tensor([base + i * (b13 + b2) + k * b13 for i in range(self.n)], dtype=torch.int64, device=dev) for k in (0, 1)]
             tptrs = [p.data_ptr() for p in self._tptrs]
         self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None, *tptrs)
         self._ws = None

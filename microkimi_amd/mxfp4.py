@@ -31,27 +31,6 @@ def dequant(packed, scales, rows, cols):
     return out
 
 
-def to_tiles(packed, scales, rows, cols, col_major=False):
-    """The tiled copy of an MXFP4 matrix on the device (mk_dev_mxfp4_to_tiles): the blocks in the operand order of the
-    block-scaled matrix instruction, chunks of 16 rows contiguous along the columns (col_major False) or chunks of 64
-    columns contiguous along the rows (True).  The layouts the one-launch MoE decode reads W1 / W3 and W2 in."""
-    import torch
-    _lib.require_device()
-    _check_shapes(packed, scales, rows, cols)
-    tiles = torch.empty(lib.mk_mxfp4_tiles_bytes(rows, cols), dtype=torch.uint8, device=packed.device)
-    check(lib.mk_dev_mxfp4_to_tiles(ptr(packed), ptr(scales), rows, cols, int(bool(col_major)), ptr(tiles), cur_stream()))
-    return tiles
-
-
-def dequant_tiles(tiles, rows, cols, col_major=False):
-    """mxfp4::dequant (src/mxfp4.rs:19-31) read from the tiled copy: f32 [rows, cols], bit-exact."""
-    import torch
-    _lib.require_device()
-    out = torch.empty((rows, cols), dtype=torch.float32, device=tiles.device)
-    check(lib.mk_dev_mxfp4_tiles_dequant(ptr(tiles), rows, cols, int(bool(col_major)), ptr(out), cur_stream()))
-    return out
-
-
 def quantize(w, search=True):
     """mxfp4::quantize (search) / quantize_naive (src/mxfp4.rs:38-138) of a device tensor [rows, cols] f32: the
     reference's (packed [rows, cols/2], scales [rows, cols/32]) bytes."""

@@ -47,9 +47,9 @@ pub struct MkExpertTable {
     pub n_experts: usize,
     /// the file's 256 x 16 f32 VQ codebook on the device, or null when every expert is MXFP4
     pub vq_codebook: *const f32,
-    /// optional (all three or none): per expert, the matrices once more as 64 x 64 tiles (mk_dev_mxfp4_to_tiles)
-    pub w1t: *const *const u8,
-    pub w3t: *const *const u8,
+    /// optional (both or none): per expert, the matrices once more in the one-launch decode kernel's order
+    /// (mk_dev_moe_pack_gate_up, mk_dev_moe_pack_down)
+    pub w13t: *const *const u8,
     pub w2t: *const *const u8,
 }
 
@@ -119,9 +119,12 @@ extern "C" {
     pub fn mk_force_q8(v: c_int);
     pub fn mk_q8_enabled() -> c_int;
     pub fn mk_dev_mxfp4_dequant(packed: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
-    pub fn mk_mxfp4_tiles_bytes(rows: usize, cols: usize) -> usize;
-    pub fn mk_dev_mxfp4_to_tiles(packed: *const u8, scales: *const u8, rows: usize, cols: usize, col_major: c_int, tiles: *mut u8, stream: *mut c_void) -> c_int;
-    pub fn mk_dev_mxfp4_tiles_dequant(tiles: *const u8, rows: usize, cols: usize, col_major: c_int, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_moe_pack_bytes(d: usize, inter: usize, down: c_int) -> usize;
+    pub fn mk_dev_moe_pack_gate_up(w1p: *const u8, w1s: *const u8, w3p: *const u8, w3s: *const u8, d: usize, inter: usize, pack: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_moe_unpack_gate_up(pack: *const u8, d: usize, inter: usize, w1p: *mut u8, w1s: *mut u8, w3p: *mut u8, w3s: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_moe_pack_down(w2p: *const u8, w2s: *const u8, d: usize, inter: usize, pack: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_moe_unpack_down(pack: *const u8, d: usize, inter: usize, w2p: *mut u8, w2s: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_moe_decode_gave_up(flag: *mut c_int) -> c_int;
     pub fn mk_dev_fp8_dequant(w: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_q8(x: *const f32, nvec: usize, n: usize, q: *mut i8, scales: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_quantize(w: *const f32, rows: usize, cols: usize, search: c_int, packed: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;

@@ -40,7 +40,7 @@ def rows_match_up_to_q8_flips(got, want, w2_of_token, d, inter, max_flips=2):
     return flips
 
 
-def build(n_experts, d, inter, cfg=2, tiles=None):
+def build(n_experts, d, inter, cfg=2, pack=None):
     from microkimi_amd import model, workloads
     host = [(workloads.mxfp4_matrix(cfg, "w1", inter, d, e), workloads.mxfp4_matrix(cfg, "w3", inter, d, e),
              workloads.mxfp4_matrix(cfg, "w2", d, inter, e)) for e in range(n_experts)]
@@ -49,7 +49,7 @@ def build(n_experts, d, inter, cfg=2, tiles=None):
     w2 = [h[2] for h in host]
     table = oracle.ExpertTable(w1, w3, w2, d, inter)
     todev = lambda lst: [(dev(p), dev(s)) for p, s in lst]
-    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter, tiles=tiles)
+    experts = model.PackedExperts(todev(w1), todev(w3), todev(w2), d, inter, pack=pack)
     return table, experts
 
 
@@ -111,6 +111,8 @@ STAGE_CASES = [
     (4096, 2048, 5, 11, 3, 4, 2, 0.05),    # DeepSeek rule on the batched path (weight inside the activation)
     (4096, 2048, 5, 2, 3, 4, 2, 1.0),      # DeepSeek rule, clamp active at hidden ~ N(0, 1)
     (96, 64, 4, 2, 2, -1, 0, 1.0),         # composed path
+    (5120, 2048, 6, 2, 3, 5, 1, 0.05),     # the one-launch kernel's other hidden width (20 rows of W2 a workgroup), SiTU
+    (5120, 2048, 6, 3, 4, -1, 2, 1.0),     # the same, DeepSeek rule, no shared expert
 ]
 
 
@@ -182,41 +184,62 @@ def test_stages_compose_to_the_layer():
         assert np.array_equal(one.view(np.uint32), two.view(np.uint32)), (d, inter, B)
 
 
-def tiles_layout_np(p, s, rows, cols, col_major):
-    """The tiled layout as include/mk_hip.h states it, element by element: the 32-block (r, b) of the matrix sits in chunk
-    ci at lane l; the 16 nibble bytes at (ci >> 1) * 2176 + (ci & 1) * 1024 + 16 l, the scale byte at (ci >> 1) * 2176 + 2048 +
-    2 l + (ci & 1)."""
-    nb = cols // 32
-    r, b = np.meshgrid(np.arange(rows), np.arange(nb), indexing="ij")
-    if col_major:
-        ci = (b >> 1) * (rows // 32) + (r >> 5)
-        lane = (r & 15) + 16 * (2 * ((r >> 4) & 1) + (b & 1))
-    else:
-        ci = (r >> 4) * (nb // 4) + (b >> 2)
-        lane = (r & 15) + 16 * (b & 3)
+def pack_gate_up_np(p1, s1, p3, s3, d, inter):
+    """The gate/up pack as include/mk_hip.h states it, element by element."""
+    nb = d // 32
+    out = np.zeros(2 * inter * nb * 17, np.uint8)
+    r, b = np.meshgrid(np.arange(inter), np.arange(nb), indexing="ij")
+    ci = (r >> 3) * (nb >> 2) + (b >> 2)
     base = (ci >> 1) * 2176
-    out = np.zeros(rows * nb * 17, np.uint8)
-    nib_at = (base + (ci & 1) * 1024 + 16 * lane)[..., None] + np.arange(16)
-    out[nib_at.reshape(-1)] = p.reshape(rows, nb, 16).reshape(-1)
-    out[(base + 2048 + 2 * lane + (ci & 1)).reshape(-1)] = s.reshape(-1)
+    for m, (p, s) in enumerate(((p1, s1), (p3, s3))):
+        lane = (r & 7) + 8 * m + 16 * (b & 3)
+        at = (base + (ci & 1) * 1024 + 16 * lane)[..., None] + np.arange(16)
+        out[at.reshape(-1)] = p.reshape(inter, nb, 16).reshape(-1)
+        out[(base + 2048 + 2 * lane + (ci & 1)).reshape(-1)] = s.reshape(-1)
     return out
 
 
-@pytest.mark.parametrize("rows,cols,col_major", [(16, 256, 0), (64, 64, 1), (1024, 512, 1), (7168, 2048, 1), (2048, 7168, 0), (512, 1024, 0)])
-def test_tiled_copy_is_the_same_matrix_bit_for_bit(rows, cols, col_major):
-    # the experts in the matrix instruction's operand order: the bytes sit where the header says, and dequant(tiles) is
-    # mxfp4::dequant bit for bit
-    torch_cuda()
+def pack_down_np(p2, s2, d, inter):
+    """The down pack as include/mk_hip.h states it, element by element (padding zero)."""
+    nbi, rw = inter // 32, d // 256
+    rb = rw - 16
+    step = (1024 + 64 * rb + 64 + 4 * rb + 127) // 128 * 128
+    out = np.zeros(256 * (inter // 128) * step, np.uint8)
+    r, b = np.meshgrid(np.arange(d), np.arange(nbi), indexing="ij")
+    c, i, kb = r // rw, r % rw, b & 3
+    base = (c * (nbi >> 2) + (b >> 2)) * step
+    noff = np.where(i < 16, 16 * (i + 16 * kb), 1024 + 16 * (kb * rb + i - 16))
+    soff = 1024 + 64 * rb + np.where(i < 16, i + 16 * kb, 64 + kb * rb + i - 16)
+    at = (base + noff)[..., None] + np.arange(16)
+    out[at.reshape(-1)] = p2.reshape(d, nbi, 16).reshape(-1)
+    out[(base + soff).reshape(-1)] = s2.reshape(-1)
+    return out
+
+
+@pytest.mark.parametrize("d,inter", [(7168, 2048), (5120, 2048), (4608, 256)])
+def test_packed_copies_are_the_same_matrices_byte_for_byte(d, inter):
+    # the experts in the one-launch kernel's order: the bytes sit where the header says, unpacking restores the reference
+    # layout byte for byte, and dequant of the restored matrices is mxfp4::dequant bit for bit
+    torch = torch_cuda()
     from microkimi_amd import mxfp4
-    rng = np.random.default_rng(rows + cols)
-    p = rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8)   # every nibble, -0.0 (nibble 8) included
-    s = rng.integers(0, 256, (rows, cols // 32), dtype=np.uint8)  # every scale byte, the subnormal byte 0 included
-    s[0, 0], s[rows - 1, cols // 32 - 1] = 0, 255
-    tiles = mxfp4.to_tiles(dev(p), dev(s), rows, cols, col_major)
-    assert np.array_equal(tiles.cpu().numpy(), tiles_layout_np(p, s, rows, cols, col_major))
-    got = mxfp4.dequant_tiles(tiles, rows, cols, col_major).cpu().numpy()
-    want = oracle.mxfp4_dequant(p, s, rows, cols)
-    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    from microkimi_amd._lib import check, lib, ptr
+    rng = np.random.default_rng(d + inter)
+    draw = lambda rows, cols: (rng.integers(0, 256, (rows, cols // 2), dtype=np.uint8), rng.integers(0, 256, (rows, cols // 32), dtype=np.uint8))
+    (p1, s1), (p3, s3), (p2, s2) = draw(inter, d), draw(inter, d), draw(d, inter)  # every nibble and every scale byte
+    dv = [dev(x) for x in (p1, s1, p3, s3, p2, s2)]
+    pk13 = torch.empty(lib.mk_moe_pack_bytes(d, inter, 0), dtype=torch.uint8, device="cuda")
+    pk2 = torch.full((lib.mk_moe_pack_bytes(d, inter, 1),), 0xAB, dtype=torch.uint8, device="cuda")
+    check(lib.mk_dev_moe_pack_gate_up(ptr(dv[0]), ptr(dv[1]), ptr(dv[2]), ptr(dv[3]), d, inter, ptr(pk13), None))
+    check(lib.mk_dev_moe_pack_down(ptr(dv[4]), ptr(dv[5]), d, inter, ptr(pk2), None))
+    assert np.array_equal(pk13.cpu().numpy(), pack_gate_up_np(p1, s1, p3, s3, d, inter))
+    assert np.array_equal(pk2.cpu().numpy(), pack_down_np(p2, s2, d, inter))
+    back = [torch.zeros_like(t) for t in dv]
+    check(lib.mk_dev_moe_unpack_gate_up(ptr(pk13), d, inter, ptr(back[0]), ptr(back[1]), ptr(back[2]), ptr(back[3]), None))
+    check(lib.mk_dev_moe_unpack_down(ptr(pk2), d, inter, ptr(back[4]), ptr(back[5]), None))
+    for t, h in zip(back, (p1, s1, p3, s3, p2, s2)):
+        assert np.array_equal(t.cpu().numpy(), h)
+    got = mxfp4.dequant(back[4], back[5], d, inter).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.mxfp4_dequant(p2, s2, d, inter).view(np.uint32))
 
 
 TWO_LAUNCH_CASES = [
@@ -229,14 +252,13 @@ TWO_LAUNCH_CASES = [
 
 
 @pytest.mark.parametrize("d,inter,n_experts,B,topk,shared,act,hs", TWO_LAUNCH_CASES)
-def test_two_launch_path_without_the_tiled_copies(d, inter, n_experts, B, topk, shared, act, hs):
-    """A table without the tiled copies takes the gate/up launch and the down launch (up to 3 tokens): both stages
-    against the oracle to TOL with nothing removed, the stages compose to the layer bit for bit, and the one-launch
-    path fed the same activation rows adds the same block terms in another order."""
+def test_two_launch_path_without_the_packed_copies(d, inter, n_experts, B, topk, shared, act, hs):
+    """A table without the packed copies takes the gate/up launch and the down launch (up to 3 tokens): both stages
+    against the oracle to TOL with nothing removed, the stages compose to the layer bit for bit, and (where the one-launch
+    kernel takes the shape) that kernel fed the same activation rows adds the same block terms in another order."""
     from microkimi_amd import model
-    table, experts = build(n_experts, d, inter, tiles=False)
-    _, with_tiles = build(n_experts, d, inter, tiles=True)
-    assert experts.table.w2t is None and with_tiles.table.w2t is not None
+    table, experts = build(n_experts, d, inter, pack=False)
+    assert experts.table.w2t is None
     host = (table_host(table, 0), table_host(table, 1))
     ids, wts, x = stage_inputs(d, inter, n_experts, B, topk, shared, hs)
     limit = 10.0 if act == 2 else 0.0
@@ -245,8 +267,6 @@ def test_two_launch_path_without_the_tiled_copies(d, inter, n_experts, B, topk, 
     got_a = a.cpu().numpy()
     worst = max(rel_l2(got_a[t, s], want_a[t, s]) for t in range(B) for s in range(got_a.shape[1]))
     assert worst <= TOL, f"worst activation row rel-L2 {worst:.2e}"
-    a_tiles = model.moe_decode_act(with_tiles, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
-    assert max(rel_l2(a_tiles[t, s], got_a[t, s]) for t in range(B) for s in range(got_a.shape[1])) <= 2e-6
     want = oracle.moe_decode(table, ids.astype(np.uint32), wts, x, shared=shared, mode=1, act_kind=act, limit=limit, threads=8)
     got = model.moe_decode_from_act(experts, dev(ids), dev(wts), dev(want_a), shared=shared, mode=1, act_kind=act).cpu().numpy()
     worst = max(rel_l2(got[t], want[t]) for t in range(B))
@@ -254,9 +274,56 @@ def test_two_launch_path_without_the_tiled_copies(d, inter, n_experts, B, topk, 
     two = model.moe_decode_from_act(experts, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
     one = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
     assert np.array_equal(one.view(np.uint32), two.view(np.uint32))
-    # the one-launch path on the same activation rows: the same block terms, added in another order
-    tile_rows = model.moe_decode_from_act(with_tiles, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
-    assert max(rel_l2(tile_rows[t], two[t]) for t in range(B)) <= 2e-6
+    if d == 7168 and inter == 2048:
+        # the one-launch kernel on the same inputs: the same block terms, added in another order
+        _, packed = build(n_experts, d, inter, pack=True)
+        assert packed.table.w2t is not None and packed.table.w13t is not None
+        a_one = model.moe_decode_act(packed, dev(ids), dev(wts), dev(x), shared=shared, mode=1, act_kind=act, limit=limit).cpu().numpy()
+        assert max(rel_l2(a_one[t, s], got_a[t, s]) for t in range(B) for s in range(got_a.shape[1])) <= 2e-6
+        rows = model.moe_decode_from_act(packed, dev(ids), dev(wts), a, shared=shared, mode=1, act_kind=act).cpu().numpy()
+        assert max(rel_l2(rows[t], two[t]) for t in range(B)) <= 2e-6
+
+
+def test_one_launch_kernel_repeated_and_captured():
+    """The one-launch kernel carries a launch tag in its exchanged values: repeated calls on one workspace, calls with
+    fewer pairs after calls with more, and replays of a captured graph all give the first call's rows bit for bit, and no
+    workgroup ever gave up waiting."""
+    torch = torch_cuda()
+    import ctypes
+    from microkimi_amd import model
+    from microkimi_amd._lib import check, lib
+    d, inter, n_experts, topk, shared = 7168, 2048, 12, 8, 11
+    table, experts = build(n_experts, d, inter)
+    assert experts.table.w13t is not None
+    res = {}
+    for B in (3, 1, 2, 3, 1):
+        ids, wts, x = stage_inputs(d, inter, n_experts, B, topk, shared, 1.0)
+        got = model.moe_decode(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=1).cpu().numpy()
+        assert np.isfinite(got).all()
+        if B in res:
+            assert np.array_equal(got.view(np.uint32), res[B].view(np.uint32)), B
+        res[B] = got
+    ids, wts, x = stage_inputs(d, inter, n_experts, 2, topk, shared, 1.0)
+    di, dw, dx = dev(ids), dev(wts), dev(x)
+    out = torch.empty((2, d), device="cuda")
+    model.moe_decode(experts, di, dw, dx, shared=shared, mode=1, out=out)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            model.moe_decode(experts, di, dw, dx, shared=shared, mode=1, out=out)
+            model.moe_decode(experts, di, dw, dx, shared=shared, mode=1, out=out)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), res[2].view(np.uint32))
+    flag = ctypes.c_int(-1)
+    check(lib.mk_dev_moe_decode_gave_up(ctypes.byref(flag)))
+    assert flag.value == 0
 
 
 def test_out_of_range_expert_id_adds_nothing():
