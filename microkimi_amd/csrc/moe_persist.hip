@@ -50,6 +50,9 @@ __host__ __device__ constexpr int pk_step_bytes(int rb) { return (1024 + 64 * rb
 // launch counter of this device (the tag of a launch is its value + 1) and the give-up flag
 __device__ unsigned g_moe_launch_ctr;
 __device__ int g_moe_fail;
+// -DMK_MOE_TRACE: every multiplying wave leaves time stamps (100 MHz) of the last launch, read with mk_debug_moe_ts:
+// 0 start, 1 hidden rows staged, 2 phase 1 done, 3 first pair of phase 2 done, 4 time spent waiting for codes in phase 2,
+// 5 end
 #ifdef MK_MOE_TRACE
 __device__ unsigned long long g_moe_ts[PK_GRID * 4 * 8];
 #define TS(i) ts[i] = __builtin_amdgcn_s_memrealtime()
@@ -221,12 +224,30 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
 #pragma unroll
         for (int b = 0; b < SB; b++) xv0[b] = reinterpret_cast<const mk_f4 *>(a.x)[min((int)threadIdx.x + b * 512, NX - 1)];
     }
+    // the pair tables: a pair's expert id and its two pointers would be two memory round trips one after the other before
+    // the first weight can be asked for; the pointer tables (when the table states its size and it fits) are read beside
+    // the ids and looked up in LDS
+    const bool tabs_in_lds = a.tab.n_experts > 0 && a.tab.n_experts <= 512;
+    const uint8_t **t13 = reinterpret_cast<const uint8_t **>(lds + L::PGU_OFF), **t2 = t13 + 512;  // (the partial sums' place, before they exist)
+    int my_e = 0;
+    bool my_ok = true;
     if ((int)threadIdx.x < P) {
         const int q = threadIdx.x, tok = q / per, sl = q - tok * per;
-        bool ok = true;
-        const int e = sl < a.topk ? mk_checked_expert(a.ids[tok * a.topk + sl], a.tab.n_experts, ok) : a.shared;
-        p13[q] = a.tab.w13t[e];
-        p2[q] = a.tab.w2t[e];
+        my_e = sl < a.topk ? mk_checked_expert(a.ids[tok * a.topk + sl], a.tab.n_experts, my_ok) : a.shared;
+    }
+    if (tabs_in_lds) {
+        if (threadIdx.x < a.tab.n_experts) {
+            t13[threadIdx.x] = a.tab.w13t[threadIdx.x];
+            t2[threadIdx.x] = a.tab.w2t[threadIdx.x];
+        }
+        __syncthreads();
+    }
+    if ((int)threadIdx.x < P) {
+        const int q = threadIdx.x, tok = q / per, sl = q - tok * per;
+        const int e = my_e;
+        const bool ok = my_ok;
+        p13[q] = tabs_in_lds ? t13[e] : a.tab.w13t[e];
+        p2[q] = tabs_in_lds ? t2[e] : a.tab.w2t[e];
         const float w = sl < a.topk ? (ok ? a.weights[tok * a.topk + sl] : 0.0f) : 1.0f;
         wg_l[q] = w;                                                     // inside the activation (DeepSeek rule)
         pw_l[q] = !ok ? 0.0f : (sl < a.topk && !a.ds_rule) ? w : 1.0f;  // in the sum over the pairs
@@ -292,6 +313,22 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
     TS(1);
 
     if (wave < 4) {
+        // (phase 2's weights: declared here because the first of them are requested before phase 1's last item is worked on)
+        constexpr int R2 = 2;  // pairs of this wave's K steps of W2 in flight (three measured slower: 41.9 against 40.5 us)
+        Step2 w2r[R2][SW];
+        const int nb_c = min(n, RB - 1);
+        auto load_pair = [&](Step2 *S, int q) {
+            q = __builtin_amdgcn_readfirstlane(min(q, P - 1));  // past the end: the last pair once more (unconditional loads)
+            const uint8_t *base = mk_uniform_ptr(p2[q]);
+#pragma unroll
+            for (int s = 0; s < SW; s++) {
+                const uint32_t off = (uint32_t)((c * NSI + wave * SW + s) * STEP);
+                S[s].wa = mk_ldg128_off_nt(base, off + lane * 16);
+                S[s].wb = mk_ldg128_off_nt(base, off + 1024 + (kb * RB + nb_c) * 16);
+                S[s].sa = mk_ldg_u8_off(base, off + 1024 + 64 * RB + lane);
+                S[s].sb = mk_ldg_u8_off(base, off + 1024 + 64 * RB + 64 + kb * RB + nb_c);
+            }
+        };
         // ------------------------------------------------------------ the multiplying waves, phase 1
         if constexpr (stage != MK_MOE_STAGE_FROM_ACT) {
             mk_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, tp = acc;  // tp: the previous step's result, taken out after the next instruction is issued
@@ -321,16 +358,11 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
                     else __hip_atomic_store(pa.lines + at, ((unsigned long long)tag << 32) | __float_as_uint(act), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             };
-            for (int it = 0; it < nitems; it++) {
+            auto do_item = [&](const Cont13 *cur, int it) {
                 const int q = it / KI, tok = q / per;
                 const uint8_t *xt = xc + tok * L::XTOK + pt * L::ROWB + code_off + (CW * wave) * 256;
                 const uint8_t *plo = has_lo ? xt : zero, *phi = has_hi ? xt : zero;
                 const float *pdx = xsc + tok * NB + (n < 8 ? ph : 0) + (CW * wave) * 8;
-                // this item's containers are in the ring; they are taken out and the ring is refilled with the next item's
-                Cont13 cur[CW];
-#pragma unroll
-                for (int i = 0; i < CW; i++) cur[i] = ring[i];
-                load_item(it + 1);
 #pragma unroll
                 for (int i = 0; i < CW; i++) {
 #pragma unroll
@@ -349,35 +381,34 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
                         dprev = dcur;
                     }
                 }
+            };
+            // an item's containers are in the ring; they are taken out and the ring is refilled with the next item's
+            Cont13 cur[CW];
+            for (int it = 0; it < nitems - 1; it++) {
+#pragma unroll
+                for (int i = 0; i < CW; i++) cur[i] = ring[i];
+                load_item(it + 1);
+                do_item(cur, it);
             }
+            // the last item: phase 2's first weights are requested in its place
+#pragma unroll
+            for (int i = 0; i < CW; i++) cur[i] = ring[i];
+            if constexpr (stage == MK_MOE_STAGE_ALL) {
+#pragma unroll
+                for (int k = 0; k < R2; k++) load_pair(w2r[k], k);
+            }
+            do_item(cur, nitems - 1);
 #pragma unroll
             for (int r = 0; r < 4; r++) acc[r] = mk_add(acc[r], mk_mul(tp[r] + mk_dpp<0xB1>(tp[r]), dprev));
             finish_item(nitems - 1);
             TS(2);
             if constexpr (stage == MK_MOE_STAGE_ACT) return;
+        } else {
+#pragma unroll
+            for (int k = 0; k < R2; k++) load_pair(w2r[k], k);
         }
 
         // ------------------------------------------------------------ the multiplying waves, phase 2
-#ifndef PK_R2
-#define PK_R2 3
-#endif
-        constexpr int R2 = PK_R2;  // pairs of this wave's K steps of W2 in flight
-        Step2 w2r[R2][SW];
-        const int nb_c = min(n, RB - 1);
-        auto load_pair = [&](Step2 *S, int q) {
-            q = __builtin_amdgcn_readfirstlane(min(q, P - 1));  // past the end: the last pair once more (unconditional loads)
-            const uint8_t *base = mk_uniform_ptr(p2[q]);
-#pragma unroll
-            for (int s = 0; s < SW; s++) {
-                const uint32_t off = (uint32_t)((c * NSI + wave * SW + s) * STEP);
-                S[s].wa = mk_ldg128_off_nt(base, off + lane * 16);
-                S[s].wb = mk_ldg128_off_nt(base, off + 1024 + (kb * RB + nb_c) * 16);
-                S[s].sa = mk_ldg_u8_off(base, off + 1024 + 64 * RB + lane);
-                S[s].sb = mk_ldg_u8_off(base, off + 1024 + 64 * RB + 64 + kb * RB + nb_c);
-            }
-        };
-#pragma unroll
-        for (int k = 0; k < R2; k++) load_pair(w2r[k], k);
         // W2_e act of pair q for this wave's K steps: partial sums of the workgroup's rows into po[q][wave]
         auto multiply = [&](const Step2 *S, int q) {
             // the pair's codes are in LDS when both exchange waves have counted it (they always count on, also after giving up)
@@ -386,9 +417,8 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
 #endif
             for (int spin = 0; pk_lds_min4(ready_l) <= q && spin < (1 << 26); spin++) __builtin_amdgcn_s_sleep(1);
 #ifdef MK_MOE_TRACE
-            if (q > 0) ts[5] += __builtin_amdgcn_s_memrealtime() - tw0;
+            ts[4] += __builtin_amdgcn_s_memrealtime() - tw0;
 #endif
-            if (q == 0) TS(3);
             const uint8_t *buf = actb + (q % RC) * ACTB;
             const float *adx = reinterpret_cast<const float *>(buf + 2 * AROWB);
             const uint8_t *xt = buf + pt * AROWB + code_off + (SW * wave) * 128;
@@ -426,8 +456,7 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if (lane == 0) *(volatile int *)(prog_l + wave) = q + 1;
-            if (q == 0) TS(4);
-            if (q == 3) TS(6);
+            if (q == 0) TS(3);
         };
         for (int q0 = 0; q0 < P; q0 += R2) {
 #pragma unroll
@@ -439,7 +468,7 @@ __global__ __launch_bounds__(512) void moe_persist_kernel(PersistArgs pa, int RC
                 }
             }
         }
-        TS(7);
+        TS(5);
     } else {
         // ------------------------------------------------------------ the exchange waves
         if constexpr (stage == MK_MOE_STAGE_ACT) return;
