@@ -583,7 +583,7 @@ def bench_gemm(torch):
     out = torch.empty((T, d), device="cuda")
 
     def step3():
-        model.moe_prefill(experts, ids_d, wts_d, x_d, out=out)
+        model.moe_prefill(experts, ids_d, wts_d, x_d, out=out, mxfp8=True)
 
     ms3 = time_region(torch, step3, 5, warmup=2)
     per_expert = 3 * (inter * d // 2 + inter * d // 32)

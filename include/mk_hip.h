@@ -64,6 +64,13 @@ int mk_init(int device);
 int mk_available(void);
 void mk_shutdown(void);
 const char *mk_last_error(void);
+/* The process-wide off switch, the counterpart of the reference's A/B override (mxfp4::no_packed_gpu,
+ * src/mxfp4.rs:327-333, MICROKIMI_NO_PACKED_GPU=1): after mk_set_enabled(0), or with MK_HIP=0 in the
+ * environment at the first call, every entry point that returns a status returns MK_ERR_NO_DEVICE before it makes any HIP
+ * call, and mk_available() is 0, so a caller's existing CPU path takes over.  mk_set_enabled(1) switches back on (it also
+ * overrides MK_HIP=0).  mk_enabled_now() reads the switch.  Work already queued on a stream is not affected. */
+void mk_set_enabled(int on);
+int mk_enabled_now(void);
 /* Device-cache budget in MiB for the host-level weight cache (MICROKIMI_GPU_CACHE_MB,
  * src/metal.rs:554-558).  0 = unlimited (default). */
 void mk_set_cache_mb(size_t mb);
@@ -253,6 +260,10 @@ int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const
 /* *flag = 1 if a workgroup of the one-launch form ever gave up waiting on this device (its rows are NaN), else 0.
  * Synchronous (a device-to-host copy).  Has no counterpart in the reference. */
 int mk_dev_moe_decode_gave_up(int *flag);
+/* count[0] (device int32) = how many of the n routed ids lie outside [0, n_experts): the pairs that the decode and prefill
+ * calls skip when the table states its size.  The reference would panic on such an index (a slice index out of range,
+ * src/model.rs:2243); a caller that wants to know asks here, on the same stream.  Asynchronous. */
+int mk_dev_moe_count_bad_ids(const int32_t *ids, size_t n, size_t n_experts, int32_t *count, void *stream);
 
 /* The two halves of mk_dev_moe_decode on their own, for callers that keep the reference's call structure (two
  * matvec_packed calls, the activation, then the third matvec_packed: src/model.rs:2246-2259, src/deepseek.rs:1080-1089)

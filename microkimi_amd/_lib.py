@@ -54,6 +54,8 @@ def _load():
         "mk_init": (i32, [i32]),
         "mk_available": (i32, []),
         "mk_shutdown": (None, []),
+        "mk_set_enabled": (None, [i32]),
+        "mk_enabled_now": (i32, []),
         "mk_last_error": (C.c_char_p, []),
         "mk_set_cache_mb": (None, [sz]),
         "mk_force_q8": (None, [i32]),
@@ -81,6 +83,7 @@ def _load():
         "mk_dev_moe_pack_down": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_dev_moe_unpack_down": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_moe_decode_gave_up": (i32, [C.POINTER(C.c_int)]),
+        "mk_dev_moe_count_bad_ids": (i32, [vp, sz, sz, vp, vp]),
         "mk_moe_decode_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_moe_decode_vq_workspace_bytes": (sz, [sz, sz, i32, sz, sz]),
         "mk_dev_moe_decode": (i32, [C.POINTER(ExpertTable), sz, sz, vp, vp, i32, vp, i32, i32, f32, vp, vp, vp]),

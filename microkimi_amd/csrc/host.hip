@@ -59,6 +59,7 @@ struct Ctx {
 Ctx g_ctx;
 
 int ensure_init() {
+    MK_REQUIRE_ENABLED();
     if (g_ctx.ready) return MK_OK;
     return mk_init(0);
 }
@@ -118,7 +119,19 @@ int mk_lds_opt_in(const void *kernel, int bytes) {
 
 extern "C" const char *mk_last_error(void) { return g_err; }
 
+int mk_enabled_state = -1;
+int mk_enabled_slow() {
+    const char *e = getenv("MK_HIP");
+    const int on = !(e && e[0] == '0' && e[1] == 0);
+    int expect = -1;
+    __atomic_compare_exchange_n(&mk_enabled_state, &expect, on, false, __ATOMIC_RELAXED, __ATOMIC_RELAXED);
+    return __atomic_load_n(&mk_enabled_state, __ATOMIC_RELAXED);
+}
+extern "C" void mk_set_enabled(int on) { __atomic_store_n(&mk_enabled_state, on ? 1 : 0, __ATOMIC_RELAXED); }
+extern "C" int mk_enabled_now(void) { return mk_enabled() ? 1 : 0; }
+
 extern "C" int mk_init(int device) {
+    MK_REQUIRE_ENABLED();
     std::lock_guard<std::mutex> lk(g_mu);
     if (g_ctx.ready) return MK_OK;
     int n = 0;
@@ -139,7 +152,12 @@ extern "C" int mk_init(int device) {
     }
     if (mk_check_hip(hipSetDevice(device), "hipSetDevice") != MK_OK) return g_ctx.status = MK_ERR_HIP;
     if (mk_check_hip(hipStreamCreate(&g_ctx.stream), "hipStreamCreate") != MK_OK) return g_ctx.status = MK_ERR_HIP;
-    if (mk_mla_static_init(nullptr) != MK_OK) return g_ctx.status = MK_ERR_HIP;
+    if (mk_mla_static_init(nullptr) != MK_OK) {
+        // a failed initialisation keeps nothing: the next mk_init starts from the beginning
+        hipStreamDestroy(g_ctx.stream);
+        g_ctx.stream = nullptr;
+        return g_ctx.status = MK_ERR_HIP;
+    }
     const char *mb = getenv("MK_GPU_CACHE_MB");
     if (mb && *mb) g_ctx.cache_cap = (size_t)strtoull(mb, nullptr, 10) << 20;
     const char *dbg = getenv("MK_GPU_DEBUG");
@@ -149,7 +167,7 @@ extern "C" int mk_init(int device) {
     return g_ctx.status = MK_OK;
 }
 
-extern "C" int mk_available(void) { return g_ctx.ready ? 1 : 0; }
+extern "C" int mk_available(void) { return g_ctx.ready && mk_enabled() ? 1 : 0; }
 
 extern "C" void mk_shutdown(void) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -649,8 +667,8 @@ extern "C" size_t mk_mla_cache_positions(const mk_mla_cache *c) { return c ? c->
 
 extern "C" int mk_mla_cache_set_hadamard(mk_mla_cache *c, int on) {
     MK_REQUIRE(c, "null pointer");
-    MK_REQUIRE(c->heads_layout, "the Hadamard option belongs to the per-head layout (mk_mla_cache_new_heads)");
     std::lock_guard<std::mutex> lk(g_mu);
+    MK_REQUIRE(c->heads_layout, "the Hadamard option belongs to the per-head layout (mk_mla_cache_new_heads)");
     MK_REQUIRE(c->n == 0, "the option can change only while the cache is empty");
     c->had = on ? 1 : 0;
     return MK_OK;

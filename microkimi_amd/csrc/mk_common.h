@@ -304,8 +304,25 @@ int mk_check_hip(hipError_t e, const char *what);
         int _s = mk_check_hip((expr), #expr);           \
         if (_s != MK_OK) return _s;                     \
     } while (0)
+// The process-wide off switch (mk_set_enabled, MK_HIP=0 in the environment): 1 on, 0 off, -1 not yet read from the
+// environment.  Every entry point that returns a status checks its arguments through MK_REQUIRE first, so the switch is
+// tested there: a disabled library returns MK_ERR_NO_DEVICE before any HIP call.
+extern int mk_enabled_state;
+int mk_enabled_slow();
+static inline bool mk_enabled() {
+    const int v = __atomic_load_n(&mk_enabled_state, __ATOMIC_RELAXED);
+    return v > 0 || (v < 0 && mk_enabled_slow());
+}
+#define MK_REQUIRE_ENABLED()                                                                          \
+    do {                                                                                              \
+        if (!mk_enabled()) {                                                                          \
+            mk_set_error("the library is switched off (mk_set_enabled(0) or MK_HIP=0)");              \
+            return MK_ERR_NO_DEVICE;                                                                  \
+        }                                                                                             \
+    } while (0)
 #define MK_REQUIRE(cond, msg)                           \
     do {                                                \
+        MK_REQUIRE_ENABLED();                           \
         if (!(cond)) {                                  \
             mk_set_error("invalid argument: %s", msg);  \
             return MK_ERR_INVALID;                      \

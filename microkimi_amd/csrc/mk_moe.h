@@ -1,10 +1,10 @@
-// Shared by the MoE decode kernels (moe.hip, moe_slab.hip).
+// Shared by the MoE decode kernels (moe.hip, moe_persist.hip).
 #pragma once
 #include "mk_common.h"
 
 // Expert id of a routed pair.  When the table states its size, an id outside it selects entry 0 with routing weight 0:
 // the pair then adds nothing to the token's row (the pointer arrays are never read out of bounds).  The reference
-// would panic on such an index; a caller that wants to know asks mk_dev_moe_count_bad_ids.
+// would panic on such an index; a caller that wants to know asks mk_dev_moe_count_bad_ids (moe.hip).
 __device__ __forceinline__ int mk_checked_expert(int e, size_t n_experts, bool &ok) {
     ok = n_experts == 0 || (unsigned)e < (unsigned)n_experts;
     return ok ? e : 0;

@@ -767,6 +767,7 @@ extern "C" int mk_dev_mla_heads_q8_attn(const int8_t *kq, const float *ks, const
     a.had_k = had ? 1.0f / 64.0f : 1.0f;
     // the reference's own head shape takes the all-heads kernel
     const bool g8 = nope == 128 && rope == 64 && vd == 128 && (pos0 + m) * nh * 128 < 0xFFFFFFFFull &&
+                      (pos0 + m) * nh * rope * 4 < 0xFFFFFFFFull &&  // the kernel's 32-bit byte offsets: q8 rows and f32 rope rows
                       ((uintptr_t)vq & 15) == 0 && ((uintptr_t)kr & 15) == 0 && ((uintptr_t)q & 15) == 0 && !MK_TUNE("MK_MLA_HEADS_GENERIC", 0);
     const bool many = g8 && m >= (size_t)MK_TUNE("MK_MLA_HEADS_PREFILL_MIN", 16);
     if (g8 && !had && !many) {

@@ -903,6 +903,26 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
 }
 }  // namespace
 
+namespace {
+// one workgroup: count[0] = number of ids outside [0, n_experts)
+__global__ __launch_bounds__(256) void count_bad_ids_kernel(const int32_t *__restrict__ ids, size_t n, unsigned n_experts, int32_t *__restrict__ count) {
+    __shared__ int part[4];
+    int c = 0;
+    for (size_t i = threadIdx.x; i < n; i += 256) c += (unsigned)ids[i] >= n_experts ? 1 : 0;
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) count[0] = part[0] + part[1] + part[2] + part[3];
+}
+}  // namespace
+
+extern "C" int mk_dev_moe_count_bad_ids(const int32_t *ids, size_t n, size_t n_experts, int32_t *count, void *stream) {
+    MK_REQUIRE(ids && count, "null pointer");
+    MK_REQUIRE(n >= 1 && n_experts >= 1 && n_experts < (1u << 31), "n and n_experts must be at least 1");
+    hipLaunchKernelGGL(count_bad_ids_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, ids, n, (unsigned)n_experts, count);
+    return mk_launch_status("count_bad_ids");
+}
+
 extern "C" int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                                  const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream) {
     return moe_decode_impl(table, B, topk, ids, weights, shared, x, mode, act_kind, limit, workspace, out, stream, STAGE_ALL, nullptr);

@@ -308,27 +308,44 @@ def moe_prefill_intermediates(experts, T, topk):
             "g": f32(lay.g, P, experts.inter), "u": f32(lay.u, P, experts.inter), "o": f32(lay.o, P, experts.d)}
 
 
-def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None, keep=False, exact=False, bf16=False):
+PREFILL_MAX_PAIRS = 16384  # (token, slot) pairs one mk_dev_moe_prefill* call takes
+
+
+def moe_prefill(experts, ids, weights, x, act_kind=ACT_SWIGLU, out=None, keep=False, exact=False, bf16=False, mxfp8=False):
     """The expert section of moe_prefill (src/model.rs:2528-2602, 2690-2700) for T prompt positions: pairs grouped by
-    expert, gate / up / activation / down per used expert on the block-scaled matrix cores (MXFP8 activations),
-    per-token weighted sum in slot order.  ids [T, topk] int32, weights [T, topk] f32, x [T, d] f32; returns [T, d].
-    keep: also store the f32 gate and up rows (moe_prefill_intermediates reads them); the result is the same.
-    exact: the reference's own arithmetic instead (f32 rows and activation against the dequantized weights, f32 products
-    and sums on the f32 matrix instruction: matvec_packed_nt per expert, src/model.rs:2580-2599); the intermediates then
-    hold ACT(gate, up) in "g", the up rows in "u" and the down rows in "o".
+    expert, gate / up / activation / down per used expert, per-token weighted sum in slot order.  ids [T, topk] int32,
+    weights [T, topk] f32, x [T, d] f32; returns [T, d].
+    The arithmetic is the reference's own unless the caller asks for less (f32 rows and activation against the
+    dequantized weights, f32 products and sums on the f32 matrix instruction: matvec_packed_nt per expert,
+    src/model.rs:2580-2599; mk_dev_moe_prefill_f32; `exact=True` names the same thing).  The intermediates then hold
+    ACT(gate, up) in "g", the up rows in "u" and the down rows in "o".
     bf16: hidden rows and activation rows rounded to bfloat16, exact weights, f32 products and sums on the bf16 matrix
-    instruction (mk_dev_moe_prefill_bf16); "g" and "u" then hold the gate and up rows."""
+    instruction (mk_dev_moe_prefill_bf16); "g" and "u" then hold the gate and up rows.
+    mxfp8: activations as MXFP8 blocks on the block-scaled matrix cores (mk_dev_moe_prefill), the fastest form and the
+    one with no counterpart in the reference: an explicit opt-in.  keep (mxfp8 only): also store the f32 gate and up
+    rows (moe_prefill_intermediates reads them); the result is the same.
+    A prompt of more than 16384 (token, slot) pairs is split into calls of whole tokens; the intermediates are then
+    those of the last call."""
     import torch
     _lib.require_device()
     T, topk = ids.shape
-    need = lib.mk_moe_prefill_workspace_bytes(T, topk, experts.n, experts.d, experts.inter)
+    if bf16 + mxfp8 + exact > 1:
+        raise ValueError("exact, bf16 and mxfp8 name three different arithmetics: pick one")
+    if keep and not mxfp8:
+        raise ValueError("keep belongs to the mxfp8 form (the others store their intermediates anyway)")
+    step = max(1, PREFILL_MAX_PAIRS // topk)
+    need = lib.mk_moe_prefill_workspace_bytes(min(T, step), topk, experts.n, experts.d, experts.inter)
     if experts._ws is None or experts._ws.numel() < need:
         experts._ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     if out is None:
         out = torch.empty((T, experts.d), dtype=torch.float32, device=x.device)
-    fn = lib.mk_dev_moe_prefill_bf16 if bf16 else lib.mk_dev_moe_prefill_f32 if exact else lib.mk_dev_moe_prefill_keep if keep else lib.mk_dev_moe_prefill
-    check(fn(C.byref(experts.table), experts.n, T, topk, ptr(ids.contiguous()), ptr(weights.contiguous()), ptr(x.contiguous()), act_kind,
-             ptr(experts._ws), ptr(out), cur_stream()))
+    fn = lib.mk_dev_moe_prefill_bf16 if bf16 else (lib.mk_dev_moe_prefill_keep if keep else lib.mk_dev_moe_prefill) if mxfp8 else lib.mk_dev_moe_prefill_f32
+    ids, weights, x = ids.contiguous(), weights.contiguous(), x.contiguous()
+    assert out.is_contiguous()
+    for t0 in range(0, T, step):
+        n = min(step, T - t0)
+        check(fn(C.byref(experts.table), experts.n, n, topk, ptr(ids[t0:t0 + n]), ptr(weights[t0:t0 + n]), ptr(x[t0:t0 + n]), act_kind,
+                 ptr(experts._ws), ptr(out[t0:t0 + n]), cur_stream()))
     return out
 
 

@@ -82,6 +82,7 @@ _lib.orc_dequant_fp8.argtypes = [_u8p, _u8p, _sz, _sz, _f32p]
 _lib.orc_quantize_fp8.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
 _lib.orc_fp8_roundtrip.argtypes = [_f32p, _sz, _sz, _u8p, _u8p]
 _lib.orc_fp8_roundtrip_emax.argtypes = [_f32p, _sz, _sz, C.c_int, _u8p, _u8p]
+_lib.orc_round_bf16.argtypes = [_f32p, _sz]
 _lib.orc_quantize_q8.argtypes = [_f32p, _sz, _i8p, _f32p]
 _lib.orc_matvec_f32.argtypes = [_f32p, _sz, _sz, _f32p, _f32p]
 _lib.orc_matvec_packed_q8.argtypes = [_u8p, _u8p, _sz, _sz, _i8p, _f32p, _f32p]
@@ -227,6 +228,14 @@ def fp8_roundtrip(x, block, emax=8):
     exps = np.empty((x.size + block - 1) // block, np.uint8)
     _lib.orc_fp8_roundtrip_emax(_p(x, _f32p), x.size, block, emax, _p(codes, _u8p), _p(exps, _u8p))
     return x, codes, exps
+
+
+def round_bf16(x):
+    """x rounded to bfloat16 (nearest, ties to even; inf and NaN unchanged), returned as f32: the input rounding of the
+    bf16 prefill section (moe_prefill with round_mxfp8=3)."""
+    y = _c(x, np.float32).copy().reshape(-1)
+    _lib.orc_round_bf16(_p(y, _f32p), y.size)
+    return y.reshape(np.shape(x))
 
 
 # --------------------------------------------------------------------- q8

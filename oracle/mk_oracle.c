@@ -1394,7 +1394,7 @@ ORC_API void orc_moe_decode(const uint8_t *const *w1p, const uint8_t *const *w1s
  * encoding of the device's prefill section; 3: hidden rows and activation
  * rounded to bfloat16 (round to nearest even), the inputs of the device's
  * bf16 prefill section. */
-static void orc_round_bf16(float *x, size_t n) {
+ORC_API void orc_round_bf16(float *x, size_t n) {
     for (size_t i = 0; i < n; i++) {
         uint32_t b;
         memcpy(&b, &x[i], 4);

@@ -7,7 +7,7 @@
 //!
 //! ```ignore
 //! #[cfg(feature = "hip")]
-//! if model::gpu_on() && rows * cols >= model::GPU_MIN_ELEMS && hip::gpu_available()
+//! if model::gpu_on() && !no_packed_gpu() && rows * cols >= model::GPU_MIN_ELEMS && hip::gpu_available()
 //!     && hip::gpu_matvec_fp4(packed, scales, rows, cols, x, out) { return; }
 //! ```
 //!
@@ -114,6 +114,8 @@ extern "C" {
     pub fn mk_init(device: c_int) -> c_int;
     pub fn mk_available() -> c_int;
     pub fn mk_shutdown();
+    pub fn mk_set_enabled(on: c_int);
+    pub fn mk_enabled_now() -> c_int;
     pub fn mk_last_error() -> *const c_char;
     pub fn mk_set_cache_mb(mb: usize);
     pub fn mk_force_q8(v: c_int);
@@ -125,6 +127,7 @@ extern "C" {
     pub fn mk_dev_moe_pack_down(w2p: *const u8, w2s: *const u8, d: usize, inter: usize, pack: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_unpack_down(pack: *const u8, d: usize, inter: usize, w2p: *mut u8, w2s: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_decode_gave_up(flag: *mut c_int) -> c_int;
+    pub fn mk_dev_moe_count_bad_ids(ids: *const i32, n: usize, n_experts: usize, count: *mut i32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_fp8_dequant(w: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_quantize_q8(x: *const f32, nvec: usize, n: usize, q: *mut i8, scales: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_quantize(w: *const f32, rows: usize, cols: usize, search: c_int, packed: *mut u8, scales: *mut u8, stream: *mut c_void) -> c_int;

@@ -63,6 +63,43 @@ def test_argument_checks_need_no_device():
     assert st == -1 and b"batch" in _lib.lib.mk_last_error()
 
 
+def test_off_switch_returns_no_device_before_anything_else():
+    # mk_set_enabled(0): every status-returning entry point answers MK_ERR_NO_DEVICE, also for arguments that it would
+    # otherwise reject (the switch is tested first) and for device-level calls (whose launch would otherwise be tried)
+    from microkimi_amd import _lib
+    lib = _lib.lib
+    assert lib.mk_enabled_now() == 1
+    lib.mk_set_enabled(0)
+    try:
+        assert lib.mk_enabled_now() == 0 and lib.mk_available() == 0
+        assert lib.mk_init(0) == -2 and b"switched off" in lib.mk_last_error()
+        st = lib.mk_dev_mxfp4_dequant(ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 48, ctypes.c_void_p(16), None)
+        assert st == -2
+        st = lib.mk_dev_mxfp4_dequant(ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 64, ctypes.c_void_p(16), None)
+        assert st == -2
+        out = np.full(4, 7.0, np.float32)
+        st = lib.mk_mxfp4_matvec(_lib.hptr(np.zeros((4, 16), np.uint8)), _lib.hptr(np.full((4, 1), 127, np.uint8)), 4, 32,
+                                 _lib.hptr(np.ones(32, np.float32)), _lib.hptr(out))
+        assert st == -2 and np.all(out == 7.0)
+        assert lib.mk_dev_moe_count_bad_ids(ctypes.c_void_p(16), 8, 4, ctypes.c_void_p(16), None) == -2
+    finally:
+        lib.mk_set_enabled(1)
+    assert lib.mk_enabled_now() == 1
+    st = lib.mk_dev_mxfp4_dequant(ctypes.c_void_p(16), ctypes.c_void_p(16), 1, 48, ctypes.c_void_p(16), None)
+    assert st == -1   # back on: the argument check answers again
+
+
+def test_off_switch_from_the_environment():
+    import subprocess
+    import sys
+    code = ("import ctypes; from microkimi_amd import _lib; l = _lib.lib; "
+            "print(l.mk_enabled_now(), l.mk_init(0), l.mk_available()); l.mk_set_enabled(1); print(l.mk_enabled_now())")
+    env = dict(os.environ, MK_HIP="0")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.split() == ["0", "-2", "0", "1"]
+
+
 def test_workloads_are_reproducible():
     from microkimi_amd import workloads as w
     p, s, x = w.config0(rows=8, cols=64)

@@ -112,6 +112,11 @@ def test_quantize_mxfp8_bit_exact():
     x[7, :64] = 0.0
     x[7, 64:96] = np.float32(448.0)  # amax / 448 is an exact power of two
     x[7, 96:128] = np.float32(0.875)
+    # mk_dev_quantize_mxfp8 keeps the reference's clamp of the scale exponent at 8 (src/deepseek.rs:316): a block above
+    # 448 * 2^8 gets byte 8 + 127 and its large values saturate at code 0x7E / 0xFE
+    x[7, 128:160] = np.linspace(-4.0e5, 4.0e5, 32, dtype=np.float32)
+    x[7, 160:192] = np.float32(448.0 * 256.0)   # exactly at the limit: exponent 8, no saturation
+    x[7, 192:224] = np.float32(448.0 * 256.0 * 1.001)
     # every e4m3 value, every midpoint between neighbours (ties) and their float neighbours, in blocks whose scale
     # is 1 (a 448 in each block) and in blocks scaled by 2^-3
     grid = np.array([oracle.e4m3_to_f32(c) for c in range(0x7F)], np.float32)  # 0 .. 448 ascending
@@ -135,6 +140,8 @@ def test_quantize_mxfp8_bit_exact():
         _, c, e = oracle.fp8_roundtrip(x[r], 32)
         assert np.array_equal(exps[r], e), r
         assert np.array_equal(codes[r], c), r
+    assert exps[7, 4] == exps[7, 5] == exps[7, 6] == 8 + 127
+    assert (codes[7, 128:138] == 0xFE).all() and (codes[7, 150:160] == 0x7E).all() and (codes[7, 160:224] == 0x7E).all()
 
 
 def _quantizer_inputs(rows, cols, seed):

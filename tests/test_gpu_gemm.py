@@ -101,7 +101,7 @@ def test_moe_prefill_on_device(T, topk, n_experts, d, inter, act):
     want = oracle.moe_prefill(table, ids, wts, x, act_kind=kind, round_mxfp8=2)
     pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
     experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
-    got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x),
+    got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x), mxfp8=True,
                             act_kind=model.ACT_SITU if act == "situ" else model.ACT_SWIGLU).cpu().numpy()
     assert np.all(np.isfinite(got))
     assert rel_l2(got, want) <= 2e-3
@@ -256,6 +256,38 @@ def test_moe_prefill_f32_random_shapes():
         assert np.isfinite(got).all() and err <= 1e-5, (case, T, topk, n_experts, d, inter, act, err)
 
 
+def test_moe_prefill_wrapper_splits_a_prompt_of_more_than_16384_pairs():
+    # one C call takes at most 16384 (token, slot) pairs; the wrapper cuts a longer prompt into calls of whole tokens.
+    # Tokens are independent, so the pieces are the rows of the separate calls, and a sample of rows is held to the oracle.
+    from microkimi_amd import model, workloads
+    from microkimi_amd._lib import MkError
+    rng = np.random.default_rng(77)
+    n_experts, topk, T, d, inter = 8, 8, 2100, 128, 128     # 16800 pairs: calls of 2048 and 52 tokens
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.int32)
+    wts = rng.random((T, topk)).astype(np.float32)
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    from microkimi_amd._lib import cur_stream, lib, ptr
+    import ctypes as C
+    import torch
+    ws = torch.empty(lib.mk_moe_prefill_workspace_bytes(T, topk, n_experts, d, inter), dtype=torch.uint8, device="cuda")
+    out = torch.empty((T, d), device="cuda")
+    st = lib.mk_dev_moe_prefill_f32(C.byref(experts.table), n_experts, T, topk, ptr(dev(ids)), ptr(dev(wts)), ptr(dev(x)), 0, ptr(ws), ptr(out),
+                                    cur_stream())
+    assert st == -1 and b"16384" in lib.mk_last_error()      # the C call itself refuses
+    got = model.moe_prefill(experts, dev(ids), dev(wts), dev(x)).cpu().numpy()
+    a = model.moe_prefill(experts, dev(ids[:2048]), dev(wts[:2048]), dev(x[:2048])).cpu().numpy()
+    b = model.moe_prefill(experts, dev(ids[2048:]), dev(wts[2048:]), dev(x[2048:])).cpu().numpy()
+    assert np.array_equal(got[:2048], a) and np.array_equal(got[2048:], b)
+    table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+    rows = np.array([0, 1, 2047, 2048, 2049, 2099])
+    want = oracle.moe_prefill(table, ids[rows].astype(np.uint32), wts[rows], x[rows], round_mxfp8=False)
+    assert rel_l2(got[rows], want) <= 1e-5
+
+
 @pytest.mark.parametrize("arith", ["mxfp8", "f32", "bf16"])
 def test_moe_prefill_skips_ids_out_of_range(arith):
     # a pair whose expert id lies outside the table adds nothing to its token (include/mk_hip.h): the result equals the
@@ -280,7 +312,7 @@ def test_moe_prefill_skips_ids_out_of_range(arith):
     want = oracle.moe_prefill(table, ref_ids.astype(np.uint32), ref_wts, x, round_mxfp8={"f32": False, "mxfp8": 2, "bf16": 3}[arith])
     pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
     experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
-    got = model.moe_prefill(experts, dev(dev_ids), dev(wts), dev(x), exact=exact, bf16=arith == "bf16").cpu().numpy()
+    got = model.moe_prefill(experts, dev(dev_ids), dev(wts), dev(x), exact=exact, bf16=arith == "bf16", mxfp8=arith == "mxfp8").cpu().numpy()
     assert np.all(np.isfinite(got)) and not got[7].any()
     assert rel_l2(got, want) <= {"f32": 1e-5, "mxfp8": 2e-3, "bf16": 3e-4}[arith]
 
@@ -329,7 +361,7 @@ def test_moe_prefill_f32_with_vq1_experts(T, topk, d, inter, act):
     want_u = oracle.vq1_matvec_nt(codebook, host[e][2], inter, d, xt, m8)[:len(toks)]
     assert len(toks) > 0 and rel_l2(mid["u"][r0:r1], want_u) <= 1e-5
     with pytest.raises(Exception):
-        model.moe_prefill(experts, dev(ids), dev(wts), dev(x), act_kind=act)
+        model.moe_prefill(experts, dev(ids), dev(wts), dev(x), act_kind=act, mxfp8=True)
 
 
 def test_config4_full_size_expert_section():
@@ -366,8 +398,8 @@ def test_config4_full_size_expert_section():
     logits, x = W.config4_tokens()
     T = x.shape[0]
     ids, wts = model.router_softmax_topk(dev(logits), topk)
-    plain = model.moe_prefill(experts, ids, wts, dev(x)).cpu().numpy()
-    got = model.moe_prefill(experts, ids, wts, dev(x), keep=True).cpu().numpy()   # the same kernels, gate / up rows stored as well
+    plain = model.moe_prefill(experts, ids, wts, dev(x), mxfp8=True).cpu().numpy()
+    got = model.moe_prefill(experts, ids, wts, dev(x), mxfp8=True, keep=True).cpu().numpy()   # the same kernels, gate / up rows stored as well
     assert np.isfinite(got).all() and np.array_equal(plain.view(np.uint32), got.view(np.uint32))
     mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}
     ids_h, wts_h = ids.cpu().numpy(), wts.cpu().numpy()

@@ -130,6 +130,28 @@ def test_matvec_packed_nt(rows, cols, m):
     assert rel_l2(got, want) <= TOL
 
 
+@pytest.mark.parametrize("rows,cols,m", [(64, 512, 1), (40, 7168, 3), (33, 64, 2)])
+def test_nt_vector_path_and_f32_matvec_give_the_same_bits(rows, cols, m):
+    # matvec_packed_nt (src/model.rs:2412-2447) and the f32 branch of matvec_packed (src/mxfp4.rs:475-539) are the same
+    # sum in the reference (the oracle's two restatements agree bit for bit, checked here too); on the device the
+    # up-to-3-positions path of mk_dev_mxfp4_matvec_nt and mk_dev_mxfp4_matvec_f32 are two kernels: same bits
+    torch = torch_cuda()
+    from microkimi_amd import model
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    p, s, _ = quantized_case(rows, cols)
+    x = oracle.pattern(7, cols * m).reshape(m, cols)
+    got = model.matvec_packed_nt(dev(p), dev(s), rows, cols, dev(x), m).cpu().numpy()
+    dp, ds = dev(p), dev(s)
+    xt = np.zeros((cols, 8), np.float32)
+    xt[:, :m] = x.T
+    want_nt = oracle.matvec_packed_nt(p, s, rows, cols, xt, 8)[:m]
+    for j in range(m):
+        out = torch.empty(rows, device="cuda")
+        check(lib.mk_dev_mxfp4_matvec_f32(ptr(dp), ptr(ds), rows, cols, ptr(dev(x[j])), ptr(out), cur_stream()))
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), got[j].view(np.uint32)), j
+        assert np.array_equal(oracle.matvec_packed(p, s, rows, cols, x[j], mode=0).view(np.uint32), want_nt[j].view(np.uint32)), j
+
+
 @pytest.mark.parametrize("sb,m", [(0, 16), (1, 16), (2, 16), (1, 3), (250, 16), (1, 600)])
 def test_matvec_packed_nt_extreme_scale_bytes(sb, m):
     # scale bytes 0..2 make every weight a subnormal or the smallest normals (byte 0 is 2^-127, src/mxfp4.rs:340-346),

@@ -27,6 +27,31 @@ def test_matvec_packed_host_slices_and_weight_cache():
     assert rel_l2(out, oracle.matvec_packed(p, s, 512, 7168, x, mode=1)) <= 1e-5
 
 
+def test_weight_cache_budget_is_an_error_not_an_eviction():
+    # MICROKIMI_GPU_CACHE_MB (src/metal.rs:554-558): a weight that does not fit the budget is not uploaded; the call fails
+    # with MK_ERR_NOMEM and a message, leaves `out` alone, and works once the budget is raised
+    torch_cuda()
+    from microkimi_amd import workloads
+    from microkimi_amd._lib import check, hptr, lib
+    rows, cols = 2048, 2048                       # 2 MiB of nibbles + 128 KiB of scale bytes
+    p, s, x = workloads.config0(rows=rows, cols=cols)
+    out = np.full(rows, 7.0, np.float32)
+    lib.mk_set_cache_mb(1)
+    try:
+        st = lib.mk_mxfp4_matvec(hptr(p), hptr(s), rows, cols, hptr(x), hptr(out))
+        assert st == -5 and b"budget exhausted" in lib.mk_last_error()
+        assert np.all(out == 7.0)
+        lib.mk_set_cache_mb(1 << 20)
+        check(lib.mk_mxfp4_matvec(hptr(p), hptr(s), rows, cols, hptr(x), hptr(out)))
+        assert rel_l2(out, oracle.matvec_packed(p, s, rows, cols, x, mode=1)) <= 1e-5
+        lib.mk_set_cache_mb(1)                    # a cached weight stays usable under a budget that is lowered afterwards
+        out2 = np.zeros(rows, np.float32)
+        check(lib.mk_mxfp4_matvec(hptr(p), hptr(s), rows, cols, hptr(x), hptr(out2)))
+        assert np.array_equal(out, out2)
+    finally:
+        lib.mk_set_cache_mb(0)
+
+
 def test_q8head_host_api():
     torch_cuda()
     from microkimi_amd import _lib

@@ -81,6 +81,33 @@ def test_decode_matches_mla_attn_flash_q8_mqa(n, nh, nope, rope, vd, qscale):
         assert rel_l2(got, want) <= TOL, (pos, rel_l2(got, want))
 
 
+def test_decode_at_the_published_shape_16384_positions_96_heads():
+    # the shape the reference's own figure is quoted on (96 heads, 128 + 64 / 128, 16k positions), at full size against the
+    # oracle: the cache is filled in chunks of 2048 positions on both sides
+    from microkimi_amd import model
+    n, nh, nope, rope, vd = 16384, 96, 128, 64, 128
+    rng = np.random.default_rng(16384)
+    want_c = oracle.MlaCache(nh, nope, rope, vd, capacity=n)
+    c = model.MlaHeadsCache(nh, nope, rope, vd, n)
+    for j0 in range(0, n, 2048):
+        k = rng.standard_normal((2048, nh * (nope + rope)), dtype=np.float32)
+        v = rng.standard_normal((2048, nh * vd), dtype=np.float32)
+        c.push(dev(k), dev(v))
+        for j in range(2048):
+            want_c.push(k[j], v[j])
+    assert c.positions() == n == want_c.n
+    assert np.array_equal(c.kq[n - 3:n].cpu().numpy(), want_c.kq[n - 3:n]) and np.array_equal(c.vq[n - 3:n].cpu().numpy(), want_c.vq[n - 3:n])
+    q = rng.standard_normal(nh * (nope + rope), dtype=np.float32) * np.float32(2.0)   # scores a few units apart: not a flat softmax
+    scale = float(np.float32(nope + rope) ** np.float32(-0.5))
+    for pos in (n - 1, 9001):
+        got = c.attn(dev(q), pos, scale).cpu().numpy()[0]
+        want = oracle.mla_attn_flash_q8_mqa(want_c, q, pos, scale)
+        assert np.isfinite(got).all()
+        assert rel_l2(got, want) <= TOL, (pos, rel_l2(got, want))
+        per_head = [rel_l2(got[h * vd:(h + 1) * vd], want[h * vd:(h + 1) * vd]) for h in range(nh)]
+        assert max(per_head) <= TOL, (pos, int(np.argmax(per_head)), max(per_head))
+
+
 @pytest.mark.parametrize("nh,n0,m,had", [(8, 300, 70, False), (3, 0, 40, False), (16, 1000, 16, True), (4, 17, 130, False)])
 def test_prefill_on_the_matrix_cores(nh, n0, m, had):
     # 16 and more queries at the reference's head shape share the K / V tiles on the matrix cores: every query against

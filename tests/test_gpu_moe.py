@@ -482,3 +482,16 @@ def test_layer_with_vq1_experts(d, inter, B, topk, shared, act, mode):
     act_rows = model.moe_decode_act(experts, dev(ids), dev(wts), dev(x), shared=shared, mode=mode, act_kind=act, limit=limit)
     again = model.moe_decode_from_act(experts, dev(ids), dev(wts), act_rows, shared=shared, mode=mode, act_kind=act).cpu().numpy()
     assert np.array_equal(again.view(np.uint32), got.view(np.uint32))
+
+
+def test_count_of_routed_ids_outside_the_table():
+    torch = torch_cuda()
+    from microkimi_amd._lib import check, cur_stream, lib, ptr
+    rng = np.random.default_rng(5)
+    for n, n_experts in [(1, 1), (8, 384), (700, 64), (16384, 384)]:
+        ids = rng.integers(0, n_experts, n).astype(np.int32)
+        bad = rng.random(n) < 0.1
+        ids[bad] = np.where(rng.random(int(bad.sum())) < 0.5, -1 - rng.integers(0, 5, int(bad.sum())), n_experts + rng.integers(0, 5, int(bad.sum())))
+        count = torch.full((1,), -7, dtype=torch.int32, device="cuda")
+        check(lib.mk_dev_moe_count_bad_ids(ptr(dev(ids)), n, n_experts, ptr(count), cur_stream()))
+        assert int(count.item()) == int(bad.sum())

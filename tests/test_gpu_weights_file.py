@@ -96,7 +96,7 @@ def test_layer_with_vq1_experts_from_a_file(tmp_path):
         assert rel_l2(got[t], want[t]) <= 1e-5
     from microkimi_amd._lib import MkError
     with pytest.raises(MkError) as e:   # the prefill call reads MXFP4 experts only
-        model.moe_prefill(ex, dev(ids), dev(wts), dev(x))
+        model.moe_prefill(ex, dev(ids), dev(wts), dev(x), mxfp8=True)
     assert e.value.status == -4
     ex.close()
     f.close()

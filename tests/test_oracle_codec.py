@@ -94,6 +94,43 @@ def test_fp8_roundtrip_block32():
         assert np.abs(y[b * 32:(b + 1) * 32] - blk).max() <= np.abs(blk).max() * 2.0 ** -4 + 1e-6
 
 
+def test_fp8_roundtrip_scale_clamp():
+    # a block whose largest value exceeds 448 * 2^8: with the reference's clamp (src/deepseek.rs:316) the scale stops at
+    # 2^8 and the values saturate at +-448 * 2^8; with the full e8m0 range the block keeps its relative precision
+    x = np.zeros(64, np.float32)
+    x[:32] = np.linspace(-4.0e5, 4.0e5, 32, dtype=np.float32)      # 4e5 > 448 * 256 = 114688
+    x[32:] = np.linspace(-1.0e5, 1.0e5, 32, dtype=np.float32)      # below the limit: both forms agree
+    y8, c8, e8 = oracle.fp8_roundtrip(x, 32, emax=8)
+    yf, cf, ef = oracle.fp8_roundtrip(x, 32, emax=127)
+    assert e8[0] == 8 + 127 and ef[0] == int(np.ceil(np.log2(4.0e5 / 448.0))) + 127 == 10 + 127
+    assert np.abs(y8[:32]).max() == 448.0 * 256.0
+    sat = np.abs(x[:32]) >= 448.0 * 256.0
+    assert sat.sum() >= 10 and np.array_equal(y8[:32][sat], np.sign(x[:32][sat]) * np.float32(448.0 * 256.0))
+    assert np.abs(yf[:32] - x[:32]).max() <= 4.0e5 * 2.0 ** -4
+    assert e8[1] == ef[1] and np.array_equal(y8[32:], yf[32:]) and np.array_equal(c8[32:], cf[32:])
+    # the lower clamp is the same in both: an all-zero block takes amax = 1e-4
+    z8, _, ez8 = oracle.fp8_roundtrip(np.zeros(32, np.float32), 32, emax=8)
+    zf, _, ezf = oracle.fp8_roundtrip(np.zeros(32, np.float32), 32, emax=127)
+    assert ez8[0] == ezf[0] == int(np.ceil(np.log2(1e-4 / 448.0))) + 127 and not z8.any() and not zf.any()
+
+
+def test_round_bf16_is_torch_bfloat16():
+    import torch
+    rng = np.random.default_rng(11)
+    bits = rng.integers(0, 2 ** 32, 200000, dtype=np.uint64).astype(np.uint32)
+    # ties (low half exactly 0x8000) with even and odd upper halves, values next to them, the largest finite
+    # numbers (which round up to infinity), subnormals, zeros, infinities
+    special = np.array([0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001, 0xBF808000, 0xBF818000, 0x7F7FFFFF, 0x7F7F8000, 0x7F7F7FFF,
+                        0xFF7FFFFF, 0x00008000, 0x00018000, 0x00007FFF, 0x80008000, 0, 0x80000000, 0x7F800000, 0xFF800000], np.uint32)
+    x = np.concatenate([bits, special]).view(np.float32)
+    x = x[~np.isnan(x)]
+    got = oracle.round_bf16(x)
+    want = torch.from_numpy(x.copy()).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    nan = oracle.round_bf16(np.array([np.nan], np.float32))
+    assert np.isnan(nan[0])
+
+
 def _block_errors(w, rows, cols, p, s):
     wq = oracle.mxfp4_dequant(p, s, rows, cols).astype(np.float64).reshape(-1, 32)
     return ((w.astype(np.float64).reshape(-1, 32) - wq) ** 2).sum(axis=1)

@@ -1,7 +1,7 @@
 """The entry point that allocates nothing (mk_dev_mla_q8_decode_static: scratch in a device array inside the library)
 against mk_dev_mla_q8_decode with a caller's workspace, through the C ABI: two calls in a row, the second on a smaller
 input, each within relative L2 1e-5 of the existing entry point (the same kernels run, so the outputs are in fact equal
-bit for bit), plus the size limit.  Collected last: it must pass alone in a fresh process and after all other tests."""
+bit for bit) and, on the smaller inputs, of the CPU oracle, plus the size limit.  Collected last: it must pass alone in a fresh process and after all other tests."""
 import ctypes as C
 
 import numpy as np
@@ -12,7 +12,7 @@ from gpu_util import dev, rel_l2, torch_cuda
 pytestmark = pytest.mark.gpu
 
 
-def run_both(ctx, nh, seed):
+def run_both(ctx, nh, seed, oracle_check=False):
     torch = torch_cuda()
     from microkimi_amd import _lib, workloads
     from microkimi_amd._lib import check, cur_stream, lib, ptr
@@ -31,15 +31,22 @@ def run_both(ctx, nh, seed):
     check(lib.mk_dev_mla_q8_decode_static(ptr(lq), ptr(ls), ptr(rq), ptr(rs), ctx - 1, ptr(q), nh, L, R, workloads.MLA_SCALE, ptr(got),
                                           cur_stream()))
     torch.cuda.synchronize()
+    if oracle_check:
+        # the existing entry point is itself held to the CPU restatement here, so that a mistake shared by both
+        # entry points (they run the same kernels) cannot pass
+        import oracle
+        ref = oracle.mla_absorbed_decode(lq.cpu().numpy(), ls.cpu().numpy().astype(np.float32), rq.cpu().numpy(),
+                                         rs.cpu().numpy().astype(np.float32), q.cpu().numpy(), nh, workloads.MLA_SCALE)
+        assert rel_l2(got.cpu().numpy(), ref) <= 1e-5
     return got.cpu().numpy(), want.cpu().numpy()
 
 
 def test_static_scratch_entry_point_two_calls_second_smaller():
     got, want = run_both(5000, 128, 1)   # many splits: partial outputs and statistics go through the scratch
     assert np.isfinite(got).all() and rel_l2(got, want) <= 1e-5
-    got2, want2 = run_both(300, 20, 2)   # smaller: fewer splits, fewer heads; the scratch still holds the first call's data
+    got2, want2 = run_both(300, 20, 2, oracle_check=True)   # smaller: fewer splits, fewer heads; the scratch still holds the first call's data
     assert np.isfinite(got2).all() and rel_l2(got2, want2) <= 1e-5
-    got3, want3 = run_both(40, 3, 3)     # a single split: no merge
+    got3, want3 = run_both(40, 3, 3, oracle_check=True)     # a single split: no merge
     assert np.isfinite(got3).all() and rel_l2(got3, want3) <= 1e-5
 
 
