@@ -284,8 +284,22 @@ struct M4 {
     static constexpr int LDS_BYTES = ST_OFF + (4 * HEADS + 4 * HEADS + 3 * HEADS) * 4;  // wmax, wsum, corr, final m, final l
 };
 
+// -DMK_MLA_TRACE: wave 0 of every workgroup leaves time stamps (100 MHz) of the last launch, read with mk_debug_mla_ts:
+// 0 start, 1 queries and first tile staged, 2 first tile's scores, 3 its probabilities, 4 its output product, 5 all tiles
+// done, 6 end
+#ifdef MK_MLA_TRACE
+__device__ unsigned long long g_mla_ts[1024 * 8];
+#define MLA_TS(i) ts[i] = __builtin_amdgcn_s_memrealtime()
+#else
+#define MLA_TS(i)
+#endif
+
 __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__restrict__ out) {
     using C4 = M4;
+#ifdef MK_MLA_TRACE
+    unsigned long long ts[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    MLA_TS(0);
     constexpr int HEADS = C4::HEADS;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -409,10 +423,11 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
     const mk_i4 zero4 = {0, 0, 0, 0};
     stage_store(st);
     __syncthreads();
+    MLA_TS(1);
 
     for (int tile = 0; tile < ntiles; tile++) {
         const int t0 = p_begin + tile * TJ;
-        const int t_next = min(t0 + TJ, last_pos);  // clamped: the last iteration's fetch is not used
+        const int t_next = min(t0 + TJ, last_pos);
         // The lane index is made opaque once per tile: every LDS address below is then recomputed from it inside the
         // loop (a few instructions each) instead of being kept in a register of its own across the whole kernel.
         int lane_v = lane;
@@ -512,7 +527,11 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
         __builtin_amdgcn_sched_barrier(0);
         // the next tile's loads go out behind the score stage (whose registers they would otherwise share); the softmax
         // exchange and the output product cover their latency
-        stage_load(st, t_next);
+#ifdef MK_MLA_TRACE
+        if (tile == 0) MLA_TS(2);
+#endif
+        const bool more = tile + 1 < ntiles;  // the last tile fetches nothing and leaves the buffer as it is
+        stage_load(st, t_next);  // (clamped to the last position; the last tile's fetch is never waited for)
         __builtin_amdgcn_sched_barrier(0);
         // ---- online softmax: one reference point per head and tile for all four waves
 #pragma unroll
@@ -553,6 +572,9 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
             l[hg] += (wsum_l[hl] + wsum_l[HEADS + hl]) + (wsum_l[2 * HEADS + hl] + wsum_l[3 * HEADS + hl]);
         }
         __builtin_amdgcn_sched_barrier(0);
+#ifdef MK_MLA_TRACE
+        if (tile == 0) MLA_TS(3);
+#endif
         // ---- out[heads][dims 128 wave ..] += P V over the tile's 64 positions
 #pragma unroll
         for (int hg = 0; hg < NHG; hg++) {
@@ -631,10 +653,16 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
             __builtin_amdgcn_sched_barrier(0);
         }
         // ---- refill the tile buffer: everybody is done reading it, then the prefetched rows go in
-        mk_lds_barrier();
-        stage_store(st);
-        mk_lds_barrier();
+#ifdef MK_MLA_TRACE
+        if (tile == 0) MLA_TS(4);
+#endif
+        if (more) {
+            mk_lds_barrier();
+            stage_store(st);
+            mk_lds_barrier();
+        }
     }
+    MLA_TS(5);
 
     // ---- store: the split's partial [HEADS][512] block, or the normalised rows when there is one split
     {
@@ -671,7 +699,21 @@ __global__ __launch_bounds__(256, 2) void mla_mfma_kernel(MlaArgs a, float *__re
             a.pl[split * a.nh + hbase + tid] = finl_l[tid];
         }
     }
+#ifdef MK_MLA_TRACE
+    MLA_TS(6);
+    if (tid == 0 && blockIdx.y * gridDim.x + blockIdx.x < 1024)
+        for (int i = 0; i < 8; i++) g_mla_ts[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + i] = ts[i];
+#endif
 }
+
+#ifdef MK_MLA_TRACE
+}  // namespace
+extern "C" int mk_debug_mla_ts(unsigned long long *out) {
+    MK_HIP_TRY(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mla_ts), sizeof(unsigned long long) * 1024 * 8));
+    return MK_OK;
+}
+namespace {
+#endif
 
 // log-sum-exp merge of the splits.  A workgroup per (head, quarter of the output dims): thread (d4, part) sums
 // every 8th split for 4 output dims with all its loads in flight at once, the eight parts meet in LDS.
