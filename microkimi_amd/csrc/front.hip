@@ -14,8 +14,10 @@
 // add (never fused), reduction ((p01 + p23) + p45) + p67, remainder sequential.
 // It is replayed here operation for operation -- lane j of a group of 8 lanes
 // owns accumulator j -- so rmsnorm outputs and router logits are the reference's
-// values bit for bit; the price is a sequential chain of cols/8 additions per
-// lane, which is fine for the small matrices this is meant for.
+// values bit for bit.  The price is a sequential chain of cols/8 additions per
+// lane; only the additions are sequential, so the other threads of the workgroup
+// form the products and lay them out in LDS in the order a chain consumes them
+// (chain-major, 16 bytes a read): a chain then runs at the latency of an add.
 #include "mk_common.h"
 
 namespace {
@@ -30,25 +32,101 @@ __device__ __forceinline__ float dot8_reduce(float acc) {
     return s;
 }
 
+// acc + p[0] + p[1] + ... + p[n-1], one addition after the other.  p: LDS, 16-byte aligned.  Batches of 32 values: the
+// next batch is requested before the current one is added (the scheduling barriers keep that order; left alone, the
+// compiler moves the requests down to their first use and every batch then waits for the whole LDS latency).
+struct ChainBatch {
+    mk_f4 v[8];
+};
+__device__ __forceinline__ void chain_load(ChainBatch &c, const mk_f4 *p4) {
+#pragma unroll
+    for (int k = 0; k < 8; k++) c.v[k] = p4[k];
+}
+__device__ __forceinline__ float chain_sum32(float acc, const ChainBatch &c) {
+#pragma unroll
+    for (int k = 0; k < 8; k++) acc = mk_add(mk_add(mk_add(mk_add(acc, c.v[k].x), c.v[k].y), c.v[k].z), c.v[k].w);
+    return acc;
+}
+__device__ __forceinline__ float chain_add(float acc, const float *p, int n) {
+    const mk_f4 *p4 = reinterpret_cast<const mk_f4 *>(p);
+    const int n32 = n >> 5;
+    if (n32 > 0) {
+        ChainBatch a, b;
+        chain_load(a, p4);
+        for (int i = 0; i < n32; i += 2) {
+            chain_load(b, p4 + 8 * min(i + 1, n32 - 1));  // (past the end: the last batch once more, unused)
+            __builtin_amdgcn_sched_barrier(0);
+            acc = chain_sum32(acc, a);
+            __builtin_amdgcn_sched_barrier(0);
+            chain_load(a, p4 + 8 * min(i + 2, n32 - 1));
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 1 < n32) acc = chain_sum32(acc, b);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    int i = n32 * 32;
+    for (; i + 4 <= n; i += 4) {
+        const mk_f4 v = p4[i >> 2];
+        acc = mk_add(mk_add(mk_add(mk_add(acc, v.x), v.y), v.z), v.w);
+    }
+    for (; i < n; i++) acc = mk_add(acc, p[i]);
+    return acc;
+}
+// floats between two chains' rows in LDS for `steps` values a chain: a multiple of 4 that is 4 modulo 64, so that the 16
+// lanes of one pass of a 16-byte read fall into 16 different groups of four banks
+__host__ __device__ constexpr int chain_stride(int steps) { return ((steps + 63) & ~63) + 4; }
+
 // One workgroup per row.  The row is staged in LDS; lanes 0..7 of wave 0 replay dot(x, x); then every
 // thread scales 8 consecutive values (x * inv * w, two multiplications in that order) and, when asked,
 // a quad of lanes quantizes its 32-block to q8.
+// prod_off: float offset of the chain-major squares inside the LDS block (8 rows of chain_stride(d / 8)), or 0 when the
+// block has no room for them (then the chain lanes square the staged values themselves).  w_off: float offset of a copy
+// of w that the waves without a chain fetch while the chain runs, or 0 (then the last loop reads w from memory).
+// Loads go out eight at a time per thread: a loop of one load and one store per trip pays a memory latency per trip.
 __global__ __launch_bounds__(256) void rmsnorm_q8_kernel(const float *__restrict__ x, int d, const float *__restrict__ w, float eps,
-                                                         float *__restrict__ out, int8_t *__restrict__ q, float *__restrict__ scales) {
+                                                         float *__restrict__ out, int8_t *__restrict__ q, float *__restrict__ scales, int prod_off,
+                                                         int w_off) {
     extern __shared__ __attribute__((aligned(16))) float xl[];  // [d], then inv
     const int t = blockIdx.x, tid = threadIdx.x;
     const float *row = x + (size_t)t * d;
-    for (int i = tid; i < d / 4; i += 256) reinterpret_cast<mk_f4 *>(xl)[i] = reinterpret_cast<const mk_f4 *>(row)[i];
+    const int chunks = d / 8, stride = chain_stride(chunks), n4 = d / 4;
+    float *prod = xl + prod_off;
+    for (int base = 0; base < n4; base += 256 * 8) {
+        mk_f4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int i = base + 256 * k + tid;
+            v[k] = reinterpret_cast<const mk_f4 *>(row)[min(i, n4 - 1)];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int i = base + 256 * k + tid;
+            if (i < n4) {
+                reinterpret_cast<mk_f4 *>(xl)[i] = v[k];
+                if (prod_off && (i >> 1) < chunks) {  // values 4 i .. 4 i + 3: accumulators 4 (i % 2) .. + 3 of chunk i / 2
+                    float *dst = prod + (4 * (i & 1)) * stride + (i >> 1);
+                    dst[0] = mk_mul(v[k].x, v[k].x);
+                    dst[stride] = mk_mul(v[k].y, v[k].y);
+                    dst[2 * stride] = mk_mul(v[k].z, v[k].z);
+                    dst[3 * stride] = mk_mul(v[k].w, v[k].w);
+                }
+            }
+        }
+    }
     for (int i = (d & ~3) + tid; i < d; i += 256) xl[i] = row[i];
     __syncthreads();
     if (tid < 64) {
         float acc = 0.0f;
-        const int j = tid & 7, chunks = d / 8;
+        const int j = tid & 7;
         if (tid < 8) {
+            if (prod_off) {
+                acc = chain_add(acc, prod + j * stride, chunks);
+            } else {
 #pragma unroll 8
-            for (int i = 0; i < chunks; i++) {
-                const float v = xl[i * 8 + j];
-                acc = mk_add(acc, mk_mul(v, v));
+                for (int i = 0; i < chunks; i++) {
+                    const float v = xl[i * 8 + j];
+                    acc = mk_add(acc, mk_mul(v, v));
+                }
             }
         }
         float s = dot8_reduce(acc);
@@ -60,20 +138,49 @@ __global__ __launch_bounds__(256) void rmsnorm_q8_kernel(const float *__restrict
             const float rt = (float)sqrt((double)mk_add(ss, eps));
             xl[d] = (float)(1.0 / (double)rt);
         }
+    } else if (w_off) {  // d % 4 == 0 here
+        float *wl = xl + w_off;
+        for (int base = 0; base < n4; base += 192 * 8) {
+            mk_f4 v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) v[k] = reinterpret_cast<const mk_f4 *>(w)[min(base + 192 * k + tid - 64, n4 - 1)];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int i = base + 192 * k + tid - 64;
+                if (i < n4) reinterpret_cast<mk_f4 *>(wl)[i] = v[k];
+            }
+        }
     }
     __syncthreads();
     const float inv = xl[d];
+    // 16-byte pieces when the row is whole groups of 8 and the output rows are aligned (w_off implies an aligned w)
+    const bool vec = d % 8 == 0 && w_off != 0 && (!out || ((uintptr_t)out & 15) == 0);
     for (int g = tid; g < (d + 7) / 8; g += 256) {  // 8 values per lane; a q8 block is a quad of lanes
         float v[8];
+        if (vec) {
+            const mk_f4 a0 = reinterpret_cast<const mk_f4 *>(xl)[2 * g], a1 = reinterpret_cast<const mk_f4 *>(xl)[2 * g + 1];
+            const mk_f4 w0 = reinterpret_cast<const mk_f4 *>(xl + w_off)[2 * g], w1 = reinterpret_cast<const mk_f4 *>(xl + w_off)[2 * g + 1];
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int i = g * 8 + k;
-            v[k] = i < d ? mk_mul(mk_mul(xl[i], inv), w[i]) : 0.0f;
-        }
-        if (out) {
+            for (int k = 0; k < 4; k++) {
+                v[k] = mk_mul(mk_mul(a0[k], inv), w0[k]);
+                v[4 + k] = mk_mul(mk_mul(a1[k], inv), w1[k]);
+            }
+            if (out) {
+                mk_f4 *dst = reinterpret_cast<mk_f4 *>(out + (size_t)t * d) + 2 * g;
+                dst[0] = mk_f4{v[0], v[1], v[2], v[3]};
+                dst[1] = mk_f4{v[4], v[5], v[6], v[7]};
+            }
+        } else {
 #pragma unroll
-            for (int k = 0; k < 8; k++)
-                if (g * 8 + k < d) out[(size_t)t * d + g * 8 + k] = v[k];
+            for (int k = 0; k < 8; k++) {
+                const int i = g * 8 + k;
+                v[k] = i < d ? mk_mul(mk_mul(xl[i], inv), w_off ? xl[w_off + i] : w[i]) : 0.0f;
+            }
+            if (out) {
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    if (g * 8 + k < d) out[(size_t)t * d + g * 8 + k] = v[k];
+            }
         }
         if (q) {  // d % 32 == 0 is checked by the host in this case
             float a = 0.0f;
@@ -111,6 +218,73 @@ __global__ __launch_bounds__(256) void matvec_f32_kernel(const float *__restrict
     if (j == 0 && r < rows) {
         for (int i = chunks * 8; i < cols; i++) s = mk_add(s, mk_mul(wr[i], xb[i]));
         out[(size_t)b * rows + r] = s;
+    }
+}
+
+// The same product with the chains fed from LDS: a workgroup per weight row and group of up to 4 tokens.  Waves 1-3 form
+// the products w[r][c] * x[t][c] of a segment of 2048 columns and store them chain-major (chain = (token, accumulator),
+// chain_stride(256) floats a chain); wave 0's lane 8 t + j adds chain (t, j) of the segment before, one addition after
+// the other.  Two segment buffers, one barrier a segment; a producer has all its loads of a segment in flight at once.
+// Needs cols % 4 == 0 and 16-byte aligned w and x.
+constexpr int MV_SEG = 2048, MV_STEPS = MV_SEG / 8, MV_STRIDE = chain_stride(MV_STEPS), MV_TB = 4, MV_NG = (MV_SEG / 4 + 191) / 192;
+__global__ __launch_bounds__(256) void matvec_f32_chain_kernel(const float *__restrict__ w, int rows, int cols, const float *__restrict__ x, int B,
+                                                               float *__restrict__ out, int tb_max) {
+    extern __shared__ __attribute__((aligned(16))) float mv_lds[];  // [2][8 tb_max][MV_STRIDE]
+    const int r = blockIdx.x, b0 = blockIdx.y * MV_TB, tb = min(MV_TB, B - b0);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int chunks = cols / 8, chain_cols = chunks * 8, nseg = (chain_cols + MV_SEG - 1) / MV_SEG;
+    const int buf_floats = 8 * tb_max * MV_STRIDE;
+    const float *wr = w + (size_t)r * cols, *xb = x + (size_t)b0 * cols;
+
+    auto produce = [&](int seg) {  // waves 1-3: 192 threads, four columns at a time, up to MV_NG column groups a thread
+        float *buf = mv_lds + (seg & 1) * buf_floats;
+        const int c0 = seg * MV_SEG, c1 = min(c0 + MV_SEG, chain_cols);
+        mk_f4 wv[MV_NG], xv[MV_TB][MV_NG];
+#pragma unroll
+        for (int k = 0; k < MV_NG; k++) {
+            const int c = min(c0 + 4 * (tid - 64 + 192 * k), cols - 4);
+            wv[k] = *reinterpret_cast<const mk_f4 *>(wr + c);
+#pragma unroll
+            for (int t = 0; t < MV_TB; t++) xv[t][k] = *reinterpret_cast<const mk_f4 *>(xb + (size_t)min(t, tb - 1) * cols + c);
+        }
+#pragma unroll
+        for (int k = 0; k < MV_NG; k++) {
+            const int c = c0 + 4 * (tid - 64 + 192 * k);
+            if (c < c1) {
+                float *dst = buf + (4 * ((c >> 2) & 1)) * MV_STRIDE + ((c - c0) >> 3);
+#pragma unroll
+                for (int t = 0; t < MV_TB; t++) {
+                    if (t < tb) {
+                        float *dt = dst + 8 * t * MV_STRIDE;
+                        dt[0] = mk_mul(wv[k].x, xv[t][k].x);
+                        dt[MV_STRIDE] = mk_mul(wv[k].y, xv[t][k].y);
+                        dt[2 * MV_STRIDE] = mk_mul(wv[k].z, xv[t][k].z);
+                        dt[3 * MV_STRIDE] = mk_mul(wv[k].w, xv[t][k].w);
+                    }
+                }
+            }
+        }
+    };
+    float acc = 0.0f;
+    if (wave != 0 && nseg > 0) produce(0);
+    __syncthreads();
+    for (int seg = 0; seg < nseg; seg++) {
+        if (wave != 0) {
+            if (seg + 1 < nseg) produce(seg + 1);
+        } else if (lane < 8 * tb) {
+            const int steps = (min((seg + 1) * MV_SEG, chain_cols) - seg * MV_SEG) >> 3;
+            acc = chain_add(acc, mv_lds + (seg & 1) * buf_floats + lane * MV_STRIDE, steps);
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+        float s = dot8_reduce(acc);
+        const int t = lane >> 3;
+        if ((lane & 7) == 0 && t < tb) {
+            const float *xt = xb + (size_t)t * cols;
+            for (int i = chain_cols; i < cols; i++) s = mk_add(s, mk_mul(wr[i], xt[i]));
+            out[(size_t)(b0 + t) * rows + r] = s;
+        }
     }
 }
 
@@ -167,34 +341,43 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict
     __syncthreads();
     float sum = 0.0f, myw = 0.0f;
     int myid = 0;
-    for (int r = 0; r < k; r++) {
-        float bv = -INFINITY;
-        int bi = 0x7FFFFFFF;
+    // A lane keeps the best of its own keys (i = lane, lane + 64, ...: the lowest index among equals); a round takes the
+    // wave's largest key, the lowest index among the lanes that hold it, and only the owner of that key looks through its
+    // keys again.  Keys that are NaN are never larger than anything and are never selected, as before.
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    auto rescan = [&]() {
+        bv = -INFINITY;
+        bi = 0x7FFFFFFF;
         for (int i = lane; i < n; i += 64) {
-            float v = key[i];
-            if (v > bv || (v == bv && i < bi)) {
+            const float v = key[i];
+            if (v > bv) {
                 bv = v;
                 bi = i;
             }
         }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            float ov = __shfl_xor(bv, off, MK_WAVE);
-            int oi = __shfl_xor(bi, off, MK_WAVE);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        const float sc = score[bi];
+        if (bi == 0x7FFFFFFF && lane < n) bi = lane;  // all of them -inf (or NaN): still a valid index, never out of range
+    };
+    rescan();
+    for (int r = 0; r < k; r++) {
+        const float top = mk_wave_max(bv);
+        int cand = bv == top ? bi : 0x7FFFFFFF;
+        cand = min(cand, mk_dpp_i<0xB1>(cand));
+        cand = min(cand, mk_dpp_i<0x4E>(cand));
+        cand = min(cand, mk_dpp_i<0x141>(cand));
+        cand = min(cand, mk_dpp_i<0x140>(cand));
+        const int best = min(min(__builtin_amdgcn_readlane(cand, 0), __builtin_amdgcn_readlane(cand, 16)),
+                             min(__builtin_amdgcn_readlane(cand, 32), __builtin_amdgcn_readlane(cand, 48)));
+        const float sc = score[best];
         if (lane == r) {
             myw = sc;
-            myid = bi;
+            myid = best;
         }
         sum += sc;  // slot order, as the reference sums the selected scores
-        __syncthreads();
-        if (lane == 0) key[bi] = -INFINITY;
-        __syncthreads();
+        if ((best & 63) == lane) {  // the owner: one wave, so its LDS write and reads stay in program order
+            key[best] = -INFINITY;
+            rescan();
+        }
     }
     if (lane < k) {
         ids[t * k + lane] = myid;
@@ -215,16 +398,38 @@ extern "C" int mk_dev_rmsnorm(const float *x, size_t B, size_t d, const float *w
     MK_REQUIRE(d >= 1 && d <= 32768 && B >= 1 && B <= 65535, "bad shape");
     MK_REQUIRE(!q || d % 32 == 0, "q8 blocks are 32 wide");
     MK_REQUIRE(((uintptr_t)x & 15) == 0 && (d % 4 == 0 || B == 1) && (!q || ((uintptr_t)q & 7) == 0), "x must be 16-byte aligned rows");
-    const size_t lds = (d + 4) * sizeof(float);
-    int st = mk_lds_opt_in(reinterpret_cast<const void *>(rmsnorm_q8_kernel), 132 * 1024);
+    size_t lds = (d + 4) * sizeof(float);
+    // the chain-major squares behind the row when both fit (the staging loop forms them from 16-byte pieces: d % 4 == 0)
+    const size_t with_prod = lds + 8 * (size_t)chain_stride((int)(d / 8)) * sizeof(float);
+    int prod_off = 0, w_off = 0;
+    if (d % 4 == 0 && d >= 128 && with_prod <= 150 * 1024) {
+        prod_off = (int)(d + 4);
+        lds = with_prod;
+    }
+    if (d % 4 == 0 && ((uintptr_t)w & 15) == 0 && lds + d * sizeof(float) <= 150 * 1024) {
+        w_off = (int)(lds / sizeof(float));
+        lds += d * sizeof(float);
+    }
+    int st = mk_lds_opt_in(reinterpret_cast<const void *>(rmsnorm_q8_kernel), 150 * 1024);
     if (st != MK_OK) return st;
-    hipLaunchKernelGGL(rmsnorm_q8_kernel, dim3((unsigned)B), dim3(256), lds, (hipStream_t)stream, x, (int)d, w, eps, out, q, scales);
+    hipLaunchKernelGGL(rmsnorm_q8_kernel, dim3((unsigned)B), dim3(256), lds, (hipStream_t)stream, x, (int)d, w, eps, out, q, scales, prod_off, w_off);
     return mk_launch_status("rmsnorm_q8");
 }
 
 extern "C" int mk_dev_matvec_f32(const float *w, size_t rows, size_t cols, const float *x, size_t B, float *out, void *stream) {
     MK_REQUIRE(w && x && out, "null pointer");
     MK_REQUIRE(rows >= 1 && rows <= (1u << 24) && cols >= 1 && cols <= (1u << 24) && B >= 1 && B <= 65535, "bad shape");
+    // rows long enough for the chains to matter, 16-byte pieces: the workgroup-per-row form
+    if (cols >= 512 && cols % 4 == 0 && (((uintptr_t)w | (uintptr_t)x) & 15) == 0 && !MK_TUNE("MK_MATVEC_F32_PLAIN", 0)) {
+        const int tb_max = (int)(B < (size_t)MV_TB ? B : (size_t)MV_TB);
+        const int nbuf = cols / 8 * 8 > (size_t)MV_SEG ? 2 : 1;
+        const size_t lds = (size_t)nbuf * 8 * tb_max * MV_STRIDE * sizeof(float);
+        int st = mk_lds_opt_in(reinterpret_cast<const void *>(matvec_f32_chain_kernel), 140 * 1024);
+        if (st != MK_OK) return st;
+        hipLaunchKernelGGL(matvec_f32_chain_kernel, dim3((unsigned)rows, (unsigned)((B + MV_TB - 1) / MV_TB)), dim3(256), lds, (hipStream_t)stream, w, (int)rows,
+                           (int)cols, x, (int)B, out, tb_max);
+        return mk_launch_status("matvec_f32_chain");
+    }
     hipLaunchKernelGGL(matvec_f32_kernel, dim3((unsigned)((rows * 8 + 255) / 256), (unsigned)B), dim3(256), 0, (hipStream_t)stream, w, (int)rows,
                        (int)cols, x, out);
     return mk_launch_status("matvec_f32");
