@@ -294,8 +294,9 @@ def bench_mxfp4_gemv(torch, cpu=True):
     return {"workload": "64 distinct 2048x7168 MXFP4 matrices, batch 1", "alg_bytes_per_matrix": per, "cpu_port": cpu_port,
             "q8_grouped_launch": {"ms": r_ms, "gbs": gbs(r_ms), "frac": gbs(r_ms) / HBM_PEAK_GBS,
                                   "frac_stream": gbs(r_ms) / HBM_PEAK_GBS, "frac_per_launch": gbs(g_ms) / HBM_PEAK_GBS,
-                                  "timing": "frac_stream: 30 launches back to back between one pair of events, median of 9 (consecutive launches overlap "
-                                            "their ends and starts); frac_per_launch: an event pair around each launch, mean of 30 (carries the events' own cost)",
+                                  "timing": "frac_stream: 30 launches back to back between one pair of events, median of 9 (the kernel plus the gap to the "
+                                            "next launch); frac_per_launch: an event pair around each launch, mean of 30 (carries the events' own cost); "
+                                            "the kernel trace under profiles/ gives the kernel alone",
                                   "ms_with_events_around_each_launch": g_ms},
             "q8_back_to_back": {"ms": s_ms, "gbs": gbs(s_ms), "frac": gbs(s_ms) / HBM_PEAK_GBS, "us_per_gemv": s_ms * 1e3 / nmat},
             "f32_back_to_back": {"ms": f_ms, "gbs": gbs(f_ms), "frac": gbs(f_ms) / HBM_PEAK_GBS}}
