@@ -367,8 +367,8 @@ def bench_moe(torch, cpu=True):
                         "tok_s": B / (ms * 1e-3), "distinct_experts": n_distinct, "pairs": B * (W.TOP_K + 1), "alg_bytes": alg,
                         "gbs": alg / (ms * 1e-3) / 1e9, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "finite": bool(torch.isfinite(out).all().item())}
-        # The layer as a decode step runs it, one graph of four calls per layer: rmsnorm, router gate matvec (256 x 7168 f32),
-        # softmax top-8, expert section.  16 gate matrices stand for 16 layers, so the routing is computed on the device and
+        # The layer as a decode step runs it: rmsnorm, router gate matvec (256 x 7168 f32), softmax top-8 (one call:
+        # mk_dev_norm_gate_route), expert section.  16 gate matrices stand for 16 layers, so the routing is computed on the device and
         # differs from call to call; the shared expert rotates as above (it may coincide with a routed one: 3 % of calls).
         if B == 1:
             gates = [torch.randn((ne, d), device="cuda", generator=g) * (d ** -0.5) for _ in range(16)]
@@ -376,9 +376,7 @@ def bench_moe(torch, cpu=True):
         picked = []
 
         def layer(k, record=False):
-            xn = model.rmsnorm(x, norm_w, 1e-6)
-            lg = model.matvec(gates[k], xn)
-            ids_k, wts_k = model.router_softmax_topk(lg, W.TOP_K)
+            xn, _, ids_k, wts_k = model.norm_gate_route(x, norm_w, 1e-6, gates[k], W.TOP_K)
             model.moe_decode(experts, ids_k, wts_k, xn, shared=(37 * k) % ne, out=out)
             if record:
                 picked.append(len(set(ids_k.cpu().numpy().reshape(-1).tolist()) | {(37 * k) % ne}))
@@ -389,8 +387,8 @@ def bench_moe(torch, cpu=True):
         if ms_chain is None:
             ms_chain = time_region(torch, lambda: [layer(k) for k in range(16)], 4, warmup=1) / 16
         alg_chain = sum(picked) / len(picked) * per_expert + ne * d * 4 + B * 4 * d * 4
-        res[f"B{B}"]["layer_chain"] = {"ms": ms_chain, "tok_s": B / (ms_chain * 1e-3), "calls": "rmsnorm, gate matvec 256 x 7168 f32, softmax top-8, expert section; "
-                                       "16 such layers captured in one graph, routing computed on the device",
+        res[f"B{B}"]["layer_chain"] = {"ms": ms_chain, "tok_s": B / (ms_chain * 1e-3), "calls": "rmsnorm + gate matvec 256 x 7168 f32 + softmax top-8 (mk_dev_norm_gate_route), expert section "
+                                       "(mk_dev_moe_decode); 16 such layers captured in one graph, routing computed on the device",
                                        "distinct_experts_mean": sum(picked) / len(picked), "alg_bytes_mean": alg_chain,
                                        "frac": alg_chain / (ms_chain * 1e-3) / 1e9 / HBM_PEAK_GBS, "finite": bool(torch.isfinite(out).all().item())}
         if cpu:

@@ -310,6 +310,18 @@ int mk_dev_rmsnorm(const float *x, size_t B, size_t d, const float *w, float eps
  * gate, latent projections). */
 int mk_dev_matvec_f32(const float *w, size_t rows, size_t cols, const float *x, size_t B, float *out, void *stream);
 
+/* The three calls above as a decode step runs them in front of its expert section (src/model.rs:2151-2173 after the
+ * layer's rmsnorm: norm, router gate matvec, routing) as ONE call of two launches: xn = rmsnorm(x) and logits = gate xn in
+ * the first (every workgroup norms the rows itself: that costs less than a launch), (ids, weights) = route(logits) in the
+ * second.  Every value is the one the separate calls give, bit for bit (the same operations in the same order).
+ * x [B][d], norm_w [d], gate [n_experts][d] f32 row-major, bias [n_experts] or NULL; xn [B][d] (may be NULL), logits
+ * [B][n_experts] (always written), ids / weights [B][k].  d % 8 == 0 and 512 <= d <= 32768, else MK_ERR_UNSUPPORTED
+ * (use the three calls).  From 5 tokens the call runs the three kernels one after the other (norming the rows once is
+ * then cheaper) and needs xn.  Has no single counterpart in the reference. */
+int mk_dev_norm_gate_route(const float *x, size_t B, size_t d, const float *norm_w, float eps, const float *gate, size_t n_experts, size_t k,
+                           int kind, const float *bias, float route_scale, float *xn, float *logits, int32_t *ids, float *weights,
+                           void *stream);
+
 /* ------------------------------------------- device level: MLA attention */
 
 /* mla_attn_flash_q8_mqa (src/model.rs:1804-1908) in the weight-absorbed form:

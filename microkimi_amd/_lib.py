@@ -93,6 +93,7 @@ def _load():
         "mk_dev_router_topk": (i32, [vp, sz, sz, sz, i32, vp, f32, vp, vp, vp]),
         "mk_dev_rmsnorm": (i32, [vp, sz, sz, vp, f32, vp, vp, vp, vp]),
         "mk_dev_matvec_f32": (i32, [vp, sz, sz, vp, sz, vp, vp]),
+        "mk_dev_norm_gate_route": (i32, [vp, sz, sz, vp, f32, vp, sz, sz, i32, vp, f32, vp, vp, vp, vp, vp]),
         "mk_mla_decode_workspace_bytes": (sz, [sz, sz, sz]),
         "mk_dev_mla_q8_decode": (i32, [vp, vp, vp, vp, sz, vp, sz, sz, sz, f32, vp, vp, vp]),
         "mk_mla_decode_static_max_heads": (sz, []),

@@ -298,27 +298,29 @@ __global__ __launch_bounds__(256) void matvec_f32_chain_kernel(const float *__re
 //   MK_ROUTER_SIGMOID       score = sigmoid(l), key = score + bias;  w = score / (sum + 1e-20)   (K3, noaux_tc)
 //   MK_ROUTER_SQRTSOFTPLUS  score = sqrt(softplus(l)), key = score + bias;  w = score / sum * route_scale   (DeepSeek-V4)
 // One wave per token; n <= 4096, k <= 64.
-__global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict__ logits, int n, int k, int kind,
-                                                         const float *__restrict__ bias, float route_scale, int32_t *__restrict__ ids,
-                                                         float *__restrict__ weights) {
-    extern __shared__ float lds_f[];  // score [n], key [n]
-    float *score = lds_f, *key = lds_f + n;
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float *row = logits + (size_t)t * n;
+// One wave routes one token.  score / key: LDS, n floats each, this wave's own; no workgroup barrier is needed (a wave's
+// LDS operations stay in program order), so several waves of a workgroup can each route a token.  COHERENT: the logits were
+// written by other workgroups of the same launch (read with agent-scope loads).
+template <bool COHERENT>
+__device__ __forceinline__ void router_wave(const float *row, int n, int k, int kind, const float *__restrict__ bias, float route_scale,
+                                            int32_t *ids_t, float *weights_t, float *score, float *key, int lane) {
+    auto logit = [&](int i) -> float {
+        if (COHERENT) return __hip_atomic_load(row + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return row[i];
+    };
     if (kind == MK_ROUTER_SOFTMAX) {
         float m = -INFINITY;
-        for (int i = lane; i < n; i += 64) m = fmaxf(m, row[i]);
+        for (int i = lane; i < n; i += 64) m = fmaxf(m, logit(i));
         m = mk_wave_max(m);
         // the reference sums exp(l - m) sequentially; the sum is only a common
         // normaliser, so its association does not change the selection order
         float z = 0.0f;
         for (int i = lane; i < n; i += 64) {
-            float e = expf(row[i] - m);
+            float e = expf(logit(i) - m);
             score[i] = e;
             z += e;
         }
         z = mk_wave_sum(z);
-        __syncthreads();
         for (int i = lane; i < n; i += 64) {
             const float p = score[i] / z;
             score[i] = p;
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict
         }
     } else {
         for (int i = lane; i < n; i += 64) {
-            const float l = row[i];
+            const float l = logit(i);
             float sc;
             if (kind == MK_ROUTER_SIGMOID) {
                 sc = 1.0f / (1.0f + expf(-l));
@@ -338,12 +340,13 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict
             key[i] = sc + (bias ? bias[i] : 0.0f);
         }
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the lanes' LDS writes above are read by other lanes below
+    __builtin_amdgcn_wave_barrier();
     float sum = 0.0f, myw = 0.0f;
     int myid = 0;
     // A lane keeps the best of its own keys (i = lane, lane + 64, ...: the lowest index among equals); a round takes the
     // wave's largest key, the lowest index among the lanes that hold it, and only the owner of that key looks through its
-    // keys again.  Keys that are NaN are never larger than anything and are never selected, as before.
+    // keys again.  Keys that are NaN are never larger than anything and are never selected.
     float bv = -INFINITY;
     int bi = 0x7FFFFFFF;
     auto rescan = [&]() {
@@ -374,19 +377,130 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict
             myid = best;
         }
         sum += sc;  // slot order, as the reference sums the selected scores
-        if ((best & 63) == lane) {  // the owner: one wave, so its LDS write and reads stay in program order
+        if ((best & 63) == lane) {  // the owner
             key[best] = -INFINITY;
             rescan();
         }
     }
     if (lane < k) {
-        ids[t * k + lane] = myid;
+        ids_t[lane] = myid;
         float wv;
         if (kind == MK_ROUTER_SIGMOID) wv = myw / (sum + 1e-20f);
         else if (kind == MK_ROUTER_SQRTSOFTPLUS) wv = myw / sum * route_scale;
         else wv = myw / sum;
-        weights[t * k + lane] = wv;
+        weights_t[lane] = wv;
     }
+}
+
+// One wave per token; n <= 4096, k <= 64.
+__global__ __launch_bounds__(64) void router_topk_kernel(const float *__restrict__ logits, int n, int k, int kind,
+                                                         const float *__restrict__ bias, float route_scale, int32_t *__restrict__ ids,
+                                                         float *__restrict__ weights) {
+    extern __shared__ float lds_f[];  // score [n], key [n]
+    const int t = blockIdx.x;
+    router_wave<false>(logits + (size_t)t * n, n, k, kind, bias, route_scale, ids + (size_t)t * k, weights + (size_t)t * k, lds_f, lds_f + n,
+                       (int)threadIdx.x);
+}
+
+// rmsnorm -> gate matvec of a decode step in one launch, every value the one the two separate kernels give.
+// Grid (n experts, groups of up to 4 tokens).  Workgroup (r, tg):
+//   1  dot(x, x) of its tokens through the chain pipeline of matvec_f32_chain_kernel (the products are the squares); every
+//      workgroup does this for itself -- a chain of d / 8 additions costs less than a launch;
+//   2  the same pipeline with the products gate[r][c] * xn[t][c], xn = (x * inv) * w as rmsnorm forms it; on the way the
+//      workgroup stores its share of the xn rows (column groups r, r + n, ...);
+//   3  stores its logit.
+// The routing stays a launch of its own: having the last workgroup of a token group route it (a counter per group) was
+// built and measured 36.8 us against 19.3 for the two launches at 256 experts x 7168 -- the release fence in front of the
+// count writes the XCD's L2 back (16 us over the launch), and 256 increments of one counter from 8 XCDs take 8 us more.
+__global__ __launch_bounds__(256) void norm_gate_kernel(const float *__restrict__ x, int B, int d, const float *__restrict__ norm_w, float eps,
+                                                              const float *__restrict__ gate, int n, float *__restrict__ xn_out,
+                                                              float *__restrict__ logits, int tb_max) {
+    extern __shared__ __attribute__((aligned(16))) float mv_lds[];  // [2][8 tb_max][MV_STRIDE]
+    __shared__ float inv_l[MV_TB];
+    const int r = blockIdx.x, tg = blockIdx.y, b0 = tg * MV_TB, tb = min(MV_TB, B - b0);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int nseg = (d + MV_SEG - 1) / MV_SEG;  // d % 8 == 0: every column is in a chain
+    const int buf_floats = 8 * tb_max * MV_STRIDE;
+    const float *gr = gate + (size_t)r * d, *xb = x + (size_t)b0 * d;
+
+    // products of one segment, by the 192 threads of waves 1-3; PASS 1: squares, PASS 2: gate * normed value
+    auto produce = [&](int seg, int pass, const float *inv) __attribute__((always_inline)) {
+        float *buf = mv_lds + (seg & 1) * buf_floats;
+        const int c0 = seg * MV_SEG, c1 = min(c0 + MV_SEG, d);
+        mk_f4 gv[MV_NG], nv[MV_NG], xv[MV_TB][MV_NG];
+#pragma unroll
+        for (int kk = 0; kk < MV_NG; kk++) {
+            const int c = min(c0 + 4 * (tid - 64 + 192 * kk), d - 4);
+            if (pass == 2) {
+                gv[kk] = *reinterpret_cast<const mk_f4 *>(gr + c);
+                nv[kk] = *reinterpret_cast<const mk_f4 *>(norm_w + c);
+            }
+#pragma unroll
+            for (int t = 0; t < MV_TB; t++) xv[t][kk] = *reinterpret_cast<const mk_f4 *>(xb + (size_t)min(t, tb - 1) * d + c);
+        }
+#pragma unroll
+        for (int kk = 0; kk < MV_NG; kk++) {
+            const int c = c0 + 4 * (tid - 64 + 192 * kk);
+            if (c < c1) {
+                float *dst = buf + (4 * ((c >> 2) & 1)) * MV_STRIDE + ((c - c0) >> 3);
+                const bool mine = pass == 2 && xn_out && ((c >> 2) % n) == r;
+#pragma unroll
+                for (int t = 0; t < MV_TB; t++) {
+                    if (t < tb) {
+                        float *dt = dst + 8 * t * MV_STRIDE;
+                        mk_f4 p;
+                        if (pass == 1) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) p[e] = mk_mul(xv[t][kk][e], xv[t][kk][e]);
+                        } else {
+                            mk_f4 y;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                y[e] = mk_mul(mk_mul(xv[t][kk][e], inv[t]), nv[kk][e]);
+                                p[e] = mk_mul(gv[kk][e], y[e]);
+                            }
+                            if (mine) *reinterpret_cast<mk_f4 *>(xn_out + (size_t)(b0 + t) * d + c) = y;
+                        }
+                        dt[0] = p.x;
+                        dt[MV_STRIDE] = p.y;
+                        dt[2 * MV_STRIDE] = p.z;
+                        dt[3 * MV_STRIDE] = p.w;
+                    }
+                }
+            }
+        }
+    };
+    float result = 0.0f;  // lane 8 t of wave 0: the dot of token t
+    auto run = [&](int pass) __attribute__((always_inline)) {
+        float inv[MV_TB] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (pass == 2) {
+#pragma unroll
+            for (int t = 0; t < MV_TB; t++) inv[t] = inv_l[t];
+        }
+        float acc = 0.0f;
+        if (wave != 0) produce(0, pass, inv);
+        __syncthreads();
+        for (int seg = 0; seg < nseg; seg++) {
+            if (wave != 0) {
+                if (seg + 1 < nseg) produce(seg + 1, pass, inv);
+            } else if (lane < 8 * tb) {
+                const int steps = (min((seg + 1) * MV_SEG, d) - seg * MV_SEG) >> 3;
+                acc = chain_add(acc, mv_lds + (seg & 1) * buf_floats + lane * MV_STRIDE, steps);
+            }
+            __syncthreads();
+        }
+        if (wave == 0) result = dot8_reduce(acc);
+    };
+    run(1);
+    if (wave == 0 && (lane & 7) == 0 && (lane >> 3) < tb) {
+        // as rmsnorm_q8_kernel: correctly rounded division and square root through double
+        const float ss = (float)((double)result / (double)d);
+        const float rt = (float)sqrt((double)mk_add(ss, eps));
+        inv_l[lane >> 3] = (float)(1.0 / (double)rt);
+    }
+    __syncthreads();
+    run(2);
+    if (wave == 0 && (lane & 7) == 0 && (lane >> 3) < tb) logits[(size_t)(b0 + (lane >> 3)) * n + r] = result;
 }
 
 }  // namespace
@@ -447,4 +561,36 @@ extern "C" int mk_dev_router_topk(const float *logits, size_t B, size_t n, size_
 
 extern "C" int mk_dev_router_softmax_topk(const float *logits, size_t B, size_t n, size_t k, int32_t *ids, float *weights, void *stream) {
     return mk_dev_router_topk(logits, B, n, k, MK_ROUTER_SOFTMAX, nullptr, 1.0f, ids, weights, stream);
+}
+
+extern "C" int mk_dev_norm_gate_route(const float *x, size_t B, size_t d, const float *norm_w, float eps, const float *gate, size_t n_experts,
+                                      size_t k, int kind, const float *bias, float route_scale, float *xn, float *logits, int32_t *ids,
+                                      float *weights, void *stream) {
+    MK_REQUIRE(x && norm_w && gate && logits && ids && weights, "null pointer");
+    MK_REQUIRE(kind >= MK_ROUTER_SOFTMAX && kind <= MK_ROUTER_SQRTSOFTPLUS, "unknown router rule");
+    MK_REQUIRE(B >= 1 && B <= 65535 && k >= 1 && k <= 64 && k <= n_experts && n_experts <= 4096, "bad batch, k or expert count");
+    MK_REQUIRE(((((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)gate | (uintptr_t)xn)) & 15) == 0, "x, norm_w, gate and xn must be 16-byte aligned");
+    if (d % 8 != 0 || d < 512 || d > 32768) {
+        mk_set_error("this call takes d %% 8 == 0 and 512 <= d <= 32768: use mk_dev_rmsnorm, mk_dev_matvec_f32, mk_dev_router_topk");
+        return MK_ERR_UNSUPPORTED;
+    }
+    if (B > (size_t)MV_TB) {
+        // from 5 tokens the rows are normed once, by a launch of their own: in the fused kernel every workgroup norms its
+        // group's rows itself, which pays for one launch but not for the second group of tokens (16 tokens: 38.7 us
+        // fused, 31.6 us as three launches, at 256 experts x 7168)
+        MK_REQUIRE(xn, "more than 4 tokens take the normed rows as a buffer (xn)");
+        int s3 = mk_dev_rmsnorm(x, B, d, norm_w, eps, xn, nullptr, nullptr, stream);
+        if (s3 != MK_OK) return s3;
+        if ((s3 = mk_dev_matvec_f32(gate, n_experts, d, xn, B, logits, stream)) != MK_OK) return s3;
+        return mk_dev_router_topk(logits, B, n_experts, k, kind, bias, route_scale, ids, weights, stream);
+    }
+    const int tb_max = (int)(B < (size_t)MV_TB ? B : (size_t)MV_TB);
+    const int nbuf = d > (size_t)MV_SEG ? 2 : 1;
+    const size_t lds = (size_t)nbuf * 8 * tb_max * MV_STRIDE * sizeof(float);
+    int st = mk_lds_opt_in(reinterpret_cast<const void *>(norm_gate_kernel), 140 * 1024);
+    if (st != MK_OK) return st;
+    hipLaunchKernelGGL(norm_gate_kernel, dim3((unsigned)n_experts, (unsigned)((B + MV_TB - 1) / MV_TB)), dim3(256), lds, (hipStream_t)stream, x, (int)B,
+                       (int)d, norm_w, eps, gate, (int)n_experts, xn, logits, tb_max);
+    if ((st = mk_launch_status("norm_gate")) != MK_OK) return st;
+    return mk_dev_router_topk(logits, B, n_experts, k, kind, bias, route_scale, ids, weights, stream);
 }

@@ -407,6 +407,24 @@ def router_softmax_topk(logits, k):
     return ids, w
 
 
+def norm_gate_route(x, norm_w, eps, gate, k, kind=ROUTER_SOFTMAX, bias=None, route_scale=1.0, want_xn=True):
+    """rmsnorm -> router gate matvec -> routing as one call of two launches (mk_dev_norm_gate_route): x [B, d], norm_w [d],
+    gate [n, d].  Returns (xn [B, d] or None, logits [B, n], ids [B, k] int32, weights [B, k]), each bit-identical to
+    rmsnorm, matvec and router_topk called one after the other."""
+    import torch
+    _lib.require_device()
+    B, d = x.shape
+    n = gate.shape[0]
+    xn = torch.empty((B, d), dtype=torch.float32, device=x.device) if want_xn else None
+    logits = torch.empty((B, n), dtype=torch.float32, device=x.device)
+    ids = torch.empty((B, k), dtype=torch.int32, device=x.device)
+    w = torch.empty((B, k), dtype=torch.float32, device=x.device)
+    check(lib.mk_dev_norm_gate_route(ptr(x.contiguous()), B, d, ptr(norm_w.contiguous()), float(eps), ptr(gate.contiguous()), n, k, kind,
+                                     None if bias is None else ptr(bias.contiguous()), float(route_scale), ptr(xn), ptr(logits), ptr(ids),
+                                     ptr(w), cur_stream()))
+    return xn, logits, ids, w
+
+
 def grouped_gemm_f32(packed_list, scales_list, rows, cols, x, offsets, bf16=False):
     """matvec_packed_nt per group (src/model.rs:2412-2447 as called at src/model.rs:2580-2599): rows
     offsets[e]..offsets[e+1] of x [m, cols] against expert e -> [m, rows] f32.  x f32: the reference's f32 arithmetic on

@@ -153,6 +153,9 @@ extern "C" {
     pub fn mk_dev_router_topk(logits: *const f32, B: usize, n: usize, k: usize, kind: c_int, bias: *const f32, route_scale: f32, ids: *mut i32, weights: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_rmsnorm(x: *const f32, B: usize, d: usize, w: *const f32, eps: f32, out: *mut f32, q: *mut i8, scales: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_matvec_f32(w: *const f32, rows: usize, cols: usize, x: *const f32, B: usize, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_norm_gate_route(x: *const f32, b: usize, d: usize, norm_w: *const f32, eps: f32, gate: *const f32, n_experts: usize, k: usize,
+                                  kind: c_int, bias: *const f32, route_scale: f32, xn: *mut f32, logits: *mut f32,
+                                  ids: *mut i32, weights: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_mla_decode_workspace_bytes(nh: usize, L: usize, n_pos: usize) -> usize;
     pub fn mk_dev_mla_q8_decode(lat_q: *const i8, lat_s: *const c_void, rope_q: *const i8, rope_s: *const c_void, pos: usize, q: *const f32, nh: usize, L: usize, R: usize, scale: f32, workspace: *mut c_void, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_mla_decode_static_max_heads() -> usize;

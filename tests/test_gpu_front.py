@@ -110,3 +110,40 @@ def test_norm_route_experts_without_host_round_trip():
     got = model.moe_decode(experts, ids, wts, x, act_kind=model.ACT_SITU).cpu().numpy()
     assert np.array_equal(ids.cpu().numpy()[0], io.astype(np.int32))
     assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-5
+
+
+@pytest.mark.parametrize("B,d,n,k,kind", [(1, 7168, 256, 8, 0), (3, 7168, 384, 6, 1), (4, 512, 16, 4, 2), (5, 2048, 64, 8, 0), (9, 4096, 4096, 64, 1),
+                                          (16, 7168, 256, 8, 0)])
+def test_norm_gate_route_gives_the_three_calls_bits(B, d, n, k, kind):
+    # mk_dev_norm_gate_route against mk_dev_rmsnorm -> mk_dev_matvec_f32 -> mk_dev_router_topk (each held to the oracle by the
+    # tests above): normed rows, logits and routing weights bit for bit, ids equal; and the rows against the oracle too
+    torch = torch_cuda()
+    from microkimi_amd import model
+    rng = np.random.default_rng(B * 1000 + n)
+    x = rng.standard_normal((B, d)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    gate = (rng.standard_normal((n, d)) * d ** -0.5).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.05).astype(np.float32) if kind else None
+    xd, nwd, gd, bd = dev(x), dev(nw), dev(gate), None if bias is None else dev(bias)
+    xn0 = model.rmsnorm(xd, nwd, 1e-6)
+    lg0 = model.matvec(gd, xn0)
+    ids0, w0 = model.router_topk(lg0, k, kind, bd, route_scale=1.5)
+    for rep in range(2):
+        xn, lg, ids, w = model.norm_gate_route(xd, nwd, 1e-6, gd, k, kind, bd, route_scale=1.5)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(xn.cpu().numpy()), bits(xn0.cpu().numpy())), rep
+        assert np.array_equal(bits(lg.cpu().numpy()), bits(lg0.cpu().numpy())), rep
+        assert np.array_equal(ids.cpu().numpy(), ids0.cpu().numpy()), rep
+        assert np.array_equal(bits(w.cpu().numpy()), bits(w0.cpu().numpy())), rep
+    assert np.array_equal(bits(xn.cpu().numpy()[0]), bits(oracle.rmsnorm(x[0], nw, 1e-6)))
+    assert np.array_equal(bits(lg.cpu().numpy()[0]), bits(oracle.matvec_f32(gate, n, d, oracle.rmsnorm(x[0], nw, 1e-6))))
+
+
+def test_norm_gate_route_refuses_what_it_does_not_take():
+    torch = torch_cuda()
+    from microkimi_amd import model
+    from microkimi_amd._lib import MkError
+    x = torch.zeros((1, 100), device="cuda")
+    with pytest.raises(MkError) as e:
+        model.norm_gate_route(x, torch.ones(100, device="cuda"), 1e-6, torch.zeros((8, 100), device="cuda"), 2)
+    assert e.value.status == -4
