@@ -258,7 +258,10 @@ size_t mk_moe_decode_vq_workspace_bytes(size_t B, size_t topk, int has_shared, s
 int mk_dev_moe_decode(const mk_expert_table *table, size_t B, size_t topk, const int32_t *ids, const float *weights, int shared,
                       const float *x, int mode, int act_kind, float limit, void *workspace, float *out, void *stream);
 /* *flag = 1 if a workgroup of the one-launch form ever gave up waiting on this device (its rows are NaN), else 0.
- * Synchronous (a device-to-host copy).  Has no counterpart in the reference. */
+ * Synchronous (a device-to-host copy).  A give-up means that the launch did not have the device to itself (calls that
+ * overlapped, or a bound set too low with MK_MOE_SPIN_LIMIT); the call that follows a give-up on the same workspace is
+ * not to be trusted either (a late workgroup of the failed launch may have tagged its values for the next one): check
+ * the flag, then drop both results.  Has no counterpart in the reference. */
 int mk_dev_moe_decode_gave_up(int *flag);
 /* count[0] (device int32) = how many of the n routed ids lie outside [0, n_experts): the pairs that the decode and prefill
  * calls skip when the table states its size.  The reference would panic on such an index (a slice index out of range,

@@ -495,3 +495,47 @@ def test_count_of_routed_ids_outside_the_table():
         count = torch.full((1,), -7, dtype=torch.int32, device="cuda")
         check(lib.mk_dev_moe_count_bad_ids(ptr(dev(ids)), n, n_experts, ptr(count), cur_stream()))
         assert int(count.item()) == int(bad.sum())
+
+
+_GIVE_UP_SCRIPT = r"""
+import ctypes, sys, numpy as np, torch
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests")
+from microkimi_amd import model, workloads
+from microkimi_amd._lib import check, lib
+d, inter, n, topk = 7168, 2048, 10, 8
+dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+host = [(workloads.mxfp4_matrix(2, "w1", inter, d, e), workloads.mxfp4_matrix(2, "w3", inter, d, e), workloads.mxfp4_matrix(2, "w2", d, inter, e))
+        for e in range(n)]
+pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+assert experts.table.w13t is not None
+rng = np.random.default_rng(0)
+x = dev(rng.standard_normal((1, d)).astype(np.float32))
+ids = dev(rng.permutation(n - 1)[:topk].astype(np.int32)[None, :])
+wts = dev(np.full((1, topk), 0.125, np.float32))
+for _ in range(3):
+    out = model.moe_decode(experts, ids, wts, x, shared=n - 1)
+    torch.cuda.synchronize()
+flag = ctypes.c_int(-1)
+check(lib.mk_dev_moe_decode_gave_up(ctypes.byref(flag)))
+o = out.cpu().numpy()
+print("RESULT", flag.value, int(np.isnan(o).sum()), int(np.isfinite(o).all()))
+"""
+
+
+def test_one_launch_kernel_gives_up_instead_of_waiting_forever():
+    # the waits of the one-launch kernel are bounded: with a bound of zero polls (MK_MOE_SPIN_LIMIT=0, read once per process,
+    # hence a process of its own) a workgroup that does not find another's values at its first look gives up, its rows
+    # become NaN, the flag goes up -- and every launch still ends.  (With luck all values are there at the first look: then
+    # the rows are finite and the flag is down.  Both are the contract; a hang or a finite wrong row is not.)
+    import os
+    import subprocess
+    import sys
+    torch_cuda()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, MK_MOE_SPIN_LIMIT="0")
+    r = subprocess.run([sys.executable, "-c", _GIVE_UP_SCRIPT, root], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("RESULT")][-1].split()
+    flag, n_nan, finite = int(line[1]), int(line[2]), int(line[3])
+    assert (flag == 1 and n_nan > 0) or (flag == 0 and finite == 1), line
