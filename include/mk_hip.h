@@ -208,7 +208,17 @@ typedef struct {
      * q8 mode at d = 7168 or 5120, inter = 2048 on a 256-CU device take the one-launch form of the layer (see
      * mk_dev_moe_decode); such calls must not overlap on one device. */
     const uint8_t *const *w13t, *const *w2t;
+    /* Optional (NULL: not there; each on its own): per expert, the scale bytes of W1, W3, W2 once more in K-tile order
+     * (mk_dev_mxfp4_scales_by_tile; d % 512 == 0 for W1 and W3, inter % 512 == 0 for W2; 1/16 of the experts' bytes again).
+     * The matrix-core kernels of mk_dev_moe_decode (from 4 tokens) and of mk_dev_moe_prefill then read these instead of
+     * w1s, w3s, w2s: same bytes, same results, whole 128-byte lines per K tile instead of an eighth of eight lines. */
+    const uint8_t *const *w1st, *const *w3st, *const *w2st;
 } mk_expert_table;
+
+/* out[(t * rows + r) * 16 + j] = scales[r * (cols / 32) + 16 t + j]: the scale bytes ([rows][cols / 32], src/mxfp4.rs:1-3) with the 16
+ * bytes a row has per 512 columns kept together and the rows of one such K tile adjacent.  cols % 512 == 0; both 16-byte
+ * aligned; rows * cols / 32 bytes. */
+int mk_dev_mxfp4_scales_by_tile(const uint8_t *scales, size_t rows, size_t cols, uint8_t *out, void *stream);
 
 /* The experts of a layer in the operand order of v_mfma_scale_f32_16x16x128_f8f6f4, for the one-launch decode kernel: the
  * same bytes as (packed, scales) in another order -- mk_dev_moe_unpack_* restores the reference layout byte for byte

@@ -27,7 +27,7 @@ class BinEntry(C.Structure):
 class ExpertTable(C.Structure):
     _fields_ = [("w1p", C.c_void_p), ("w1s", C.c_void_p), ("w3p", C.c_void_p), ("w3s", C.c_void_p), ("w2p", C.c_void_p),
                 ("w2s", C.c_void_p), ("d", C.c_size_t), ("inter", C.c_size_t), ("n_experts", C.c_size_t), ("vq_codebook", C.c_void_p),
-                ("w13t", C.c_void_p), ("w2t", C.c_void_p)]
+                ("w13t", C.c_void_p), ("w2t", C.c_void_p), ("w1st", C.c_void_p), ("w3st", C.c_void_p), ("w2st", C.c_void_p)]
 
 
 class Prof(C.Structure):
@@ -61,6 +61,7 @@ def _load():
         "mk_force_q8": (None, [i32]),
         "mk_q8_enabled": (i32, []),
         "mk_dev_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
+        "mk_dev_mxfp4_scales_by_tile": (i32, [vp, sz, sz, vp, vp]),
         "mk_dev_fp8_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_dev_quantize_q8": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_quantize_mxfp8": (i32, [vp, sz, sz, vp, vp, vp]),

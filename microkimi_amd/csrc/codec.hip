@@ -110,7 +110,28 @@ __global__ __launch_bounds__(256) void mk_quantize_mxfp8_kernel(const float *__r
     if ((i & 3) == 0) exps[i >> 2] = (uint8_t)eb;
 }
 
+// The scale bytes of an MXFP4 matrix, [rows][cols / 32], once more as [cols / 512][rows][16]: the 16 bytes that a row has
+// per 512 columns, rows of one K tile together.  One thread per 16 bytes.
+__global__ __launch_bounds__(256) void mk_scales_by_tile_kernel(const uint4 *__restrict__ scales, uint4 *__restrict__ out, size_t rows, size_t kt) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * kt) return;
+    const size_t t = i / rows, r = i - t * rows;
+    out[i] = scales[r * kt + t];
+}
+
 // ------------------------------------------------------------------ C ABI
+extern "C" int mk_dev_mxfp4_scales_by_tile(const uint8_t *scales, size_t rows, size_t cols, uint8_t *out, void *stream) {
+    MK_REQUIRE(scales && out, "null pointer");
+    MK_REQUIRE(cols % 512 == 0, "cols must be a multiple of 512");
+    MK_REQUIRE(((uintptr_t)scales & 15) == 0 && ((uintptr_t)out & 15) == 0, "scales and out must be 16-byte aligned");
+    const size_t n = rows * (cols / 512);
+    if (n == 0) return MK_OK;
+    MK_REQUIRE(n <= 0x7fffffffull * 256, "matrix too large");
+    hipLaunchKernelGGL(mk_scales_by_tile_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, (const uint4 *)scales,
+                       (uint4 *)out, rows, cols / 512);
+    return mk_launch_status("mxfp4_scales_by_tile");
+}
+
 extern "C" int mk_dev_mxfp4_dequant(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, float *out, void *stream) {
     MK_REQUIRE(packed && scales && out, "null pointer");
     MK_REQUIRE(cols % 32 == 0, "cols must be a multiple of 32");

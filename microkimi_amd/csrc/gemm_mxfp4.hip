@@ -126,6 +126,11 @@ constexpr int a_buf_bytes(int mc) { return a_wsc_off(mc) + 256 * 16; }          
 struct GemmArgs {
     const uint8_t *const *packed_ptrs[2];
     const uint8_t *const *scales_ptrs[2];
+    // optional: the same scale bytes in [K tile of 512 columns][row][16] order (mk_dev_mxfp4_scales_by_tile).  A row's 16
+    // bytes per K tile are an eighth of a 128-byte line of the plain array, and that line is asked for in eight K tiles:
+    // the scale lines of the workgroups resident on an XCD outgrow its L2 and were fetched 2.9 times; in this order a
+    // workgroup's 4 KB per K tile are whole lines that are used once
+    const uint8_t *const *scales_t_ptrs[2];
     int rows, cols;
     const uint8_t *codes;
     const uint8_t *exps;
@@ -217,7 +222,8 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // per value instead of 8 written and 8 read back by a kernel of its own.
 template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
-                                          uint8_t *lds, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr) {
+                                          uint8_t *lds, const uint8_t *scales_t, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr,
+                                          const uint8_t *scales3_t = nullptr) {
     static_assert(!GU || (FULL && PIN && !DEEP && MC <= 2), "the gate/up form exists for the small-group pass");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
@@ -263,8 +269,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     mk_i4 st[2 * MC], ste, stw;
     // (gate/up form: thread i is row slot (wave i / 64, row tile (i / 16) % 4, row i % 16) of the workgroup)
     const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * 256 + tid;
-    const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? scales3 : scales;
-    const uint32_t wsoff = (uint32_t)min(ws_row, a.rows - 1) * (uint32_t)nb;
+    const bool ws_tiles = scales_t != nullptr;  // (uniform)
+    const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? (ws_tiles ? scales3_t : scales3) : (ws_tiles ? scales_t : scales);
+    const uint32_t ws_r = (uint32_t)min(ws_row, a.rows - 1);
+    const uint32_t wsoff = ws_tiles ? ws_r * 16u : ws_r * (uint32_t)nb, ws_step = ws_tiles ? (uint32_t)a.rows * 16u : 16u;
     uint32_t coff[2 * MC];  // the host checks that tokens x cols stays below 2^32
 #pragma unroll
     for (int k = 0; k < 2 * MC; k++) {
@@ -277,7 +285,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
         for (int k = 0; k < 2 * MC; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
         ste = mk_ldg128_off(a.exps, eoff + ku * 16);
-        stw = mk_ldg128_off(ws_base, wsoff + ku * 16);
+        stw = mk_ldg128_off(ws_base, wsoff + ku * ws_step);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
@@ -545,15 +553,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     if (count <= 0 || (count <= 32 ? 2 : 4) != MC) return;
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
+    const uint8_t *scales_t = a.scales_t_ptrs[m] ? mk_uniform_ptr(a.scales_t_ptrs[m][e]) : nullptr;
     float *out = a.out[m];
     if (MC == 2) {
-        if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
-        else gemm_pass<2, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds);
+        if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds, scales_t);
+        else gemm_pass<2, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds, scales_t);
     } else {
         // the 64-token passes of a group are dealt to gridDim.y workgroups: a few large groups still fill the chip
 #pragma unroll 1
         for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
-            gemm_pass<MC, true, false, true, true>(a, packed, scales, out, rb, base, tok1, lds);
+            gemm_pass<MC, true, false, true, true>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
     }
 }
 
@@ -576,11 +585,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     if (count <= 0) return;
     const uint8_t *p1 = mk_uniform_ptr(a.packed_ptrs[0][e]), *s1 = mk_uniform_ptr(a.scales_ptrs[0][e]);
     const uint8_t *p3 = mk_uniform_ptr(a.packed_ptrs[1][e]), *s3 = mk_uniform_ptr(a.scales_ptrs[1][e]);
+    const bool tiles = a.scales_t_ptrs[0] && a.scales_t_ptrs[1];
+    const uint8_t *t1 = tiles ? mk_uniform_ptr(a.scales_t_ptrs[0][e]) : nullptr, *t3 = tiles ? mk_uniform_ptr(a.scales_t_ptrs[1][e]) : nullptr;
     if (count <= 16) {
-        gemm_pass<1, true, true, true, false, true>(a, p1, s1, nullptr, rb, tok0, tok1, lds, p3, s3);
+        gemm_pass<1, true, true, true, false, true>(a, p1, s1, nullptr, rb, tok0, tok1, lds, t1, p3, s3, t3);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 32) gemm_pass<2, true, true, true, false, true>(a, p1, s1, nullptr, rb, base, tok1, lds, p3, s3);
+        for (int base = tok0; base < tok1; base += 32) gemm_pass<2, true, true, true, false, true>(a, p1, s1, nullptr, rb, base, tok1, lds, t1, p3, s3, t3);
     }
 }
 
@@ -602,7 +613,7 @@ int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
 // gate and up of the prefill section in one launch (the matrices share the token rows); see mk_common.h
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                             size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
-                            float *const *out, void *stream) {
+                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs) {
     MK_REQUIRE(n_mats == 1 || n_mats == 2, "one or two matrices per group");
     for (int k = 0; k < n_mats; k++) MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k], "null pointer");
     MK_REQUIRE(codes && exps && offsets, "null pointer");
@@ -617,6 +628,7 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         for (int k = 0; k < n_mats; k++) {
             a.packed_ptrs[k] = packed_ptrs[k];
             a.scales_ptrs[k] = scales_ptrs[k];
+            a.scales_t_ptrs[k] = scales_t_ptrs ? scales_t_ptrs[k] : nullptr;
             a.out[k] = out[k];
         }
         a.rows = (int)rows;
@@ -645,7 +657,7 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
 int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                                       size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
                                       const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
-                                      float *keep_u, void *stream) {
+                                      float *keep_u, void *stream, const uint8_t *const *w1st, const uint8_t *const *w3st) {
     MK_REQUIRE(w1p && w1s && w3p && w3s && codes && exps && offsets && act_codes && act_exps, "null pointer");
     if (!(cols % 512 == 0 && rows % 128 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0 &&
           ((uintptr_t)codes & 15) == 0 && ((uintptr_t)act_codes & 3) == 0 && n_groups * (rows / 128) < 0x7FFFFFFFull))
@@ -656,6 +668,8 @@ int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *
     a.scales_ptrs[0] = w1s;
     a.packed_ptrs[1] = w3p;
     a.scales_ptrs[1] = w3s;
+    a.scales_t_ptrs[0] = w1st;
+    a.scales_t_ptrs[1] = w3st;
     a.out[0] = keep_g;
     a.out[1] = keep_u;
     a.keep = keep_g && keep_u;
@@ -680,5 +694,5 @@ extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, cons
                                          size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
                                          void *stream) {
     MK_REQUIRE(packed_ptrs && scales_ptrs && codes && exps && offsets && out, "null pointer");
-    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream);
+    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream, nullptr);
 }

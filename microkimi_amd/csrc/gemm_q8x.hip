@@ -38,6 +38,7 @@ constexpr int QX_LDS = QX_ZERO_OFF + ((QX_ZERO_BYTES + 255) / 256) * 256;
 struct Q8xArgs {
     const uint8_t *const *packed_ptrs[2];  // by expert id
     const uint8_t *const *scales_ptrs[2];
+    const uint8_t *const *scales_t_ptrs[2];  // optional: the scale bytes in K-tile order (see gemm_mxfp4.hip)
     int rows, cols;
     const int8_t *xq;       // [activation rows][cols]
     const float *xs;        // [activation rows][cols / 32]
@@ -69,8 +70,8 @@ __device__ __forceinline__ void qx_split(uint32_t q4, uint32_t &a_codes, uint32_
 
 // One pass: up to QX_TOK tokens (NP pairs) of a group against the workgroup's 256 rows.
 template <int NP, int WAVES>
-__device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
-                                         uint8_t *lds) {
+__device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed, const uint8_t *scales, const uint8_t *scales_t, float *out, int rb,
+                                         int base, int tok1, uint8_t *lds) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
@@ -83,7 +84,10 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
 #pragma unroll
         for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(row0 + rt * 16 + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
     const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
-    const uint32_t wsoff = (uint32_t)min(rb * (64 * WAVES) + tid, a.rows - 1) * (uint32_t)nb;
+    const bool ws_tiles = scales_t != nullptr;  // (uniform)
+    const uint8_t *ws_base = ws_tiles ? scales_t : scales;
+    const uint32_t ws_r = (uint32_t)min(rb * (64 * WAVES) + tid, a.rows - 1);
+    const uint32_t wsoff = ws_tiles ? ws_r * 16u : ws_r * (uint32_t)nb, ws_step = ws_tiles ? (uint32_t)a.rows * 16u : 16u;
 
     // this lane as a column of the instruction: token t2 of the pair, phase p, part (0: a codes, 1: b codes)
     const int t2 = n >> 3, ph = (n >> 1) & 3, part = n & 1;
@@ -111,7 +115,7 @@ __device__ __forceinline__ void q8x_pass(const Q8xArgs &a, const uint8_t *packed
     auto stage_load = [&](int kt) __attribute__((always_inline)) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
         stq = mk_ldg128_off(a.xq, qoff + ku * 512);
-        stw = mk_ldg128_off(scales, wsoff + ku * 16);
+        stw = mk_ldg128_off(ws_base, wsoff + ku * ws_step);
         stdx = mk_ldg_f32_off(a.xs, (dxoff + ku * 16 + (sch & 15)) * 4);  // unconditional: a load under a branch forces a full wait
     };
     auto stage_store = [&](uint8_t *buf) __attribute__((always_inline)) {
@@ -268,11 +272,12 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
     const int e = a.gexp[gi];
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
+    const uint8_t *scales_t = a.scales_t_ptrs[m] ? mk_uniform_ptr(a.scales_t_ptrs[m][e]) : nullptr;
     float *out = a.out[m];
     for (int i = threadIdx.x * 16; i < QX_LDS - QX_ZERO_OFF; i += 64 * WAVES * 16) *reinterpret_cast<mk_i4 *>(lds + QX_ZERO_OFF + i) = mk_i4{0, 0, 0, 0};
 #pragma unroll 1
     for (int pass = first_pass; tok0 + QX_TOK * pass < tok1; pass += pass_step)
-        q8x_pass<QX_TOK / 2, WAVES>(a, packed, scales, out, rb, tok0 + QX_TOK * pass, tok1, lds);
+        q8x_pass<QX_TOK / 2, WAVES>(a, packed, scales, scales_t, out, rb, tok0 + QX_TOK * pass, tok1, lds);
 }
 
 }  // namespace
@@ -280,7 +285,8 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
 // All groups' rows against one (n_mats = 1) or two matrices per expert; see mk_common.h.
 int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t rows, size_t cols,
                    const int8_t *xq, const float *xs, const int32_t *arow, const int32_t *goff, const int32_t *gexp, const int32_t *ngroups,
-                   const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream) {
+                   const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream,
+                   const uint8_t *const *const *scales_t_ptrs) {
     MK_REQUIRE(n_mats == 1 || n_mats == 2, "one or two matrices per group");
     MK_REQUIRE(cols % 512 == 0 && cols > 0 && rows >= 1, "cols must be a positive multiple of 512");
     MK_REQUIRE(rows * (cols / 2) < 0xFFFFFFFFull, "matrix too large for 32-bit byte offsets");
@@ -288,6 +294,7 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     for (int k = 0; k < n_mats; k++) {
         a.packed_ptrs[k] = packed_ptrs[k];
         a.scales_ptrs[k] = scales_ptrs[k];
+        a.scales_t_ptrs[k] = scales_t_ptrs ? scales_t_ptrs[k] : nullptr;
         a.out[k] = out[k];
     }
     a.rows = (int)rows;
@@ -351,5 +358,5 @@ extern "C" int mk_dev_mxfp4_matvec_q8_batched(const uint8_t *packed, const uint8
     const uint8_t *const *pp = reinterpret_cast<const uint8_t *const *>(ws);
     const uint8_t *const *sp = reinterpret_cast<const uint8_t *const *>(ws + 8);
     const int32_t *w = reinterpret_cast<const int32_t *>(ws + 16);
-    return mk_q8x_grouped(1, &pp, &sp, rows, cols, xq, xs, nullptr, w, w + 2, w + 3, w + 4, 1, m, &out, stream);
+    return mk_q8x_grouped(1, &pp, &sp, rows, cols, xq, xs, nullptr, w, w + 2, w + 3, w + 4, 1, m, &out, stream, nullptr);
 }

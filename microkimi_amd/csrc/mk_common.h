@@ -348,9 +348,11 @@ int mk_mla_static_init(void **out_ptr);
 
 // mk_dev_mxfp4_grouped_gemm for n_mats (1 or 2) weight matrices per group that multiply the same token rows, in one launch
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].
+// scales_t_ptrs (may be null, and so may its entries): the matrices' scale bytes in K-tile order
+// (mk_dev_mxfp4_scales_by_tile), read instead of scales_ptrs by the kernels that walk K in tiles of 512.
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                             size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
-                            float *const *out, void *stream);
+                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs = nullptr);
 // matvec_packed_nt (f32 products and sums, gemv_mxfp4.hip) for groups of rows that each meet their own n_mats (1 or 2)
 // matrices: group e owns the grouped rows offsets[e] .. offsets[e+1]; grouped row p multiplies activation row
 // xrow[p] / xdiv of x (xrow null: row p itself); matrix k's [. x rows] result goes to out[k] at the grouped row.  m: the
@@ -370,4 +372,4 @@ int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_p
 int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                                       size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
                                       const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
-                                      float *keep_u, void *stream);
+                                      float *keep_u, void *stream, const uint8_t *const *w1st = nullptr, const uint8_t *const *w3st = nullptr);

@@ -32,7 +32,8 @@ int mk_vq1_grouped_sweep(const float *lut, const int32_t *vec_index, const uint8
 
 int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t rows, size_t cols,
                    const int8_t *xq, const float *xs, const int32_t *arow, const int32_t *goff, const int32_t *gexp, const int32_t *ngroups,
-                   const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream);
+                   const int32_t *gbig, size_t max_groups, size_t max_group_rows, float *const *out, void *stream,
+                   const uint8_t *const *const *scales_t_ptrs);
 
 namespace {
 
@@ -814,7 +815,10 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
             const uint8_t *const *pp[2] = {table->w1p, table->w3p};
             const uint8_t *const *sp[2] = {table->w1s, table->w3s};
             float *gu[2] = {w.g, w.u};
-            if ((s = mk_q8x_grouped(2, pp, sp, inter, d, w.xq, w.xs, w.rtok, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, gu, stream)) != MK_OK) return s;
+            const uint8_t *const *tp[2] = {table->w1st, table->w3st};
+            if ((s = mk_q8x_grouped(2, pp, sp, inter, d, w.xq, w.xs, w.rtok, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, gu, stream,
+                                    table->w1st && table->w3st ? tp : nullptr)) != MK_OK)
+                return s;
         }
         {
             const size_t n_blocks = P * inter / 32;
@@ -828,7 +832,10 @@ int moe_decode_impl(const mk_expert_table *table, size_t B, size_t topk, const i
             const uint8_t *const *pp[1] = {table->w2p};
             const uint8_t *const *sp[1] = {table->w2s};
             float *oo[1] = {w.o};
-            if ((s = mk_q8x_grouped(1, pp, sp, d, inter, w.aq, w.as, nullptr, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, oo, stream)) != MK_OK) return s;
+            const uint8_t *const *tp[1] = {table->w2st};
+            if ((s = mk_q8x_grouped(1, pp, sp, d, inter, w.aq, w.as, nullptr, w.goff, w.gexp, w.ngroups, w.ngroups + 1, P, B, oo, stream,
+                                    table->w2st ? tp : nullptr)) != MK_OK)
+                return s;
         }
         hipLaunchKernelGGL(moe_combine_grouped_kernel, dim3((unsigned)((d + 255) / 256), (unsigned)B), dim3(256), 0, st, w.o, w.pt.pw, w.pos, per,
                            (int)topk, (int)d, act_kind == MK_ACT_DS ? 1 : 0, out);

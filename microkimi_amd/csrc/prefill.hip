@@ -306,18 +306,28 @@ int moe_prefill_impl(const mk_expert_table *table, size_t n_experts, size_t T, s
     s = MK_TUNE("MK_PREFILL_SEPARATE", 0) ? MK_ERR_UNSUPPORTED
                                          : mk_mxfp4_grouped_gemm_gate_up_act(table->w1p, table->w1s, table->w3p, table->w3s, n_experts, inter, d, w.codes,
                                                                              w.exps, w.offsets, P, act_kind, w.codes2, w.exps2, keep ? w.g : nullptr,
-                                                                             keep ? w.u : nullptr, stream);
+                                                                             keep ? w.u : nullptr, stream, table->w1st, table->w3st);
     if (s == MK_ERR_UNSUPPORTED) {
         const uint8_t *const *pp[2] = {table->w1p, table->w3p};
         const uint8_t *const *sp[2] = {table->w1s, table->w3s};
         float *gu[2] = {w.g, w.u};
-        if ((s = mk_mxfp4_grouped_gemm_n(2, pp, sp, n_experts, inter, d, w.codes, w.exps, w.offsets, P, gu, stream)) != MK_OK) return s;
+        const uint8_t *const *tp[2] = {table->w1st, table->w3st};
+        if ((s = mk_mxfp4_grouped_gemm_n(2, pp, sp, n_experts, inter, d, w.codes, w.exps, w.offsets, P, gu, stream,
+                                         table->w1st && table->w3st ? tp : nullptr)) != MK_OK)
+            return s;
         hipLaunchKernelGGL(prefill_act_mxfp8_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
                            (int)n_experts, (int)inter, act_kind, w.codes2, w.exps2);
         s = mk_launch_status("prefill_act_mxfp8");
     }
     if (s != MK_OK) return s;
-    if ((s = mk_dev_mxfp4_grouped_gemm(table->w2p, table->w2s, n_experts, d, inter, w.codes2, w.exps2, w.offsets, P, w.o, stream)) != MK_OK) return s;
+    {
+        const uint8_t *const *pd[1] = {table->w2p};
+        const uint8_t *const *sd[1] = {table->w2s};
+        const uint8_t *const *td[1] = {table->w2st};
+        float *od[1] = {w.o};
+        if ((s = mk_mxfp4_grouped_gemm_n(1, pd, sd, n_experts, d, inter, w.codes2, w.exps2, w.offsets, P, od, stream, table->w2st ? td : nullptr)) != MK_OK)
+            return s;
+    }
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");

@@ -281,7 +281,13 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     const bool with_pack = !any_vq && (d == 7168 || d == 5120) && inter == 2048 && pk2 > 0 && mk_env_int("MK_EXPERT_PACK", 1) != 0;
     const size_t pack_off = off;
     if (with_pack) off += (pk13 + pk2) * n_experts;
-    const size_t tab_off = off, total = off + 8 * n_experts * sizeof(void *);
+    // and every matrix's scale bytes in K-tile order for the matrix-core kernels (mk_dev_mxfp4_scales_by_tile), when the shapes
+    // allow it and MK_EXPERT_SCALE_TILES is not 0: 1/16 of the experts' bytes again
+    const size_t st_per = align_up(d * inter / 32, 256);
+    const bool with_st = !any_vq && d % 512 == 0 && inter % 512 == 0 && mk_env_int("MK_EXPERT_SCALE_TILES", 1) != 0;
+    const size_t st_off = off;
+    if (with_st) off += 3 * st_per * n_experts;
+    const size_t tab_off = off, total = off + 11 * n_experts * sizeof(void *);
     mk_expert_set *s = new mk_expert_set;
     if (hipMalloc(&s->dev, total) != hipSuccess) {
         (void)hipGetLastError();
@@ -293,7 +299,7 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->n = n_experts;
     uint8_t *base = (uint8_t *)s->dev;
     // pass 2: one copy per blob straight out of the mapping, then the pointer arrays
-    std::vector<const uint8_t *> ptrs(8 * n_experts, nullptr);
+    std::vector<const uint8_t *> ptrs(11 * n_experts, nullptr);
     for (size_t e = 0; e < n_experts; e++) {
         for (int k = 0; k < 3; k++) {
             const Blob &b = blobs[e * 3 + k];
@@ -317,7 +323,17 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
         ptrs[6 * n_experts + e] = t13;
         ptrs[7 * n_experts + e] = t2;
     }
-    if (with_pack && hipDeviceSynchronize() != hipSuccess) {
+    for (size_t e = 0; with_st && e < n_experts; e++) {
+        for (int k = 0; k < 3; k++) {
+            uint8_t *t = base + st_off + (3 * e + k) * st_per;
+            if (mk_dev_mxfp4_scales_by_tile(ptrs[(size_t)(2 * k + 1) * n_experts + e], k == 2 ? d : inter, k == 2 ? inter : d, t, nullptr) != MK_OK) {
+                mk_expert_set_free(s);
+                return MK_ERR_HIP;
+            }
+            ptrs[(size_t)(8 + k) * n_experts + e] = t;
+        }
+    }
+    if ((with_pack || with_st) && hipDeviceSynchronize() != hipSuccess) {
         (void)hipGetLastError();
         mk_expert_set_free(s);
         mk_set_error("the packed copies of the experts failed");
@@ -348,6 +364,9 @@ extern "C" int mk_bin_load_experts(const mk_binfile *f, const char *layer_prefix
     s->table.vq_codebook = any_vq ? reinterpret_cast<const float *>(base + cb_off) : nullptr;
     s->table.w13t = with_pack ? tab + 6 * n_experts : nullptr;
     s->table.w2t = with_pack ? tab + 7 * n_experts : nullptr;
+    s->table.w1st = with_st ? tab + 8 * n_experts : nullptr;
+    s->table.w3st = with_st ? tab + 9 * n_experts : nullptr;
+    s->table.w2st = with_st ? tab + 10 * n_experts : nullptr;
     *out = s;
     return MK_OK;
 }

@@ -200,9 +200,11 @@ class PackedExperts:
     the file's 256 x 16 f32 `vq_codebook`.  Built from lists of device tensors.  pack: also keep every expert's matrices
     in the order the one-launch decode kernel streams them (mk_dev_moe_pack_gate_up / _down; as many bytes again), which
     lets up to 3 decode tokens take that kernel (calls on it must not overlap on one device); None = when the shapes are
-    the ones it takes (d 7168 or 5120, inter 2048) and no expert is VQ1."""
+    the ones it takes (d 7168 or 5120, inter 2048) and no expert is VQ1.  scales_by_tile: also keep every matrix's scale
+    bytes in K-tile order (mk_dev_mxfp4_scales_by_tile; 1/16 of the experts' bytes again) for the matrix-core kernels of
+    moe_decode from 4 tokens and of moe_prefill; None = when d and inter are multiples of 512 and no expert is VQ1."""
 
-    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, pack=None):
+    def __init__(self, w1, w3, w2, d, inter, vq_codebook=None, pack=None, scales_by_tile=None):
         import torch
         self.d, self.inter, self.n = d, inter, len(w1)
         self._keep = (w1, w3, w2, vq_codebook)
@@ -230,7 +232,24 @@ class PackedExperts:
                 check(lib.mk_dev_moe_pack_down(ptr(w2[i][0]), ptr(w2[i][1]), d, inter, at + b13, cur_stream()))
             self._tptrs = [torch.tensor([base + i * (b13 + b2) + k * b13 for i in range(self.n)], dtype=torch.int64, device=dev) for k in (0, 1)]
             tptrs = [p.data_ptr() for p in self._tptrs]
-        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None, *tptrs)
+        # the scale bytes once more in K-tile order for the matrix-core kernels (None = when the shapes allow it)
+        st_fits = not any_vq and d % 512 == 0 and inter % 512 == 0
+        if scales_by_tile is None:
+            scales_by_tile = st_fits
+        stptrs = [None, None, None]
+        if scales_by_tile:
+            if not st_fits:
+                raise ValueError("the K-tile ordered scale bytes need MXFP4 experts with d and inter multiples of 512")
+            per = d * inter // 32
+            self._st = torch.empty(self.n * 3 * per, dtype=torch.uint8, device=dev)
+            base = self._st.data_ptr()
+            for i in range(self.n):
+                for k, (lst, r, c) in enumerate(((w1, inter, d), (w3, inter, d), (w2, d, inter))):
+                    check(lib.mk_dev_mxfp4_scales_by_tile(ptr(lst[i][1]), r, c, base + (3 * i + k) * per, cur_stream()))
+            self._stptrs = [torch.tensor([base + (3 * i + k) * per for i in range(self.n)], dtype=torch.int64, device=dev) for k in range(3)]
+            stptrs = [p.data_ptr() for p in self._stptrs]
+        self.table = ExpertTable(*[p.data_ptr() for p in self._ptrs], d, inter, self.n, vq_codebook.data_ptr() if self.has_vq else None, *tptrs,
+                                 *stptrs)
         self._ws = None
 
 

@@ -51,6 +51,10 @@ pub struct MkExpertTable {
     /// (mk_dev_moe_pack_gate_up, mk_dev_moe_pack_down)
     pub w13t: *const *const u8,
     pub w2t: *const *const u8,
+    /// optional (each on its own): per expert, the scale bytes of W1, W3, W2 in K-tile order (mk_dev_mxfp4_scales_by_tile)
+    pub w1st: *const *const u8,
+    pub w3st: *const *const u8,
+    pub w2st: *const *const u8,
 }
 
 /// mk_bin_entry: one directory entry of an MKIM file (weights::Entry, src/weights.rs:31-37).
@@ -121,6 +125,7 @@ extern "C" {
     pub fn mk_force_q8(v: c_int);
     pub fn mk_q8_enabled() -> c_int;
     pub fn mk_dev_mxfp4_dequant(packed: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4_scales_by_tile(scales: *const u8, rows: usize, cols: usize, out: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_moe_pack_bytes(d: usize, inter: usize, down: c_int) -> usize;
     pub fn mk_dev_moe_pack_gate_up(w1p: *const u8, w1s: *const u8, w3p: *const u8, w3s: *const u8, d: usize, inter: usize, pack: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_dev_moe_unpack_gate_up(pack: *const u8, d: usize, inter: usize, w1p: *mut u8, w1s: *mut u8, w3p: *mut u8, w3s: *mut u8, stream: *mut c_void) -> c_int;

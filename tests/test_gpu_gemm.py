@@ -219,6 +219,32 @@ def test_moe_prefill_bf16_on_device(T, topk, n_experts, d, inter, act):
             assert rel_l2(mid[name][r], Wd @ xb) <= 1e-5, (name, r)
 
 
+@pytest.mark.parametrize("T,topk,n_experts,d,inter", [(40, 2, 4, 1024, 512), (300, 3, 5, 512, 1024)])
+def test_moe_prefill_mxfp8_with_and_without_the_tile_ordered_scale_bytes(T, topk, n_experts, d, inter):
+    # the MXFP8 section's kernels read the same scale bytes from either place: the same bits, intermediates included
+    from microkimi_amd import model, workloads
+    rng = np.random.default_rng(T + d)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    w1, w3, w2 = pk(0), pk(1), pk(2)
+    x = dev((rng.standard_normal((T, d)) * 0.05).astype(np.float32))
+    ids = dev(np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.int32))
+    wts = dev(rng.random((T, topk)).astype(np.float32))
+    res = []
+    for tiles in (True, False):
+        experts = model.PackedExperts(w1, w3, w2, d, inter, scales_by_tile=tiles)
+        assert bool(experts.table.w1st) == tiles
+        for keep in (False, True):
+            out = model.moe_prefill(experts, ids, wts, x, mxfp8=True, keep=keep).cpu().numpy()
+            mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()} if keep else {}
+            res.append((out, mid))
+    for (a, ma), (b, mb) in zip(res[:2], res[2:]):
+        assert np.isfinite(a).all() and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        for k in ma:
+            assert np.array_equal(ma[k].view(np.uint32), mb[k].view(np.uint32)), k
+
+
 def test_moe_prefill_bf16_refuses_other_shapes():
     # d or inter not in multiples of 512, or a layer with VQ1 experts: MK_ERR_UNSUPPORTED, nothing computed
     from microkimi_amd import model, workloads

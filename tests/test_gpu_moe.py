@@ -361,6 +361,42 @@ def test_batched_path_all_tokens_on_the_same_experts():
     rows_match_up_to_q8_flips(got, want, lambda t: [w2_dev[2], w2_dev[0], w2_dev[shared]], d, inter)
 
 
+def test_scale_bytes_by_tile_are_the_same_bytes():
+    # out[(t * rows + r) * 16 + j] = scales[r * (cols / 32) + 16 t + j]; a cols that is not a multiple of 512 is refused
+    from microkimi_amd import _lib
+    import torch
+    rng = np.random.default_rng(5)
+    for rows, cols in ((1, 512), (37, 1024), (256, 7168), (300, 2048)):
+        sc = rng.integers(0, 256, size=(rows, cols // 32), dtype=np.uint8)
+        out = torch.zeros(rows * cols // 32, dtype=torch.uint8, device="cuda")
+        _lib.check(_lib.lib.mk_dev_mxfp4_scales_by_tile(_lib.ptr(dev(sc)), rows, cols, _lib.ptr(out), None))
+        torch.cuda.synchronize()
+        want = sc.reshape(rows, cols // 512, 16).transpose(1, 0, 2)
+        assert np.array_equal(out.cpu().numpy().reshape(cols // 512, rows, 16), want)
+    st = _lib.lib.mk_dev_mxfp4_scales_by_tile(_lib.ptr(out), 4, 768, _lib.ptr(out), None)
+    assert st == -1 and b"512" in _lib.lib.mk_last_error()
+
+
+@pytest.mark.parametrize("B,topk,shared", [(4, 2, -1), (16, 3, 5), (13, 2, 3)])
+def test_batched_path_with_and_without_the_tile_ordered_scale_bytes(B, topk, shared):
+    """The matrix-core path reads the scale bytes from the K-tile ordered copies when the table has them and from the
+    reference layout when it has not: the same bytes, so the same bits."""
+    from microkimi_amd import model
+    d, inter, n_experts = 1024, 512, 6
+    host = build(n_experts, d, inter)[1]._keep
+    with_st = model.PackedExperts(host[0], host[1], host[2], d, inter, scales_by_tile=True)
+    without = model.PackedExperts(host[0], host[1], host[2], d, inter, scales_by_tile=False)
+    assert with_st.table.w1st and with_st.table.w3st and with_st.table.w2st
+    assert not (without.table.w1st or without.table.w3st or without.table.w2st)
+    rng = np.random.default_rng(B * 7 + topk)
+    ids = np.stack([rng.permutation(5)[:topk] for _ in range(B)]).astype(np.int32)
+    wts = rng.random((B, topk)).astype(np.float32)
+    x = (rng.standard_normal((B, d)) * 0.02).astype(np.float32)
+    a = model.moe_decode(with_st, dev(ids), dev(wts), dev(x), shared=shared, mode=1).cpu().numpy()
+    b = model.moe_decode(without, dev(ids), dev(wts), dev(x), shared=shared, mode=1).cpu().numpy()
+    assert np.isfinite(a).all() and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_moe_decode_f32_mode():
     from microkimi_amd import model
     d, inter, n_experts, B, topk = 2048, 1024, 6, 2, 3
