@@ -678,6 +678,7 @@ typedef __bf16 mk_bf2 __attribute__((ext_vector_type(2)));
 struct Bf16GroupedArgs {
     const uint8_t *const *packed[2];
     const uint8_t *const *scales[2];
+    const uint8_t *const *scales_t[2];  // optional: the scale bytes in [K tile][row][16] order (16-byte aligned), read instead
     float *out[2];
     const uint16_t *x;       // [grouped rows][cols] bf16
     const int32_t *offsets;  // [groups + 1]
@@ -715,13 +716,16 @@ __global__ __launch_bounds__(64 * RW) __attribute__((amdgpu_waves_per_eu(4))) vo
 #pragma unroll
     for (int h = 0; h < 2; h++) wline[h] = packed + (size_t)min(row0 + 8 * h + (lane >> 3), a.rows - 1) * (cols / 2) + (lane & 7) * 16;
     const int rot_idx = (((lane & 7) << 3) | (((lane >> 3) & 1) << 2) | (lane >> 4)) * 4;
-    const uint8_t *srow = scales + (size_t)min(row0 + i, a.rows - 1) * nb;
-    const int sc_al = ((uintptr_t)scales & 15) == 0 ? 16 : ((uintptr_t)scales & 3) == 0 ? 4 : 1;  // (nb % 16 == 0)
+    // a wave's 16 rows x 16 scale bytes of a K tile: 16 eighths of lines in the reference layout, two whole lines in K-tile order
+    const uint8_t *scales_t = a.scales_t[mat] ? a.scales_t[mat][grp] : nullptr;
+    const uint8_t *srow = scales_t ? scales_t + (size_t)min(row0 + i, a.rows - 1) * 16 : scales + (size_t)min(row0 + i, a.rows - 1) * nb;
+    const size_t sstep = scales_t ? (size_t)a.rows * 16 : 16;
+    const int sc_al = scales_t || ((uintptr_t)scales & 15) == 0 ? 16 : ((uintptr_t)scales & 3) == 0 ? 4 : 1;  // (nb % 16 == 0)
     auto load_w = [&](int kt, mk_i4 (&wl)[4], mk_i4 &sc) {
         const size_t ku = (size_t)min(kt, ktiles - 1);
 #pragma unroll
         for (int j = 0; j < 4; j++) wl[j] = mk_ldg128_nt(wline[j & 1] + ku * 256 + (j >> 1) * 128);
-        const uint8_t *sp = srow + ku * 16;  // the scale bytes of the row's 16 blocks in the K tile
+        const uint8_t *sp = srow + ku * sstep;  // the scale bytes of the row's 16 blocks in the K tile
         if (sc_al == 16) sc = *reinterpret_cast<const mk_i4 *>(sp);
         else if (sc_al == 4) sc = mk_i4{(int)mk_ldg_u32(sp), (int)mk_ldg_u32(sp + 4), (int)mk_ldg_u32(sp + 8), (int)mk_ldg_u32(sp + 12)};
         else {
@@ -991,7 +995,8 @@ int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptr
 }
 
 int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
-                               size_t rows, size_t cols, const uint16_t *x, const int32_t *offsets, float *const *out, void *stream) {
+                               size_t rows, size_t cols, const uint16_t *x, const int32_t *offsets, float *const *out, void *stream,
+                               const uint8_t *const *const *scales_t_ptrs) {
     MK_REQUIRE((n_mats == 1 || n_mats == 2) && packed_ptrs && scales_ptrs && x && offsets && out, "bad argument");
     if (cols == 0 || cols % 512 != 0 || rows % 4 != 0) {
         mk_set_error("the bf16 grouped product takes cols % 512 == 0 and rows % 4 == 0");
@@ -1002,6 +1007,7 @@ int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_p
     for (int k = 0; k < n_mats; k++) {
         MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k] && ((uintptr_t)out[k] & 15) == 0, "null or unaligned pointer");
         a.packed[k] = packed_ptrs[k], a.scales[k] = scales_ptrs[k], a.out[k] = out[k];
+        a.scales_t[k] = scales_t_ptrs ? scales_t_ptrs[k] : nullptr;
     }
     a.x = x, a.offsets = offsets, a.rows = (int)rows, a.nb = (int)(cols / 32);
     constexpr int RW = 8;
@@ -1020,7 +1026,7 @@ extern "C" int mk_dev_mxfp4_grouped_gemm_bf16(const uint8_t *const *packed_ptrs,
                                               size_t cols, const uint16_t *x, const int32_t *offsets, size_t m, float *out, void *stream) {
     MK_REQUIRE(packed_ptrs && scales_ptrs && x && offsets && out, "null pointer");
     (void)m;
-    return mk_mxfp4_grouped_gemm_bf16(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, x, offsets, &out, stream);
+    return mk_mxfp4_grouped_gemm_bf16(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, x, offsets, &out, stream, nullptr);
 }
 
 extern "C" int mk_dev_mxfp4_matvec_nt(const uint8_t *packed, const uint8_t *scales, size_t rows, size_t cols, const float *x, size_t m,

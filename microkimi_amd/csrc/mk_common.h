@@ -364,8 +364,10 @@ int mk_mxfp4_grouped_gemm_nt(int n_mats, const uint8_t *const *const *packed_ptr
                              const float *vq_codebook, float *const *out, void *stream);
 // The grouped product with bfloat16 activation rows x [grouped rows][cols] (gemv_mxfp4.hip): exact bf16 weights, f32
 // products and sums on the bf16 matrix instruction.  MK_ERR_UNSUPPORTED unless cols % 512 == 0 and rows % 4 == 0.
+// scales_t_ptrs: as for mk_mxfp4_grouped_gemm_n.
 int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
-                               size_t rows, size_t cols, const uint16_t *x, const int32_t *offsets, float *const *out, void *stream);
+                               size_t rows, size_t cols, const uint16_t *x, const int32_t *offsets, float *const *out, void *stream,
+                               const uint8_t *const *const *scales_t_ptrs = nullptr);
 // The gate and up matrices of every group against the same token rows, the activation ACT(gate, up) and its MXFP8 form
 // (e4m3 codes [m][rows], e8m0 bytes [m][rows / 32], whole exponent range) in one launch; the f32 gate / up rows are
 // written too when keep_g and keep_u are given.  MK_ERR_UNSUPPORTED (nothing launched) for shapes it does not take.

@@ -404,7 +404,9 @@ extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_ex
     const uint8_t *const *pp[2] = {table->w1p, table->w3p};
     const uint8_t *const *sp[2] = {table->w1s, table->w3s};
     float *gu[2] = {w.g, w.u};
-    if ((s = mk_mxfp4_grouped_gemm_bf16(2, pp, sp, n_experts, inter, d, w.xb, w.offsets, gu, stream)) != MK_OK) return s;
+    const uint8_t *const *tp[2] = {table->w1st, table->w3st};
+    if ((s = mk_mxfp4_grouped_gemm_bf16(2, pp, sp, n_experts, inter, d, w.xb, w.offsets, gu, stream, table->w1st && table->w3st ? tp : nullptr)) != MK_OK)
+        return s;
     // (the hidden rows are used up: the activation rows take their place)
     hipLaunchKernelGGL(prefill_act_bf16_kernel, dim3((unsigned)((P * (inter / 8) + 255) / 256)), dim3(256), 0, st, w.g, w.u, w.offsets,
                        (int)n_experts, (int)inter, act_kind, w.xb);
@@ -412,7 +414,8 @@ extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_ex
     const uint8_t *const *pd[1] = {table->w2p};
     const uint8_t *const *sd[1] = {table->w2s};
     float *od[1] = {w.o};
-    if ((s = mk_mxfp4_grouped_gemm_bf16(1, pd, sd, n_experts, d, inter, w.xb, w.offsets, od, stream)) != MK_OK) return s;
+    const uint8_t *const *td[1] = {table->w2st};
+    if ((s = mk_mxfp4_grouped_gemm_bf16(1, pd, sd, n_experts, d, inter, w.xb, w.offsets, od, stream, table->w2st ? td : nullptr)) != MK_OK) return s;
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");

@@ -220,8 +220,8 @@ def test_moe_prefill_bf16_on_device(T, topk, n_experts, d, inter, act):
 
 
 @pytest.mark.parametrize("T,topk,n_experts,d,inter", [(40, 2, 4, 1024, 512), (300, 3, 5, 512, 1024)])
-def test_moe_prefill_mxfp8_with_and_without_the_tile_ordered_scale_bytes(T, topk, n_experts, d, inter):
-    # the MXFP8 section's kernels read the same scale bytes from either place: the same bits, intermediates included
+def test_moe_prefill_with_and_without_the_tile_ordered_scale_bytes(T, topk, n_experts, d, inter):
+    # the MXFP8 and bf16 sections' kernels read the same scale bytes from either place: the same bits, intermediates included
     from microkimi_amd import model, workloads
     rng = np.random.default_rng(T + d)
     host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
@@ -239,7 +239,9 @@ def test_moe_prefill_mxfp8_with_and_without_the_tile_ordered_scale_bytes(T, topk
             out = model.moe_prefill(experts, ids, wts, x, mxfp8=True, keep=keep).cpu().numpy()
             mid = {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()} if keep else {}
             res.append((out, mid))
-    for (a, ma), (b, mb) in zip(res[:2], res[2:]):
+        out = model.moe_prefill(experts, ids, wts, x, bf16=True).cpu().numpy()
+        res.append((out, {k: v.cpu().numpy() for k, v in model.moe_prefill_intermediates(experts, T, topk).items()}))
+    for (a, ma), (b, mb) in zip(res[:3], res[3:]):
         assert np.isfinite(a).all() and np.array_equal(a.view(np.uint32), b.view(np.uint32))
         for k in ma:
             assert np.array_equal(ma[k].view(np.uint32), mb[k].view(np.uint32)), k
