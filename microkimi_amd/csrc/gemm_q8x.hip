@@ -46,9 +46,9 @@ struct Q8xArgs {
     const int32_t *goff;    // [groups + 1] first grouped row of every group
     const int32_t *gexp;    // [groups] expert id
     const int32_t *ngroups; // number of groups (device)
-    const int32_t *gbig;    // the group with the most rows (device): its passes beyond the first get workgroups of their own
+    const int32_t *gbig;    // the group with the most rows (device): every one of its passes gets workgroups of its own
     int regular;            // workgroups of the regular part of the grid (groups x matrices x row blocks)
-    int extra_sets;         // sets of workgroups behind it that take the later passes of the largest group in turn
+    int extra_sets;         // passes of the largest group beyond the first (0: it is a regular group like the others)
     float *out[2];          // [grouped rows][rows]
     int n_mats, row_blocks;
 };
@@ -248,24 +248,34 @@ template <int WAVES>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3))) void q8x_grouped_kernel(Q8xArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int per_group = a.n_mats * a.row_blocks;
-    // Regular workgroups: (group, matrix, row block), all passes of the group one after the other -- except for the
-    // group with the most rows (in a decode batch the shared expert, which has every token): the regular workgroup
-    // takes its first pass and the workgroups behind the regular part of the grid take one later pass each, so that
-    // this group's workgroups do not run several times as long as the others.
+    // The group with the most rows (in a decode batch the shared expert, which has every token) comes first and has one
+    // workgroup per (matrix, row block, pass): workgroup ids go round the eight XCDs in turn, so the passes of a row block
+    // get ids 8 apart -- same XCD, dispatched together -- and walk the same weight lines at the same time: one of them
+    // fetches a line from HBM, the others find it in their XCD's L2.  Behind them the regular workgroups: (group, matrix,
+    // row block), all passes of the group one after the other.
     int gi, r0, first_pass, pass_step;
     const int big = *a.gbig;
-    if ((int)blockIdx.x < a.regular) {
-        gi = blockIdx.x / per_group;
-        r0 = blockIdx.x % per_group;
-        if (gi >= *a.ngroups) return;
-        first_pass = 0;
-        pass_step = (gi == big && a.extra_sets > 0) ? 0x10000 : 1;
-    } else {
-        const int x = blockIdx.x - a.regular;
+    const int passes = a.extra_sets + 1, nbig = a.extra_sets > 0 ? passes * per_group : 0;
+    if ((int)blockIdx.x < nbig) {
+        const int x = blockIdx.x, blk = x / (8 * passes), in = x % (8 * passes);
+        const int full = per_group / 8 * 8;  // (the row blocks beyond the last whole set of eight: pass-major)
+        if (blk * 8 < full) {
+            r0 = blk * 8 + (in & 7);
+            first_pass = in >> 3;
+        } else {
+            const int y = x - full * passes, rem = per_group - full;
+            r0 = full + y % rem;
+            first_pass = y / rem;
+        }
         gi = big;
+        pass_step = 0x10000;  // whatever the group's size, every pass is taken by exactly one workgroup
+    } else {
+        const int x = blockIdx.x - nbig;
+        gi = x / per_group;
         r0 = x % per_group;
-        first_pass = 1 + x / per_group;
-        pass_step = a.extra_sets;  // whatever the group's size, every pass is taken by exactly one workgroup
+        if (gi >= *a.ngroups || (gi == big && nbig > 0)) return;
+        first_pass = 0;
+        pass_step = 1;
     }
     const int m = r0 / a.row_blocks, rb = r0 % a.row_blocks;
     const int tok0 = a.goff[gi], tok1 = a.goff[gi + 1];
@@ -312,7 +322,7 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     const size_t wg_rows = 64 * (size_t)waves;
     a.row_blocks = (int)((rows + wg_rows - 1) / wg_rows);
     const size_t passes = (max_group_rows + QX_TOK - 1) / QX_TOK;
-    const size_t regular = max_groups * n_mats * a.row_blocks, grid = regular + (passes - 1) * n_mats * a.row_blocks;
+    const size_t regular = max_groups * n_mats * a.row_blocks, grid = regular + (passes > 1 ? passes : 0) * n_mats * a.row_blocks;
     MK_REQUIRE(passes >= 1 && grid < 0x7FFFFFFFull, "too many workgroups");
     a.regular = (int)regular;
     a.extra_sets = (int)(passes - 1);
