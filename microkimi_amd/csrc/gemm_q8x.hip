@@ -255,18 +255,13 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(3)))
     // row block), all passes of the group one after the other.
     int gi, r0, first_pass, pass_step;
     const int big = *a.gbig;
-    const int passes = a.extra_sets + 1, nbig = a.extra_sets > 0 ? passes * per_group : 0;
+    const int passes = a.extra_sets + 1, nbig = a.extra_sets > 0 ? passes * ((per_group + 7) / 8 * 8) : 0;
     if ((int)blockIdx.x < nbig) {
+        // (row blocks padded to whole sets of eight: the workgroups of the padding leave at once)
         const int x = blockIdx.x, blk = x / (8 * passes), in = x % (8 * passes);
-        const int full = per_group / 8 * 8;  // (the row blocks beyond the last whole set of eight: pass-major)
-        if (blk * 8 < full) {
-            r0 = blk * 8 + (in & 7);
-            first_pass = in >> 3;
-        } else {
-            const int y = x - full * passes, rem = per_group - full;
-            r0 = full + y % rem;
-            first_pass = y / rem;
-        }
+        r0 = blk * 8 + (in & 7);
+        if (r0 >= per_group) return;
+        first_pass = in >> 3;
         gi = big;
         pass_step = 0x10000;  // whatever the group's size, every pass is taken by exactly one workgroup
     } else {
@@ -322,7 +317,8 @@ int mk_q8x_grouped(int n_mats, const uint8_t *const *const *packed_ptrs, const u
     const size_t wg_rows = 64 * (size_t)waves;
     a.row_blocks = (int)((rows + wg_rows - 1) / wg_rows);
     const size_t passes = (max_group_rows + QX_TOK - 1) / QX_TOK;
-    const size_t regular = max_groups * n_mats * a.row_blocks, grid = regular + (passes > 1 ? passes : 0) * n_mats * a.row_blocks;
+    const size_t per_group = (size_t)n_mats * a.row_blocks;
+    const size_t regular = max_groups * per_group, grid = regular + (passes > 1 ? passes : 0) * ((per_group + 7) / 8 * 8);
     MK_REQUIRE(passes >= 1 && grid < 0x7FFFFFFFull, "too many workgroups");
     a.regular = (int)regular;
     a.extra_sets = (int)(passes - 1);
