@@ -282,14 +282,22 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     const uint32_t eoff = (uint32_t)min(base + (tid & (16 * MC - 1)), tok1 - 1) * (uint32_t)nb;
     auto stage_load = [&](int kt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
+#ifdef MK_GEMM_FP4_PROBE
+        constexpr int STG = MC >= 4 ? MC : 2 * MC;  // (half the bytes a token row has in a K tile)
+#else
+        constexpr int STG = 2 * MC;
+#endif
 #pragma unroll
-        for (int k = 0; k < 2 * MC; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
+        for (int k = 0; k < STG; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
         ste = mk_ldg128_off(a.exps, eoff + ku * 16);
         stw = mk_ldg128_off(ws_base, wsoff + ku * ws_step);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
         for (int k = 0; k < 2 * MC; k++) {
+#ifdef MK_GEMM_FP4_PROBE
+            if (MC >= 4 && k >= MC) break;
+#endif
             const int i = tid + 256 * k;
             *reinterpret_cast<mk_i4 *>(buf + (i >> 5) * A_STRIDE + (i & 31) * 16) = st[k];
         }
@@ -336,12 +344,20 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 #pragma unroll
             for (int s = 0; s < KT_STEPS; s++) {
                 const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + s * 128);
+#ifdef MK_GEMM_FP4_PROBE
+                // timing only (the results mean nothing): the activation operand taken as e2m1 -- 16 bytes a lane instead of
+                // 32, both operands fp4, the instruction at its fp4 rate -- to see what MXFP4 activations would buy
+                const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], 0, 0, 0, 0};
+                constexpr int AFMT = 4;
+#else
                 const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + s * 128 + 64);
                 const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                constexpr int AFMT = 0;
+#endif
                 const int asb = ae[s * 4];
                 const mk_i8v b0 = {w0[s][0], w0[s][1], w0[s][2], w0[s][3], 0, 0, 0, 0}, b1 = {w1[s][0], w1[s][1], w1[s][2], w1[s][3], 0, 0, 0, 0};
-                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b0, av, acc[rt][c], 4, 0, 0, (int)sc0[s * 4], 0, asb);
-                acc[rt + 1][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b1, av, acc[rt + 1][c], 4, 0, 0, (int)sc1[s * 4], 0, asb);
+                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b0, av, acc[rt][c], 4, AFMT, 0, (int)sc0[s * 4], 0, asb);
+                acc[rt + 1][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b1, av, acc[rt + 1][c], 4, AFMT, 0, (int)sc1[s * 4], 0, asb);
             }
         }
     };
