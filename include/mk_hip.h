@@ -101,6 +101,16 @@ int mk_dev_quantize_q8(const float *x, size_t nvec, size_t n, int8_t *q, float *
  * is the activation format of mk_dev_mxfp4_grouped_gemm. */
 int mk_dev_quantize_mxfp8(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream);
 
+/* bfloat16 (round to nearest even) of `nvec` rows of `n` floats, every value as the sum of TWO e4m3 terms with an e8m0
+ * block exponent each per 32 values: hi = the leading four significant bits of the bfloat16 value, lo = the other four;
+ * hi * 2^(eh - 127) + lo * 2^(el - 127) is the bfloat16 value exactly unless it lies more than 2^13 below the largest of
+ * its block (then its last bits round off, an error below 2^-17 of that largest value); a value that is not finite
+ * becomes the e4m3 NaN.  Layout per row and K tile of 512 values: codes [n / 512][2][512] (hi row, lo row), exps
+ * [n / 512][2][16].  This is the activation format of mk_dev_mxfp4_grouped_gemm_split and, inside, of
+ * mk_dev_moe_prefill_bf16: bfloat16 activations on the block-scaled matrix instruction (no counterpart in the
+ * reference, whose prefill is f32: src/model.rs:2412-2447).  n % 512 == 0; x 16-byte, codes 8-byte aligned. */
+int mk_dev_quantize_bf16_split(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream);
+
 /* mxfp4::quantize (search != 0) / quantize_naive (search == 0) (src/mxfp4.rs:38-138): per 32-group
  * e = ceil(log2(maxabs / 6)) clamped to [-127, 128], with `search` the better of e - 1, e, e + 1 by squared error in f64
  * (e wins ties), nearest E2M1 level by the midpoints, sign from the sign bit.  w [rows][cols] f32 ->
@@ -425,6 +435,17 @@ int mk_dev_mxfp4_grouped_gemm_f32(const uint8_t *const *packed_ptrs, const uint8
 int mk_dev_mxfp4_grouped_gemm_bf16(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
                                    size_t cols, const uint16_t *x, const int32_t *offsets, size_t m, float *out, void *stream);
 
+/* mk_dev_mxfp4_grouped_gemm with bfloat16 token rows in the two-term form of mk_dev_quantize_bf16_split (codes
+ * [m][cols / 512][2][512], exps [m][cols / 512][2][16], 16-byte aligned): both terms of a value meet the same weight
+ * registers on v_mfma_scale_f32_16x16x128_f8f6f4 and are summed in f32, so y[i][r] = sum_k dequant(W_e)[r][k] * bf16(x)[i][k]
+ * (matvec_packed_nt of src/model.rs:2412-2447 on bfloat16-rounded rows) up to the arithmetic of the instruction, which
+ * keeps fewer bits of a step's 128 products than a chain of f32 additions would: relative L2 about 1e-5 over a group,
+ * up to 3e-5 measured on single rows with a wide range of magnitudes (the bfloat16 rounding of the rows themselves is
+ * 2e-3).  Groups of any size (passes of 32 rows).  MK_ERR_UNSUPPORTED unless cols % 512 == 0. */
+int mk_dev_mxfp4_grouped_gemm_split(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                    size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
+                                    void *stream);
+
 /* Bytes of device scratch mk_dev_moe_prefill needs. */
 size_t mk_moe_prefill_workspace_bytes(size_t T, size_t topk, size_t n_experts, size_t d, size_t inter);
 
@@ -478,13 +499,18 @@ int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_experts, size_
                            const float *x, int act_kind, void *workspace, float *out, void *stream);
 
 /* The same section with bfloat16 activations: the hidden rows and the activation rows are rounded to bfloat16 (nearest
- * even) once, the MXFP4 weights are exact in bfloat16, and v_mfma_f32_16x16x32_bf16 gives f32 products and f32 sums: the
- * results are those of moe_prefill (src/model.rs:2528-2602) on bfloat16-rounded inputs, with the order of the sums as
- * the only further difference (about 2e-3 of a row's norm from the reference's f32 arithmetic, where the MXFP8 call
- * differs by 2-5 %).  Same arguments, workspace and intermediates as mk_dev_moe_prefill_f32 (g holds the gate rows
- * here: the activation is kept as bfloat16 elsewhere in the workspace).  MK_ERR_UNSUPPORTED unless d and inter are
- * multiples of 512, and for a table with VQ1 experts.  Weights whose value lies below 2^-126 may be flushed to zero by
- * the hardware conversion. */
+ * even) once, the MXFP4 weights are exact, products exact and sums f32: the results are those of moe_prefill
+ * (src/model.rs:2528-2602) on bfloat16-rounded inputs, about 2e-3 of a row's norm from the reference's f32 arithmetic
+ * (the MXFP8 call differs by 2-5 %).  Two forms compute it.  The default keeps every bfloat16 value as two e4m3 terms
+ * (mk_dev_quantize_bf16_split) and runs the block-scaled matrix instruction, v_mfma_scale_f32_16x16x128_f8f6f4, twice
+ * per step against the same weight registers (the kernels of mk_dev_moe_prefill; gate, up, activation and its two-term
+ * form in one launch): exact inputs, and the instruction's own arithmetic, which stays about 1e-5 (relative L2 of a row)
+ * from f32 sums.  MK_PREFILL_BF16_MFMA=1 selects v_mfma_f32_16x16x32_bf16 with the weights converted exactly
+ * (3e-7 from f32 sums, 1.2 times the time).  A hidden or activation value that is not finite makes the rows it enters
+ * NaN.  Same arguments, workspace and intermediates as mk_dev_moe_prefill_f32 (g holds the gate rows here and u the
+ * up rows: the activation is kept in its matrix-instruction form elsewhere in the workspace).  MK_ERR_UNSUPPORTED unless
+ * d and inter are multiples of 512, and for a table with VQ1 experts.  Weights whose value lies below 2^-126 may be
+ * flushed to zero by the hardware conversion (bf16 instruction form). */
 int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
                             const float *x, int act_kind, void *workspace, float *out, void *stream);
 

@@ -62,6 +62,8 @@ def _load():
         "mk_q8_enabled": (i32, []),
         "mk_dev_mxfp4_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_dev_mxfp4_scales_by_tile": (i32, [vp, sz, sz, vp, vp]),
+        "mk_dev_quantize_bf16_split": (i32, [vp, sz, sz, vp, vp, vp]),
+        "mk_dev_mxfp4_grouped_gemm_split": (i32, [vp, vp, sz, sz, sz, vp, vp, vp, sz, vp, vp]),
         "mk_dev_fp8_dequant": (i32, [vp, vp, sz, sz, vp, vp]),
         "mk_dev_quantize_q8": (i32, [vp, sz, sz, vp, vp, vp]),
         "mk_dev_quantize_mxfp8": (i32, [vp, sz, sz, vp, vp, vp]),

@@ -119,7 +119,40 @@ __global__ __launch_bounds__(256) void mk_scales_by_tile_kernel(const uint4 *__r
     out[i] = scales[r * kt + t];
 }
 
+// bfloat16 of every value as two e4m3 terms (mk_bf16_split8), rows of n values, in the K-tile layout of the two-term GEMM
+__global__ __launch_bounds__(256) void mk_quantize_bf16_split_kernel(const float *__restrict__ x, size_t n_groups8, int n, uint8_t *__restrict__ codes,
+                                                                     uint8_t *__restrict__ exps) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;  // group of 8 values
+    if (i >= n_groups8) return;                               // (n % 32 == 0: whole quads leave together)
+    const int per_row = n / 8;
+    const size_t r = i / per_row, c = i % per_row;
+    const mk_f4 a = reinterpret_cast<const mk_f4 *>(x)[2 * i], b = reinterpret_cast<const mk_f4 *>(x)[2 * i + 1];
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t hi[2], lo[2], eh, el;
+    mk_bf16_split8<false>(v, hi, lo, eh, el);
+    const size_t kt = c >> 6, within = (c & 63) * 8;
+    uint8_t *dst = codes + r * (2 * (size_t)n) + kt * 1024 + within;
+    *reinterpret_cast<mk_u2 *>(dst) = mk_u2{hi[0], hi[1]};
+    *reinterpret_cast<mk_u2 *>(dst + 512) = mk_u2{lo[0], lo[1]};
+    if ((c & 3) == 0) {
+        uint8_t *ed = exps + r * (size_t)(n / 16) + kt * 32 + ((c & 63) >> 2);
+        ed[0] = (uint8_t)eh;
+        ed[16] = (uint8_t)el;
+    }
+}
+
 // ------------------------------------------------------------------ C ABI
+extern "C" int mk_dev_quantize_bf16_split(const float *x, size_t nvec, size_t n, uint8_t *codes, uint8_t *exps, void *stream) {
+    MK_REQUIRE(x && codes && exps, "null pointer");
+    MK_REQUIRE(n % 512 == 0 && n <= 0x7FFFFFFFull, "n must be a multiple of 512");
+    MK_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)codes & 7) == 0, "x must be 16-byte and codes 8-byte aligned");
+    const size_t n8 = nvec * (n / 8);
+    if (n8 == 0) return MK_OK;
+    MK_REQUIRE(n8 <= 0x7fffffffull * 256, "too many values");
+    hipLaunchKernelGGL(mk_quantize_bf16_split_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, n8, (int)n, codes, exps);
+    return mk_launch_status("quantize_bf16_split");
+}
+
 extern "C" int mk_dev_mxfp4_scales_by_tile(const uint8_t *scales, size_t rows, size_t cols, uint8_t *out, void *stream) {
     MK_REQUIRE(scales && out, "null pointer");
     MK_REQUIRE(cols % 512 == 0, "cols must be a multiple of 512");

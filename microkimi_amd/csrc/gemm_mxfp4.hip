@@ -116,10 +116,12 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 // through readfirstlane, which hides the loop counter from the induction
 // variable widening that would otherwise rebuild 64-bit pointers per lane.
 constexpr int KT_STEPS = 4;
-constexpr int A_STRIDE = 512 + 32;  // LDS row stride of the activation tile: rows 8 banks apart (with 4 or 16 banks the 16-byte operand reads counted 2.5 times the bank-conflict cycles)
-constexpr int a_codes_bytes(int mc) { return 16 * mc * A_STRIDE; }
-constexpr int a_wsc_off(int mc) { return a_codes_bytes(mc) + 16 * mc * 16; }      // codes, then 16 scale bytes per token,
-constexpr int a_buf_bytes(int mc) { return a_wsc_off(mc) + 256 * 16; }            // then the K tile's 16 scale bytes of the 256 weight rows
+// LDS row stride of the activation tile: rows 8 banks apart (with 4 or 16 banks the 16-byte operand reads counted 2.5
+// times the bank-conflict cycles).  TWO (see gemm_pass): a token row has two code rows and two exponent rows per K tile.
+constexpr int a_stride(bool two = false) { return (two ? 1024 : 512) + 32; }
+constexpr int a_codes_bytes(int mc, bool two = false) { return 16 * mc * a_stride(two); }
+constexpr int a_wsc_off(int mc, bool two = false) { return a_codes_bytes(mc, two) + 16 * mc * (two ? 32 : 16); }  // codes, then the scale bytes per token,
+constexpr int a_buf_bytes(int mc, bool two = false) { return a_wsc_off(mc, two) + 256 * 16; }  // then the K tile's 16 scale bytes of the 256 weight rows
 
 // One launch covers n_mats (1 or 2) weight matrices per group that share the activation rows (gate and up): matrix m
 // of group e is packed_ptrs[m][e], its result goes to out[m].
@@ -220,11 +222,19 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // epilogue forms ACT(g, u), quantizes each token's 32 values to MXFP8 (mk_mxfp8_quantize8's arithmetic with the whole
 // e8m0 range; the block's maximum crosses the four lanes of a token) and stores codes and exponent bytes: 1.03 bytes
 // per value instead of 8 written and 8 read back by a kernel of its own.
-template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false>
+// TWO: every activation value is the sum of two e4m3 terms with block exponents of their own -- the exact split of a
+// bfloat16 value x = hi + lo, hi its leading four significant bits and lo the other four (mk_bf16_split8) -- kept per
+// K tile as [hi codes 512][lo codes 512] and [hi exponents 16][lo exponents 16].  The K tile then is 1024 products deep:
+// two matrix instructions per step against the same weight registers into the same accumulators, nothing else changes.
+// The products are exact and the sums f32, so this is the bfloat16 GEMM (apart from values more than 2^13 below their
+// block's largest, whose last bits fall off the e4m3 grid) at the streaming rate of the MXFP8 one.
+template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false, bool TWO = false>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds, const uint8_t *scales_t, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr,
                                           const uint8_t *scales3_t = nullptr) {
     static_assert(!GU || (FULL && PIN && !DEEP && MC <= 2), "the gate/up form exists for the small-group pass");
+    static_assert(!TWO || (FULL && PIN && !DEEP && MC <= 2), "the two-term form exists for the small-group pass");
+    constexpr int AW = TWO ? 2 : 1, AS = a_stride(TWO);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
@@ -266,20 +276,21 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // tile: thread i fetches row i's once.  Fetched by the lanes that use them (a lane per row, four lanes of a
     // row the same 16 bytes) they were 4 of a wave's 29 loads per K tile and about half of its vector-cache
     // accesses: a 16-byte load whose lanes sit in 16 different lines is looked up once per lane and pass.
-    mk_i4 st[2 * MC], ste, stw;
+    mk_i4 st[2 * MC * AW], ste, stw;
     // (gate/up form: thread i is row slot (wave i / 64, row tile (i / 16) % 4, row i % 16) of the workgroup)
     const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * 256 + tid;
     const bool ws_tiles = scales_t != nullptr;  // (uniform)
     const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? (ws_tiles ? scales3_t : scales3) : (ws_tiles ? scales_t : scales);
     const uint32_t ws_r = (uint32_t)min(ws_row, a.rows - 1);
     const uint32_t wsoff = ws_tiles ? ws_r * 16u : ws_r * (uint32_t)nb, ws_step = ws_tiles ? (uint32_t)a.rows * 16u : 16u;
-    uint32_t coff[2 * MC];  // the host checks that tokens x cols stays below 2^32
+    uint32_t coff[2 * MC * AW];  // the host checks that tokens x cols (x 2) stays below 2^32
 #pragma unroll
-    for (int k = 0; k < 2 * MC; k++) {
+    for (int k = 0; k < 2 * MC * AW; k++) {
         const int i = tid + 256 * k;
-        coff[k] = (uint32_t)min(base + (i >> 5), tok1 - 1) * (uint32_t)cols + (i & 31) * 16;
+        coff[k] = (uint32_t)min(base + i / (32 * AW), tok1 - 1) * (uint32_t)(cols * AW) + (i % (32 * AW)) * 16;
     }
-    const uint32_t eoff = (uint32_t)min(base + (tid & (16 * MC - 1)), tok1 - 1) * (uint32_t)nb;
+    // (thread i: token i / AW, exponent row i % AW)
+    const uint32_t eoff = (uint32_t)min(base + (tid & (16 * MC * AW - 1)) / AW, tok1 - 1) * (uint32_t)(nb * AW) + (tid % AW) * 16;
     auto stage_load = [&](int kt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
 #ifdef MK_GEMM_FP4_PROBE
@@ -288,21 +299,21 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         constexpr int STG = 2 * MC;
 #endif
 #pragma unroll
-        for (int k = 0; k < STG; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * 512);
-        ste = mk_ldg128_off(a.exps, eoff + ku * 16);
+        for (int k = 0; k < STG * AW; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * (512 * AW));
+        ste = mk_ldg128_off(a.exps, eoff + ku * (16 * AW));
         stw = mk_ldg128_off(ws_base, wsoff + ku * ws_step);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
-        for (int k = 0; k < 2 * MC; k++) {
+        for (int k = 0; k < 2 * MC * AW; k++) {
 #ifdef MK_GEMM_FP4_PROBE
             if (MC >= 4 && k >= MC) break;
 #endif
             const int i = tid + 256 * k;
-            *reinterpret_cast<mk_i4 *>(buf + (i >> 5) * A_STRIDE + (i & 31) * 16) = st[k];
+            *reinterpret_cast<mk_i4 *>(buf + (i / (32 * AW)) * AS + (i % (32 * AW)) * 16) = st[k];
         }
-        if (tid < 16 * MC) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC) + tid * 16) = ste;
-        *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC) + tid * 16) = stw;
+        if (tid < 16 * MC * AW) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC, TWO) + tid * 16) = ste;
+        *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC, TWO) + tid * 16) = stw;
     };
     mk_f4 acc[4][MC];
 #pragma unroll
@@ -311,11 +322,11 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto mma_unit = [&](const mk_i4 *w, int rt, const uint8_t *buf) {
-        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC) + (wave * 64 + rt * 16 + n) * 16);
+        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC, TWO) + (wave * 64 + rt * 16 + n) * 16);
 #pragma unroll
         for (int c = 0; c < MC; c++) {
-            const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC) + (c * 16 + n) * 16);
-            const uint8_t *arow = buf + (c * 16 + n) * A_STRIDE + kb * 16;
+            const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * (16 * AW));
+            const uint8_t *arow = buf + (c * 16 + n) * AS + kb * 16;
 #pragma unroll
             for (int s = 0; s < KT_STEPS; s++) {
                 const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + s * 128);
@@ -329,6 +340,18 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 else
                     acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*M: fp8 rows*/, 4 /*N: fp4 weights*/, 0, asb, 0, wsb);
             }
+            if constexpr (TWO) {  // the second term of every value against the same weight registers
+                const mk_i4 ael = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 32 + 16);
+#pragma unroll
+                for (int s = 0; s < KT_STEPS; s++) {
+                    const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + 512 + s * 128);
+                    const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + 512 + s * 128 + 64);
+                    const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                    const mk_i8v bv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
+                    acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[rt][c], 4, 0, 0, (int)((uint32_t)sc[s] >> (8 * kb)), 0,
+                                                                                  (int)((uint32_t)ael[s] >> (8 * kb)));
+                }
+            }
         }
     };
     // Two row tiles against one read of the activation operands (large groups: with four token tiles the LDS reads of a
@@ -336,11 +359,11 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf) {
         // the scale bytes are read one at a time where they are used: held as 16-byte rows they cost the registers that
         // make the difference between two waves per SIMD with and without a spill
-        const uint8_t *sc0 = buf + a_wsc_off(MC) + (wave * 64 + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
+        const uint8_t *sc0 = buf + a_wsc_off(MC, TWO) + (wave * 64 + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
 #pragma unroll
         for (int c = 0; c < MC; c++) {
-            const uint8_t *ae = buf + a_codes_bytes(MC) + (c * 16 + n) * 16 + kb;
-            const uint8_t *arow = buf + (c * 16 + n) * A_STRIDE + kb * 16;
+            const uint8_t *ae = buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 16 + kb;
+            const uint8_t *arow = buf + (c * 16 + n) * AS + kb * 16;
 #pragma unroll
             for (int s = 0; s < KT_STEPS; s++) {
                 const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + s * 128);
@@ -417,7 +440,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO);
             stage_load(kt + 1);
             if constexpr (PIN && FULL && MC >= 4) {
                 // large groups: two row tiles per read of the activation operands (93-109 -> 82-95 us on 8 experts x 512 tokens)
@@ -443,7 +466,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 }
             }
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO));
             __syncthreads();
         }
     } else {
@@ -454,7 +477,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO);
             stage_load(kt + 1);
             load_unit(wb, kt, 1);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
@@ -472,7 +495,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             compute_unit(wb, 3, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO));
             __syncthreads();
         }
     }
@@ -485,6 +508,26 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             for (int i = 0; i < 4; i++) {
                 v[i] = mk_act(a.act_kind, acc[0][c][i], acc[2][c][i], 0.0f, 1.0f);
                 v[4 + i] = mk_act(a.act_kind, acc[1][c][i], acc[3][c][i], 0.0f, 1.0f);
+            }
+            if constexpr (TWO) {
+                // bfloat16 of the activation as two e4m3 terms, in the K-tile layout the down projection stages
+                uint32_t hi[2], lo[2], eh, el;
+                mk_bf16_split8<true>(v, hi, lo, eh, el);
+                const int t = base + c * 16 + n;
+                if (t < tok1 && row0 + 31 < a.rows) {
+                    const int r = row0 + kb * 4;
+                    uint8_t *dst = a.act_codes + (size_t)t * (2 * (size_t)a.rows) + (r >> 9) * 1024 + (r & 511);
+                    *reinterpret_cast<uint32_t *>(dst) = hi[0];
+                    *reinterpret_cast<uint32_t *>(dst + 16) = hi[1];
+                    *reinterpret_cast<uint32_t *>(dst + 512) = lo[0];
+                    *reinterpret_cast<uint32_t *>(dst + 528) = lo[1];
+                    if (kb == 0) {
+                        uint8_t *ed = a.act_exps + (size_t)t * (a.rows / 16) + (r >> 9) * 32 + ((r & 511) >> 5);
+                        ed[0] = (uint8_t)eh;
+                        ed[16] = (uint8_t)el;
+                    }
+                }
+                continue;
             }
             float amax = 0.0f;
 #pragma unroll
@@ -546,7 +589,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 // Two instantiations share the grid: groups of up to 32 tokens (the prefill
 // case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
 // workgroup whose group belongs to the other one exits.
-template <int MC>
+template <int MC, bool TWO = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
@@ -566,12 +609,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const int m = r / a.row_blocks, rb = r % a.row_blocks;
     const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
     const int count = tok1 - tok0;
-    if (count <= 0 || (count <= 32 ? 2 : 4) != MC) return;
+    if (count <= 0 || (!TWO && (count <= 32 ? 2 : 4) != MC)) return;
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
     const uint8_t *scales_t = a.scales_t_ptrs[m] ? mk_uniform_ptr(a.scales_t_ptrs[m][e]) : nullptr;
     float *out = a.out[m];
-    if (MC == 2) {
+    if constexpr (TWO) {
+        // any group size: passes of 32 token rows, one after the other
+        if (count <= 16) {
+            gemm_pass<1, true, true, true, false, false, true>(a, packed, scales, out, rb, tok0, tok1, lds, scales_t);
+        } else {
+#pragma unroll 1
+            for (int base = tok0; base < tok1; base += 32) gemm_pass<2, true, true, true, false, false, true>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
+        }
+    } else if (MC == 2) {
         if (count <= 16) gemm_pass<1, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds, scales_t);
         else gemm_pass<2, true, true, true>(a, packed, scales, out, rb, tok0, tok1, lds, scales_t);
     } else {
@@ -584,6 +635,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
 
 // The gate/up form: workgroup -> (group, block of 128 rows), both matrices.  Groups of up to 16 tokens take one token
 // tile, larger ones passes of 32 tokens (a group beyond 32 passes over its weights again: the prefill shape has none).
+template <bool TWO = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_gu_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int per_group = a.row_blocks;  // blocks of 128 rows
@@ -604,23 +656,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const bool tiles = a.scales_t_ptrs[0] && a.scales_t_ptrs[1];
     const uint8_t *t1 = tiles ? mk_uniform_ptr(a.scales_t_ptrs[0][e]) : nullptr, *t3 = tiles ? mk_uniform_ptr(a.scales_t_ptrs[1][e]) : nullptr;
     if (count <= 16) {
-        gemm_pass<1, true, true, true, false, true>(a, p1, s1, nullptr, rb, tok0, tok1, lds, t1, p3, s3, t3);
+        gemm_pass<1, true, true, true, false, true, TWO>(a, p1, s1, nullptr, rb, tok0, tok1, lds, t1, p3, s3, t3);
     } else {
 #pragma unroll 1
-        for (int base = tok0; base < tok1; base += 32) gemm_pass<2, true, true, true, false, true>(a, p1, s1, nullptr, rb, base, tok1, lds, t1, p3, s3, t3);
+        for (int base = tok0; base < tok1; base += 32)
+            gemm_pass<2, true, true, true, false, true, TWO>(a, p1, s1, nullptr, rb, base, tok1, lds, t1, p3, s3, t3);
     }
 }
 
-template <int MC>
+template <int MC, bool TWO = false>
 int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
     // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
     // average group size (one per 64 tokens, at most 16); a workgroup without a pass exits at once.
     unsigned passes = 1;
     if (MC == 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
     const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC>), 2 * a_buf_bytes(MC));
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO>), 2 * a_buf_bytes(MC, TWO));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL(mxfp4_grouped_gemm_stream_kernel<MC>, grid, dim3(256), 2 * a_buf_bytes(MC), st, a);
+    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO>), grid, dim3(256), 2 * a_buf_bytes(MC, TWO), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
 }
 
@@ -629,8 +682,9 @@ int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
 // gate and up of the prefill section in one launch (the matrices share the token rows); see mk_common.h
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                             size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
-                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs) {
+                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs, bool two) {
     MK_REQUIRE(n_mats == 1 || n_mats == 2, "one or two matrices per group");
+    MK_REQUIRE(!two || (cols % 512 == 0 && m * cols * 2 < 0xFFFFFFFFull), "the two-term form takes cols in multiples of 512");
     for (int k = 0; k < n_mats; k++) MK_REQUIRE(packed_ptrs[k] && scales_ptrs[k] && out[k], "null pointer");
     MK_REQUIRE(codes && exps && offsets, "null pointer");
     MK_REQUIRE(cols % 128 == 0 && cols > 0, "cols must be a positive multiple of 128");
@@ -655,10 +709,12 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         a.n_groups = (int)n_groups;
         a.n_mats = n_mats;
         a.row_blocks = (int)row_blocks;
+        if (two) return launch_stream<2, true>(a, m, (hipStream_t)stream);
         int st = launch_stream<2>(a, m, (hipStream_t)stream);
         if (st == MK_OK && m > 32) st = launch_stream<4>(a, m, (hipStream_t)stream);
         return st;
     }
+    MK_REQUIRE(!two, "the two-term form needs the streaming kernel's shapes");
     for (int k = 0; k < n_mats; k++) {
         hipLaunchKernelGGL(mxfp4_grouped_gemm_kernel, dim3((unsigned)((rows + 63) / 64), (unsigned)n_groups), dim3(256), 0, (hipStream_t)stream,
                            packed_ptrs[k], scales_ptrs[k], (int)rows, (int)cols, codes, exps, offsets, out[k]);
@@ -673,8 +729,9 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
 int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                                       size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
                                       const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
-                                      float *keep_u, void *stream, const uint8_t *const *w1st, const uint8_t *const *w3st) {
+                                      float *keep_u, void *stream, const uint8_t *const *w1st, const uint8_t *const *w3st, bool two) {
     MK_REQUIRE(w1p && w1s && w3p && w3s && codes && exps && offsets && act_codes && act_exps, "null pointer");
+    if (two && (rows % 512 != 0 || m * cols * 2 >= 0xFFFFFFFFull)) return MK_ERR_UNSUPPORTED;
     if (!(cols % 512 == 0 && rows % 128 == 0 && rows * (cols / 2) < 0xFFFFFFFFull && m * cols < 0xFFFFFFFFull && ((uintptr_t)exps & 15) == 0 &&
           ((uintptr_t)codes & 15) == 0 && ((uintptr_t)act_codes & 3) == 0 && n_groups * (rows / 128) < 0x7FFFFFFFull))
         return MK_ERR_UNSUPPORTED;
@@ -700,9 +757,16 @@ int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *
     a.act_kind = act_kind;
     a.act_codes = act_codes;
     a.act_exps = act_exps;
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_gu_kernel), 2 * a_buf_bytes(2));
+    if (two) {
+        const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_gu_kernel<true>), 2 * a_buf_bytes(2, true));
+        if (s != MK_OK) return s;
+        hipLaunchKernelGGL(mxfp4_grouped_gemm_gu_kernel<true>, dim3((unsigned)(n_groups * (rows / 128))), dim3(256), 2 * a_buf_bytes(2, true),
+                           (hipStream_t)stream, a);
+        return mk_launch_status("mxfp4_grouped_gemm_gu");
+    }
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_gu_kernel<false>), 2 * a_buf_bytes(2));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL(mxfp4_grouped_gemm_gu_kernel, dim3((unsigned)(n_groups * (rows / 128))), dim3(256), 2 * a_buf_bytes(2), (hipStream_t)stream, a);
+    hipLaunchKernelGGL(mxfp4_grouped_gemm_gu_kernel<false>, dim3((unsigned)(n_groups * (rows / 128))), dim3(256), 2 * a_buf_bytes(2), (hipStream_t)stream, a);
     return mk_launch_status("mxfp4_grouped_gemm_gu");
 }
 
@@ -710,5 +774,17 @@ extern "C" int mk_dev_mxfp4_grouped_gemm(const uint8_t *const *packed_ptrs, cons
                                          size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m, float *out,
                                          void *stream) {
     MK_REQUIRE(packed_ptrs && scales_ptrs && codes && exps && offsets && out, "null pointer");
-    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream, nullptr);
+    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream, nullptr, false);
+}
+
+extern "C" int mk_dev_mxfp4_grouped_gemm_split(const uint8_t *const *packed_ptrs, const uint8_t *const *scales_ptrs, size_t n_groups, size_t rows,
+                                               size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
+                                               float *out, void *stream) {
+    MK_REQUIRE(packed_ptrs && scales_ptrs && codes && exps && offsets && out, "null pointer");
+    if (cols == 0 || cols % 512 != 0 || rows * (cols / 2) >= 0xFFFFFFFFull || m * cols * 2 >= 0xFFFFFFFFull) {
+        mk_set_error("the two-term grouped product takes cols in multiples of 512 and operands below 4 GiB");
+        return MK_ERR_UNSUPPORTED;
+    }
+    MK_REQUIRE(((uintptr_t)exps & 15) == 0, "exps must be 16-byte aligned");
+    return mk_mxfp4_grouped_gemm_n(1, &packed_ptrs, &scales_ptrs, n_groups, rows, cols, codes, exps, offsets, m, &out, stream, nullptr, true);
 }

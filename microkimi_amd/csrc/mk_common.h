@@ -284,6 +284,62 @@ __device__ __forceinline__ void mk_mxfp8_quantize8(const float (&v)[8], uint32_t
     c1 = (uint32_t)w1;
 }
 
+// bfloat16 (round to nearest even) of 8 consecutive values of a 32-block as TWO e4m3 terms per value with a block
+// exponent each: x = hi + lo, hi = the leading four significant bits of the bfloat16 value (sign, exponent, three
+// mantissa bits) and lo the other four -- both exact on the e4m3 grid of their block unless the value lies more than
+// 2^13 below the block's largest (then its last bits round off: below 2^-17 of that largest value).  A dot product over
+// hi and lo against exact weights with f32 sums is the bfloat16 dot product.  ROWS: the block's other values sit in the
+// lanes c + 16, + 32, + 48 (matrix-instruction results); otherwise in the aligned quad of lanes.  Codes: lowest byte
+// first, [0] = v[0..3], [1] = v[4..7].  A value that is not finite gets the e4m3 NaN code.
+template <bool ROWS>
+__device__ __forceinline__ void mk_bf16_split8(const float (&v)[8], uint32_t (&hi)[2], uint32_t (&lo)[2], uint32_t &exp_hi, uint32_t &exp_lo) {
+    float h[8], l[8], ah = 0.0f, al = 0.0f;
+    uint32_t bad[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float b = (float)(__bf16)v[i];
+        const uint32_t bits = __float_as_uint(b);
+        const bool fin = (bits & 0x7F800000u) != 0x7F800000u;
+        h[i] = __uint_as_float(bits & 0xFFF00000u);
+        l[i] = fin ? b - h[i] : 0.0f;
+        if (!fin) bad[i >> 2] |= 0x7Fu << (8 * (i & 3));
+        ah = fmaxf(ah, fabsf(h[i]));
+        al = fmaxf(al, fabsf(l[i]));
+    }
+    if constexpr (ROWS) {
+        ah = mk_rows_max(ah);
+        al = mk_rows_max(al);
+    } else {
+        ah = fmaxf(ah, mk_dpp<0xB1>(ah));
+        ah = fmaxf(ah, mk_dpp<0x4E>(ah));
+        al = fmaxf(al, mk_dpp<0xB1>(al));
+        al = fmaxf(al, mk_dpp<0x4E>(al));
+    }
+    auto encode = [](const float (&x)[8], float amax, uint32_t (&codes)[2], uint32_t &exp_byte) {
+        int e = mk_ceil_log2f(fmaxf(amax, 1e-30f) / 448.0f);
+        e = max(-127, min(127, e));
+        exp_byte = (uint32_t)(e + 127);
+        const float inv = mk_scale_from_byte(254u - exp_byte);  // 2^-e, exact
+        float q[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = fminf(fmaxf(x[i] * inv, -448.0f), 448.0f);
+        int w0 = 0, w1 = 0;
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], w0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], w1, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
+        codes[0] = (uint32_t)w0;
+        codes[1] = (uint32_t)w1;
+    };
+    encode(h, ah, hi, exp_hi);
+    encode(l, al, lo, exp_lo);
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const uint32_t m = ((bad[k] >> 6) & 0x01010101u) * 0xFFu;  // bytes of the values that are not finite
+        hi[k] = (hi[k] & ~m) | (bad[k] & m);
+    }
+}
+
 // silu(x) = x / (1 + exp(-x)) (src/deepseek.rs:97-100)
 __device__ __forceinline__ float mk_silu(float x) { return x / (1.0f + expf(-x)); }
 // situ (src/model.rs:619-621)
@@ -350,9 +406,11 @@ int mk_mla_static_init(void **out_ptr);
 // (gemm_mxfp4.hip): matrix k of group e is packed_ptrs[k][e] / scales_ptrs[k][e], its [m x rows] result goes to out[k].
 // scales_t_ptrs (may be null, and so may its entries): the matrices' scale bytes in K-tile order
 // (mk_dev_mxfp4_scales_by_tile), read instead of scales_ptrs by the kernels that walk K in tiles of 512.
+// two: the token rows are bfloat16 values as two e4m3 terms each (mk_bf16_split8): codes [m][cols / 512][2][512], exps
+// [m][cols / 512][2][16]; cols % 512 == 0.  (The gate/up call then writes the activation in that form too; rows % 512 == 0.)
 int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs, const uint8_t *const *const *scales_ptrs, size_t n_groups,
                             size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps, const int32_t *offsets, size_t m,
-                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs = nullptr);
+                            float *const *out, void *stream, const uint8_t *const *const *scales_t_ptrs = nullptr, bool two = false);
 // matvec_packed_nt (f32 products and sums, gemv_mxfp4.hip) for groups of rows that each meet their own n_mats (1 or 2)
 // matrices: group e owns the grouped rows offsets[e] .. offsets[e+1]; grouped row p multiplies activation row
 // xrow[p] / xdiv of x (xrow null: row p itself); matrix k's [. x rows] result goes to out[k] at the grouped row.  m: the
@@ -374,4 +432,5 @@ int mk_mxfp4_grouped_gemm_bf16(int n_mats, const uint8_t *const *const *packed_p
 int mk_mxfp4_grouped_gemm_gate_up_act(const uint8_t *const *w1p, const uint8_t *const *w1s, const uint8_t *const *w3p, const uint8_t *const *w3s,
                                       size_t n_groups, size_t rows, size_t cols, const uint8_t *codes, const uint8_t *exps,
                                       const int32_t *offsets, size_t m, int act_kind, uint8_t *act_codes, uint8_t *act_exps, float *keep_g,
-                                      float *keep_u, void *stream, const uint8_t *const *w1st = nullptr, const uint8_t *const *w3st = nullptr);
+                                      float *keep_u, void *stream, const uint8_t *const *w1st = nullptr, const uint8_t *const *w3st = nullptr,
+                                      bool two = false);

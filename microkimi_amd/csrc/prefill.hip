@@ -33,7 +33,10 @@ struct PrefillWs {
     float *g, *u;             // [P][inter]
     uint8_t *codes2, *exps2;  // [P][inter], [P][inter/32]
     float *o;                 // [P][d]
-    uint16_t *xb;             // [P][max(d, inter)] bf16: the hidden rows, then the activation rows, of the bf16 section
+    uint16_t *xb;             // [P][max(d, inter)] bf16: the hidden rows, then the activation rows, of the bf16 section (matrix-instruction form)
+    // bf16 section, two-term form (mk_bf16_split8): [P][d / 512][2][512] codes and [P][d / 512][2][16] exponents of the
+    // hidden rows, the same for the activation rows
+    uint8_t *split_codes, *split_exps, *split_codes2, *split_exps2;
     size_t bytes;
 };
 
@@ -57,6 +60,10 @@ PrefillWs carve(void *base, size_t P, size_t n_experts, size_t d, size_t inter) 
     w.exps2 = take(P * (inter / 32));
     w.o = (float *)take(P * d * 4);
     w.xb = (uint16_t *)take(P * (d > inter ? d : inter) * 2);
+    w.split_codes = take(P * d * 2);
+    w.split_exps = take(P * (d / 32) * 2);
+    w.split_codes2 = take(P * inter * 2);
+    w.split_exps2 = take(P * (inter / 32) * 2);
     w.bytes = off;
     return w;
 }
@@ -217,6 +224,33 @@ __global__ __launch_bounds__(256) void prefill_gather_bf16_kernel(const float *_
     reinterpret_cast<bf8 *>(xb)[i] = v;
 }
 
+// bfloat16 of the hidden row of each grouped pair as two e4m3 terms per value (mk_bf16_split8), in the K-tile layout the
+// two-term GEMM stages: a lane takes 8 consecutive values, four lanes a 32-block
+__global__ __launch_bounds__(256) void prefill_gather_split_kernel(const float *__restrict__ x, const int32_t *__restrict__ order,
+                                                                   const int32_t *__restrict__ offsets, int n_experts, int topk, int d,
+                                                                   uint8_t *__restrict__ codes, uint8_t *__restrict__ exps) {
+    const int per_row = d / 8;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of 8 values
+    const size_t rows = (size_t)offsets[n_experts];                  // pairs with a valid expert id
+    if (i >= rows * per_row) return;  // (d % 32 == 0: whole quads leave together)
+    const size_t r = i / per_row, c = i % per_row;
+    const int t = order[r] / topk;
+    const mk_f4 *src = reinterpret_cast<const mk_f4 *>(x + (size_t)t * d) + 2 * c;
+    const mk_f4 a = src[0], b = src[1];
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t hi[2], lo[2], eh, el;
+    mk_bf16_split8<false>(v, hi, lo, eh, el);
+    const size_t kt = c >> 6, within = (c & 63) * 8;  // K tile of 512 columns, byte inside it
+    uint8_t *dst = codes + r * (2 * (size_t)d) + kt * 1024 + within;
+    *reinterpret_cast<mk_u2 *>(dst) = mk_u2{hi[0], hi[1]};
+    *reinterpret_cast<mk_u2 *>(dst + 512) = mk_u2{lo[0], lo[1]};
+    if ((c & 3) == 0) {
+        uint8_t *ed = exps + r * (size_t)(d / 16) + kt * 32 + ((c & 63) >> 2);
+        ed[0] = (uint8_t)eh;
+        ed[16] = (uint8_t)el;
+    }
+}
+
 // act = ACT(gate, up) in f32, stored as bfloat16 (round to nearest even)
 __global__ __launch_bounds__(256) void prefill_act_bf16_kernel(const float *__restrict__ g, const float *__restrict__ u,
                                                                const int32_t *__restrict__ offsets, int n_experts, int inter, int act_kind,
@@ -372,8 +406,9 @@ extern "C" int mk_dev_moe_prefill_f32(const mk_expert_table *table, size_t n_exp
 }
 
 // The section with bfloat16 hidden rows and activation rows against the exact weights (bf16 matrix instruction).
-extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
-                                       const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+namespace {
+int moe_prefill_bf16_impl(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids, const float *weights,
+                          const float *x, int act_kind, void *workspace, float *out, void *stream, bool keep) {
     MK_REQUIRE(table && ids && weights && x && workspace && out, "null pointer");
     MK_REQUIRE(act_kind == MK_ACT_SWIGLU || act_kind == MK_ACT_SITU, "moe_prefill knows the SwiGLU and SiTU activations");
     if (table->vq_codebook) {
@@ -398,6 +433,27 @@ extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_ex
                        w.offsets);
     int s = mk_launch_status("prefill_group");
     if (s != MK_OK) return s;
+    // Two forms.  The two-term form (every bfloat16 value as two e4m3 terms on the block-scaled matrix instruction, the
+    // streaming kernels of the MXFP8 section) is the default; MK_PREFILL_BF16_MFMA=1 selects the bfloat16 matrix instruction.
+    if (!MK_TUNE("MK_PREFILL_BF16_MFMA", 0) && P * d * 2 < 0xFFFFFFFFull && P * inter * 2 < 0xFFFFFFFFull) {
+        hipLaunchKernelGGL(prefill_gather_split_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
+                           (int)n_experts, (int)topk, (int)d, w.split_codes, w.split_exps);
+        if ((s = mk_launch_status("prefill_gather_split")) != MK_OK) return s;
+        s = mk_mxfp4_grouped_gemm_gate_up_act(table->w1p, table->w1s, table->w3p, table->w3s, n_experts, inter, d, w.split_codes, w.split_exps,
+                                              w.offsets, P, act_kind, w.split_codes2, w.split_exps2, keep ? w.g : nullptr, keep ? w.u : nullptr, stream,
+                                              table->w1st, table->w3st, true);
+        if (s != MK_OK) return s;  // (d and inter in multiples of 512: the launch takes every such shape)
+        const uint8_t *const *pd[1] = {table->w2p};
+        const uint8_t *const *sd[1] = {table->w2s};
+        const uint8_t *const *td[1] = {table->w2st};
+        float *od[1] = {w.o};
+        if ((s = mk_mxfp4_grouped_gemm_n(1, pd, sd, n_experts, d, inter, w.split_codes2, w.split_exps2, w.offsets, P, od, stream,
+                                         table->w2st ? td : nullptr, true)) != MK_OK)
+            return s;
+        hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights,
+                           (int)topk, (int)d, out);
+        return mk_launch_status("prefill_combine");
+    }
     hipLaunchKernelGGL(prefill_gather_bf16_kernel, dim3((unsigned)((P * (d / 8) + 255) / 256)), dim3(256), 0, st, x, w.order, w.offsets,
                        (int)n_experts, (int)topk, (int)d, w.xb);
     if ((s = mk_launch_status("prefill_gather_bf16")) != MK_OK) return s;
@@ -419,6 +475,14 @@ extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_ex
     hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((d / 4 + 255) / 256), (unsigned)T), dim3(256), 0, st, w.o, w.pos, weights, (int)topk,
                        (int)d, out);
     return mk_launch_status("prefill_combine");
+}
+
+}  // namespace
+
+extern "C" int mk_dev_moe_prefill_bf16(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,
+                                       const float *weights, const float *x, int act_kind, void *workspace, float *out, void *stream) {
+    // (the f32 gate and up rows are stored too: the launch is bound by its loads and the stores cost nothing measurable)
+    return moe_prefill_bf16_impl(table, n_experts, T, topk, ids, weights, x, act_kind, workspace, out, stream, true);
 }
 
 extern "C" int mk_dev_moe_prefill(const mk_expert_table *table, size_t n_experts, size_t T, size_t topk, const int32_t *ids,

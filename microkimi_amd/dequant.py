@@ -45,3 +45,17 @@ def quantize_mxfp8(x):
     exps = torch.empty(x.shape[:-1] + (n // 32,), dtype=torch.uint8, device=x.device)
     check(lib.mk_dev_quantize_mxfp8(ptr(x), nvec, n, ptr(codes), ptr(exps), cur_stream()))
     return codes, exps
+
+
+def quantize_bf16_split(x):
+    """bfloat16 of x [..., n] (n % 512 == 0) as two e4m3 terms per value (mk_dev_quantize_bf16_split): codes
+    [..., n / 512, 2, 512] and exps [..., n / 512, 2, 16], the activation format of model.grouped_gemm_split."""
+    import torch
+    _lib.require_device()
+    x = x.contiguous()
+    n = x.shape[-1]
+    nvec = x.numel() // n
+    codes = torch.empty(x.shape[:-1] + (n // 512, 2, 512), dtype=torch.uint8, device=x.device)
+    exps = torch.empty(x.shape[:-1] + (n // 512, 2, 16), dtype=torch.uint8, device=x.device)
+    check(lib.mk_dev_quantize_bf16_split(ptr(x), nvec, n, ptr(codes), ptr(exps), cur_stream()))
+    return codes, exps

@@ -462,6 +462,22 @@ def grouped_gemm_f32(packed_list, scales_list, rows, cols, x, offsets, bf16=Fals
     return out
 
 
+def grouped_gemm_split(packed_list, scales_list, rows, cols, codes, exps, offsets):
+    """matvec_packed_nt per group (src/model.rs:2412-2447) on bfloat16-rounded rows given as two e4m3 terms per value
+    (dequant.quantize_bf16_split), on the block-scaled matrix cores: rows offsets[e]..offsets[e+1] against expert e
+    -> [m, rows] f32."""
+    import torch
+    _lib.require_device()
+    dev = codes.device
+    pp = torch.tensor([t.data_ptr() for t in packed_list], dtype=torch.int64, device=dev)
+    sp = torch.tensor([t.data_ptr() for t in scales_list], dtype=torch.int64, device=dev)
+    m = codes.shape[0]
+    out = torch.empty((m, rows), dtype=torch.float32, device=dev)
+    check(lib.mk_dev_mxfp4_grouped_gemm_split(ptr(pp), ptr(sp), len(packed_list), rows, cols, ptr(codes), ptr(exps), ptr(offsets), m, ptr(out),
+                                              cur_stream()))
+    return out
+
+
 def grouped_gemm_mxfp8(packed_list, scales_list, rows, cols, codes, exps, offsets):
     """Per-expert batched evaluation of moe_prefill (src/model.rs:2539-2602) on the block-scaled matrix cores:
     rows offsets[e]..offsets[e+1] of the MXFP8 activations (codes, exps) against expert e -> [m, rows] f32."""

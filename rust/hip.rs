@@ -125,6 +125,8 @@ extern "C" {
     pub fn mk_force_q8(v: c_int);
     pub fn mk_q8_enabled() -> c_int;
     pub fn mk_dev_mxfp4_dequant(packed: *const u8, scales: *const u8, rows: usize, cols: usize, out: *mut f32, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_quantize_bf16_split(x: *const f32, nvec: usize, n: usize, codes: *mut u8, exps: *mut u8, stream: *mut c_void) -> c_int;
+    pub fn mk_dev_mxfp4_grouped_gemm_split(packed_ptrs: *const *const u8, scales_ptrs: *const *const u8, n_groups: usize, rows: usize, cols: usize, codes: *const u8, exps: *const u8, offsets: *const i32, m: usize, out: *mut f32, stream: *mut c_void) -> c_int;
     pub fn mk_dev_mxfp4_scales_by_tile(scales: *const u8, rows: usize, cols: usize, out: *mut u8, stream: *mut c_void) -> c_int;
     pub fn mk_moe_pack_bytes(d: usize, inter: usize, down: c_int) -> usize;
     pub fn mk_dev_moe_pack_gate_up(w1p: *const u8, w1s: *const u8, w3p: *const u8, w3s: *const u8, d: usize, inter: usize, pack: *mut u8, stream: *mut c_void) -> c_int;

@@ -171,6 +171,117 @@ def test_grouped_gemm_f32_and_bf16(rows, cols, counts, bf16):
             assert rel_l2(got[r0:r1], xin[r0:r1] @ Wd.T) <= 1e-5, e
 
 
+def decode_split(codes, exps):
+    """The values a two-term row stands for: codes [m, kt, 2, 512] e4m3, exps [m, kt, 2, 16] e8m0 -> (hi + lo) [m, kt * 512] f64."""
+    c = codes.astype(np.int32)
+    e, mant = (c >> 3) & 15, c & 7
+    v = np.where(e == 0, mant / 8.0 * 2.0 ** -6, (1 + mant / 8.0) * 2.0 ** (e - 7.0))
+    v = np.where((c & 127) == 127, np.nan, v) * np.where(c & 128, -1.0, 1.0)
+    m, kt = codes.shape[:2]
+    v = v.reshape(m, kt, 2, 16, 32) * (2.0 ** (exps.astype(np.float64) - 127))[..., None]
+    return (v[:, :, 0] + v[:, :, 1]).reshape(m, kt * 512)
+
+
+def test_bf16_split_is_the_bfloat16_value():
+    # mk_dev_quantize_bf16_split: hi + lo is bfloat16(x) exactly for every value within 2^13 of its block's largest,
+    # and within 2^-17 of that largest value otherwise; zeros, a zero block, huge and tiny blocks; NaN / inf -> NaN
+    torch = torch_cuda()
+    from microkimi_amd import dequant
+    rng = np.random.default_rng(11)
+    n = 1024
+    x = rng.standard_normal((40, n)).astype(np.float32)
+    x[1] *= 1e-3
+    x[2] *= 3e5
+    x[3] = (x[3] * np.exp(rng.uniform(-30, 12, n))).astype(np.float32)       # 60 binades inside the blocks
+    x[4, :32] = 0.0
+    x[5] = np.float32(2.0) ** rng.integers(-20, 20, n).astype(np.float32)    # powers of two: lo is zero everywhere
+    x[6] = (x[6] * 1e-30).astype(np.float32)
+    x[7] = (x[7] * 1e30).astype(np.float32)
+    x[8, ::7] = 0.0
+    codes, exps = dequant.quantize_bf16_split(dev(x))
+    got = decode_split(codes.cpu().numpy(), exps.cpu().numpy())
+    want = bf16_round(x).astype(np.float64)
+    blockmax = np.abs(want).reshape(40, n // 32, 32).max(axis=2, keepdims=True)
+    near = (np.abs(want).reshape(40, n // 32, 32) >= blockmax * 2.0 ** -13).reshape(40, n)
+    assert np.array_equal(got[near], want[near])
+    slack = np.broadcast_to(blockmax * 2.0 ** -17, (40, n // 32, 32)).reshape(40, n)
+    assert np.all(np.abs(got - want)[~near] <= slack[~near])
+    assert near.mean() > 0.9 and (~near).sum() > 100   # both kinds of value were there
+    y = x[:2].copy()
+    y[0, 5], y[0, 40], y[1, 100] = np.inf, -np.inf, np.nan
+    codes, exps = dequant.quantize_bf16_split(dev(y))
+    got = decode_split(codes.cpu().numpy(), exps.cpu().numpy())
+    assert np.isnan(got[0, 5]) and np.isnan(got[0, 40]) and np.isnan(got[1, 100])
+    ok = near[:2].copy()
+    ok[0, :64] = False   # (the blocks that hold an infinity: their other values underflow against it)
+    ok[1, 100] = False
+    assert np.array_equal(got[ok], bf16_round(y).astype(np.float64)[ok])
+
+
+@pytest.mark.parametrize("rows,cols,counts", [(128, 512, [5, 0, 20, 33]), (64, 1024, [3, 70]), (256, 512, [0, 0, 16, 1, 32, 0, 7, 9]),
+                                              (2048, 7168, [9, 24]), (7168, 2048, [16, 1, 40]), (300, 512, [1, 17, 65])])
+def test_grouped_gemm_split(rows, cols, counts):
+    # the two-term grouped product: every group's rows against the f64 product of its dequantized matrix and the
+    # bfloat16-rounded rows; group sizes around the 16-row tile and the 32-row pass, empty groups, ragged weight rows
+    torch_cuda()
+    from microkimi_amd import dequant, model, workloads
+    rng = np.random.default_rng(rows + cols)
+    mats = [workloads.mxfp4_matrix(4, "w1", rows, cols, e) for e in range(len(counts))]
+    m = int(sum(counts))
+    x = rng.standard_normal((m, cols)).astype(np.float32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    codes, exps = dequant.quantize_bf16_split(dev(x))
+    got = model.grouped_gemm_split([dev(p) for p, _ in mats], [dev(s) for _, s in mats], rows, cols, codes, exps, dev(offsets)).cpu().numpy()
+    xin = bf16_round(x).astype(np.float64)
+    for e, (p, s) in enumerate(mats):
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        if r1 > r0:
+            Wd = oracle.mxfp4_dequant(p, s, rows, cols).astype(np.float64)
+            want = xin[r0:r1] @ Wd.T
+            # the block-scaled instruction keeps fewer bits of a step's 128 products than a chain of f32 additions would:
+            # 1e-5 over a group, single rows up to a few times that
+            assert rel_l2(got[r0:r1], want) <= 1.5e-5, e
+            assert max(rel_l2(got[i], want[i - r0]) for i in range(r0, r1)) <= 4e-5, e
+    with pytest.raises(Exception, match="512"):
+        model.grouped_gemm_split([dev(mats[0][0])], [dev(mats[0][1])], rows, 256, codes, exps, dev(offsets[:2]))
+
+
+_BF16_MFMA_SCRIPT = r"""
+import sys
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests")
+import numpy as np, oracle
+from gpu_util import dev, rel_l2
+from microkimi_amd import model, workloads
+T, topk, ne, d, inter = 70, 2, 3, 1024, 512
+rng = np.random.default_rng(5)
+host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e), workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(ne)]
+table = oracle.ExpertTable([h[0] for h in host], [h[1] for h in host], [h[2] for h in host], d, inter)
+x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+ids = np.stack([rng.permutation(ne)[:topk] for _ in range(T)]).astype(np.uint32)
+wts = rng.random((T, topk)).astype(np.float32)
+pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+got = model.moe_prefill(experts, dev(ids.astype(np.int32)), dev(wts), dev(x), bf16=True).cpu().numpy()
+want = oracle.moe_prefill(table, ids, wts, x, round_mxfp8=3)
+print("RESULT", rel_l2(got, want), int(np.isfinite(got).all()))
+"""
+
+
+def test_moe_prefill_bf16_on_the_bf16_matrix_instruction():
+    # MK_PREFILL_BF16_MFMA=1 (read once per process, hence a process of its own): the same section on
+    # v_mfma_f32_16x16x32_bf16 instead of the two-term form, against the same oracle
+    import os
+    import subprocess
+    import sys
+    torch_cuda()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, MK_PREFILL_BF16_MFMA="1")
+    r = subprocess.run([sys.executable, "-c", _BF16_MFMA_SCRIPT, root], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = [l for l in r.stdout.splitlines() if l.startswith("RESULT")][-1].split()
+    assert float(line[1]) <= 3e-4 and int(line[2]) == 1, line
+
+
 def bf16_round(a):
     """bfloat16, round to nearest even, of an f32 array (as f32 values)."""
     b = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
@@ -510,6 +621,11 @@ def test_config4_full_size_expert_section():
     print(f"config 4 full size, f32 mode: worst token row vs the pure-f32 reference path {worst_exact:.2e}")
     print(f"config 4 full size, bf16 mode: worst token row vs the bf16-input oracle {worst_bf16:.2e}, vs the pure-f32 reference path {worst_bf16_f32:.2e}")
     assert worst <= 2e-3
-    assert worst_bf16 <= 3e-4 and worst_bf16_f32 <= 6e-3
+    # bf16 mode against the oracle on bf16-rounded rows: what is left is activation values whose bfloat16 rounding falls
+    # the other way (one such value moves its row by 2^-9 of that value).  The gate and up rows carry 5e-6 of arithmetic
+    # noise here (the block-scaled matrix instruction adds into its accumulator by truncation) where the bfloat16 matrix
+    # instruction (MK_PREFILL_BF16_MFMA=1) carries 3e-7, so more values fall the other way: 4.3e-4 against 6.3e-5
+    # measured.  The distance to the f32 reference, which is the rounding to bfloat16 itself, is the same for both: 1.7e-3.
+    assert worst_bf16 <= 8e-4 and worst_bf16_f32 <= 3e-3
     assert worst_exact <= 1e-5
     assert worst_f32 < 0.06  # the e4m3 rounding of the activations: reported, not a parity claim
