@@ -678,17 +678,24 @@ def bench_gemm(torch):
                                  "ms": ms4, "tok_s": T / (ms4 * 1e-3), "tflops": fl3 / (ms4 * 1e-3) / 1e12,
                                  "mfma_frac_fp32_peak": fl3 / (ms4 * 1e-3) / 1e12 / 157.3,
                                  "finite": bool(torch.isfinite(out).all().item())}
-    # and with bfloat16 activations (exact weights, bf16 matrix instruction)
+    # and with bfloat16 activations (exact weights; every bfloat16 value as two e4m3 terms on the block-scaled matrix
+    # instruction, or the bf16 matrix instruction with MK_PREFILL_BF16_MFMA=1)
 
     def step5():
         model.moe_prefill(experts, ids_d, wts_d, x_d, out=out, bf16=True)
 
     ms5 = time_region(torch, step5, 5, warmup=2)
-    res["expert_section_bf16"] = {"workload": "the same section, mk_dev_moe_prefill_bf16: group, gather + bf16, gate + up (one launch), activation + bf16, down, combine",
+    bf16_mfma = os.environ.get("MK_PREFILL_BF16_MFMA", "0") not in ("", "0")
+    res["expert_section_bf16"] = {"workload": "the same section, mk_dev_moe_prefill_bf16: group, gather + bf16 "
+                                              + ("(bf16 matrix instruction), gate + up (one launch), activation + bf16, down, combine" if bf16_mfma else
+                                                 "as two e4m3 terms, gate + up + SwiGLU + bf16 as two terms (one launch, block-scaled matrix "
+                                                 "instruction, two instructions a step), down, combine"),
                                   "ms": ms5, "tok_s": T / (ms5 * 1e-3), "tflops": fl3 / (ms5 * 1e-3) / 1e12,
-                                  "mfma_frac_bf16_peak": fl3 / (ms5 * 1e-3) / 1e12 / 2500.0, "weight_bytes": used * per_expert,
-                                  "weight_gbs": used * per_expert / (ms5 * 1e-3) / 1e9, "finite": bool(torch.isfinite(out).all().item()),
-                                  "rel_l2_to_f32_section": dist(out)}
+                                  # useful flops (one product per bfloat16 value) against the peak of the instruction that runs
+                                  ("mfma_frac_bf16_peak" if bf16_mfma else "mfma_frac_fp8_peak"): fl3 / (ms5 * 1e-3) / 1e12 / (2500.0 if bf16_mfma else 5000.0),
+                                  "weight_bytes": used * per_expert, "weight_gbs": used * per_expert / (ms5 * 1e-3) / 1e9,
+                                  "hbm_frac": used * per_expert / (ms5 * 1e-3) / 1e9 / 8000.0,
+                                  "finite": bool(torch.isfinite(out).all().item()), "rel_l2_to_f32_section": dist(out)}
     # BASELINE states this configuration in bf16: the bf16 section leads, the other two arithmetics stand beside it with
     # their distance to the f32 section's result (which the parity tests hold within 1e-5 of the CPU oracle)
     res["lead"] = {"section": "expert_section_bf16", "ms": ms5, "tok_s": T / (ms5 * 1e-3), "dtype": "bf16 activations, exact MXFP4 weights, f32 sums",
