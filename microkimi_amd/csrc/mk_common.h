@@ -316,7 +316,9 @@ __device__ __forceinline__ void mk_bf16_split8(const float (&v)[8], uint32_t (&h
         al = fmaxf(al, mk_dpp<0x4E>(al));
     }
     auto encode = [](const float (&x)[8], float amax, uint32_t (&codes)[2], uint32_t &exp_byte) {
-        int e = mk_ceil_log2f(fmaxf(amax, 1e-30f) / 448.0f);
+        // the smallest e with amax <= 448 * 2^e, from the bits of amax = m * 2^k: k - 8, one more when m > 1.75
+        const uint32_t ab = __float_as_uint(amax);
+        int e = (int)(ab >> 23) - 127 - 8 + ((ab & 0x7FFFFFu) > 0x600000u ? 1 : 0);
         e = max(-127, min(127, e));
         exp_byte = (uint32_t)(e + 127);
         const float inv = mk_scale_from_byte(254u - exp_byte);  // 2^-e, exact

@@ -129,22 +129,25 @@ __global__ __launch_bounds__(GROUP_WAVES * 64) void prefill_group_kernel(const i
     }
     __syncthreads();
     for (int e = threadIdx.x; e <= n_experts; e += blockDim.x) offsets[e] = eoff[e];
-    for (int i0 = wave * C; i0 < min((wave + 1) * C, P); i0 += 64) {
+    // bits an expert id takes: the lanes of a chunk that hold the same id are found with one ballot per bit
+    int nbits = 1;
+    while ((1 << nbits) < n_experts) nbits++;
+    const int i_end = min((wave + 1) * C, P);
+    int e_next = wave * C + lane < P ? ids[wave * C + lane] : -1;  // (the next chunk's ids are asked for a chunk ahead)
+    for (int i0 = wave * C; i0 < i_end; i0 += 64) {
         const int i = i0 + lane;
-        const int e = i < P ? ids[i] : -1;
-        const bool valid = e >= 0 && e < n_experts;
+        const int e = e_next;
+        e_next = (i0 + 64 < i_end && i + 64 < P) ? ids[i + 64] : -1;
+        const bool valid = i < P && e >= 0 && e < n_experts;
         if (i < P && !valid) pos[i] = -1;
-        // rank of the lane among the lanes of this chunk that hold the same expert, and the size of that group:
-        // one pass over the 64 lanes (scalar broadcast of each lane's key), no serial walk over the distinct keys
-        int rank = 0, same = 0;
-        const int key = valid ? e : -1 - lane;  // invalid lanes match nobody
-#pragma unroll 8
-        for (int j = 0; j < 64; j++) {
-            const int kj = __builtin_amdgcn_readlane(key, j);
-            const int eq = kj == key ? 1 : 0;
-            same += eq;
-            rank += (j < lane) ? eq : 0;
+        // rank of the lane among the lanes of this chunk that hold the same expert, and the size of that group
+        unsigned long long same_mask = __ballot(valid);
+        for (int b = 0; b < nbits; b++) {
+            const bool bit = (e >> b) & 1;
+            const unsigned long long m = __ballot(valid && bit);
+            same_mask &= bit ? m : ~m;
         }
+        const int same = __popcll(same_mask), rank = __popcll(same_mask & ((1ull << lane) - 1ull));
         int start = 0;
         if (valid) start = eoff[e] + mine[e];  // every lane reads before any lane of this wave advances the counter
         __builtin_amdgcn_wave_barrier();       // ... also in the compiler's schedule: the reads above stay above the update
