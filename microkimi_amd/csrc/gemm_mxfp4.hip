@@ -121,7 +121,7 @@ constexpr int KT_STEPS = 4;
 constexpr int a_stride(bool two = false) { return (two ? 1024 : 512) + 32; }
 constexpr int a_codes_bytes(int mc, bool two = false) { return 16 * mc * a_stride(two); }
 constexpr int a_wsc_off(int mc, bool two = false) { return a_codes_bytes(mc, two) + 16 * mc * (two ? 32 : 16); }  // codes, then the scale bytes per token,
-constexpr int a_buf_bytes(int mc, bool two = false) { return a_wsc_off(mc, two) + 256 * 16; }  // then the K tile's 16 scale bytes of the 256 weight rows
+constexpr int a_buf_bytes(int mc, bool two = false, int nw = 4) { return a_wsc_off(mc, two) + 64 * nw * 16; }  // then the K tile's 16 scale bytes of the workgroup's weight rows
 
 // One launch covers n_mats (1 or 2) weight matrices per group that share the activation rows (gate and up): matrix m
 // of group e is packed_ptrs[m][e], its result goes to out[m].
@@ -228,17 +228,21 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // two matrix instructions per step against the same weight registers into the same accumulators, nothing else changes.
 // The products are exact and the sums f32, so this is the bfloat16 GEMM (apart from values more than 2^13 below their
 // block's largest, whose last bits fall off the e4m3 grid) at the streaming rate of the MXFP8 one.
-template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false, bool TWO = false>
+// NW: waves of the workgroup (4, or 8 for large groups: 512 weight rows share one staged activation tile, which halves the
+// activation bytes a CU fetches per FLOP -- the pass for large groups is bound by what a CU can load, about 30 B/ns).
+template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false, bool TWO = false, int NW = 4>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds, const uint8_t *scales_t, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr,
                                           const uint8_t *scales3_t = nullptr) {
     static_assert(!GU || (FULL && PIN && !DEEP && MC <= 2), "the gate/up form exists for the small-group pass");
     static_assert(!TWO || (FULL && PIN && !DEEP && MC <= 2), "the two-term form exists for the small-group pass");
+    static_assert(NW == 4 || (NW == 8 && !GU && !TWO), "eight waves: the plain pass only");
     constexpr int AW = TWO ? 2 : 1, AS = a_stride(TWO);
+    constexpr int NTH = 64 * NW, STG_N = 2 * MC * AW * 4 / NW;  // threads; 16-byte chunks of the activation tile per thread
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
-    const int row0 = GU ? rb * 128 + wave * 32 : rb * 256 + wave * 64;
+    const int row0 = GU ? rb * 128 + wave * 32 : rb * NTH + wave * 64;
     // first row of the wave's row tile rt
     auto tile_row = [&](int rt) { return GU ? row0 + (rt & 1) * 16 : row0 + rt * 16; };
     // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
@@ -276,17 +280,17 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // tile: thread i fetches row i's once.  Fetched by the lanes that use them (a lane per row, four lanes of a
     // row the same 16 bytes) they were 4 of a wave's 29 loads per K tile and about half of its vector-cache
     // accesses: a 16-byte load whose lanes sit in 16 different lines is looked up once per lane and pass.
-    mk_i4 st[2 * MC * AW], ste, stw;
+    mk_i4 st[STG_N], ste, stw;
     // (gate/up form: thread i is row slot (wave i / 64, row tile (i / 16) % 4, row i % 16) of the workgroup)
-    const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * 256 + tid;
+    const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * NTH + tid;
     const bool ws_tiles = scales_t != nullptr;  // (uniform)
     const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? (ws_tiles ? scales3_t : scales3) : (ws_tiles ? scales_t : scales);
     const uint32_t ws_r = (uint32_t)min(ws_row, a.rows - 1);
     const uint32_t wsoff = ws_tiles ? ws_r * 16u : ws_r * (uint32_t)nb, ws_step = ws_tiles ? (uint32_t)a.rows * 16u : 16u;
-    uint32_t coff[2 * MC * AW];  // the host checks that tokens x cols (x 2) stays below 2^32
+    uint32_t coff[STG_N];  // the host checks that tokens x cols (x 2) stays below 2^32
 #pragma unroll
-    for (int k = 0; k < 2 * MC * AW; k++) {
-        const int i = tid + 256 * k;
+    for (int k = 0; k < STG_N; k++) {
+        const int i = tid + NTH * k;
         coff[k] = (uint32_t)min(base + i / (32 * AW), tok1 - 1) * (uint32_t)(cols * AW) + (i % (32 * AW)) * 16;
     }
     // (thread i: token i / AW, exponent row i % AW)
@@ -294,22 +298,22 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     auto stage_load = [&](int kt) {
         const uint32_t ku = (uint32_t)__builtin_amdgcn_readfirstlane(min(kt, ktiles - 1));
 #ifdef MK_GEMM_FP4_PROBE
-        constexpr int STG = MC >= 4 ? MC : 2 * MC;  // (half the bytes a token row has in a K tile)
+        constexpr int STG = MC >= 4 ? STG_N / 2 : STG_N;  // (half the bytes a token row has in a K tile)
 #else
-        constexpr int STG = 2 * MC;
+        constexpr int STG = STG_N;
 #endif
 #pragma unroll
-        for (int k = 0; k < STG * AW; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * (512 * AW));
+        for (int k = 0; k < STG; k++) st[k] = mk_ldg128_off(a.codes, coff[k] + ku * (512 * AW));
         ste = mk_ldg128_off(a.exps, eoff + ku * (16 * AW));
         stw = mk_ldg128_off(ws_base, wsoff + ku * ws_step);
     };
     auto stage_store = [&](uint8_t *buf) {
 #pragma unroll
-        for (int k = 0; k < 2 * MC * AW; k++) {
+        for (int k = 0; k < STG_N; k++) {
 #ifdef MK_GEMM_FP4_PROBE
-            if (MC >= 4 && k >= MC) break;
+            if (MC >= 4 && k >= STG_N / 2) break;
 #endif
-            const int i = tid + 256 * k;
+            const int i = tid + NTH * k;
             *reinterpret_cast<mk_i4 *>(buf + (i / (32 * AW)) * AS + (i % (32 * AW)) * 16) = st[k];
         }
         if (tid < 16 * MC * AW) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC, TWO) + tid * 16) = ste;
@@ -440,7 +444,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, NW);
             stage_load(kt + 1);
             if constexpr (PIN && FULL && MC >= 4) {
                 // large groups: two row tiles per read of the activation operands (93-109 -> 82-95 us on 8 experts x 512 tokens)
@@ -466,7 +470,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 }
             }
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, NW));
             __syncthreads();
         }
     } else {
@@ -477,7 +481,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, NW);
             stage_load(kt + 1);
             load_unit(wb, kt, 1);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
@@ -495,7 +499,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             compute_unit(wb, 3, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, NW));
             __syncthreads();
         }
     }
@@ -589,8 +593,8 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 // Two instantiations share the grid: groups of up to 32 tokens (the prefill
 // case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
 // workgroup whose group belongs to the other one exits.
-template <int MC, bool TWO = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
+template <int MC, bool TWO = false, int NW = 4>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
     // the plain order the workgroups of one group land on all of them and each fetches the group's activation rows for
@@ -629,7 +633,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         // the 64-token passes of a group are dealt to gridDim.y workgroups: a few large groups still fill the chip
 #pragma unroll 1
         for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
-            gemm_pass<MC, true, false, true, true>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
+            gemm_pass<MC, true, false, true, true, false, false, NW>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
     }
 }
 
@@ -664,16 +668,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     }
 }
 
-template <int MC, bool TWO = false>
-int launch_stream(const GemmArgs &a, size_t m, hipStream_t st) {
+template <int MC, bool TWO = false, int NW = 4>
+int launch_stream(GemmArgs a, size_t m, hipStream_t st) {
     // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
     // average group size (one per 64 tokens, at most 16); a workgroup without a pass exits at once.
     unsigned passes = 1;
     if (MC == 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
+    a.row_blocks = (a.rows + 64 * NW - 1) / (64 * NW);
     const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO>), 2 * a_buf_bytes(MC, TWO));
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW>), 2 * a_buf_bytes(MC, TWO, NW));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO>), grid, dim3(256), 2 * a_buf_bytes(MC, TWO), st, a);
+    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW>), grid, dim3(64 * NW), 2 * a_buf_bytes(MC, TWO, NW), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
 }
 
@@ -711,7 +716,7 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         a.row_blocks = (int)row_blocks;
         if (two) return launch_stream<2, true>(a, m, (hipStream_t)stream);
         int st = launch_stream<2>(a, m, (hipStream_t)stream);
-        if (st == MK_OK && m > 32) st = launch_stream<4>(a, m, (hipStream_t)stream);
+        if (st == MK_OK && m > 32) st = MK_TUNE("MK_GEMM_LARGE_WAVES", 8) == 8 ? launch_stream<4, false, 8>(a, m, (hipStream_t)stream) : launch_stream<4>(a, m, (hipStream_t)stream);
         return st;
     }
     MK_REQUIRE(!two, "the two-term form needs the streaming kernel's shapes");
