@@ -121,7 +121,7 @@ constexpr int KT_STEPS = 4;
 constexpr int a_stride(bool two = false) { return (two ? 1024 : 512) + 32; }
 constexpr int a_codes_bytes(int mc, bool two = false) { return 16 * mc * a_stride(two); }
 constexpr int a_wsc_off(int mc, bool two = false) { return a_codes_bytes(mc, two) + 16 * mc * (two ? 32 : 16); }  // codes, then the scale bytes per token,
-constexpr int a_buf_bytes(int mc, bool two = false, int nw = 4) { return a_wsc_off(mc, two) + 64 * nw * 16; }  // then the K tile's 16 scale bytes of the workgroup's weight rows
+constexpr int a_buf_bytes(int mc, bool two = false, int wg_rows = 256) { return a_wsc_off(mc, two) + wg_rows * 16; }  // then the K tile's 16 scale bytes of the workgroup's weight rows
 
 // One launch covers n_mats (1 or 2) weight matrices per group that share the activation rows (gate and up): matrix m
 // of group e is packed_ptrs[m][e], its result goes to out[m].
@@ -230,19 +230,23 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
 // block's largest, whose last bits fall off the e4m3 grid) at the streaming rate of the MXFP8 one.
 // NW: waves of the workgroup (4, or 8 for large groups: 512 weight rows share one staged activation tile, which halves the
 // activation bytes a CU fetches per FLOP -- the pass for large groups is bound by what a CU can load, about 30 B/ns).
-template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false, bool TWO = false, int NW = 4>
+// RT: 16-row tiles a wave owns (4; 2 with eight token tiles for large groups: 32 rows x 128 tokens a wave keeps the same 64
+// accumulator registers and moves 0.8 x the bytes per FLOP of 64 rows x 64 tokens).
+template <int MC, bool FULL, bool NT, bool PIN, bool DEEP = false, bool GU = false, bool TWO = false, int NW = 4, int RT = 4>
 __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *packed, const uint8_t *scales, float *out, int rb, int base, int tok1,
                                           uint8_t *lds, const uint8_t *scales_t, const uint8_t *packed3 = nullptr, const uint8_t *scales3 = nullptr,
                                           const uint8_t *scales3_t = nullptr) {
     static_assert(!GU || (FULL && PIN && !DEEP && MC <= 2), "the gate/up form exists for the small-group pass");
     static_assert(!TWO || (FULL && PIN && !DEEP && MC <= 2), "the two-term form exists for the small-group pass");
     static_assert(NW == 4 || (NW == 8 && !GU && !TWO), "eight waves: the plain pass only");
+    static_assert(RT == 4 || (RT == 2 && DEEP && PIN && FULL && !GU && !TWO), "two row tiles a wave: the deep pass only");
+    constexpr int WG_ROWS = 16 * RT * NW;
     constexpr int AW = TWO ? 2 : 1, AS = a_stride(TWO);
     constexpr int NTH = 64 * NW, STG_N = 2 * MC * AW * 4 / NW;  // threads; 16-byte chunks of the activation tile per thread
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, kb = lane >> 4;
     const int cols = a.cols, nb = cols / 32, ktiles = cols / 512;
-    const int row0 = GU ? rb * 128 + wave * 32 : rb * NTH + wave * 64;
+    const int row0 = GU ? rb * 128 + wave * 32 : rb * WG_ROWS + wave * (16 * RT);
     // first row of the wave's row tile rt
     auto tile_row = [&](int rt) { return GU ? row0 + (rt & 1) * 16 : row0 + rt * 16; };
     // this lane's weight row in each of the wave's four row tiles (clamped; stores are guarded)
@@ -252,9 +256,9 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // of all 16 rows, lane (kb, n) reading bytes 16 kb .. of row n (every line is then requested by two loads).
     static_assert(KT_STEPS == 4, "two lines of 128 bytes per row and K tile");
     const int r3 = lane >> 3, c8 = lane & 7;
-    uint32_t woff[4][FULL ? 2 : 1];
+    uint32_t woff[RT][FULL ? 2 : 1];
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++) {
+    for (int rt = 0; rt < RT; rt++) {
         if constexpr (FULL) {
 #pragma unroll
             for (int h = 0; h < 2; h++) woff[rt][h] = (uint32_t)min(tile_row(rt) + 8 * h + r3, a.rows - 1) * (uint32_t)(cols / 2) + c8 * 16;
@@ -282,7 +286,8 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // accesses: a 16-byte load whose lanes sit in 16 different lines is looked up once per lane and pass.
     mk_i4 st[STG_N], ste, stw;
     // (gate/up form: thread i is row slot (wave i / 64, row tile (i / 16) % 4, row i % 16) of the workgroup)
-    const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * NTH + tid;
+    // (two row tiles a wave: the workgroup has fewer rows than threads, the upper threads fetch a row again and store nothing)
+    const int ws_row = GU ? rb * 128 + (tid >> 6) * 32 + ((tid >> 4) & 1) * 16 + (tid & 15) : rb * WG_ROWS + min(tid, WG_ROWS - 1);
     const bool ws_tiles = scales_t != nullptr;  // (uniform)
     const uint8_t *ws_base = (GU && ((tid >> 5) & 1)) ? (ws_tiles ? scales3_t : scales3) : (ws_tiles ? scales_t : scales);
     const uint32_t ws_r = (uint32_t)min(ws_row, a.rows - 1);
@@ -317,16 +322,16 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             *reinterpret_cast<mk_i4 *>(buf + (i / (32 * AW)) * AS + (i % (32 * AW)) * 16) = st[k];
         }
         if (tid < 16 * MC * AW) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC, TWO) + tid * 16) = ste;
-        *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC, TWO) + tid * 16) = stw;
+        if (WG_ROWS >= NTH || tid < WG_ROWS) *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC, TWO) + tid * 16) = stw;
     };
-    mk_f4 acc[4][MC];
+    mk_f4 acc[RT][MC];
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++)
+    for (int rt = 0; rt < RT; rt++)
 #pragma unroll
         for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto mma_unit = [&](const mk_i4 *w, int rt, const uint8_t *buf) {
-        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC, TWO) + (wave * 64 + rt * 16 + n) * 16);
+        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16);
 #pragma unroll
         for (int c = 0; c < MC; c++) {
             const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * (16 * AW));
@@ -363,7 +368,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf) {
         // the scale bytes are read one at a time where they are used: held as 16-byte rows they cost the registers that
         // make the difference between two waves per SIMD with and without a spill
-        const uint8_t *sc0 = buf + a_wsc_off(MC, TWO) + (wave * 64 + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
+        const uint8_t *sc0 = buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
 #pragma unroll
         for (int c = 0; c < MC; c++) {
             const uint8_t *ae = buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 16 + kb;
@@ -435,21 +440,21 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     if constexpr (DEEP) {
         // Four register blocks, one per row tile: the unit of row tile rt for K tile kt + 1 is requested as soon as the
         // unit of K tile kt has been used, three units of matrix work ahead of its use.
-        mk_i4 w4[4][KT_STEPS];
+        mk_i4 w4[RT][KT_STEPS];
 #pragma unroll
-        for (int rt = 0; rt < 4; rt++) load_unit(w4[rt], 0, rt);
+        for (int rt = 0; rt < RT; rt++) load_unit(w4[rt], 0, rt);
         stage_load(0);
         __syncthreads();  // the previous pass (if any) has finished with the LDS buffers
         stage_store(lds);
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, NW);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, WG_ROWS);
             stage_load(kt + 1);
             if constexpr (PIN && FULL && MC >= 4) {
                 // large groups: two row tiles per read of the activation operands (93-109 -> 82-95 us on 8 experts x 512 tokens)
 #pragma unroll
-                for (int rt = 0; rt < 4; rt += 2) {
+                for (int rt = 0; rt < RT; rt += 2) {
                     __builtin_amdgcn_sched_barrier(0);
                     exchange_in_place(w4[rt]);
                     exchange_in_place(w4[rt + 1]);
@@ -462,7 +467,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 }
             } else {
 #pragma unroll
-                for (int rt = 0; rt < 4; rt++) {
+                for (int rt = 0; rt < RT; rt++) {
                     if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
                     compute_unit(w4[rt], rt, buf);
                     if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
@@ -470,7 +475,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 }
             }
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, NW));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, WG_ROWS));
             __syncthreads();
         }
     } else {
@@ -481,7 +486,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         __syncthreads();
 #pragma unroll 1
         for (int kt = 0; kt < ktiles; kt++) {
-            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, NW);
+            const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, WG_ROWS);
             stage_load(kt + 1);
             load_unit(wb, kt, 1);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
@@ -499,7 +504,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
             compute_unit(wb, 3, buf);
             if constexpr (PIN) __builtin_amdgcn_sched_barrier(0);
-            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, NW));
+            stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, WG_ROWS));
             __syncthreads();
         }
     }
@@ -567,7 +572,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         return;
     }
 #pragma unroll
-    for (int rt = 0; rt < 4; rt += 2) {
+    for (int rt = 0; rt < RT; rt += 2) {
         if constexpr (PIN) {
 #pragma unroll
             for (int c = 0; c < MC; c++) store_tile_pair<NT>(out, a.rows, base + c * 16, tok1, row0 + rt * 16, n, kb, acc[rt][c], acc[rt + 1][c]);
@@ -593,7 +598,7 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
 // Two instantiations share the grid: groups of up to 32 tokens (the prefill
 // case; one or two token tiles) and larger ones, in passes of 64 tokens.  A
 // workgroup whose group belongs to the other one exits.
-template <int MC, bool TWO = false, int NW = 4>
+template <int MC, bool TWO = false, int NW = 4, int RT = 4>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void mxfp4_grouped_gemm_stream_kernel(GemmArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // Workgroup -> (group, matrix, row block).  Consecutive workgroup ids go round the 8 XCDs, each with its own L2: with
@@ -613,7 +618,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int m = r / a.row_blocks, rb = r % a.row_blocks;
     const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
     const int count = tok1 - tok0;
-    if (count <= 0 || (!TWO && (count <= 32 ? 2 : 4) != MC)) return;
+    if (count <= 0 || (!TWO && (count <= 32) != (MC == 2))) return;
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
     const uint8_t *scales_t = a.scales_t_ptrs[m] ? mk_uniform_ptr(a.scales_t_ptrs[m][e]) : nullptr;
@@ -633,7 +638,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         // the 64-token passes of a group are dealt to gridDim.y workgroups: a few large groups still fill the chip
 #pragma unroll 1
         for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
-            gemm_pass<MC, true, false, true, true, false, false, NW>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
+            gemm_pass<MC, true, false, true, true, false, false, NW, RT>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
     }
 }
 
@@ -668,17 +673,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     }
 }
 
-template <int MC, bool TWO = false, int NW = 4>
+template <int MC, bool TWO = false, int NW = 4, int RT = 4>
 int launch_stream(GemmArgs a, size_t m, hipStream_t st) {
     // Large groups: the group sizes live on the device, so the number of workgroups per (group, row block) follows the
     // average group size (one per 64 tokens, at most 16); a workgroup without a pass exits at once.
     unsigned passes = 1;
-    if (MC == 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
-    a.row_blocks = (a.rows + 64 * NW - 1) / (64 * NW);
+    if (MC >= 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
+    constexpr int WG_ROWS = 16 * RT * NW;
+    a.row_blocks = (a.rows + WG_ROWS - 1) / WG_ROWS;
     const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
-    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW>), 2 * a_buf_bytes(MC, TWO, NW));
+    const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW, RT>), 2 * a_buf_bytes(MC, TWO, WG_ROWS));
     if (s != MK_OK) return s;
-    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW>), grid, dim3(64 * NW), 2 * a_buf_bytes(MC, TWO, NW), st, a);
+    hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW, RT>), grid, dim3(64 * NW), 2 * a_buf_bytes(MC, TWO, WG_ROWS), st, a);
     return mk_launch_status("mxfp4_grouped_gemm_stream");
 }
 
@@ -716,7 +722,11 @@ int mk_mxfp4_grouped_gemm_n(int n_mats, const uint8_t *const *const *packed_ptrs
         a.row_blocks = (int)row_blocks;
         if (two) return launch_stream<2, true>(a, m, (hipStream_t)stream);
         int st = launch_stream<2>(a, m, (hipStream_t)stream);
-        if (st == MK_OK && m > 32) st = MK_TUNE("MK_GEMM_LARGE_WAVES", 8) == 8 ? launch_stream<4, false, 8>(a, m, (hipStream_t)stream) : launch_stream<4>(a, m, (hipStream_t)stream);
+        if (st == MK_OK && m > 32) {
+            const int form = MK_TUNE("MK_GEMM_LARGE_FORM", 2);  // 0: 4 waves x 64 rows x 64 tokens; 1: 8 waves x 64 x 64; 2: 8 waves x 32 rows x 128 tokens
+            st = form == 2 ? launch_stream<8, false, 8, 2>(a, m, (hipStream_t)stream)
+                 : form == 1 ? launch_stream<4, false, 8>(a, m, (hipStream_t)stream) : launch_stream<4>(a, m, (hipStream_t)stream);
+        }
         return st;
     }
     MK_REQUIRE(!two, "the two-term form needs the streaming kernel's shapes");
