@@ -27,6 +27,7 @@
 #include <algorithm>
 
 #include "mk_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -365,12 +366,13 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     };
     // Two row tiles against one read of the activation operands (large groups: with four token tiles the LDS reads of a
     // unit, 32 KB per wave, take longer than its 16 matrix instructions; shared by two units they take half)
-    auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf) {
+    auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf, auto c_begin, auto c_end) {
+        constexpr int C0 = decltype(c_begin)::value, C1 = decltype(c_end)::value;  // token tiles [C0, C1)
         // the scale bytes are read one at a time where they are used: held as 16-byte rows they cost the registers that
         // make the difference between two waves per SIMD with and without a spill
         const uint8_t *sc0 = buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
 #pragma unroll
-        for (int c = 0; c < MC; c++) {
+        for (int c = C0; c < C1; c++) {
             const uint8_t *ae = buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 16 + kb;
             const uint8_t *arow = buf + (c * 16 + n) * AS + kb * 16;
 #pragma unroll
@@ -451,14 +453,40 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         for (int kt = 0; kt < ktiles; kt++) {
             const uint8_t *buf = lds + (kt & 1) * a_buf_bytes(MC, TWO, WG_ROWS);
             stage_load(kt + 1);
-            if constexpr (PIN && FULL && MC >= 4) {
+            if constexpr (PIN && FULL && RT == 2) {
+                // One pair of row tiles: its weights are in use until the K tile's last matrix instruction, so the next K
+                // tile's are asked for half way, into the registers the staged activation chunks leave when they are
+                // stored (the other LDS buffer is free since the last barrier); left to the end of the K tile the loads
+                // had nothing but the barrier in front of their first use.
+                mk_i4 wn[2][KT_STEPS];
+                __builtin_amdgcn_sched_barrier(0);
+                exchange_in_place(w4[0]);
+                exchange_in_place(w4[1]);
+                mma_unit2(w4[0], w4[1], 0, buf, std::integral_constant<int, 0>{}, std::integral_constant<int, MC / 2>{});
+                pin_acc(0);
+                pin_acc(1);
+                __builtin_amdgcn_sched_barrier(0);
+                stage_store(lds + ((kt + 1) & 1) * a_buf_bytes(MC, TWO, WG_ROWS));
+                __builtin_amdgcn_sched_barrier(0);
+                load_unit(wn[0], kt + 1, 0);
+                load_unit(wn[1], kt + 1, 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_unit2(w4[0], w4[1], 0, buf, std::integral_constant<int, MC / 2>{}, std::integral_constant<int, MC>{});
+                pin_acc(0);
+                pin_acc(1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < KT_STEPS; j++) w4[0][j] = wn[0][j], w4[1][j] = wn[1][j];
+                __syncthreads();
+                continue;
+            } else if constexpr (PIN && FULL && MC >= 4) {
                 // large groups: two row tiles per read of the activation operands (93-109 -> 82-95 us on 8 experts x 512 tokens)
 #pragma unroll
                 for (int rt = 0; rt < RT; rt += 2) {
                     __builtin_amdgcn_sched_barrier(0);
                     exchange_in_place(w4[rt]);
                     exchange_in_place(w4[rt + 1]);
-                    mma_unit2(w4[rt], w4[rt + 1], rt, buf);
+                    mma_unit2(w4[rt], w4[rt + 1], rt, buf, std::integral_constant<int, 0>{}, std::integral_constant<int, MC>{});
                     pin_acc(rt);
                     pin_acc(rt + 1);
                     __builtin_amdgcn_sched_barrier(0);
