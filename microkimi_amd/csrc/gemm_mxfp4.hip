@@ -633,20 +633,31 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // the plain order the workgroups of one group land on all of them and each fetches the group's activation rows for
     // itself (prefill gate GEMM: 235 MB of 2.45 GB).  When the group count allows it, XCD x takes the groups x, x + 8, ...
     // and runs all workgroups of a group itself.
-    const int per_group = a.n_mats * a.row_blocks;
+    const int per_group = a.n_mats * a.row_blocks, n_items = a.n_groups * per_group;
+    if constexpr (!TWO && MC >= 4) {
+        // The launch for large groups follows every launch for small ones, because the group sizes live on the device.
+        // When no group has more than 32 rows (the prefill shape) it has nothing to do: found here, once per workgroup,
+        // and the grid is a few hundred workgroups that walk the items -- workgroups of this size go one to a CU, and
+        // one per item, each leaving at its own count, took 12-20 us to drain.
+        int big = 0;
+        for (int g = threadIdx.x; g < a.n_groups; g += blockDim.x) big |= (a.offsets[g + 1] - a.offsets[g] > 32) ? 1 : 0;
+        if (!__syncthreads_or(big)) return;
+    }
+#pragma unroll 1
+    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
     int e, r;
     if (a.n_groups % 8 == 0) {
-        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        const int x = item & 7, j = item >> 3;
         e = x + 8 * (j / per_group);
         r = j % per_group;
     } else {
-        e = blockIdx.x / per_group;
-        r = blockIdx.x % per_group;
+        e = item / per_group;
+        r = item % per_group;
     }
     const int m = r / a.row_blocks, rb = r % a.row_blocks;
     const int tok0 = a.offsets[e], tok1 = a.offsets[e + 1];
     const int count = tok1 - tok0;
-    if (count <= 0 || (!TWO && (count <= 32) != (MC == 2))) return;
+    if (count <= 0 || (!TWO && (count <= 32) != (MC == 2))) continue;
     const uint8_t *packed = mk_uniform_ptr(a.packed_ptrs[m][e]);
     const uint8_t *scales = mk_uniform_ptr(a.scales_ptrs[m][e]);
     const uint8_t *scales_t = a.scales_t_ptrs[m] ? mk_uniform_ptr(a.scales_t_ptrs[m][e]) : nullptr;
@@ -668,6 +679,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         for (int base = tok0 + 16 * MC * (int)blockIdx.y; base < tok1; base += 16 * MC * (int)gridDim.y)
             gemm_pass<MC, true, false, true, true, false, false, NW, RT>(a, packed, scales, out, rb, base, tok1, lds, scales_t);
     }
+    }  // items
 }
 
 // The gate/up form: workgroup -> (group, block of 128 rows), both matrices.  Groups of up to 16 tokens take one token
@@ -709,7 +721,8 @@ int launch_stream(GemmArgs a, size_t m, hipStream_t st) {
     if (MC >= 4) passes = (unsigned)std::min<size_t>(16, std::max<size_t>(1, (m / a.n_groups + 16 * MC - 1) / (16 * MC)));
     constexpr int WG_ROWS = 16 * RT * NW;
     a.row_blocks = (a.rows + WG_ROWS - 1) / WG_ROWS;
-    const dim3 grid((unsigned)(a.n_groups * a.n_mats * a.row_blocks), passes);
+    const size_t n_items = (size_t)a.n_groups * a.n_mats * a.row_blocks;
+    const dim3 grid((unsigned)(MC >= 4 ? std::min<size_t>(n_items, 512) : n_items), passes);  // (512: a multiple of the 8 XCDs)
     const int s = mk_lds_opt_in(reinterpret_cast<const void *>(mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW, RT>), 2 * a_buf_bytes(MC, TWO, WG_ROWS));
     if (s != MK_OK) return s;
     hipLaunchKernelGGL((mxfp4_grouped_gemm_stream_kernel<MC, TWO, NW, RT>), grid, dim3(64 * NW), 2 * a_buf_bytes(MC, TWO, WG_ROWS), st, a);
