@@ -358,6 +358,26 @@ def test_moe_prefill_with_and_without_the_tile_ordered_scale_bytes(T, topk, n_ex
             assert np.array_equal(ma[k].view(np.uint32), mb[k].view(np.uint32)), k
 
 
+def test_moe_prefill_bf16_non_finite_hidden_value_gives_nan_rows():
+    # a hidden value that is not finite makes the token's row NaN (its e4m3 code is the NaN), the other tokens' rows stay as they were
+    from microkimi_amd import model, workloads
+    T, topk, n_experts, d, inter = 20, 2, 3, 512, 512
+    rng = np.random.default_rng(9)
+    host = [(workloads.mxfp4_matrix(4, "w1", inter, d, e), workloads.mxfp4_matrix(4, "w3", inter, d, e),
+             workloads.mxfp4_matrix(4, "w2", d, inter, e)) for e in range(n_experts)]
+    pk = lambda k: [(dev(h[k][0]), dev(h[k][1])) for h in host]
+    experts = model.PackedExperts(pk(0), pk(1), pk(2), d, inter)
+    x = (rng.standard_normal((T, d)) * 0.05).astype(np.float32)
+    ids = dev(np.stack([rng.permutation(n_experts)[:topk] for _ in range(T)]).astype(np.int32))
+    wts = dev(rng.random((T, topk)).astype(np.float32))
+    clean = model.moe_prefill(experts, ids, wts, dev(x), bf16=True).cpu().numpy()
+    x[3, 17], x[11, 400] = np.inf, np.nan
+    got = model.moe_prefill(experts, ids, wts, dev(x), bf16=True).cpu().numpy()
+    assert np.isnan(got[3]).all() and np.isnan(got[11]).all()
+    others = [t for t in range(T) if t not in (3, 11)]
+    assert np.array_equal(got[others].view(np.uint32), clean[others].view(np.uint32))
+
+
 def test_moe_prefill_bf16_refuses_other_shapes():
     # d or inter not in multiples of 512, or a layer with VQ1 experts: MK_ERR_UNSUPPORTED, nothing computed
     from microkimi_amd import model, workloads
