@@ -63,6 +63,18 @@ def test_argument_checks_need_no_device():
     assert st == -1 and b"batch" in _lib.lib.mk_last_error()
 
 
+def test_argument_checks_of_the_two_term_and_scale_layout_entry_points():
+    # shapes these entry points do not take are refused before anything is launched
+    from microkimi_amd import _lib
+    lib, p16 = _lib.lib, ctypes.c_void_p(16)
+    assert lib.mk_dev_mxfp4_scales_by_tile(p16, 8, 768, p16, None) == -1 and b"512" in lib.mk_last_error()
+    assert lib.mk_dev_mxfp4_scales_by_tile(p16, 8, 1024, ctypes.c_void_p(8), None) == -1 and b"aligned" in lib.mk_last_error()
+    assert lib.mk_dev_quantize_bf16_split(p16, 2, 256, p16, p16, None) == -1 and b"512" in lib.mk_last_error()
+    assert lib.mk_dev_quantize_bf16_split(None, 2, 512, p16, p16, None) == -1
+    st = lib.mk_dev_mxfp4_grouped_gemm_split(p16, p16, 1, 64, 256, p16, p16, p16, 4, p16, None)
+    assert st == -4 and b"512" in lib.mk_last_error()   # MK_ERR_UNSUPPORTED
+
+
 def test_off_switch_returns_no_device_before_anything_else():
     # mk_set_enabled(0): every status-returning entry point answers MK_ERR_NO_DEVICE, also for arguments that it would
     # otherwise reject (the switch is tested first) and for device-level calls (whose launch would otherwise be tried)
