@@ -110,8 +110,8 @@ __global__ __launch_bounds__(256) void mxfp4_grouped_gemm_kernel(const uint8_t *
 //     bytes in flight;
 //   * the 16 scale bytes per weight row and K tile are fetched once per
 //     workgroup (thread i: row i, one 16-byte load) and staged in LDS with the
-//     activation tile; a lane reads its row's 16 bytes from there and shifts out
-//     the byte of its step and K block.
+//     activation tile, transposed to [K block][step]; a lane reads the dword of
+//     its row and K block from there and shifts out the byte of its step.
 //
 // Loads take the form "uniform base + 32-bit lane offset".  The K offset goes
 // through readfirstlane, which hides the loop counter from the induction
@@ -188,6 +188,23 @@ __device__ __forceinline__ void store_tile_pair(float *out, int rows, int t0, in
     const mk_f4 first = __builtin_bit_cast(mk_f4, fi), second = __builtin_bit_cast(mk_f4, si);
     store_tile<NT>(out, rows, t0 + (n & 7), tok1, row + (up ? 16 : 0) + kb * 4, first);
     store_tile<NT>(out, rows, t0 + 8 + (n & 7), tok1, row + (up ? 16 : 0) + kb * 4, second);
+}
+
+// The 16 scale bytes a row has in a K tile, [step][K block of the step], as [K block][step]: a lane (K block kb) then finds
+// the bytes of its four steps in ONE dword of LDS, and the byte of a step is a shift by a constant.
+__device__ __forceinline__ mk_i4 mk_scale_bytes_by_kb(const mk_i4 v) {
+    const uint32_t d0 = (uint32_t)v[0], d1 = (uint32_t)v[1], d2 = (uint32_t)v[2], d3 = (uint32_t)v[3];
+    // v_perm_b32(hi, lo, sel): selector bytes 0-3 pick from lo, 4-7 from hi
+    const uint32_t a01 = __builtin_amdgcn_perm(d1, d0, 0x05010400u);  // d0.b0 d1.b0 d0.b1 d1.b1
+    const uint32_t b01 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);  // d0.b2 d1.b2 d0.b3 d1.b3
+    const uint32_t a23 = __builtin_amdgcn_perm(d3, d2, 0x05010400u);
+    const uint32_t b23 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+    mk_i4 o;
+    o[0] = (int)__builtin_amdgcn_perm(a23, a01, 0x05040100u);  // kb 0: d0.b0 d1.b0 d2.b0 d3.b0
+    o[1] = (int)__builtin_amdgcn_perm(a23, a01, 0x07060302u);  // kb 1
+    o[2] = (int)__builtin_amdgcn_perm(b23, b01, 0x05040100u);  // kb 2
+    o[3] = (int)__builtin_amdgcn_perm(b23, b01, 0x07060302u);  // kb 3
+    return o;
 }
 
 // PIN: the loads and the matrix instructions stay where the source puts them.  Left alone, instruction selection places
@@ -322,8 +339,8 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
             const int i = tid + NTH * k;
             *reinterpret_cast<mk_i4 *>(buf + (i / (32 * AW)) * AS + (i % (32 * AW)) * 16) = st[k];
         }
-        if (tid < 16 * MC * AW) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC, TWO) + tid * 16) = ste;
-        if (WG_ROWS >= NTH || tid < WG_ROWS) *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC, TWO) + tid * 16) = stw;
+        if (tid < 16 * MC * AW) *reinterpret_cast<mk_i4 *>(buf + a_codes_bytes(MC, TWO) + tid * 16) = mk_scale_bytes_by_kb(ste);
+        if (WG_ROWS >= NTH || tid < WG_ROWS) *reinterpret_cast<mk_i4 *>(buf + a_wsc_off(MC, TWO) + tid * 16) = mk_scale_bytes_by_kb(stw);
     };
     mk_f4 acc[RT][MC];
 #pragma unroll
@@ -332,10 +349,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
         for (int c = 0; c < MC; c++) acc[rt][c] = mk_f4{0.0f, 0.0f, 0.0f, 0.0f};
 
     auto mma_unit = [&](const mk_i4 *w, int rt, const uint8_t *buf) {
-        const mk_i4 sc = *reinterpret_cast<const mk_i4 *>(buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16);
+        const uint32_t sc = *reinterpret_cast<const uint32_t *>(buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb * 4);
 #pragma unroll
         for (int c = 0; c < MC; c++) {
-            const mk_i4 ae = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * (16 * AW));
+            const uint32_t ae = *reinterpret_cast<const uint32_t *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * (16 * AW) + kb * 4);
             const uint8_t *arow = buf + (c * 16 + n) * AS + kb * 16;
 #pragma unroll
             for (int s = 0; s < KT_STEPS; s++) {
@@ -343,23 +360,22 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + s * 128 + 64);
                 const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                 const mk_i8v bv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
-                const int asb = (int)((uint32_t)ae[s] >> (8 * kb));  // the instruction reads byte 0
-                const int wsb = (int)((uint32_t)sc[s] >> (8 * kb));
+                const int asb = (int)(ae >> (8 * s));  // the instruction reads byte 0
+                const int wsb = (int)(sc >> (8 * s));
                 if constexpr (PIN)
                     acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[rt][c], 4 /*M: fp4 weights*/, 0 /*N: fp8 rows*/, 0, wsb, 0, asb);
                 else
                     acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[rt][c], 0 /*M: fp8 rows*/, 4 /*N: fp4 weights*/, 0, asb, 0, wsb);
             }
             if constexpr (TWO) {  // the second term of every value against the same weight registers
-                const mk_i4 ael = *reinterpret_cast<const mk_i4 *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 32 + 16);
+                const uint32_t ael = *reinterpret_cast<const uint32_t *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 32 + 16 + kb * 4);
 #pragma unroll
                 for (int s = 0; s < KT_STEPS; s++) {
                     const mk_i4 a0 = *reinterpret_cast<const mk_i4 *>(arow + 512 + s * 128);
                     const mk_i4 a1 = *reinterpret_cast<const mk_i4 *>(arow + 512 + s * 128 + 64);
                     const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                     const mk_i8v bv = {w[s][0], w[s][1], w[s][2], w[s][3], 0, 0, 0, 0};
-                    acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[rt][c], 4, 0, 0, (int)((uint32_t)sc[s] >> (8 * kb)), 0,
-                                                                                  (int)((uint32_t)ael[s] >> (8 * kb)));
+                    acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[rt][c], 4, 0, 0, (int)(sc >> (8 * s)), 0, (int)(ael >> (8 * s)));
                 }
             }
         }
@@ -368,12 +384,12 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
     // unit, 32 KB per wave, take longer than its 16 matrix instructions; shared by two units they take half)
     auto mma_unit2 = [&](const mk_i4 *w0, const mk_i4 *w1, int rt, const uint8_t *buf, auto c_begin, auto c_end) {
         constexpr int C0 = decltype(c_begin)::value, C1 = decltype(c_end)::value;  // token tiles [C0, C1)
-        // the scale bytes are read one at a time where they are used: held as 16-byte rows they cost the registers that
-        // make the difference between two waves per SIMD with and without a spill
-        const uint8_t *sc0 = buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb, *sc1 = sc0 + 256;
+        // (a lane's scale bytes of the K tile are one dword each: staged as [K block][step], see mk_scale_bytes_by_kb)
+        const uint32_t sc0 = *reinterpret_cast<const uint32_t *>(buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb * 4);
+        const uint32_t sc1 = *reinterpret_cast<const uint32_t *>(buf + a_wsc_off(MC, TWO) + (wave * (16 * RT) + rt * 16 + n) * 16 + kb * 4 + 256);
 #pragma unroll
         for (int c = C0; c < C1; c++) {
-            const uint8_t *ae = buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 16 + kb;
+            const uint32_t ae = *reinterpret_cast<const uint32_t *>(buf + a_codes_bytes(MC, TWO) + (c * 16 + n) * 16 + kb * 4);
             const uint8_t *arow = buf + (c * 16 + n) * AS + kb * 16;
 #pragma unroll
             for (int s = 0; s < KT_STEPS; s++) {
@@ -388,10 +404,10 @@ __device__ __forceinline__ void gemm_pass(const GemmArgs &a, const uint8_t *pack
                 const mk_i8v av = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                 constexpr int AFMT = 0;
 #endif
-                const int asb = ae[s * 4];
+                const int asb = (int)(ae >> (8 * s));
                 const mk_i8v b0 = {w0[s][0], w0[s][1], w0[s][2], w0[s][3], 0, 0, 0, 0}, b1 = {w1[s][0], w1[s][1], w1[s][2], w1[s][3], 0, 0, 0, 0};
-                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b0, av, acc[rt][c], 4, AFMT, 0, (int)sc0[s * 4], 0, asb);
-                acc[rt + 1][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b1, av, acc[rt + 1][c], 4, AFMT, 0, (int)sc1[s * 4], 0, asb);
+                acc[rt][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b0, av, acc[rt][c], 4, AFMT, 0, (int)(sc0 >> (8 * s)), 0, asb);
+                acc[rt + 1][c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b1, av, acc[rt + 1][c], 4, AFMT, 0, (int)(sc1 >> (8 * s)), 0, asb);
             }
         }
     };
